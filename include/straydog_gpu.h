@@ -1,0 +1,118 @@
+/* The part of Straydog's GPU C ABI that this MI355X (gfx950) attention library implements.
+ *
+ * Every function keeps the name, argument order, argument meaning and error convention of the
+ * reference declaration it replaces (cited per function as gpu/straydog_gpu.h:LINE of the reference
+ * checkout, with the reference body it stands in for), so the Rust host's bindings call it unchanged.
+ * Conventions (reference gpu/straydog_gpu.h:1-5): a negative int or a null pointer is a failure that
+ * sd_error() then describes for the calling thread; other int results are 0 or a query's answer;
+ * handles are opaque; no exception crosses this boundary.  Ops are queued on the device's one compute
+ * stream and return at once; only reads (sd_buffer_read, sd_download) wait for the stream.  Every
+ * pointer an op takes must lie inside one allocation of the same device (reference gpu/ops.hpp:4-26).
+ *
+ * The attention *stages* that the reference reaches only through whole-layer span calls, and the
+ * synthetic paged/batched configurations, are in straydog_gpu_ext.h (sdx_*).
+ */
+#ifndef STRAYDOG_GPU_H
+#define STRAYDOG_GPU_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- Errors and devices ---- */
+/* reference straydog_gpu.h:17 (gpu/core.hpp:172): the calling thread's last failure text, valid until its next call. */
+const char* sd_error(void);
+/* reference straydog_gpu.h:18 */
+int sd_device_count(void);
+/* reference straydog_gpu.h:21: name (NUL-terminated, cut to capacity), free and total bytes of device `ordinal`. */
+int sd_device_info(int ordinal, char* name, size_t capacity, uint64_t* free_bytes, uint64_t* total_bytes);
+/* reference straydog_gpu.h:35-36 (gpu/kernels.cpp:3511-3614): a device handle with a VRAM budget in bytes that every
+ * allocation is charged against; one compute stream. */
+void* sd_create(int ordinal, uint64_t budget);
+void sd_destroy(void* handle);
+/* reference straydog_gpu.h:37: bytes allocated so far and the budget. */
+int sd_memory(void* handle, uint64_t* used, uint64_t* budget);
+
+/* ---- Allocations and transfers ---- */
+/* reference straydog_gpu.h:44 (gpu/host_io.hpp:81-109): a new allocation holding a copy of `data`; the caller's
+ * memory is free on return, the bytes land in stream order. */
+void* sd_upload(void* handle, const void* data, uint64_t bytes);
+/* reference straydog_gpu.h:49: an allocation whose bytes arrive later (only its 64-byte tail is zeroed). */
+void* sd_allocate(void* handle, uint64_t bytes);
+/* reference straydog_gpu.h:58: stage caller memory into all of an allocation. */
+int sd_write(void* handle, void* pointer, const void* data, uint64_t bytes);
+/* reference straydog_gpu.h:64-68 */
+int sd_release(void* handle, void* pointer);
+int sd_allocation_bytes(void* handle, const void* pointer, uint64_t* bytes);
+int sd_zero(void* handle, void* pointer);
+/* reference straydog_gpu.h:69 (gpu/host_io.hpp:113-140): copy out and wait for the stream. */
+int sd_download(void* handle, void* pointer, void* output, uint64_t bytes);
+/* reference straydog_gpu.h:152-156 (gpu/kernels.cpp:4555-4592): a zero-filled buffer (synchronised before return),
+ * writes staged in stream order, reads that wait for the stream. */
+void* sd_buffer(void* handle, uint64_t bytes);
+int sd_buffer_write(void* handle, void* buffer, uint64_t offset, const void* data, uint64_t bytes);
+int sd_buffer_read(void* handle, const void* buffer, uint64_t offset, void* output, uint64_t bytes);
+
+/* ---- K/V format ---- */
+/* reference straydog_gpu.h:113 (gpu/kernels.cpp:4266-4274): the bytes of a K/V row of the Qwen state, 512 (FP16) or
+ * 272 (Q8_0: 256 int8 then eight FP16 block scales, gpu/core.hpp:397-403).  Default 272. */
+int sd_kv_format(void* handle, uint32_t row);
+
+/* ---- Attention ops ---- */
+/* reference straydog_gpu.h:528 (gpu/kernels.cpp:4387-4419, kernels :79-165): selection-list attention of `steps` rows at
+ * positions base.. over the Qwen state (4 planes of `context` rows: K head 0, K head 1, V head 0, V head 1).  Host
+ * pointers: input = [steps*24*256 q | steps*2*256 k | steps*2*256 v | steps*selected indices as floats | steps counts],
+ * output = steps*24*256 floats.  The rows' K/V are written first; scale 1/16; an index is attended when
+ * 0 <= index <= base+step and index < context. */
+int sd_attention_sequence(void* handle, void* state, uint64_t context, uint64_t base, uint64_t steps, uint64_t selected,
+                          const float* input, uint64_t input_count, float* output, uint64_t output_count);
+/* reference straydog_gpu.h:451 (gpu/token_mixing.hpp:652-693, kernels :356-520): causal grouped-query attention of
+ * q (rows x heads x dim) at `positions` over FP32 caches keys/values (context x kv_heads x dim), each row up to its
+ * position (clipped to the cache), times sigmoid(gate) when given.  scratch: rows x heads x splits x (dim + 2) floats,
+ * splits = min(64, max(1, 256 / (rows x heads))). */
+int sd_op_attention(void* handle, const float* q, const float* keys, const float* values, uint64_t context, const int32_t* positions,
+                    uint64_t rows, uint64_t heads, uint64_t kv_heads, uint64_t dim, float scale, const float* gate, float* scratch,
+                    uint64_t scratch_bytes, float* out);
+/* reference straydog_gpu.h:385 (gpu/kernels.cpp:5311-5476, kernels gpu/ops.hpp:1240-1677): latent attention.  Each query
+ * attends the window rows of `raw` ending at its position (position p in row p % raw_rows) and the compressed rows
+ * `selected` lists (-1: none), keys = values, with a per-head sink in the max and the denominator.  `compressed` may
+ * carry bit 0 (BF16 rows, gpu/ops.hpp:1205-1214).  rope_dims rotates q's last values by positions * frequencies on the
+ * way in and the output back.  scratch is optional and unused by this implementation. */
+int sd_op_sparse_attention(void* handle, const float* q, const float* raw, uint64_t raw_rows, const int32_t* positions, uint64_t window,
+                           const float* compressed, uint64_t compressed_rows, const int32_t* selected, uint64_t selections,
+                           const float* sinks, uint64_t rows, uint64_t heads, uint64_t dim, float scale, uint64_t rope_dims,
+                           const float* frequencies, float* scratch, uint64_t scratch_bytes, float* out);
+/* reference straydog_gpu.h:271 (gpu/kernels.cpp:4942-4956, kernel gpu/ops.hpp:107-120): the last rope_dims values of each of
+ * a row's `vectors` vectors of `width` rotated in adjacent pairs by positions[row] * frequencies[pair] (sine and cosine in
+ * double); inverse: by the angle times -1. */
+int sd_op_rope(void* handle, float* x, uint64_t rows, uint64_t vectors, uint64_t width, uint64_t rope_dims, const int32_t* positions,
+               const float* frequencies, int inverse);
+/* reference straydog_gpu.h:407 (gpu/kernels.cpp:5478-5485, kernel gpu/ops.hpp:1681-1694): per-channel softmax pooling. */
+int sd_op_compress(void* handle, const float* kv, const float* gate, uint64_t groups, uint64_t ratio, uint64_t dim, float* out);
+/* reference straydog_gpu.h:408 (gpu/kernels.cpp:5487-5499, kernel gpu/ops.hpp:1700-1739): scores[row][g] =
+ * scale * sum_h relu(q[row][h] . keys[g]) * weights[row][h] for g < visible[row], -inf beyond, in the canonical
+ * order (fmaf over the columns in order, each head's term rounded, heads added in order).  keys may be BF16-tagged. */
+int sd_op_index_scores(void* handle, const float* q, const float* keys, const float* weights, const int32_t* visible, uint64_t rows,
+                       uint64_t groups, uint64_t heads, uint64_t dim, float scale, float* scores);
+/* reference straydog_gpu.h:409 (gpu/kernels.cpp:5669-5676, gpu/ops.hpp:1766-1941): each row's k highest scores' indices in
+ * ascending index order; ties keep the lower index; -inf never kept; -1 fills empty slots. */
+int sd_op_top_k(void* handle, const float* scores, uint64_t rows, uint64_t groups, uint64_t k, int32_t* out);
+/* reference straydog_gpu.h:414 (gpu/kernels.cpp:5524-5540, gpu/ops.hpp:1942-1975): a row's candidate blocks. */
+int sd_op_index_candidates(void* handle, const float* scores, const int32_t* visible, uint64_t rows, uint64_t groups, uint64_t blocks,
+                           uint64_t block, int32_t* out, float* scratch, uint64_t scratch_bytes);
+/* reference straydog_gpu.h:419 (gpu/kernels.cpp:5561-5618, gpu/ops.hpp:1993-2230): rope of q (q itself unchanged),
+ * sd_op_index_scores and sd_op_top_k in one call: the same scores and indices, bit for bit. */
+int sd_op_index_select(void* handle, const float* q, const float* keys, const float* weights, const int32_t* visible, uint64_t rows,
+                       uint64_t groups, uint64_t heads, uint64_t dim, float scale, uint64_t rope_dims, const int32_t* positions,
+                       const float* frequencies, float* scores, uint64_t k, int32_t* out, const int32_t* candidates, uint64_t blocks,
+                       uint64_t block);
+/* reference straydog_gpu.h:459 (gpu/token_mixing.hpp:728-744): out = x as BF16, nearest even, a NaN stays a NaN. */
+int sd_op_to_bf16(void* handle, const float* x, uint64_t count, void* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,83 @@
+/* Extension entry points of the MI355X attention library (sdx_*).
+ *
+ * The reference reaches its decode / verify / prefill attention only inside whole-layer span calls
+ * (sd_decode_span, sd_verify_span, sd_prefill_span: gpu/straydog_gpu.h:526,536,571 of the reference), which also
+ * run GEMVs, hyper-connections and MoE.  These entry points expose the attention *stage* of those spans on its
+ * own, generalised to a paged, batched K/V cache, with the same conventions as straydog_gpu.h: device-resident
+ * arguments (positions are read on the device so a recorded graph replays without new host arguments, as
+ * gpu/qsa_decode.hpp:1-4 does), ops queued on the handle's stream, negative result = failure described by
+ * sd_error().  Each one cites the reference code whose arithmetic it stands in for.
+ */
+#ifndef STRAYDOG_GPU_EXT_H
+#define STRAYDOG_GPU_EXT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* A paged K/V cache.  Page p holds, for page_tokens consecutive positions, 2*kv_heads planes: the keys of K/V head
+ * h in plane h, its values in plane kv_heads + h (the reference's plane order, gpu/core.hpp:397-403, inside a page).
+ * A plane is page_tokens rows of row_bytes: Q8_0 (row_bytes = dim + dim/16: dim int8 then dim/32 FP16 block scales,
+ * the reference's kv_row_q8 rule, 272 bytes at dim 256 and 136 at dim 128) or FP16 (row_bytes = 2*dim).
+ * Byte offset of (page, plane, token) = ((page * 2*kv_heads + plane) * page_tokens + token) * row_bytes.
+ * page_tokens is a multiple of 32; dim is 128 or 256. */
+typedef struct sdx_kv_pool {
+    void* pages;
+    uint64_t page_count;
+    uint32_t page_tokens;
+    uint32_t kv_heads;
+    uint32_t dim;
+    uint32_t row_bytes;
+} sdx_kv_pool;
+
+/* Append K/V rows (reference write_attention_kv + kv_encode, gpu/kernels.cpp:58-98): row r of sequence s goes to
+ * position positions[s] + r through page_table[s * table_stride + position / page_tokens].  keys/values are
+ * [seqs][span][kv_heads][dim], FP32 (input_f16 = 0) or FP16 (1).  Q8_0 encoding is bit-exact kv_encode. */
+int sdx_kv_write(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
+                 const void* keys, const void* values, int input_f16, uint64_t seqs, uint64_t span);
+
+/* Causal grouped-query attention over the paged cache: the attention step of a decode (span 1), a speculative
+ * verify (span <= 8) or a prefill chunk (any span), i.e. qsa_decode_parts/qsa_decode_merge, qsa_flash and
+ * qsa_prompt_attention of the reference (gpu/sparse_attention_compute.hpp:41-170, :176-279,
+ * gpu/qsa_prompt_attention.hpp:47-213) with the dense selection 0..position.  Row r of sequence s attends
+ * positions t <= positions[s] + r.  q/out are [seqs][span][heads][dim], FP32 or FP16 each; softmax and sums in
+ * FP32; K/V and probabilities enter the matrix cores as FP16.  max_context bounds positions[s] + span (it sizes the
+ * launch; positions themselves stay on the device).  scratch holds the split partial results:
+ * sdx_paged_attention_scratch bytes. */
+uint64_t sdx_paged_attention_scratch(uint64_t seqs, uint64_t span, uint64_t heads, uint64_t dim, uint64_t max_context);
+int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride,
+                        const int32_t* positions, uint64_t max_context, const void* q, int q_f16, uint64_t seqs, uint64_t span,
+                        uint64_t heads, float scale, void* out, int out_f16, void* scratch, uint64_t scratch_bytes);
+
+/* Top-k indexed sparse attention over BF16 latent K/V for a batch of sequences (one decode row each):
+ * stage 1+2 = sd_op_index_scores + sd_op_top_k per sequence (gpu/ops.hpp:1700-1739, 1766-1941) with each sequence's own
+ * keys [batch][groups][dim] BF16; q_index [batch][heads][dim] BF16; weights [batch][heads] FP32; visible [batch].
+ * scores (optional, [batch][groups] FP32) receives the canonical scores; indices [batch][k] int32, ascending,
+ * ties to the lowest index, -1 padding: bit-exact. */
+int sdx_index_top_k(void* handle, const void* q_index, const void* keys, const float* weights, const int32_t* visible, uint64_t batch,
+                    uint64_t groups, uint64_t heads, uint64_t dim, float scale, float* scores, uint64_t k, int32_t* indices);
+/* stage 3 = op_sparse_attention_kernel's arithmetic (gpu/ops.hpp:1240-1297) without window or sink, keys = the
+ * selected rows' kdim columns, values = their first vdim columns: q [batch][heads][kdim] BF16, latents
+ * [batch][groups][kdim] BF16, selected [batch][k] (-1 skipped), out [batch][heads][vdim] FP32. */
+int sdx_latent_attention(void* handle, const void* q, const void* latents, const int32_t* selected, uint64_t batch, uint64_t groups,
+                         uint64_t k, uint64_t heads, uint64_t kdim, uint64_t vdim, float scale, float* out);
+
+/* Harness helpers: wait for the handle's stream; events on that stream (ids >= 2) and the time between two;
+ * counter-based N(0,1) / U[lo,hi) fills for synthetic benchmark inputs; a plain copy kernel for measuring the
+ * HBM ceiling and calibrating byte counters. */
+int sdx_synchronize(void* handle);
+int64_t sdx_event_record(void* handle);
+int sdx_event_elapsed(void* handle, int64_t begin, int64_t end, float* milliseconds);
+int sdx_events_clear(void* handle);
+int sdx_device_compute_units(void* handle);
+int sdx_fill_normal(void* handle, void* out, uint64_t count, uint64_t seed, int out_kind /* 0 f32, 1 f16, 2 bf16 */);
+int sdx_fill_uniform(void* handle, float* out, uint64_t count, uint64_t seed, float lo, float hi);
+int sdx_copy(void* handle, void* target, const void* source, uint64_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

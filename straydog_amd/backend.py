@@ -1,0 +1,196 @@
+"""Host-side mirror of the reference's safe wrappers over the C ABI for the attention path:
+`Backend` / `Buffer` of crates/straydog-engine/src/gpu.rs:735 and ops.rs:846-886, 1139-1245 (same method
+names, argument order and meaning; a failed call raises with sd_error()'s text, as `check` does in
+crates/straydog-gpu/src/lib.rs:24-43).  Device pointers are plain integers; host data are numpy arrays.
+Everything runs in the HIP library; nothing here computes.
+"""
+import ctypes
+
+import numpy as np
+
+from . import abi
+
+
+class StraydogError(RuntimeError):
+    pass
+
+
+class Buffer:
+    """A zero-filled device allocation (ops.rs Buffer): base address and size."""
+
+    def __init__(self, pointer, size):
+        self.pointer, self.size = pointer, size
+
+    def base(self):
+        return self.pointer
+
+    def at(self, offset_bytes):
+        return self.pointer + offset_bytes
+
+
+def _host(array):
+    return array.ctypes.data_as(ctypes.c_void_p)
+
+
+def tagged_bf16(pointer):
+    """The reference's state_tag: bit 0 marks a BF16 row pointer passed where FP32 is declared (gpu/ops.hpp:1205-1214)."""
+    return pointer | 1
+
+
+class Backend:
+    def __init__(self, ordinal=0, budget=1 << 30, library=None):
+        self.lib = library or abi.load()
+        self.handle = self.lib.sd_create(ordinal, budget)
+        if not self.handle:
+            raise StraydogError(self.error())
+
+    def error(self):
+        text = self.lib.sd_error()
+        return text.decode("utf-8", "replace") if text else ""
+
+    def check(self, code):
+        if code is None or code < 0:
+            raise StraydogError(self.error())
+        return code
+
+    def close(self):
+        if self.handle:
+            self.lib.sd_destroy(self.handle)
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *_):
+        self.close()
+
+    # ---- allocations and transfers -------------------------------------------------
+    def memory(self):
+        used, budget = abi.c_u64(), abi.c_u64()
+        self.check(self.lib.sd_memory(self.handle, ctypes.byref(used), ctypes.byref(budget)))
+        return used.value, budget.value
+
+    def buffer(self, size):
+        pointer = self.lib.sd_buffer(self.handle, size)
+        if not pointer:
+            raise StraydogError(self.error())
+        return Buffer(pointer, size)
+
+    def release(self, buffer):
+        self.check(self.lib.sd_release(self.handle, buffer.pointer))
+
+    def write_buffer(self, buffer, offset, values):
+        values = np.ascontiguousarray(values)
+        self.check(self.lib.sd_buffer_write(self.handle, buffer.pointer, offset, _host(values), values.nbytes))
+
+    def read_buffer(self, buffer, offset, dtype, count):
+        out = np.empty(count, dtype=dtype)
+        self.check(self.lib.sd_buffer_read(self.handle, buffer.pointer, offset, _host(out), out.nbytes))
+        return out
+
+    def upload(self, values):
+        """A buffer holding `values` (the tests' upload helper: buffer + write_buffer)."""
+        values = np.ascontiguousarray(values)
+        buffer = self.buffer(max(values.nbytes, 4))
+        if values.nbytes:
+            self.write_buffer(buffer, 0, values)
+        return buffer
+
+    def synchronize(self):
+        self.check(self.lib.sdx_synchronize(self.handle))
+
+    def kv_format(self, row):
+        self.check(self.lib.sd_kv_format(self.handle, row))
+
+    # ---- reference ops ---------------------------------------------------------------
+    def attention_sequence(self, state, context, base, steps, selected, packed):
+        packed = np.ascontiguousarray(packed, dtype=np.float32)
+        out = np.empty(steps * 24 * 256, dtype=np.float32)
+        self.check(self.lib.sd_attention_sequence(self.handle, state, context, base, steps, selected, _host(packed), packed.size,
+                                                  _host(out), out.size))
+        return out
+
+    def attention(self, q, keys, values, context, positions, rows, heads, kv_heads, dim, scale, gate, scratch, out):
+        self.check(self.lib.sd_op_attention(self.handle, q, keys, values, context, positions, rows, heads, kv_heads, dim, scale,
+                                            gate, scratch.pointer if scratch else None, scratch.size if scratch else 0, out))
+
+    def sparse_attention(self, q, raw, raw_rows, positions, window, compressed, compressed_rows, selected, selections, sinks, rows,
+                         heads, dim, scale, rope_dims, frequencies, scratch, out):
+        self.check(self.lib.sd_op_sparse_attention(self.handle, q, raw, raw_rows, positions, window, compressed, compressed_rows,
+                                                   selected, selections, sinks, rows, heads, dim, scale, rope_dims, frequencies,
+                                                   scratch.pointer if scratch else None, scratch.size if scratch else 0, out))
+
+    def rope(self, x, rows, vectors, width, rope_dims, positions, frequencies, inverse=False):
+        self.check(self.lib.sd_op_rope(self.handle, x, rows, vectors, width, rope_dims, positions, frequencies, int(inverse)))
+
+    def compress(self, kv, gate, groups, ratio, dim, out):
+        self.check(self.lib.sd_op_compress(self.handle, kv, gate, groups, ratio, dim, out))
+
+    def index_scores(self, q, keys, weights, visible, rows, groups, heads, dim, scale, scores):
+        self.check(self.lib.sd_op_index_scores(self.handle, q, keys, weights, visible, rows, groups, heads, dim, scale, scores))
+
+    def top_k(self, scores, rows, groups, k, out):
+        self.check(self.lib.sd_op_top_k(self.handle, scores, rows, groups, k, out))
+
+    def index_candidates(self, scores, visible, rows, groups, blocks, block, out, scratch):
+        self.check(self.lib.sd_op_index_candidates(self.handle, scores, visible, rows, groups, blocks, block, out, scratch.pointer,
+                                                   scratch.size))
+
+    def index_select(self, q, keys, weights, visible, rows, groups, heads, dim, scale, rope, scores, k, out, within=None):
+        rope_dims, positions, frequencies = rope if rope else (0, None, None)
+        candidates, blocks, block = within if within else (None, 0, 0)
+        self.check(self.lib.sd_op_index_select(self.handle, q, keys, weights, visible, rows, groups, heads, dim, scale, rope_dims,
+                                               positions, frequencies, scores, k, out, candidates, blocks, block))
+
+    def to_bf16(self, x, count, out):
+        self.check(self.lib.sd_op_to_bf16(self.handle, x, count, out))
+
+    # ---- paged cache extensions --------------------------------------------------------
+    def kv_pool(self, pages, page_tokens, kv_heads, dim, row_bytes):
+        size = pages * 2 * kv_heads * page_tokens * row_bytes
+        buffer = self.buffer(size)
+        return abi.KvPool(buffer.pointer, pages, page_tokens, kv_heads, dim, row_bytes), buffer
+
+    def kv_write(self, pool, page_table, table_stride, positions, keys, values, input_f16, seqs, span):
+        self.check(self.lib.sdx_kv_write(self.handle, ctypes.byref(pool), page_table, table_stride, positions, keys, values,
+                                         int(input_f16), seqs, span))
+
+    def paged_attention_scratch(self, seqs, span, heads, dim, max_context):
+        return int(self.lib.sdx_paged_attention_scratch(seqs, span, heads, dim, max_context))
+
+    def paged_attention(self, pool, page_table, table_stride, positions, max_context, q, q_f16, seqs, span, heads, scale, out,
+                        out_f16, scratch):
+        self.check(self.lib.sdx_paged_attention(self.handle, ctypes.byref(pool), page_table, table_stride, positions, max_context,
+                                                q, int(q_f16), seqs, span, heads, scale, out, int(out_f16), scratch.pointer,
+                                                scratch.size))
+
+    def index_top_k(self, q_index, keys, weights, visible, batch, groups, heads, dim, scale, scores, k, indices):
+        self.check(self.lib.sdx_index_top_k(self.handle, q_index, keys, weights, visible, batch, groups, heads, dim, scale, scores,
+                                            k, indices))
+
+    def latent_attention(self, q, latents, selected, batch, groups, k, heads, kdim, vdim, scale, out):
+        self.check(self.lib.sdx_latent_attention(self.handle, q, latents, selected, batch, groups, k, heads, kdim, vdim, scale, out))
+
+    # ---- harness helpers ----------------------------------------------------------------
+    def event(self):
+        return self.check(self.lib.sdx_event_record(self.handle))
+
+    def elapsed_ms(self, begin, end):
+        ms = abi.c_float()
+        self.check(self.lib.sdx_event_elapsed(self.handle, begin, end, ctypes.byref(ms)))
+        return ms.value
+
+    def events_clear(self):
+        self.check(self.lib.sdx_events_clear(self.handle))
+
+    def compute_units(self):
+        return self.check(self.lib.sdx_device_compute_units(self.handle))
+
+    def fill_normal(self, out, count, seed, kind=0):
+        self.check(self.lib.sdx_fill_normal(self.handle, out, count, seed, kind))
+
+    def fill_uniform(self, out, count, seed, lo=0.0, hi=1.0):
+        self.check(self.lib.sdx_fill_uniform(self.handle, out, count, seed, lo, hi))
+
+    def copy(self, target, source, size):
+        self.check(self.lib.sdx_copy(self.handle, target, source, size))

@@ -1,0 +1,345 @@
+// Devices, allocations and transfers of the C ABI (reference gpu/kernels.cpp:3511-3614 sd_create, :4555-4592 sd_buffer*,
+// gpu/host_io.hpp:81-180 upload/download/allocate), for one MI355X per handle.
+#include "device.hpp"
+
+#include "../../include/straydog_gpu.h"
+#include "../../include/straydog_gpu_ext.h"
+
+#include <algorithm>
+
+namespace sd {
+
+thread_local std::string last_error;
+
+Device& device(void* handle) {
+    if (!handle) throw std::runtime_error("Straydog device handle is null");
+    Device& d = *static_cast<Device*>(handle);
+    SD_CHECK(hipSetDevice(d.ordinal));
+    return d;
+}
+
+static std::string budget_exceeded(const Device& d, size_t bytes) {
+    const size_t left = d.budget > d.used ? d.budget - d.used : 0;
+    return "Straydog VRAM budget exceeded (" + std::to_string(bytes >> 20) + " MiB asked, " + std::to_string(left >> 20) + " MiB of " +
+           std::to_string(d.budget >> 20) + " MiB left)";
+}
+
+void* allocate(Device& d, size_t bytes, bool zero) {
+    const size_t available = d.budget > d.used ? d.budget - d.used : 0;
+    if (!bytes || bytes > available || allocation_tail > available - bytes) throw std::runtime_error(budget_exceeded(d, bytes));
+    void* pointer = nullptr;
+    SD_CHECK(hipMalloc(&pointer, bytes + allocation_tail));
+    {
+        std::lock_guard<std::mutex> lock(d.mutex);
+        d.allocations.emplace(static_cast<const uint8_t*>(pointer), bytes);
+        d.used += bytes + allocation_tail;
+    }
+    if (zero) SD_CHECK(hipMemsetAsync(pointer, 0, bytes + allocation_tail, d.stream));
+    else SD_CHECK(hipMemsetAsync(static_cast<uint8_t*>(pointer) + bytes, 0, allocation_tail, d.stream));
+    return pointer;
+}
+
+void release(Device& d, void* pointer) {
+    size_t bytes = 0;
+    {
+        std::lock_guard<std::mutex> lock(d.mutex);
+        const auto found = d.allocations.find(static_cast<const uint8_t*>(pointer));
+        if (found == d.allocations.end()) throw std::runtime_error("Straydog release: not an allocation of this device");
+        bytes = found->second;
+        d.allocations.erase(found);
+        d.used -= bytes + allocation_tail;
+    }
+    SD_CHECK(hipStreamSynchronize(d.stream));
+    SD_CHECK(hipFree(pointer));
+}
+
+// Caller memory goes through the page-locked arena a half at a time, so the caller's buffer is free on return and
+// the bytes land in stream order; a half is reused only after the copy that read it has finished.
+void upload(Device& d, void* target, const void* data, size_t bytes) {
+    const size_t half = io_arena_bytes / 2;
+    const uint8_t* from = static_cast<const uint8_t*>(data);
+    uint8_t* to = static_cast<uint8_t*>(target);
+    static thread_local int turn = 0;
+    while (bytes) {
+        const size_t part = std::min(bytes, half);
+        uint8_t* slot = d.arena + (turn & 1) * half;
+        hipEvent_t done = d.events[turn & 1];
+        SD_CHECK(hipEventSynchronize(done));
+        std::memcpy(slot, from, part);
+        SD_CHECK(hipMemcpyAsync(to, slot, part, hipMemcpyHostToDevice, d.stream));
+        SD_CHECK(hipEventRecord(done, d.stream));
+        from += part; to += part; bytes -= part; ++turn;
+    }
+}
+
+void download(Device& d, void* output, const void* source, size_t bytes) {
+    uint8_t* to = static_cast<uint8_t*>(output);
+    const uint8_t* from = static_cast<const uint8_t*>(source);
+    // both halves may hold an upload in flight: wait for the stream once, then the arena is ours
+    SD_CHECK(hipStreamSynchronize(d.stream));
+    while (bytes) {
+        const size_t part = std::min(bytes, io_arena_bytes);
+        SD_CHECK(hipMemcpyAsync(d.arena, from, part, hipMemcpyDeviceToHost, d.stream));
+        SD_CHECK(hipStreamSynchronize(d.stream));
+        std::memcpy(to, d.arena, part);
+        from += part; to += part; bytes -= part;
+    }
+}
+
+void* workspace(Device& d, size_t bytes) {
+    if (bytes <= d.workspace_bytes) return d.workspace;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    SD_CHECK(hipStreamIsCapturing(d.stream, &capturing));
+    if (capturing != hipStreamCaptureStatusNone) throw std::runtime_error("Straydog attention workspace cannot grow while a graph is recorded");
+    if (d.workspace) release(d, d.workspace);
+    d.workspace = nullptr; d.workspace_bytes = 0;
+    const size_t rounded = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+    d.workspace = allocate(d, rounded, true);
+    d.workspace_bytes = rounded;
+    return d.workspace;
+}
+
+void op_span(Device& d, const void* pointer, size_t bytes, const char* what) {
+    const uint8_t* at = static_cast<const uint8_t*>(pointer);
+    std::lock_guard<std::mutex> lock(d.mutex);
+    auto next = d.allocations.upper_bound(at);
+    if (at && next != d.allocations.begin()) {
+        --next;
+        const uint8_t* base = next->first;
+        if (bytes <= next->second && size_t(at - base) <= next->second - bytes) return;
+    }
+    throw std::runtime_error(std::string("Straydog op: ") + what + " is outside this device's allocations");
+}
+
+void op_state_span(Device& d, const void* pointer, size_t count, const char* what) {
+    op_span(d, state_base(pointer), checked_product({uint64_t(count), state_bf16(pointer) ? 2u : 4u}), what);
+}
+
+}  // namespace sd
+
+using namespace sd;
+
+extern "C" {
+
+const char* sd_error(void) { return last_error.c_str(); }
+
+int sd_device_count(void) {
+    int count = 0;
+    const hipError_t error = hipGetDeviceCount(&count);
+    if (error != hipSuccess) { last_error = gpu_error_text(error); (void)hipGetLastError(); return error == hipErrorNoDevice ? 0 : -1; }
+    return count;
+}
+
+int sd_device_info(int ordinal, char* name, size_t capacity, uint64_t* free_bytes, uint64_t* total_bytes) {
+    try {
+        hipDeviceProp_t properties;
+        SD_CHECK(hipGetDeviceProperties(&properties, ordinal));
+        if (name && capacity) { std::strncpy(name, properties.name, capacity - 1); name[capacity - 1] = '\0'; }
+        SD_CHECK(hipSetDevice(ordinal));
+        size_t free_now = 0, total = 0;
+        SD_CHECK(hipMemGetInfo(&free_now, &total));
+        if (free_bytes) *free_bytes = free_now;
+        if (total_bytes) *total_bytes = total;
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+void* sd_create(int ordinal, uint64_t budget) {
+    Device* d = nullptr;
+    try {
+        int count = 0;
+        SD_CHECK(hipGetDeviceCount(&count));
+        if (ordinal < 0 || ordinal >= count) throw std::runtime_error("Straydog device ordinal out of range");
+        SD_CHECK(hipSetDevice(ordinal));
+        hipDeviceProp_t properties;
+        SD_CHECK(hipGetDeviceProperties(&properties, ordinal));
+        if (std::string(properties.gcnArchName).rfind("gfx950", 0) != 0)
+            throw std::runtime_error(std::string("this Straydog attention library is built for gfx950 (MI355X) only; device is ") + properties.gcnArchName);
+        d = new Device;
+        d->ordinal = ordinal;
+        d->budget = size_t(budget);
+        d->compute_units = unsigned(properties.multiProcessorCount);
+        SD_CHECK(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
+        SD_CHECK(hipHostMalloc(reinterpret_cast<void**>(&d->arena), io_arena_bytes, hipHostMallocDefault));
+        d->events.resize(2);
+        for (auto& event : d->events) { SD_CHECK(hipEventCreateWithFlags(&event, hipEventDisableTiming)); SD_CHECK(hipEventRecord(event, d->stream)); }
+        return d;
+    } catch (const std::exception& e) {
+        last_error = e.what();
+        if (d) sd_destroy(d);
+        return nullptr;
+    }
+}
+
+void sd_destroy(void* handle) {
+    if (!handle) return;
+    Device* d = static_cast<Device*>(handle);
+    (void)hipSetDevice(d->ordinal);
+    if (d->stream) (void)hipStreamSynchronize(d->stream);
+    for (const auto& entry : d->allocations) (void)hipFree(const_cast<uint8_t*>(entry.first));
+    for (auto& event : d->events) if (event) (void)hipEventDestroy(event);
+    if (d->arena) (void)hipHostFree(d->arena);
+    if (d->stream) (void)hipStreamDestroy(d->stream);
+    delete d;
+}
+
+int sd_memory(void* handle, uint64_t* used, uint64_t* budget) {
+    try {
+        Device& d = device(handle);
+        if (used) *used = d.used;
+        if (budget) *budget = d.budget;
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+void* sd_upload(void* handle, const void* data, uint64_t bytes) {
+    try {
+        Device& d = device(handle);
+        if (!data) throw std::runtime_error("invalid Straydog upload");
+        void* pointer = allocate(d, size_t(bytes), false);
+        upload(d, pointer, data, size_t(bytes));
+        return pointer;
+    } catch (const std::exception& e) { last_error = e.what(); return nullptr; }
+}
+
+void* sd_allocate(void* handle, uint64_t bytes) {
+    try { return allocate(device(handle), size_t(bytes), false); }
+    catch (const std::exception& e) { last_error = e.what(); return nullptr; }
+}
+
+int sd_write(void* handle, void* pointer, const void* data, uint64_t bytes) {
+    try {
+        Device& d = device(handle);
+        std::unique_lock<std::mutex> lock(d.mutex);
+        const auto found = d.allocations.find(static_cast<const uint8_t*>(pointer));
+        if (!data || found == d.allocations.end() || found->second != bytes) throw std::runtime_error("invalid Straydog write");
+        lock.unlock();
+        upload(d, pointer, data, size_t(bytes));
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sd_release(void* handle, void* pointer) {
+    try { release(device(handle), pointer); return 0; }
+    catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sd_allocation_bytes(void* handle, const void* pointer, uint64_t* bytes) {
+    try {
+        Device& d = device(handle);
+        std::lock_guard<std::mutex> lock(d.mutex);
+        const auto found = d.allocations.find(static_cast<const uint8_t*>(pointer));
+        if (found == d.allocations.end() || !bytes) throw std::runtime_error("Straydog: not an allocation of this device");
+        *bytes = found->second + allocation_tail;
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sd_zero(void* handle, void* pointer) {
+    try {
+        Device& d = device(handle);
+        size_t bytes = 0;
+        {
+            std::lock_guard<std::mutex> lock(d.mutex);
+            const auto found = d.allocations.find(static_cast<const uint8_t*>(pointer));
+            if (found == d.allocations.end()) throw std::runtime_error("Straydog zero: not an allocation of this device");
+            bytes = found->second;
+        }
+        SD_CHECK(hipMemsetAsync(pointer, 0, bytes, d.stream));
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sd_download(void* handle, void* pointer, void* output, uint64_t bytes) {
+    try {
+        Device& d = device(handle);
+        if (!output) throw std::runtime_error("invalid Straydog download");
+        op_span(d, pointer, size_t(bytes), "a downloaded allocation");
+        download(d, output, pointer, size_t(bytes));
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+void* sd_buffer(void* handle, uint64_t bytes) {
+    try {
+        Device& d = device(handle);
+        void* pointer = allocate(d, size_t(bytes), true);
+        // Return only after the zeros land (reference gpu/kernels.cpp:4566-4568).
+        SD_CHECK(hipStreamSynchronize(d.stream));
+        return pointer;
+    } catch (const std::exception& e) { last_error = e.what(); return nullptr; }
+}
+
+int sd_buffer_write(void* handle, void* buffer, uint64_t offset, const void* data, uint64_t bytes) {
+    try {
+        Device& d = device(handle);
+        if (!data || offset > UINT64_MAX - bytes) throw std::runtime_error("invalid Straydog buffer write");
+        op_span(d, static_cast<uint8_t*>(buffer) + offset, size_t(bytes), "a written buffer");
+        upload(d, static_cast<uint8_t*>(buffer) + offset, data, size_t(bytes));
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sd_buffer_read(void* handle, const void* buffer, uint64_t offset, void* output, uint64_t bytes) {
+    try {
+        Device& d = device(handle);
+        if (!output || offset > UINT64_MAX - bytes) throw std::runtime_error("invalid Straydog buffer read");
+        op_span(d, static_cast<const uint8_t*>(buffer) + offset, size_t(bytes), "a read buffer");
+        download(d, output, static_cast<const uint8_t*>(buffer) + offset, size_t(bytes));
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sd_kv_format(void* handle, uint32_t row) {
+    try {
+        Device& d = device(handle);
+        if (row != 512 && row != 272) throw std::runtime_error("invalid Straydog K/V format");
+        d.kv_row = row;
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+// ---- extensions: stream waits and event timing for harnesses ----
+
+int sdx_synchronize(void* handle) {
+    try { Device& d = device(handle); SD_CHECK(hipStreamSynchronize(d.stream)); return 0; }
+    catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int64_t sdx_event_record(void* handle) {
+    try {
+        Device& d = device(handle);
+        hipEvent_t event;
+        SD_CHECK(hipEventCreate(&event));
+        SD_CHECK(hipEventRecord(event, d.stream));
+        d.events.push_back(event);
+        return int64_t(d.events.size() - 1);
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sdx_event_elapsed(void* handle, int64_t begin, int64_t end, float* milliseconds) {
+    try {
+        Device& d = device(handle);
+        if (begin < 2 || end < 2 || size_t(begin) >= d.events.size() || size_t(end) >= d.events.size() || !milliseconds)
+            throw std::runtime_error("invalid Straydog event");
+        SD_CHECK(hipEventSynchronize(d.events[size_t(end)]));
+        SD_CHECK(hipEventElapsedTime(milliseconds, d.events[size_t(begin)], d.events[size_t(end)]));
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sdx_events_clear(void* handle) {
+    try {
+        Device& d = device(handle);
+        SD_CHECK(hipStreamSynchronize(d.stream));
+        while (d.events.size() > 2) { SD_CHECK(hipEventDestroy(d.events.back())); d.events.pop_back(); }
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sdx_device_compute_units(void* handle) {
+    try { return int(device(handle).compute_units); }
+    catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+}  // extern "C"

@@ -1,0 +1,93 @@
+// The device behind an opaque handle: one HIP device, one compute stream, a VRAM budget, and the table of
+// its allocations that every op checks its pointers against.  Mirrors the conventions of the reference's
+// Device (gpu/core.hpp:649-979, check/SD_OP_BEGIN/END :426-435, op_span gpu/ops.hpp:4-26, checked sizes
+// gpu/core.hpp:1415-1429) for the attention entry points only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstring>
+#include <initializer_list>
+#include <map>
+#include <mutex>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace sd {
+
+// Every allocation carries this many spare bytes so an unaligned wide load at its end stays inside it
+// (reference gpu/core.hpp:209-211).
+constexpr size_t allocation_tail = 64;
+// Page-locked staging for uploads and downloads (reference gpu/core.hpp:405: 32 MiB per device).
+constexpr size_t io_arena_bytes = size_t(32) << 20;
+
+extern thread_local std::string last_error;
+
+inline const char* gpu_error_text(hipError_t error) {
+    const char* text = hipGetErrorString(error);
+    return text && *text ? text : "GPU error";
+}
+
+inline void check_at(hipError_t error, const char* file, int line) {
+    if (error == hipSuccess) return;
+    const std::string path(file);
+    throw std::runtime_error(std::string(gpu_error_text(error)) + " (" + path.substr(path.find_last_of("/\\") + 1) + ":" +
+                             std::to_string(line) + ", code " + std::to_string(int(error)) + ")");
+}
+#define SD_CHECK(error) ::sd::check_at((error), __FILE__, __LINE__)
+
+struct Device {
+    int ordinal = 0;
+    hipStream_t stream = nullptr;
+    size_t budget = 0, used = 0;
+    std::map<const uint8_t*, size_t> allocations;   // base -> requested bytes
+    std::mutex mutex;
+    uint8_t* arena = nullptr;                       // page-locked staging, io_arena_bytes
+    uint32_t kv_row = 272;                          // sd_kv_format: 272 (Q8_0) or 512 (FP16)
+    unsigned compute_units = 0;
+    // Workspaces the attention ops own (allocated on first use, outside any graph capture).
+    void* sequence_input = nullptr; size_t sequence_input_bytes = 0;
+    void* sequence_output = nullptr; size_t sequence_output_bytes = 0;
+    void* workspace = nullptr; size_t workspace_bytes = 0;
+    std::vector<hipEvent_t> events;
+};
+
+Device& device(void* handle);                         // sets the HIP device of the handle; throws on null
+void* allocate(Device& d, size_t bytes, bool zero);   // budget-checked hipMalloc (+ tail)
+void release(Device& d, void* pointer);
+void upload(Device& d, void* target, const void* data, size_t bytes);     // caller memory -> device, in stream order
+void download(Device& d, void* output, const void* source, size_t bytes);  // device -> caller memory, waits
+// A workspace of at least `bytes` that lives with the device; grows only outside graph capture.
+void* workspace(Device& d, size_t bytes);
+
+// [pointer, pointer + bytes) must lie inside one live allocation of this device.
+void op_span(Device& d, const void* pointer, size_t bytes, const char* what);
+// The same for a pointer that may carry the BF16 tag in bit 0: `count` values of 2 or 4 bytes.
+void op_state_span(Device& d, const void* pointer, size_t count, const char* what);
+
+inline bool state_bf16(const void* p) { return reinterpret_cast<uintptr_t>(p) & 1u; }
+inline const void* state_base(const void* p) { return reinterpret_cast<const void*>(reinterpret_cast<uintptr_t>(p) & ~uintptr_t(1)); }
+
+inline size_t checked_product(std::initializer_list<uint64_t> factors) {
+    uint64_t total = 1;
+    for (const uint64_t f : factors) {
+        if (f && total > UINT64_MAX / f) throw std::runtime_error("Straydog op: a size overflows");
+        total *= f;
+    }
+    if (total > (uint64_t(1) << 48)) throw std::runtime_error("Straydog op: a size overflows");
+    return size_t(total);
+}
+inline size_t checked_floats(std::initializer_list<uint64_t> factors) { return checked_product({uint64_t(checked_product(factors)), 4}); }
+inline unsigned checked_blocks(size_t count, unsigned threads = 256) {
+    const size_t blocks = (count + threads - 1) / threads;
+    if (!blocks || blocks > 0x7fffffffu) throw std::runtime_error("Straydog op: a launch is out of range");
+    return unsigned(blocks);
+}
+
+}  // namespace sd
+
+// The body of an extern "C" op: the device the handle names, failures as the thread's error text.
+#define SD_OP_BEGIN try { ::sd::Device& value = ::sd::device(handle);
+#define SD_OP_END SD_CHECK(hipGetLastError()); return 0; } catch (const std::exception& e) { ::sd::last_error = e.what(); return -1; }

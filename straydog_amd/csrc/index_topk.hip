@@ -1,0 +1,443 @@
+// The sparse path's indexer: BF16 rounding, compression pooling, rope, indexer scores in the canonical order,
+// radix top-k, candidate blocks, and their fused entry points.
+//   reference: gpu/token_mixing.hpp:728-744 (to_bf16), gpu/ops.hpp:107-120 (rope), :1681-1694 (compress),
+//   :1700-1739 (index scores), :1766-1941 (top-k), :1942-1975 (candidates), gpu/kernels.cpp:5478-5676 (entries).
+// Bit-exactness rules kept here: a score is, per head, a chain of fmaf over the columns in order; the head's term
+// max(dot, 0) * weight is rounded on its own (no contraction with the sum); the terms are added in head order; the
+// scale is applied last.  Top-k compares order-preserving integer keys, keeps the lowest indices among ties and
+// emits ascending indices.
+#include "device.hpp"
+#include "../../include/straydog_gpu.h"
+#include "../../include/straydog_gpu_ext.h"
+
+using namespace sd;
+
+namespace {
+
+__device__ __forceinline__ float bf16_value(uint16_t bits) { return __uint_as_float(uint32_t(bits) << 16); }
+
+__global__ void to_bf16_kernel(const float* x, size_t count, uint16_t* out) {
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) {
+        const uint32_t bits = __float_as_uint(x[i]);
+        out[i] = (bits & 0x7fffffffu) > 0x7f800000u ? uint16_t((bits >> 16) | 0x40u) : uint16_t((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+    }
+}
+
+__global__ void compress_kernel(const float* kv, const float* gate, size_t groups, size_t ratio, size_t dim, float* out) {
+    const size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (index >= groups * dim) return;
+    const size_t group = index / dim, col = index % dim;
+    if (!gate) { out[index] = kv[group * dim + col]; return; }
+    float top = -INFINITY;
+    for (size_t r = 0; r < ratio; ++r) top = fmaxf(top, gate[(group * ratio + r) * dim + col]);
+    float sum = 0.0f, acc = 0.0f;
+    for (size_t r = 0; r < ratio; ++r) {
+        const float w = expf(gate[(group * ratio + r) * dim + col] - top);
+        sum += w;
+        acc += w * kv[(group * ratio + r) * dim + col];
+    }
+    out[index] = acc / sum;
+}
+
+// The last 2 * pairs values of each vector rotated in adjacent pairs by positions[row] * frequencies[pair]
+// (angle, sine and cosine in double).  `from` may differ from `to` (the fused entry leaves q as it was).
+__global__ void rope_kernel(const float* from, float* to, size_t count, size_t vectors, size_t width, size_t pairs, const int32_t* positions,
+                            const float* frequencies, int inverse, int copy_rest) {
+    const size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (copy_rest) {   // one thread per value: plain copy of the unrotated part
+        const size_t values = count;   // here count = rows * vectors * width
+        if (index >= values) return;
+        const size_t col = index % width;
+        if (col < width - 2 * pairs) { to[index] = from[index]; return; }
+        if ((col - (width - 2 * pairs)) & 1) return;
+        const size_t row = index / (vectors * width), pair = (col - (width - 2 * pairs)) / 2;
+        const double angle = double(positions[row]) * double(frequencies[pair]) * (inverse ? -1.0 : 1.0);
+        double s, c;
+        sincos(angle, &s, &c);
+        const double a = from[index], b = from[index + 1];
+        to[index] = float(a * c - b * s);
+        to[index + 1] = float(a * s + b * c);
+        return;
+    }
+    if (index >= count) return;
+    const size_t row = index / (vectors * pairs), rest = index % (vectors * pairs), vector = rest / pairs, pair = rest % pairs;
+    const size_t at = (row * vectors + vector) * width + (width - 2 * pairs) + 2 * pair;
+    const double angle = double(positions[row]) * double(frequencies[pair]) * (inverse ? -1.0 : 1.0);
+    double s, c;
+    sincos(angle, &s, &c);
+    const double a = from[at], b = from[at + 1];
+    to[at] = float(a * c - b * s);
+    to[at + 1] = float(a * s + b * c);
+}
+
+// A row's candidate group `v` (gpu/ops.hpp:1948-1951): groups of its candidate blocks in candidate order.
+__device__ __forceinline__ size_t candidate_group(const int32_t* candidates, size_t block, size_t v, size_t groups) {
+    const int32_t b = candidates[v / block];
+    return b < 0 ? groups : size_t(b) * block + v % block;
+}
+
+// Indexer scores, a thread per scored group.  q is uniform over the workgroup, so its values arrive through
+// scalar loads and every fmaf is (scalar q, vector key, vector sum).  H = 32 or 64 heads are carried at once,
+// the key's columns 32 at a time; each chain still adds its columns in order.
+template<int H, bool BF16>
+__global__ void __launch_bounds__(256) index_scores_kernel(const float* __restrict__ q, const void* __restrict__ keys, size_t key_batch_stride,
+                                                           const float* __restrict__ weights, const int32_t* __restrict__ visible,
+                                                           size_t groups, size_t heads, size_t dim, float scale, float* __restrict__ scores,
+                                                           size_t score_stride, const int32_t* __restrict__ candidates, size_t blocks,
+                                                           size_t block) {
+    const size_t row = blockIdx.y, place = size_t(blockIdx.x) * 256 + threadIdx.x;
+    const size_t scored = candidates ? blocks * block : groups;
+    const int32_t* row_candidates = candidates ? candidates + row * blocks : nullptr;
+    const size_t g = !row_candidates ? place : place < scored ? candidate_group(row_candidates, block, place, groups) : groups;
+    const int32_t seen = visible[row];
+    const size_t limit = min(groups, size_t(seen > 0 ? seen : 0));
+    const size_t key_row = min(g, groups - 1);
+    const float* row_q = q + row * heads * dim;
+    float acc[H];
+    #pragma unroll
+    for (int h = 0; h < H; ++h) acc[h] = 0.0f;
+    for (size_t d0 = 0; d0 < dim; d0 += 32) {
+        float k[32];
+        if (BF16) {
+            const uint16_t* from = static_cast<const uint16_t*>(keys) + row * key_batch_stride + key_row * dim + d0;
+            if (d0 + 32 <= dim && (reinterpret_cast<uintptr_t>(from) & 15) == 0) {
+                #pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const uint4 raw = reinterpret_cast<const uint4*>(from)[v];
+                    const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+                    #pragma unroll
+                    for (int i = 0; i < 4; ++i) { k[8 * v + 2 * i] = __uint_as_float(words[i] << 16); k[8 * v + 2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u); }
+                }
+            } else {
+                #pragma unroll
+                for (int c = 0; c < 32; ++c) k[c] = d0 + c < dim ? bf16_value(from[c]) : 0.0f;
+            }
+        } else {
+            const float* from = static_cast<const float*>(keys) + row * key_batch_stride + key_row * dim + d0;
+            #pragma unroll
+            for (int c = 0; c < 32; ++c) k[c] = d0 + c < dim ? from[c] : 0.0f;
+        }
+        const int width = int(min(size_t(32), dim - d0));
+        #pragma unroll
+        for (int h = 0; h < H; ++h) {
+            if (size_t(h) < heads) {
+                const float* query = row_q + size_t(h) * dim + d0;
+                if (width == 32) {
+                    #pragma unroll
+                    for (int c = 0; c < 32; ++c) acc[h] = __builtin_fmaf(query[c], k[c], acc[h]);
+                } else {
+                    for (int c = 0; c < width; ++c) acc[h] = __builtin_fmaf(query[c], k[c], acc[h]);
+                }
+            }
+        }
+    }
+    if (place >= scored) return;
+    float total = 0.0f;
+    #pragma unroll
+    for (int h = 0; h < H; ++h) {
+        if (size_t(h) < heads) {
+            // the term is rounded before it joins the sum: keep the multiply and the add apart
+            const float term = __fmul_rn(fmaxf(acc[h], 0.0f), weights[row * heads + h]);
+            total = __fadd_rn(total, term);
+        }
+    }
+    scores[row * score_stride + place] = g < limit ? __fmul_rn(total, scale) : -INFINITY;
+}
+
+// ---- top-k -------------------------------------------------------------------------------------------------
+
+__device__ __forceinline__ uint32_t top_k_key(float value) {
+    const uint32_t bits = __float_as_uint(value == 0.0f ? 0.0f : value);   // -0 ties +0
+    return bits & 0x80000000u ? ~bits : bits | 0x80000000u;
+}
+
+constexpr int TOPK_THREADS = 1024, TOPK_WAVES = TOPK_THREADS / 64, TOPK_RUN = 8;
+
+// Exclusive prefix of `value` over the workgroup in thread order, and the workgroup's sum.
+__device__ __forceinline__ uint32_t block_scan(uint32_t value, uint32_t* wave_sums, uint32_t& total) {
+    const unsigned lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    uint32_t inclusive = value;
+    #pragma unroll
+    for (unsigned offset = 1; offset < 64; offset *= 2) {
+        const uint32_t other = __shfl_up(inclusive, offset);
+        if (lane >= offset) inclusive += other;
+    }
+    __syncthreads();
+    if (lane == 63) wave_sums[wave] = inclusive;
+    __syncthreads();
+    uint32_t before = 0, sum = 0;
+    #pragma unroll
+    for (int w = 0; w < TOPK_WAVES; ++w) {
+        const uint32_t c = wave_sums[w];
+        before += unsigned(w) < wave ? c : 0u;
+        sum += c;
+    }
+    total = sum;
+    return before + inclusive - value;
+}
+
+// One workgroup per row.  The k-th highest key by four 8-bit radix passes (MSB first, a 256-bin histogram per pass
+// in LDS), then one ordered pass: thread t owns runs of TOPK_RUN consecutive places so a workgroup scan of the kept
+// counts gives every kept place its slot in ascending index order.  score(place) and index(place) let the same code
+// serve plain rows and candidate-ordered rows.
+template<class Score, class Index>
+__device__ void top_k_row(Score score, Index index, size_t places, size_t k, int32_t* out) {
+    __shared__ uint32_t bins[256];
+    __shared__ uint32_t wave_sums[TOPK_WAVES];
+    __shared__ uint32_t picked_bin, picked_rank, picked_count, live_total;
+    const unsigned t = threadIdx.x;
+    const uint32_t floor = top_k_key(-INFINITY);
+    uint32_t prefix = 0, rank = uint32_t(k), equal_count = 0;
+    bool all = false;
+    for (int byte = 3; byte >= 0 && !all; --byte) {
+        const int shift = 8 * byte;
+        if (t < 256) bins[t] = 0;
+        __syncthreads();
+        for (size_t place = t; place < places; place += TOPK_THREADS) {
+            const uint32_t key = top_k_key(score(place));
+            if (key > floor && (byte == 3 || (key >> (shift + 8)) == (prefix >> (shift + 8)))) atomicAdd(&bins[(key >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        // thread i < 256 holds bin 255 - i: the scan counts keys in higher bins
+        const uint32_t count = t < 256 ? bins[255 - t] : 0u;
+        uint32_t every;
+        const uint32_t above = block_scan(count, wave_sums, every);
+        if (t < 256 && above < rank && above + count >= rank) { picked_bin = 255 - t; picked_rank = rank - above; picked_count = count; }
+        if (t == 0) live_total = every;
+        __syncthreads();
+        if (byte == 3 && live_total <= k) { all = true; break; }
+        prefix |= picked_bin << shift;
+        rank = picked_rank;
+        equal_count = picked_count;
+        __syncthreads();
+    }
+    // keys above `prefix` are kept; of the equal_count keys equal to it the first `rank` (lowest indices)
+    const uint32_t threshold = prefix, need = all ? 0u : rank;
+    (void)equal_count;
+    uint32_t slot = 0, ties_seen = 0;
+    const size_t tile = size_t(TOPK_THREADS) * TOPK_RUN;
+    for (size_t base = 0; base < places; base += tile) {
+        const size_t first = base + size_t(t) * TOPK_RUN;
+        uint32_t keys[TOPK_RUN];
+        uint32_t greater = 0, ties = 0;
+        #pragma unroll
+        for (int i = 0; i < TOPK_RUN; ++i) {
+            keys[i] = first + i < places ? top_k_key(score(first + i)) : floor;
+            const bool live = keys[i] > floor;
+            greater += live && (all || keys[i] > threshold);
+            ties += live && !all && keys[i] == threshold;
+        }
+        uint32_t tile_greater, tile_ties;
+        const uint32_t greater_before = block_scan(greater, wave_sums, tile_greater);
+        uint32_t tie_before = ties_seen + block_scan(ties, wave_sums, tile_ties);
+        // slot of this thread's first kept place: kept before it = greater before + ties before that were still needed
+        uint32_t at = slot + greater_before + (min(tie_before, need) - min(ties_seen, need));
+        #pragma unroll
+        for (int i = 0; i < TOPK_RUN; ++i) {
+            const bool live = keys[i] > floor;
+            bool keep = live && (all || keys[i] > threshold);
+            if (live && !all && keys[i] == threshold) { keep = tie_before < need; ++tie_before; }
+            if (keep) out[at++] = index(first + i);
+        }
+        slot += tile_greater + (min(ties_seen + tile_ties, need) - min(ties_seen, need));
+        ties_seen += tile_ties;
+    }
+    for (size_t i = slot + t; i < k; i += TOPK_THREADS) out[i] = -1;
+}
+
+__global__ void __launch_bounds__(TOPK_THREADS) top_k_kernel(const float* scores, size_t groups, size_t score_stride, size_t k, int32_t* out) {
+    const float* s = scores + size_t(blockIdx.x) * score_stride;
+    top_k_row([s](size_t g) { return s[g]; }, [](size_t g) { return int32_t(g); }, groups, k, out + size_t(blockIdx.x) * k);
+}
+
+// Top-k over a row's candidate groups: scores are stored in candidate order (sd_op_index_select with candidates).
+__global__ void __launch_bounds__(TOPK_THREADS) top_k_candidates_kernel(const float* scores, size_t score_stride, size_t groups, const int32_t* candidates,
+                                                                        size_t blocks, size_t block, size_t k, int32_t* out) {
+    const float* s = scores + size_t(blockIdx.x) * score_stride;
+    const int32_t* c = candidates + size_t(blockIdx.x) * blocks;
+    top_k_row([=](size_t v) { return candidate_group(c, block, v, groups) < groups ? s[v] : -INFINITY; },
+              [=](size_t v) { return int32_t(candidate_group(c, block, v, groups)); }, blocks * block, k, out + size_t(blockIdx.x) * k);
+}
+
+// Each block's highest score; the block of the row's last visible group is +inf (always kept).
+__global__ void __launch_bounds__(256) block_tops_kernel(const float* scores, const int32_t* visible, size_t groups, size_t block, size_t count,
+                                                         float* tops) {
+    const size_t row = blockIdx.y, b = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (b >= count) return;
+    const float* s = scores + row * groups;
+    const int32_t raw = visible[row];
+    const size_t seen = min(groups, size_t(raw > 0 ? raw : 0));
+    float top = seen && b == (seen - 1) / block ? INFINITY : -INFINITY;
+    for (size_t g = b * block, end = min(groups, g + block); g < end; ++g) top = fmaxf(top, s[g]);
+    tops[row * count + b] = top;
+}
+
+__global__ void widen_bf16_kernel(const uint16_t* from, float* to, size_t count) {
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) to[i] = bf16_value(from[i]);
+}
+
+void widen_bf16(Device& d, const void* from, float* to, size_t count) {
+    widen_bf16_kernel<<<unsigned(std::min<size_t>(checked_blocks(count), 65536)), 256, 0, d.stream>>>(static_cast<const uint16_t*>(from), to, count);
+    SD_CHECK(hipGetLastError());
+}
+
+void launch_scores(Device& d, const float* q, const void* keys, bool bf16, size_t key_batch_stride, const float* weights, const int32_t* visible,
+                   size_t rows, size_t groups, size_t heads, size_t dim, float scale, float* scores, size_t score_stride,
+                   const int32_t* candidates, size_t blocks, size_t block) {
+    const size_t scored = candidates ? blocks * block : groups;
+    const dim3 grid(checked_blocks(scored), unsigned(rows));
+#define SD_SCORES(H, B) index_scores_kernel<H, B><<<grid, 256, 0, d.stream>>>(q, keys, key_batch_stride, weights, visible, groups, heads, dim, scale, \
+                                                                              scores, score_stride, candidates, blocks, block)
+    if (heads <= 32) { if (bf16) SD_SCORES(32, true); else SD_SCORES(32, false); }
+    else { if (bf16) SD_SCORES(64, true); else SD_SCORES(64, false); }
+#undef SD_SCORES
+    SD_CHECK(hipGetLastError());
+}
+
+}  // namespace
+
+extern "C" {
+
+int sd_op_to_bf16(void* handle, const float* x, uint64_t count, void* out) {
+    SD_OP_BEGIN
+    if (!count) return 0;
+    op_span(value, x, checked_floats({count}), "values to round");
+    op_span(value, out, checked_product({count, 2}), "BF16 values");
+    to_bf16_kernel<<<unsigned(std::min<size_t>(checked_blocks(size_t(count)), 65536)), 256, 0, value.stream>>>(x, size_t(count), static_cast<uint16_t*>(out));
+    SD_OP_END
+}
+
+int sd_op_compress(void* handle, const float* kv, const float* gate, uint64_t groups, uint64_t ratio, uint64_t dim, float* out) {
+    SD_OP_BEGIN
+    if (!groups || !ratio || !dim) throw std::runtime_error("invalid Straydog compress shape");
+    op_span(value, kv, checked_floats({groups, ratio, dim}), "rows to compress");
+    if (gate) op_span(value, gate, checked_floats({groups, ratio, dim}), "a compression gate");
+    op_span(value, out, checked_floats({groups, dim}), "compressed rows");
+    compress_kernel<<<checked_blocks(checked_product({groups, dim})), 256, 0, value.stream>>>(kv, gate, size_t(groups), size_t(ratio), size_t(dim), out);
+    SD_OP_END
+}
+
+/* reference straydog_gpu.h:271 (gpu/kernels.cpp:4942-4956, kernel gpu/ops.hpp:107-120) */
+int sd_op_rope(void* handle, float* x, uint64_t rows, uint64_t vectors, uint64_t width, uint64_t rope_dims, const int32_t* positions,
+               const float* frequencies, int inverse) {
+    SD_OP_BEGIN
+    if (!rows || !vectors || !rope_dims || rope_dims % 2 || rope_dims > width) throw std::runtime_error("invalid Straydog rope shape");
+    op_span(value, x, checked_floats({rows, vectors, width}), "a rotated buffer");
+    op_span(value, positions, checked_floats({rows}), "rope positions");
+    op_span(value, frequencies, checked_floats({rope_dims / 2}), "rope frequencies");
+    const size_t count = checked_product({rows, vectors, rope_dims / 2});
+    rope_kernel<<<checked_blocks(count), 256, 0, value.stream>>>(x, x, count, size_t(vectors), size_t(width), size_t(rope_dims / 2), positions,
+                                                                 frequencies, inverse, 0);
+    SD_OP_END
+}
+
+int sd_op_index_scores(void* handle, const float* q, const float* keys, const float* weights, const int32_t* visible, uint64_t rows,
+                       uint64_t groups, uint64_t heads, uint64_t dim, float scale, float* scores) {
+    SD_OP_BEGIN
+    if (!rows || rows > 65535 || !groups || groups > (uint64_t(1) << 31) || !heads || heads > 64 || !dim) throw std::runtime_error("invalid Straydog index shape");
+    op_span(value, q, checked_floats({rows, heads, dim}), "index queries");
+    op_state_span(value, keys, checked_product({groups, dim}), "index keys");
+    op_span(value, weights, checked_floats({rows, heads}), "index weights");
+    op_span(value, visible, checked_floats({rows}), "visible counts");
+    op_span(value, scores, checked_floats({rows, groups}), "index scores");
+    launch_scores(value, q, state_base(keys), state_bf16(keys), 0, weights, visible, size_t(rows), size_t(groups), size_t(heads), size_t(dim), scale,
+                  scores, size_t(groups), nullptr, 0, 1);
+    SD_OP_END
+}
+
+int sd_op_top_k(void* handle, const float* scores, uint64_t rows, uint64_t groups, uint64_t k, int32_t* out) {
+    SD_OP_BEGIN
+    if (!rows || rows > 0x7fffffffu || !groups || !k || groups > (uint64_t(1) << 31) || k > (uint64_t(1) << 31)) throw std::runtime_error("invalid Straydog top-k shape");
+    op_span(value, scores, checked_floats({rows, groups}), "scores");
+    op_span(value, out, checked_floats({rows, k}), "top-k indices");
+    top_k_kernel<<<unsigned(rows), TOPK_THREADS, 0, value.stream>>>(scores, size_t(groups), size_t(groups), size_t(k), out);
+    SD_OP_END
+}
+
+int sd_op_index_candidates(void* handle, const float* scores, const int32_t* visible, uint64_t rows, uint64_t groups, uint64_t blocks,
+                           uint64_t block, int32_t* out, float* scratch, uint64_t scratch_bytes) {
+    SD_OP_BEGIN
+    if (!rows || rows > 65535 || !groups || groups > (uint64_t(1) << 31) || !blocks || blocks > (uint64_t(1) << 20) || !block || block > 4096)
+        throw std::runtime_error("invalid Straydog index candidates");
+    const uint64_t count = (groups + block - 1) / block;
+    op_span(value, scores, checked_floats({rows, groups}), "index scores");
+    op_span(value, visible, checked_floats({rows}), "visible counts");
+    op_span(value, out, checked_floats({rows, blocks}), "index candidates");
+    if (checked_floats({rows, count}) > scratch_bytes) throw std::runtime_error("Straydog index candidates need more scratch");
+    op_span(value, scratch, checked_floats({rows, count}), "index candidates' scratch");
+    block_tops_kernel<<<dim3(checked_blocks(size_t(count)), unsigned(rows)), 256, 0, value.stream>>>(scores, visible, size_t(groups), size_t(block),
+                                                                                                 size_t(count), scratch);
+    SD_CHECK(hipGetLastError());
+    top_k_kernel<<<unsigned(rows), TOPK_THREADS, 0, value.stream>>>(scratch, size_t(count), size_t(count), size_t(blocks), out);
+    SD_OP_END
+}
+
+int sd_op_index_select(void* handle, const float* q, const float* keys, const float* weights, const int32_t* visible, uint64_t rows,
+                       uint64_t groups, uint64_t heads, uint64_t dim, float scale, uint64_t rope_dims, const int32_t* positions,
+                       const float* frequencies, float* scores, uint64_t k, int32_t* out, const int32_t* candidates, uint64_t blocks,
+                       uint64_t block) {
+    SD_OP_BEGIN
+    if (!rows || rows > 65535 || !groups || groups > (uint64_t(1) << 31) || !heads || heads > 64 || !dim || !k || k > (uint64_t(1) << 31) ||
+        rope_dims % 2 || rope_dims > dim || rope_dims > 128)
+        throw std::runtime_error("invalid Straydog index shape");
+    uint64_t scored = groups;
+    if (candidates) {
+        if (!blocks || !block || blocks > (uint64_t(1) << 20) || block > 4096) throw std::runtime_error("invalid Straydog index candidates");
+        op_span(value, candidates, checked_floats({rows, blocks}), "index candidates");
+        scored = blocks * block;
+    }
+    op_span(value, q, checked_floats({rows, heads, dim}), "index queries");
+    op_state_span(value, keys, checked_product({groups, dim}), "index keys");
+    op_span(value, weights, checked_floats({rows, heads}), "index weights");
+    op_span(value, visible, checked_floats({rows}), "visible counts");
+    op_span(value, positions, checked_floats({rows}), "query positions");
+    if (rope_dims) op_span(value, frequencies, checked_floats({rope_dims / 2}), "rope frequencies");
+    op_span(value, scores, checked_floats({rows, std::max(groups, scored)}), "index scores");
+    op_span(value, out, checked_floats({rows, k}), "top-k indices");
+    const float* rotated = q;
+    if (rope_dims) {
+        // q itself stays as it was: the rotated copy lives in the device's workspace
+        const size_t count = checked_product({rows, heads, dim});
+        float* copy = static_cast<float*>(workspace(value, count * 4));
+        rope_kernel<<<checked_blocks(count), 256, 0, value.stream>>>(q, copy, count, size_t(heads), size_t(dim), size_t(rope_dims / 2), positions,
+                                                                     frequencies, 0, 1);
+        SD_CHECK(hipGetLastError());
+        rotated = copy;
+    }
+    // scores rows are `scored` wide with candidates (candidate order), `groups` wide without
+    const size_t stride = candidates ? size_t(scored) : size_t(groups);
+    launch_scores(value, rotated, state_base(keys), state_bf16(keys), 0, weights, visible, size_t(rows), size_t(groups), size_t(heads), size_t(dim),
+                  scale, scores, stride, candidates, size_t(blocks), size_t(block ? block : 1));
+    if (candidates)
+        top_k_candidates_kernel<<<unsigned(rows), TOPK_THREADS, 0, value.stream>>>(scores, stride, size_t(groups), candidates, size_t(blocks),
+                                                                                   size_t(block), size_t(k), out);
+    else
+        top_k_kernel<<<unsigned(rows), TOPK_THREADS, 0, value.stream>>>(scores, size_t(groups), stride, size_t(k), out);
+    SD_OP_END
+}
+
+int sdx_index_top_k(void* handle, const void* q_index, const void* keys, const float* weights, const int32_t* visible, uint64_t batch,
+                    uint64_t groups, uint64_t heads, uint64_t dim, float scale, float* scores, uint64_t k, int32_t* indices) {
+    SD_OP_BEGIN
+    if (!batch || batch > 65535 || !groups || groups > (uint64_t(1) << 31) || !heads || heads > 64 || !dim || !k || k > (uint64_t(1) << 31))
+        throw std::runtime_error("invalid Straydog index shape");
+    op_span(value, q_index, checked_product({batch, heads, dim, 2}), "index queries");
+    op_span(value, keys, checked_product({batch, groups, dim, 2}), "index keys");
+    op_span(value, weights, checked_floats({batch, heads}), "index weights");
+    op_span(value, visible, checked_floats({batch}), "visible counts");
+    op_span(value, indices, checked_floats({batch, k}), "top-k indices");
+    // workspace: the queries widened to FP32 (exact), and the scores when the caller does not want them
+    const size_t q_bytes = checked_floats({batch, heads, dim}), score_bytes = checked_floats({batch, groups});
+    uint8_t* space = static_cast<uint8_t*>(workspace(value, q_bytes + 256 + (scores ? 0 : score_bytes)));
+    float* wide_q = reinterpret_cast<float*>(space);
+    float* row_scores = scores ? scores : reinterpret_cast<float*>(space + ((q_bytes + 255) & ~size_t(255)));
+    if (scores) op_span(value, scores, score_bytes, "index scores");
+    widen_bf16(value, q_index, wide_q, size_t(batch * heads * dim));
+    launch_scores(value, wide_q, keys, true, size_t(groups * dim), weights, visible, size_t(batch), size_t(groups), size_t(heads), size_t(dim), scale,
+                  row_scores, size_t(groups), nullptr, 0, 1);
+    top_k_kernel<<<unsigned(batch), TOPK_THREADS, 0, value.stream>>>(row_scores, size_t(groups), size_t(groups), size_t(k), indices);
+    SD_OP_END
+}
+
+}  // extern "C"
+

@@ -1,0 +1,138 @@
+// Appending rows to the paged K/V cache, and small utility kernels (fills, copy).
+// The Q8_0 arithmetic is the reference's kv_encode/kv_put (gpu/kernels.cpp:58-74): scale = f16(max|x| / 127) over a
+// 32-value block, q = clamp(rint(x / f32(scale)), -127, 127), q = 0 when the scale is 0.
+#include "device.hpp"
+#include "kv_codec.hpp"
+#include "../../include/straydog_gpu_ext.h"
+
+#include <hip/hip_fp16.h>
+
+using namespace sd;
+
+namespace {
+
+// A thread holds 4 consecutive values of a row; the 8 threads of a 32-value block are adjacent lanes, so the
+// block's largest magnitude is three xor-shuffles away.  One 4-byte store per thread; lane 0 of a block stores the scale.
+template<bool F16_IN>
+__global__ void __launch_bounds__(256) kv_write_kernel(uint8_t* pages, unsigned page_tokens, unsigned kv_heads, unsigned dim, unsigned row_bytes,
+                                                       const int32_t* page_table, size_t table_stride, const int32_t* positions,
+                                                       const void* keys, const void* values, size_t span, size_t total) {
+    const size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x;   // one per 4 values of [K|V][seq][row][head][dim/4]
+    const bool live = index < total;
+    const size_t quads = dim / 4, per_kind = total / 2;
+    const size_t at = live ? index % per_kind : 0;
+    const bool is_value = live && index >= per_kind;
+    const size_t quad = at % quads, head = at / quads % kv_heads, row = at / quads / kv_heads % span, seq = at / quads / kv_heads / span;
+    const void* source = is_value ? values : keys;
+    float x[4];
+    const size_t first = ((seq * span + row) * kv_heads + head) * dim + quad * 4;
+    if (F16_IN) {
+        const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const __half*>(source) + first);
+        const __half2 a = *reinterpret_cast<const __half2*>(&raw.x), b = *reinterpret_cast<const __half2*>(&raw.y);
+        x[0] = __low2float(a); x[1] = __high2float(a); x[2] = __low2float(b); x[3] = __high2float(b);
+    } else {
+        const float4 raw = *reinterpret_cast<const float4*>(static_cast<const float*>(source) + first);
+        x[0] = raw.x; x[1] = raw.y; x[2] = raw.z; x[3] = raw.w;
+    }
+    const size_t position = size_t(positions[seq]) + row;
+    const size_t page = size_t(page_table[seq * table_stride + position / page_tokens]);
+    const size_t plane = is_value ? kv_heads + head : head;
+    uint8_t* out = pages + ((page * 2 * kv_heads + plane) * page_tokens + position % page_tokens) * row_bytes;
+    kv_store_quad(out, unsigned(quad), dim, row_bytes != 2 * dim, x, live);
+}
+
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {   // splitmix64 finaliser
+    z += 0x9e3779b97f4a7c15ull;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+
+__global__ void fill_normal_kernel(void* out, size_t count, uint64_t seed, int kind) {
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) {
+        const uint64_t bits = mix64(seed ^ (i * 0xd1342543de82ef95ull));
+        const float u = (float(uint32_t(bits >> 40)) + 0.5f) * (1.0f / 16777216.0f);
+        const float v = (float(uint32_t(bits) >> 8) + 0.5f) * (1.0f / 16777216.0f);
+        const float value = sqrtf(-2.0f * logf(u)) * cosf(6.2831853f * v);
+        if (kind == 0) static_cast<float*>(out)[i] = value;
+        else if (kind == 1) static_cast<__half*>(out)[i] = __float2half_rn(value);
+        else {
+            const uint32_t b = __float_as_uint(value);
+            static_cast<uint16_t*>(out)[i] = uint16_t((b + 0x7fffu + ((b >> 16) & 1u)) >> 16);
+        }
+    }
+}
+
+__global__ void fill_uniform_kernel(float* out, size_t count, uint64_t seed, float lo, float hi) {
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) {
+        const uint64_t bits = mix64(seed ^ (i * 0xd1342543de82ef95ull));
+        out[i] = lo + (hi - lo) * (float(uint32_t(bits >> 40)) * (1.0f / 16777216.0f));
+    }
+}
+
+// Plain streaming copy, 16 bytes a lane: the measured HBM ceiling and the calibration of byte counters.
+__global__ void __launch_bounds__(256) copy_kernel(uint4* target, const uint4* source, size_t count) {
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x)
+        target[i] = source[i];
+}
+
+}  // namespace
+
+namespace sd {
+void validate_pool(Device& d, const sdx_kv_pool* pool) {
+    if (!pool || !pool->pages || !pool->page_count || !pool->page_tokens || pool->page_tokens % 32 || !pool->kv_heads ||
+        (pool->dim != 128 && pool->dim != 256) || (pool->row_bytes != pool->dim + pool->dim / 16 && pool->row_bytes != 2 * pool->dim))
+        throw std::runtime_error("invalid Straydog K/V pool");
+    op_span(d, pool->pages, checked_product({pool->page_count, 2, pool->kv_heads, pool->page_tokens, pool->row_bytes}), "a K/V pool");
+}
+}  // namespace sd
+
+extern "C" {
+
+int sdx_kv_write(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
+                 const void* keys, const void* values, int input_f16, uint64_t seqs, uint64_t span) {
+    SD_OP_BEGIN
+    validate_pool(value, pool);
+    if (!seqs || !span || !table_stride) throw std::runtime_error("invalid Straydog K/V write shape");
+    const size_t element = input_f16 ? 2 : 4;
+    op_span(value, page_table, checked_floats({seqs, table_stride}), "a page table");
+    op_span(value, positions, checked_floats({seqs}), "K/V positions");
+    op_span(value, keys, checked_product({seqs, span, pool->kv_heads, pool->dim, element}), "new keys");
+    op_span(value, values, checked_product({seqs, span, pool->kv_heads, pool->dim, element}), "new values");
+    const size_t total = checked_product({2, seqs, span, pool->kv_heads, pool->dim / 4});
+    auto* pages = static_cast<uint8_t*>(pool->pages);
+    if (input_f16)
+        kv_write_kernel<true><<<checked_blocks(total), 256, 0, value.stream>>>(pages, pool->page_tokens, pool->kv_heads, pool->dim, pool->row_bytes,
+            page_table, size_t(table_stride), positions, keys, values, size_t(span), total);
+    else
+        kv_write_kernel<false><<<checked_blocks(total), 256, 0, value.stream>>>(pages, pool->page_tokens, pool->kv_heads, pool->dim, pool->row_bytes,
+            page_table, size_t(table_stride), positions, keys, values, size_t(span), total);
+    SD_OP_END
+}
+
+int sdx_fill_normal(void* handle, void* out, uint64_t count, uint64_t seed, int out_kind) {
+    SD_OP_BEGIN
+    if (!count || out_kind < 0 || out_kind > 2) throw std::runtime_error("invalid Straydog fill");
+    op_span(value, out, checked_product({count, out_kind == 0 ? 4u : 2u}), "a filled buffer");
+    fill_normal_kernel<<<unsigned(std::min<size_t>(checked_blocks(size_t(count)), 65536)), 256, 0, value.stream>>>(out, size_t(count), seed, out_kind);
+    SD_OP_END
+}
+
+int sdx_fill_uniform(void* handle, float* out, uint64_t count, uint64_t seed, float lo, float hi) {
+    SD_OP_BEGIN
+    if (!count) throw std::runtime_error("invalid Straydog fill");
+    op_span(value, out, checked_floats({count}), "a filled buffer");
+    fill_uniform_kernel<<<unsigned(std::min<size_t>(checked_blocks(size_t(count)), 65536)), 256, 0, value.stream>>>(out, size_t(count), seed, lo, hi);
+    SD_OP_END
+}
+
+int sdx_copy(void* handle, void* target, const void* source, uint64_t bytes) {
+    SD_OP_BEGIN
+    if (!bytes || bytes % 16) throw std::runtime_error("invalid Straydog copy");
+    op_span(value, target, size_t(bytes), "a copy's target");
+    op_span(value, source, size_t(bytes), "a copy's source");
+    copy_kernel<<<value.compute_units * 16, 256, 0, value.stream>>>(static_cast<uint4*>(target), static_cast<const uint4*>(source), size_t(bytes / 16));
+    SD_OP_END
+}
+
+}  // extern "C"

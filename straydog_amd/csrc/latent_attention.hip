@@ -1,0 +1,216 @@
+// Latent sparse attention: each query attends a sliding window of raw rows and the compressed rows its selection
+// lists, the same row serving as key and value, with an optional per-head sink that enters the maximum and the
+// denominator only (reference gpu/ops.hpp:1240-1297, rope :1318-1328, entry gpu/kernels.cpp:5311-5476; CPU twin
+// crates/straydog-engine/examples/ds41_reference.rs:385-411).  The batched entry of the sparse top-k path uses the
+// same kernel without window or sink, keys kdim wide and values their first vdim columns.
+//
+// A workgroup owns one row and 8 of its heads, so a gathered row is read once for 8 heads: scores with 8 adjacent
+// lanes (the heads) sharing a key row, a wave per head for the softmax, then a thread per output column.
+#include "device.hpp"
+#include "../../include/straydog_gpu.h"
+#include "../../include/straydog_gpu_ext.h"
+
+using namespace sd;
+
+namespace {
+
+constexpr int HB = 8, THREADS = 256, PAD = 4, MAX_COLS = 4;
+
+struct LatentArgs {
+    const float* q;                 // [rows][heads][kdim]
+    const uint16_t* q_bf16;         // or BF16 queries (the batched entry)
+    const float* raw; size_t raw_rows;
+    const int32_t* positions; size_t window;
+    const void* compressed; size_t compressed_batch_stride;   // values per row of the batch (0: one table for every row)
+    const int32_t* selected; size_t selections;
+    const float* sinks;
+    size_t heads, kdim, vdim;
+    float scale;
+    size_t pairs; const float* frequencies;
+    float* out;
+};
+
+template<bool BF16>
+__device__ __forceinline__ float latent_value(const void* row, size_t col) {
+    if (BF16) return __uint_as_float(uint32_t(static_cast<const uint16_t*>(row)[col]) << 16);
+    return static_cast<const float*>(row)[col];
+}
+
+template<bool BF16>
+__global__ void __launch_bounds__(THREADS) latent_attention_kernel(LatentArgs a) {
+    const size_t row = blockIdx.y, head0 = size_t(blockIdx.x) * HB;
+    const unsigned t = threadIdx.x, lane = t % 64, wave = t / 64;
+    const size_t heads_here = min(size_t(HB), a.heads - head0);
+    const int64_t p = a.positions ? a.positions[row] : 0;
+    const int64_t first = a.window ? (p - int64_t(a.window) + 1 < 0 ? 0 : p - int64_t(a.window) + 1) : 0;
+    const size_t raw_count = a.window ? size_t(p - first + 1) : 0, total = raw_count + a.selections;
+    const size_t stride = a.kdim + PAD;
+    extern __shared__ float lds[];
+    float* qs = lds;                         // [HB][kdim + PAD]; reused for the output rows at the end
+    float* w = qs + HB * stride;             // [HB][total]
+    float* denominators = w + HB * total;    // [HB]
+    // queries, their last 2 * pairs values rotated (angle, sine and cosine in double)
+    const size_t rotated = a.kdim - 2 * a.pairs;
+    for (size_t i = t; i < heads_here * a.kdim; i += THREADS) {
+        const size_t h = i / a.kdim, c = i % a.kdim, at = (row * a.heads + head0 + h) * a.kdim;
+        const auto load = [&](size_t col) { return a.q_bf16 ? __uint_as_float(uint32_t(a.q_bf16[at + col]) << 16) : a.q[at + col]; };
+        float value = load(c);
+        if (c >= rotated) {
+            const size_t pair = (c - rotated) / 2;
+            double s, co;
+            sincos(double(p) * double(a.frequencies[pair]), &s, &co);
+            const double x = load(rotated + 2 * pair), y = load(rotated + 2 * pair + 1);
+            value = (c - rotated) & 1 ? float(x * s + y * co) : float(x * co - y * s);
+        }
+        qs[h * stride + c] = value;
+    }
+    __syncthreads();
+    const auto key_row = [&](size_t index, bool& bf16) -> const void* {
+        if (index < raw_count) { bf16 = false; return a.raw + size_t(first + int64_t(index)) % a.raw_rows * a.kdim; }
+        const int32_t at = a.selected[row * a.selections + (index - raw_count)];
+        bf16 = BF16;
+        if (at < 0) return nullptr;
+        const size_t offset = row * a.compressed_batch_stride + size_t(at) * a.kdim;
+        return BF16 ? static_cast<const void*>(static_cast<const uint16_t*>(a.compressed) + offset)
+                    : static_cast<const void*>(static_cast<const float*>(a.compressed) + offset);
+    };
+    // scores: 32 keys a pass, the 8 heads of a key in adjacent lanes
+    {
+        const size_t h = t % HB;
+        for (size_t index = t / HB; index < total; index += THREADS / HB) {
+            bool bf16;
+            const void* key = key_row(index, bf16);
+            float dot = 0.0f;
+            if (key && h < heads_here) {
+                const float* query = qs + h * stride;
+                if (bf16) for (size_t c = 0; c < a.kdim; ++c) dot += query[c] * latent_value<true>(key, c);
+                else for (size_t c = 0; c < a.kdim; ++c) dot += query[c] * latent_value<false>(key, c);
+            }
+            if (h < heads_here) w[h * total + index] = key ? dot * a.scale : -INFINITY;
+        }
+    }
+    __syncthreads();
+    // softmax weights: a wave per head
+    for (size_t h = wave; h < heads_here; h += THREADS / 64) {
+        const float sink = a.sinks ? a.sinks[head0 + h] : -INFINITY;
+        float top = sink;
+        for (size_t i = lane; i < total; i += 64) top = fmaxf(top, w[h * total + i]);
+        for (unsigned offset = 32; offset; offset /= 2) top = fmaxf(top, __shfl_xor(top, offset));
+        float sum = 0.0f;
+        for (size_t i = lane; i < total; i += 64) {
+            const float s = w[h * total + i];
+            const float weight = s == -INFINITY ? 0.0f : expf(s - top);
+            w[h * total + i] = weight;
+            sum += weight;
+        }
+        for (unsigned offset = 32; offset; offset /= 2) sum += __shfl_xor(sum, offset);
+        if (!lane) denominators[h] = sum + (a.sinks ? expf(sink - top) : 0.0f);
+    }
+    __syncthreads();
+    // weighted rows: a thread per output column, every head of the workgroup at once
+    float acc[HB][MAX_COLS];
+    #pragma unroll
+    for (int h = 0; h < HB; ++h)
+        #pragma unroll
+        for (int c = 0; c < MAX_COLS; ++c) acc[h][c] = 0.0f;
+    for (size_t index = 0; index < total; ++index) {
+        bool bf16;
+        const void* key = key_row(index, bf16);
+        if (!key) continue;
+        #pragma unroll
+        for (int c = 0; c < MAX_COLS; ++c) {
+            const size_t col = t + size_t(c) * THREADS;
+            if (col >= a.vdim) break;
+            const float v = bf16 ? latent_value<true>(key, col) : latent_value<false>(key, col);
+            #pragma unroll
+            for (int h = 0; h < HB; ++h) acc[h][c] += w[size_t(h) * total + index] * v;
+        }
+    }
+    // (w rows of absent heads are never written: their products are discarded below)
+    float* rows_out = qs;   // [HB][vdim]
+    #pragma unroll
+    for (int h = 0; h < HB; ++h)
+        #pragma unroll
+        for (int c = 0; c < MAX_COLS; ++c) {
+            const size_t col = t + size_t(c) * THREADS;
+            if (size_t(h) < heads_here && col < a.vdim) rows_out[size_t(h) * a.vdim + col] = acc[h][c] / denominators[h];
+        }
+    __syncthreads();
+    const size_t back = a.vdim - 2 * a.pairs;
+    for (size_t i = t; i < heads_here * a.vdim; i += THREADS) {
+        const size_t h = i / a.vdim, c = i % a.vdim;
+        float value = rows_out[i];
+        if (c >= back) {
+            const size_t pair = (c - back) / 2;
+            double s, co;
+            sincos(double(p) * double(a.frequencies[pair]) * -1.0, &s, &co);
+            const double x = rows_out[h * a.vdim + back + 2 * pair], y = rows_out[h * a.vdim + back + 2 * pair + 1];
+            value = (c - back) & 1 ? float(x * s + y * co) : float(x * co - y * s);
+        }
+        a.out[(row * a.heads + head0 + h) * a.vdim + c] = value;
+    }
+}
+
+void launch(Device& d, const LatentArgs& args, size_t rows, size_t total_keys, bool bf16) {
+    const size_t shared = (HB * (args.kdim + PAD) + HB * total_keys + HB) * 4;
+    if (shared > 160 * 1024 - 256) throw std::runtime_error("invalid Straydog attention shape");
+    static bool raised = false;
+    if (!raised) {
+        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attention_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
+        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attention_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
+        raised = true;
+    }
+    const dim3 grid(unsigned((args.heads + HB - 1) / HB), unsigned(rows));
+    if (bf16) latent_attention_kernel<true><<<grid, THREADS, shared, d.stream>>>(args);
+    else latent_attention_kernel<false><<<grid, THREADS, shared, d.stream>>>(args);
+}
+
+}  // namespace
+
+extern "C" {
+
+int sd_op_sparse_attention(void* handle, const float* q, const float* raw, uint64_t raw_rows, const int32_t* positions, uint64_t window,
+                           const float* compressed, uint64_t compressed_rows, const int32_t* selected, uint64_t selections,
+                           const float* sinks, uint64_t rows, uint64_t heads, uint64_t dim, float scale, uint64_t rope_dims,
+                           const float* frequencies, float* scratch, uint64_t scratch_bytes, float* out) {
+    SD_OP_BEGIN
+    (void)scratch; (void)scratch_bytes;
+    if (!rows || rows > 65535 || !heads || !dim || dim > 1024 || !window || !raw_rows || rope_dims % 2 || rope_dims > dim || rope_dims > 128)
+        throw std::runtime_error("invalid Straydog attention shape");
+    if (rope_dims) op_span(value, frequencies, checked_floats({rope_dims / 2}), "rope frequencies");
+    op_span(value, q, checked_floats({rows, heads, dim}), "attention queries");
+    op_span(value, raw, checked_floats({raw_rows, dim}), "window rows");
+    op_span(value, positions, checked_floats({rows}), "query positions");
+    if (selections) {
+        op_state_span(value, compressed, checked_product({compressed_rows, dim}), "compressed rows");
+        op_span(value, selected, checked_floats({rows, selections}), "selected rows");
+    }
+    op_span(value, sinks, checked_floats({heads}), "attention sinks");
+    op_span(value, out, checked_floats({rows, heads, dim}), "an attention output");
+    LatentArgs args{};
+    args.q = q; args.raw = raw; args.raw_rows = size_t(raw_rows); args.positions = positions; args.window = size_t(window);
+    args.compressed = state_base(compressed); args.selected = selected; args.selections = size_t(selections); args.sinks = sinks;
+    args.heads = size_t(heads); args.kdim = args.vdim = size_t(dim); args.scale = scale; args.pairs = size_t(rope_dims / 2);
+    args.frequencies = frequencies; args.out = out;
+    launch(value, args, size_t(rows), size_t(window + selections), state_bf16(compressed));
+    SD_OP_END
+}
+
+int sdx_latent_attention(void* handle, const void* q, const void* latents, const int32_t* selected, uint64_t batch, uint64_t groups,
+                         uint64_t k, uint64_t heads, uint64_t kdim, uint64_t vdim, float scale, float* out) {
+    SD_OP_BEGIN
+    if (!batch || batch > 65535 || !groups || !k || !heads || !kdim || !vdim || vdim > kdim || kdim > 1024)
+        throw std::runtime_error("invalid Straydog attention shape");
+    op_span(value, q, checked_product({batch, heads, kdim, 2}), "attention queries");
+    op_span(value, latents, checked_product({batch, groups, kdim, 2}), "latent rows");
+    op_span(value, selected, checked_floats({batch, k}), "selected rows");
+    op_span(value, out, checked_floats({batch, heads, vdim}), "an attention output");
+    LatentArgs args{};
+    args.q_bf16 = static_cast<const uint16_t*>(q); args.compressed = latents; args.compressed_batch_stride = size_t(groups * kdim);
+    args.selected = selected; args.selections = size_t(k); args.heads = size_t(heads); args.kdim = size_t(kdim); args.vdim = size_t(vdim);
+    args.scale = scale; args.out = out;
+    launch(value, args, size_t(batch), size_t(k), true);
+    SD_OP_END
+}
+
+}  // extern "C"

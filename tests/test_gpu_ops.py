@@ -1,0 +1,337 @@
+"""GPU parity of the reference ABI's attention ops, written after the reference's own model-free tests:
+crates/straydog-engine/tests/attention_gpu.rs (causal GQA against an F64 reference with a derived bound, output
+guards), tests/fused_gpu.rs:326-428 (top-k against its rule on adversarial ties; index_select == rope + index_scores
++ top_k bit for bit, run twice; candidates), tests/ds_state_bf16_gpu.rs (BF16 rounding; BF16-tagged rows == the FP32
+values they stand for, bit for bit), and sd_attention_sequence / sd_op_sparse_attention / sd_op_compress against the
+CPU oracle."""
+import numpy as np
+import pytest
+
+from gpu_util import backend, close_enough
+from test_oracle_attention import SHAPES, _attention_gpu_case
+from test_oracle_index_topk import Random, _adversarial
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    with backend(4 << 30) as handle:
+        yield handle
+
+
+def _read(gpu, buffer, dtype, count):
+    return gpu.read_buffer(buffer, 0, dtype, count)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("zero_queries", [False, True])
+def test_causal_gqa_matches_f64_softmax(gpu, oracle, shape, zero_queries):
+    rows, heads, kv_heads, dim, context = shape
+    if zero_queries and shape != (17, 4, 2, 256, 35):
+        pytest.skip("the reference runs zero queries on one shape")
+    q, keys, values, positions, gate, scale = _attention_gpu_case(*shape, zero_queries=zero_queries)
+    qs, ks, vs, gs, ps = (gpu.upload(x) for x in (q, keys, values, gate, positions))
+    scratch = gpu.buffer(rows * heads * 64 * (dim + 2) * 4)
+    guard, canary = 7, np.float32(12345.125)
+    output = gpu.upload(np.full(q.size + 2 * guard, canary, dtype=np.float32))
+    for gated in (False, True):
+        gpu.attention(qs.base(), ks.base(), vs.base(), context, ps.base(), rows, heads, kv_heads, dim, float(scale),
+                      gs.base() if gated else None, scratch, output.at(guard * 4))
+        actual = _read(gpu, output, np.float32, q.size + 2 * guard)
+        assert np.all(actual[:guard] == canary) and np.all(actual[guard + q.size:] == canary), "output guard"
+        want, bound = oracle.op_attention_f64(q, keys, values, positions, scale, gate if gated else None)
+        got = actual[guard:guard + q.size].reshape(q.shape)
+        assert np.all(np.isfinite(got))
+        ratio = np.abs(got - want) / bound
+        assert ratio.max() <= 1.0, f"{shape} gated={gated}: error/bound {ratio.max():.3f}"
+    for b in (qs, ks, vs, gs, ps, scratch, output):
+        gpu.release(b)
+
+
+def test_attention_refuses_bad_arguments(gpu):
+    from straydog_amd.backend import StraydogError
+    b = gpu.buffer(1 << 20)
+    with pytest.raises(StraydogError, match="scratch too small"):
+        gpu.attention(b.base(), b.base(), b.base(), 8, b.base(), 1, 2, 1, 64, 0.1, None, None, b.base())
+    with pytest.raises(StraydogError, match="invalid Straydog attention shape"):
+        gpu.attention(b.base(), b.base(), b.base(), 8, b.base(), 1, 3, 2, 64, 0.1, None, b, b.base())
+    with pytest.raises(StraydogError, match="overflows|outside"):
+        gpu.attention(b.base(), b.base(), b.base(), 1 << 62, b.base(), 1, 2, 1, 64, 0.1, None, b, b.base())
+    gpu.release(b)
+
+
+@pytest.mark.parametrize("row_bytes", [272, 512])
+def test_attention_sequence_matches_the_oracle(gpu, oracle, row_bytes):
+    rng = np.random.default_rng(70 + row_bytes)
+    context, base, steps, selected = 600, 300, 5, 2052
+    gpu.kv_format(row_bytes)
+    state_host = np.zeros(context * 4 * row_bytes, dtype=np.uint8)
+    old_k = rng.standard_normal((1, base, 2, 256)).astype(np.float32)
+    old_v = rng.standard_normal((1, base, 2, 256)).astype(np.float32)
+    oracle.kv_write(state_host, row_bytes, context, 2, 256, np.zeros((1, 1), np.int32), np.zeros(1, np.int32), old_k, old_v)
+    state = gpu.upload(state_host)
+    q = rng.standard_normal((steps, 24, 256)).astype(np.float32)
+    k = rng.standard_normal((steps, 2, 256)).astype(np.float32)
+    v = rng.standard_normal((steps, 2, 256)).astype(np.float32)
+    indices = np.full((steps, selected), -1.0, dtype=np.float32)
+    counts = np.zeros(steps, dtype=np.float32)
+    for s in range(steps):
+        picked = np.sort(rng.permutation(base + s + 1)[: 200 + 13 * s])
+        extra = [base + s + 3, -2.0, context + 1]        # ignored: past the row's position, negative, past the context
+        row = np.concatenate([picked, extra]).astype(np.float32)
+        indices[s, :row.size] = row
+        counts[s] = row.size
+    packed = np.concatenate([q.ravel(), k.ravel(), v.ravel(), indices.ravel(), counts]).astype(np.float32)
+    got = gpu.attention_sequence(state.base(), context, base, steps, selected, packed)
+    want = oracle.attention_sequence(state_host, row_bytes, context, base, steps, selected, packed)
+    assert np.abs(got - want).max() < 2e-5
+    # the rows' K/V were written as the oracle writes them
+    after = _read(gpu, state, np.uint8, state_host.size)
+    assert np.array_equal(after, state_host)
+    from straydog_amd.backend import StraydogError
+    with pytest.raises(StraydogError, match="selection count"):
+        bad = packed.copy(); bad[-1] = 0.0
+        gpu.attention_sequence(state.base(), context, base, steps, selected, bad)
+    with pytest.raises(StraydogError, match="workspace mismatch"):
+        gpu.attention_sequence(state.base(), context, base, steps, selected, packed[:-1])
+    gpu.release(state)
+    gpu.kv_format(272)
+
+
+def test_to_bf16_rounds_to_nearest_even(gpu, oracle):
+    rng = np.random.default_rng(2)
+    bits = np.concatenate([rng.integers(0, 2 ** 32, 50000, dtype=np.uint64).astype(np.uint32),
+                           np.array([0, 0x80000000, 0x3f808000, 0x3f818000, 0x3f807fff, 0x3f808001, 0x7f7fffff, 0x7f800000, 0xff800000,
+                                     0x7f800001, 0x7fc00000, 0xffc00001, 1, 0x8000, 0x18000], dtype=np.uint32)])
+    x = gpu.upload(bits)
+    out = gpu.buffer(bits.size * 2)
+    gpu.to_bf16(x.base(), bits.size, out.base())
+    assert np.array_equal(_read(gpu, out, np.uint16, bits.size), oracle.to_bf16(bits.view(np.float32)))
+    gpu.release(x); gpu.release(out)
+
+
+def test_compress_matches_the_oracle(gpu, oracle):
+    rng = np.random.default_rng(3)
+    groups, ratio, dim = 37, 4, 512
+    kv = rng.standard_normal((groups * ratio, dim)).astype(np.float32)
+    gate = (rng.standard_normal((groups * ratio, dim)) * 3).astype(np.float32)
+    kb, gb, out = gpu.upload(kv), gpu.upload(gate), gpu.buffer(groups * dim * 4)
+    gpu.compress(kb.base(), gb.base(), groups, ratio, dim, out.base())
+    assert np.abs(_read(gpu, out, np.float32, groups * dim).reshape(groups, dim) - oracle.compress(kv, gate, ratio)).max() < 1e-6
+    gpu.compress(kb.base(), None, groups, 1, dim, out.base())
+    assert np.array_equal(_read(gpu, out, np.float32, groups * dim), kv[:groups].ravel())
+    for b in (kb, gb, out):
+        gpu.release(b)
+
+
+@pytest.mark.parametrize("groups", [511, 512, 513, 600, 4096, 30000, 65536, 131072])
+def test_top_k_matches_its_reference_with_many_ties(gpu, oracle, groups):
+    random = Random(0x2f6b91d3c0a54e77 ^ groups)
+    k, rows = 512, 2
+    if groups > 30000:      # the pure-Python generator is slow: vectorise the same distribution
+        rng = np.random.default_rng(groups)
+        draw = rng.integers(0, 97, size=(rows, groups))
+        scores = (rng.integers(0, 17, size=(rows, groups)) * 0.25 - 2.0).astype(np.float32)
+        scores[draw <= 6] = -np.inf
+        scores[draw == 7] = np.inf
+        scores[draw == 8] = -0.0
+        scores.reshape(-1)[999::1000] += np.float32(0.125)
+    else:
+        scores = _adversarial(random, rows, groups)
+    sb, out = gpu.upload(scores), gpu.buffer(rows * k * 4)
+    for _ in range(2):      # twice: nothing left over from the first run
+        gpu.top_k(sb.base(), rows, groups, k, out.base())
+        got = _read(gpu, out, np.int32, rows * k).reshape(rows, k)
+        assert np.array_equal(got, oracle.top_k(scores, k)), groups
+    gpu.release(sb); gpu.release(out)
+
+
+def test_top_k_edge_cases(gpu, oracle):
+    cases = [np.array([[1.0, 1.0, 1.0, 2.0, -np.inf, 1.0]], np.float32), np.full((1, 700), -np.inf, np.float32),
+             np.zeros((3, 9000), np.float32), np.array([[0.0, -0.0, -1.0, np.inf]], np.float32)]
+    for scores in cases:
+        for k in (1, 3, 600, 2048):
+            sb, out = gpu.upload(scores), gpu.buffer(scores.shape[0] * k * 4)
+            gpu.top_k(sb.base(), scores.shape[0], scores.shape[1], k, out.base())
+            got = _read(gpu, out, np.int32, scores.shape[0] * k).reshape(scores.shape[0], k)
+            assert np.array_equal(got, oracle.top_k(scores, k)), (scores.shape, k)
+            gpu.release(sb); gpu.release(out)
+
+
+def _bf16_round(oracle, x):
+    bits = oracle.to_bf16(x)
+    return bits, (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+@pytest.mark.parametrize("rows,groups,heads,dim", [(1, 3000, 32, 128), (4, 2000, 64, 128), (2, 300, 5, 96), (1, 1000, 33, 40)])
+def test_index_scores_are_bit_exact(gpu, oracle, rows, groups, heads, dim):
+    rng = np.random.default_rng(rows * 1000 + groups)
+    q = (rng.standard_normal((rows, heads, dim)) * 2).astype(np.float32)
+    keys = rng.standard_normal((groups, dim)).astype(np.float32)
+    weights = rng.standard_normal((rows, heads)).astype(np.float32)
+    visible = np.array([groups - 3 * r for r in range(rows)], dtype=np.int32)
+    scale = float(1.0 / (np.sqrt(np.float32(dim)) * np.sqrt(np.float32(heads))))
+    qb, kb, wb, vb, out = gpu.upload(q), gpu.upload(keys), gpu.upload(weights), gpu.upload(visible), gpu.buffer(rows * groups * 4)
+    gpu.index_scores(qb.base(), kb.base(), wb.base(), vb.base(), rows, groups, heads, dim, scale, out.base())
+    got = _read(gpu, out, np.float32, rows * groups).reshape(rows, groups)
+    want = oracle.index_scores(q, keys, weights, visible, scale)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # BF16-tagged keys give the bits of the FP32 values they stand for
+    key_bits, key_values = _bf16_round(oracle, keys)
+    hb = gpu.upload(key_bits)
+    from straydog_amd.backend import tagged_bf16
+    gpu.index_scores(qb.base(), tagged_bf16(hb.base()), wb.base(), vb.base(), rows, groups, heads, dim, scale, out.base())
+    tagged = _read(gpu, out, np.float32, rows * groups).reshape(rows, groups)
+    assert np.array_equal(tagged.view(np.uint32), oracle.index_scores(q, key_values, weights, visible, scale).view(np.uint32))
+    for b in (qb, kb, wb, vb, out, hb):
+        gpu.release(b)
+
+
+def test_an_index_select_matches_rope_scores_and_top_k(gpu, oracle):
+    # fused_gpu.rs:390-428
+    random = np.random.default_rng(0xa54f)
+    heads, dim, rope_dims, k = 32, 128, 64, 512
+    frequencies = (np.float32(1.6e5) ** (-(2.0 * np.arange(rope_dims // 2, dtype=np.float32)) / np.float32(rope_dims))).astype(np.float32)
+    fb = gpu.upload(frequencies)
+    for rows, groups in [(1, 3000), (4, 2000), (1, 300)]:
+        q = (random.random((rows, heads, dim)) * 4 - 2).astype(np.float32)
+        keys = (random.random((groups, dim)) * 2 - 1).astype(np.float32)
+        weights = (random.random((rows, heads)) * 2 - 1).astype(np.float32)
+        visible = np.array([groups - 3 * r for r in range(rows)], dtype=np.int32)
+        at = np.array([20000 + 7 * r for r in range(rows)], dtype=np.int32)
+        scale = float(1.0 / (np.sqrt(np.float32(dim)) * np.sqrt(np.float32(heads))))
+        kb, wb, vb, pb = gpu.upload(keys), gpu.upload(weights), gpu.upload(visible), gpu.upload(at)
+        q1, s1, o1 = gpu.upload(q), gpu.buffer(rows * groups * 4), gpu.buffer(rows * k * 4)
+        gpu.rope(q1.base(), rows, heads, dim, rope_dims, pb.base(), fb.base(), False)
+        gpu.index_scores(q1.base(), kb.base(), wb.base(), vb.base(), rows, groups, heads, dim, scale, s1.base())
+        gpu.top_k(s1.base(), rows, groups, k, o1.base())
+        scores_1, out_1 = _read(gpu, s1, np.uint32, rows * groups), _read(gpu, o1, np.int32, rows * k)
+        q2 = gpu.upload(q)
+        for run in range(2):
+            s2, o2 = gpu.buffer(rows * groups * 4), gpu.buffer(rows * k * 4)
+            gpu.index_select(q2.base(), kb.base(), wb.base(), vb.base(), rows, groups, heads, dim, scale, (rope_dims, pb.base(), fb.base()),
+                             s2.base(), k, o2.base())
+            assert np.array_equal(_read(gpu, s2, np.uint32, rows * groups), scores_1), (rows, run)
+            assert np.array_equal(_read(gpu, o2, np.int32, rows * k), out_1), (rows, run)
+            gpu.release(s2); gpu.release(o2)
+        assert np.array_equal(_read(gpu, q2, np.uint32, q.size), q.view(np.uint32).ravel()), "q unchanged"
+        # and against the oracle: rotate on the host in double, then the canonical scores and the rule
+        rotated = q.copy()
+        for r in range(rows):
+            angle = float(at[r]) * frequencies.astype(np.float64)
+            a, b = rotated[r, :, dim - rope_dims::2].astype(np.float64), rotated[r, :, dim - rope_dims + 1::2].astype(np.float64)
+            rotated[r, :, dim - rope_dims::2] = (a * np.cos(angle) - b * np.sin(angle)).astype(np.float32)
+            rotated[r, :, dim - rope_dims + 1::2] = (a * np.sin(angle) + b * np.cos(angle)).astype(np.float32)
+        rope_got = _read(gpu, q1, np.float32, q.size).reshape(q.shape)
+        assert np.abs(rope_got - rotated).max() <= 2.4e-7 * 4      # within an ulp of the host's double sincos
+        want_scores = oracle.index_scores(rope_got, keys, weights, visible, scale)
+        assert np.array_equal(want_scores.view(np.uint32).ravel(), scores_1)
+        assert np.array_equal(oracle.top_k(want_scores, k).ravel(), out_1)
+        for b in (kb, wb, vb, pb, q1, s1, o1, q2):
+            gpu.release(b)
+    gpu.release(fb)
+
+
+def test_the_two_level_indexer_matches_its_reference(gpu, oracle):
+    # fused_gpu.rs:476-566 without the projection launch
+    rng = np.random.default_rng(0x1f83)
+    heads, dim, k, blocks, block = 32, 128, 512, 2048, 8
+    for rows, groups in [(1, 20000), (3, 23001)]:
+        keys = (rng.random((groups, dim)) * 2 - 1).astype(np.float32)
+        seen = np.array([16000 if r == 1 else groups - 13 * r for r in range(rows)], dtype=np.int32)
+        scale = float(1.0 / (np.sqrt(np.float32(dim)) * np.sqrt(np.float32(heads))))
+        q = (rng.random((rows, heads, dim)) * 4 - 2).astype(np.float32)
+        weights = (rng.random((rows, heads)) * 2 - 1).astype(np.float32)
+        kb, vb, qb, wb = gpu.upload(keys), gpu.upload(seen), gpu.upload(q), gpu.upload(weights)
+        scores, out = gpu.buffer(rows * groups * 4), gpu.buffer(rows * k * 4)
+        gpu.index_select(qb.base(), kb.base(), wb.base(), vb.base(), rows, groups, heads, dim, scale, None, scores.base(), k, out.base())
+        cand = gpu.buffer(rows * blocks * 4)
+        count = (groups + block - 1) // block
+        scratch = gpu.buffer(rows * count * 4)
+        gpu.index_candidates(scores.base(), vb.base(), rows, groups, blocks, block, cand.base(), scratch)
+        source = _read(gpu, scores, np.float32, rows * groups).reshape(rows, groups)
+        chosen = _read(gpu, cand, np.int32, rows * blocks).reshape(rows, blocks)
+        assert np.array_equal(chosen, oracle.index_candidates(source, seen, blocks, block))
+        keep = np.zeros((rows, groups), dtype=bool)
+        for r in range(rows):
+            for b in chosen[r][chosen[r] >= 0]:
+                keep[r, b * block:(b + 1) * block] = True
+        q2 = (rng.random((rows, heads, dim)) * 4 - 2).astype(np.float32)
+        w2 = (rng.random((rows, heads)) * 2 - 1).astype(np.float32)
+        qb2, wb2 = gpu.upload(q2), gpu.upload(w2)
+        every = oracle.index_scores(q2, keys, w2, seen, scale)
+        masked = np.where(keep, every, -np.inf).astype(np.float32)
+        for run in range(2):
+            s3, o3 = gpu.buffer(rows * max(groups, blocks * block) * 4), gpu.buffer(rows * k * 4)
+            gpu.index_select(qb2.base(), kb.base(), wb2.base(), vb.base(), rows, groups, heads, dim, scale, None, s3.base(), k, o3.base(),
+                             (cand.base(), blocks, block))
+            got = _read(gpu, o3, np.int32, rows * k).reshape(rows, k)
+            assert np.array_equal(got, oracle.top_k(masked, k)), (rows, run)
+            gpu.release(s3); gpu.release(o3)
+        for b in (kb, vb, qb, wb, scores, out, cand, scratch, qb2, wb2):
+            gpu.release(b)
+
+
+def test_sparse_attention_matches_the_oracle_and_bf16_rows_match_f32(gpu, oracle):
+    # ds_state_bf16_gpu.rs:69-110 and the oracle's closed form (window ring, sink, -1 selections, rope in and out)
+    rng = np.random.default_rng(11)
+    from straydog_amd.backend import tagged_bf16
+    for rows, heads, dim, window, raw_rows, n, selections, rope_dims in [(3, 64, 512, 128, 128, 900, 512, 64), (5, 10, 64, 5, 8, 40, 7, 16),
+                                                                         (2, 32, 128, 16, 16, 64, 33, 0)]:
+        q = rng.standard_normal((rows, heads, dim)).astype(np.float32)
+        raw = rng.standard_normal((raw_rows, dim)).astype(np.float32)
+        comp_bits, comp = _bf16_round(oracle, rng.standard_normal((n, dim)).astype(np.float32))
+        positions = np.array([2, 500, 131, 77, 9][:rows], dtype=np.int32)
+        selected = np.stack([rng.permutation(n)[:selections] for _ in range(rows)]).astype(np.int32)
+        selected[0, ::5] = -1
+        sinks = rng.standard_normal(heads).astype(np.float32)
+        freqs = (1.6e5 ** (-(2.0 * np.arange(max(rope_dims // 2, 1))) / max(rope_dims, 1))).astype(np.float32)
+        scale = float(1.0 / np.sqrt(dim))
+        qb, rb, pb, sb, kb, fb = (gpu.upload(x) for x in (q, raw, positions, selected, sinks, freqs))
+        cf, ch = gpu.upload(comp), gpu.upload(comp_bits)
+        out = gpu.buffer(q.size * 4)
+        results = []
+        for compressed in (cf.base(), tagged_bf16(ch.base())):
+            gpu.sparse_attention(qb.base(), rb.base(), raw_rows, pb.base(), window, compressed, n, sb.base(), selections, kb.base(), rows, heads,
+                                 dim, scale, rope_dims, fb.base() if rope_dims else None, None, out.base())
+            results.append(_read(gpu, out, np.float32, q.size).reshape(q.shape))
+        assert np.array_equal(results[0].view(np.uint32), results[1].view(np.uint32)), "BF16 rows and their FP32 values differ"
+        want = oracle.latent_attention(q, raw, positions, window, comp, selected, sinks, dim, scale, rope_dims, freqs if rope_dims else None)
+        assert np.abs(results[0] - want).max() < 5e-5
+        for b in (qb, rb, pb, sb, kb, fb, cf, ch, out):
+            gpu.release(b)
+
+
+def test_batched_sparse_path_small(gpu, oracle):
+    # BASELINE config 4 in small: index scores -> top-k (bit-exact) -> gather attention over BF16 latents, per sequence
+    rng = np.random.default_rng(12)
+    batch, groups, iheads, idim, k, heads, kdim, vdim = 3, 5000, 64, 128, 256, 64, 576, 512
+    q_bits, q_vals = _bf16_round(oracle, rng.standard_normal((batch, iheads, idim)).astype(np.float32))
+    key_bits, key_vals = _bf16_round(oracle, rng.standard_normal((batch, groups, idim)).astype(np.float32))
+    weights = rng.random((batch, iheads)).astype(np.float32)
+    visible = np.array([groups, groups - 100, 200], dtype=np.int32)    # the last row has fewer visible groups than k: -1 padding
+    qb, kb, wb, vb = gpu.upload(q_bits), gpu.upload(key_bits), gpu.upload(weights), gpu.upload(visible)
+    scores, indices = gpu.buffer(batch * groups * 4), gpu.buffer(batch * k * 4)
+    gpu.index_top_k(qb.base(), kb.base(), wb.base(), vb.base(), batch, groups, iheads, idim, 1.0, scores.base(), k, indices.base())
+    got_scores = _read(gpu, scores, np.float32, batch * groups).reshape(batch, groups)
+    got_indices = _read(gpu, indices, np.int32, batch * k).reshape(batch, k)
+    for b in range(batch):
+        want = oracle.index_scores(q_vals[b:b + 1], key_vals[b], weights[b:b + 1], visible[b:b + 1], 1.0)
+        assert np.array_equal(got_scores[b].view(np.uint32), want[0].view(np.uint32))
+        assert np.array_equal(got_indices[b], oracle.top_k(want, k)[0])
+    # without a scores buffer the indices are the same
+    gpu.index_top_k(qb.base(), kb.base(), wb.base(), vb.base(), batch, groups, iheads, idim, 1.0, None, k, indices.base())
+    assert np.array_equal(_read(gpu, indices, np.int32, batch * k).reshape(batch, k), got_indices)
+    aq_bits, aq = _bf16_round(oracle, rng.standard_normal((batch, heads, kdim)).astype(np.float32))
+    lat_bits, lat = _bf16_round(oracle, rng.standard_normal((batch, groups, kdim)).astype(np.float32))
+    ab, lb, out = gpu.upload(aq_bits), gpu.upload(lat_bits), gpu.buffer(batch * heads * vdim * 4)
+    scale = float(1.0 / np.sqrt(kdim))
+    gpu.latent_attention(ab.base(), lb.base(), indices.base(), batch, groups, k, heads, kdim, vdim, scale, out.base())
+    got = _read(gpu, out, np.float32, batch * heads * vdim).reshape(batch, heads, vdim)
+    for b in range(batch):
+        want = oracle.latent_attention(aq[b:b + 1], None, None, 0, lat_bits[b], got_indices[b:b + 1], None, vdim, scale)
+        close_enough(got[b], want[0], f"sequence {b}")
+        assert np.abs(got[b] - want[0]).max() < 5e-5
+    for b in (qb, kb, wb, vb, scores, indices, ab, lb, out):
+        gpu.release(b)

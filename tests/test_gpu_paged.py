@@ -1,0 +1,163 @@
+"""GPU parity of the paged K/V cache path through the C ABI: sdx_kv_write (bit-exact Q8_0 / FP16 rows against the
+oracle's kv_encode restatement) and sdx_paged_attention (decode and verify spans) against the oracle's fp32
+attention on identical seeded inputs, within max-abs 2e-3 and relative 1e-2; plus properties that hold at any size
+(page permutation leaves the output bit-identical, a verify row equals the single-token call at its position, zero
+queries give the mean of the values)."""
+import numpy as np
+import pytest
+
+from gpu_util import backend, close_enough, make_pool
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    with backend() as handle:
+        yield handle
+
+
+@pytest.mark.parametrize("dim,fmt", [(128, "q8"), (256, "q8"), (128, "f16"), (256, "f16")])
+@pytest.mark.parametrize("input_f16", [False, True])
+def test_kv_write_rows_are_bit_exact(gpu, oracle, dim, fmt, input_f16):
+    rng = np.random.default_rng(100 + dim + input_f16)
+    row_bytes = dim + dim // 16 if fmt == "q8" else 2 * dim
+    seqs, span, kv_heads, page_tokens = 3, 5, 2, 32
+    starts = np.array([0, 30, 77], dtype=np.int32)        # row runs that cross page boundaries
+    pages_per = [(int(s) + span + page_tokens - 1) // page_tokens for s in starts]
+    total = sum(pages_per) + 1
+    order = rng.permutation(total)
+    table = np.zeros((seqs, max(pages_per)), dtype=np.int32)
+    at = 0
+    for s in range(seqs):
+        table[s, :pages_per[s]] = order[at:at + pages_per[s]]
+        at += pages_per[s]
+    magnitude = 10.0 ** rng.integers(-3, 3, size=(seqs, span, kv_heads, 1))
+    keys = (rng.standard_normal((seqs, span, kv_heads, dim)) * magnitude).astype(np.float32)
+    values = (rng.standard_normal((seqs, span, kv_heads, dim)) * magnitude).astype(np.float32)
+    keys[0, 0, 0, :32] = 0.0                              # an all-zero block: zero scale, zero bytes
+    keys[1, 2, 1, 5] = 500.0                              # one large value leaves the other blocks alone
+    values[2, 4, 0, 64:96] = -3.0                         # a block of equal magnitudes
+    if input_f16:
+        keys, values = keys.astype(np.float16), values.astype(np.float16)
+    host = np.zeros(oracle.pool_bytes(total, kv_heads, page_tokens, row_bytes), dtype=np.uint8)
+    oracle.kv_write(host, row_bytes, page_tokens, kv_heads, dim, table, starts, keys.astype(np.float32), values.astype(np.float32))
+    pool, buffer = gpu.kv_pool(total, page_tokens, kv_heads, dim, row_bytes)
+    tb, pb, kb, vb = gpu.upload(table), gpu.upload(starts), gpu.upload(keys), gpu.upload(values)
+    gpu.kv_write(pool, tb.base(), table.shape[1], pb.base(), kb.base(), vb.base(), input_f16, seqs, span)
+    got = gpu.read_buffer(buffer, 0, np.uint8, host.size)
+    assert np.array_equal(got, host)
+    for b in (tb, pb, kb, vb, buffer):
+        gpu.release(b)
+
+
+def _run(gpu, pool, table, table_buffer, positions, q, span, heads, scale, q_f16, out_f16, max_context=None):
+    seqs = len(positions)
+    dim = pool.dim
+    max_context = max_context or int(max(positions)) + span
+    max_context = min(max(max_context, 1), table.shape[1] * pool.page_tokens)
+    scratch = gpu.buffer(max(gpu.paged_attention_scratch(seqs, span, heads, dim, max_context), 4))
+    qb = gpu.upload(q.astype(np.float16) if q_f16 else q.astype(np.float32))
+    pb = gpu.upload(np.asarray(positions, dtype=np.int32))
+    out = gpu.buffer(seqs * span * heads * dim * (2 if out_f16 else 4))
+    gpu.paged_attention(pool, table_buffer.base(), table.shape[1], pb.base(), max_context, qb.base(), q_f16, seqs, span, heads, scale,
+                        out.base(), out_f16, scratch)
+    result = gpu.read_buffer(out, 0, np.float16 if out_f16 else np.float32, seqs * span * heads * dim).astype(np.float32)
+    for b in (scratch, qb, pb, out):
+        gpu.release(b)
+    return result.reshape(seqs, span, heads, dim)
+
+
+def test_config0_single_sequence_decode(gpu, oracle):
+    # BASELINE config 0: 1 query token, 16 query heads over 2 K/V heads, head_dim 128, context 4096, fp32 q and output
+    rng = np.random.default_rng(0x9e3779b97f4a7c15 & 0xffffffff)
+    heads, kv_heads, dim, context, page_tokens, row_bytes = 16, 2, 128, 4096, 256, 136
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, [context], kv_heads, dim, page_tokens, row_bytes)
+    q = rng.standard_normal((1, 1, heads, dim)).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    got = _run(gpu, pool, table, tb, [context - 1], q, 1, heads, scale, False, False)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array([context - 1], np.int32), q, scale)
+    worst, relative, size = close_enough(got, want, "config 0")
+    print(f"config 0: max-abs {worst:.2e}, relative L2 {relative:.2e}, output magnitude {size:.2e}")
+    gpu.release(buffer); gpu.release(tb)
+
+
+@pytest.mark.parametrize("dim,fmt,heads,kv_heads", [(128, "q8", 32, 4), (128, "q8", 4, 4), (128, "q8", 12, 1), (256, "q8", 24, 2),
+                                                    (128, "f16", 16, 2), (256, "f16", 8, 2)])
+def test_ragged_batched_decode(gpu, oracle, dim, fmt, heads, kv_heads):
+    # BASELINE config 1 in small: ragged lengths around every boundary of the kernel (1 token, a step of 32, a page, a chunk)
+    rng = np.random.default_rng(7 + dim + heads)
+    row_bytes = dim + dim // 16 if fmt == "q8" else 2 * dim
+    page_tokens = 64
+    lengths = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 700, 1500]
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, lengths, kv_heads, dim, page_tokens, row_bytes)
+    seqs = len(lengths)
+    q = rng.standard_normal((seqs, 1, heads, dim)).astype(np.float16).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    positions = [n - 1 for n in lengths]
+    got = _run(gpu, pool, table, tb, positions, q, 1, heads, scale, True, True)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array(positions, np.int32), q, scale)
+    for s in range(seqs):
+        close_enough(got[s], want[s], f"length {lengths[s]}")
+    # the same pages at other places, the table renamed with them: bit-identical output
+    page_bytes = 2 * kv_heads * page_tokens * row_bytes
+    pages = host.reshape(-1, page_bytes)
+    perm = rng.permutation(pages.shape[0])
+    moved = np.ascontiguousarray(pages[perm]).reshape(-1)
+    renamed = np.argsort(perm).astype(np.int32)[table]
+    gpu.write_buffer(buffer, 0, moved)
+    tb2 = gpu.upload(renamed)
+    again = _run(gpu, pool, renamed, tb2, positions, q, 1, heads, scale, True, True)
+    assert np.array_equal(again.view(np.uint32), got.view(np.uint32))
+    for b in (buffer, tb, tb2):
+        gpu.release(b)
+
+
+@pytest.mark.parametrize("span,heads,kv_heads", [(5, 32, 4), (8, 8, 2), (2, 16, 1), (4, 16, 1)])
+def test_verify_span_rows(gpu, oracle, span, heads, kv_heads):
+    # BASELINE config 3 in small: span rows attend all of the context and causally inside the span
+    rng = np.random.default_rng(31 + span)
+    dim, row_bytes, page_tokens = 128, 136, 64
+    contexts = [0, 27, 64, 300, 1029]
+    lengths = [c + span for c in contexts]
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, lengths, kv_heads, dim, page_tokens, row_bytes)
+    seqs = len(lengths)
+    q = rng.standard_normal((seqs, span, heads, dim)).astype(np.float16).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    got = _run(gpu, pool, table, tb, contexts, q, span, heads, scale, True, False)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array(contexts, np.int32), q, scale)
+    close_enough(got, want, f"span {span}")
+    # row r of the span is the single-token decode at position context + r
+    for r in range(span):
+        single = _run(gpu, pool, table, tb, [c + r for c in contexts], q[:, r:r + 1], 1, heads, scale, True, False,
+                      max_context=max(lengths))
+        close_enough(single[:, 0], want[:, r], f"row {r} alone")
+        assert np.abs(single[:, 0] - got[:, r]).max() < 2e-4
+    gpu.release(buffer); gpu.release(tb)
+
+
+def test_zero_queries_give_the_mean_of_the_values(gpu, oracle):
+    rng = np.random.default_rng(5)
+    heads, kv_heads, dim, row_bytes, page_tokens = 8, 2, 128, 136, 32
+    lengths = [45, 200]
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, lengths, kv_heads, dim, page_tokens, row_bytes)
+    q = np.zeros((2, 1, heads, dim), dtype=np.float32)
+    got = _run(gpu, pool, table, tb, [n - 1 for n in lengths], q, 1, heads, 0.088, False, False)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array([n - 1 for n in lengths], np.int32), q, 0.088)
+    assert np.abs(got - want).max() < 1e-4
+    gpu.release(buffer); gpu.release(tb)
+
+
+def test_refusals(gpu):
+    from straydog_amd.backend import StraydogError
+    pool, buffer = gpu.kv_pool(2, 32, 1, 128, 136)
+    small = gpu.buffer(64)
+    with pytest.raises(StraydogError, match="outside this device's allocations"):
+        gpu.paged_attention(pool, 0x1000, 1, small.base(), 32, small.base(), 0, 1, 1, 8, 0.1, small.base(), 0, small)
+    with pytest.raises(StraydogError, match="scratch too small"):
+        table = gpu.upload(np.zeros(4, np.int32))
+        q = gpu.buffer(8 * 128 * 4)
+        gpu.paged_attention(pool, table.base(), 1, table.base(), 32, q.base(), 0, 1, 1, 8, 0.1, q.base(), 0, small)
+    bad = type(pool)(buffer.pointer, 2, 33, 1, 128, 136)
+    with pytest.raises(StraydogError, match="invalid Straydog K/V pool"):
+        gpu.kv_write(bad, small.base(), 1, small.base(), small.base(), small.base(), False, 1, 1)
