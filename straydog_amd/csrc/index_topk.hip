@@ -16,6 +16,18 @@ namespace {
 
 __device__ __forceinline__ float bf16_value(uint16_t bits) { return __uint_as_float(uint32_t(bits) << 16); }
 
+// sum + round(a * b): the product is rounded on its own, never contracted with the add into a fused multiply-add
+// (the rule of the reference's canonical score order, gpu/ops.hpp:2171-2187).
+__device__ __forceinline__ float add_rounded_product(float sum, float a, float b) {
+    #pragma clang fp contract(off)
+    const float product = a * b;
+    return sum + product;
+}
+__device__ __forceinline__ float rounded_product(float a, float b) {
+    #pragma clang fp contract(off)
+    return a * b;
+}
+
 __global__ void to_bf16_kernel(const float* x, size_t count, uint16_t* out) {
     for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) {
         const uint32_t bits = __float_as_uint(x[i]);
@@ -137,11 +149,10 @@ __global__ void __launch_bounds__(256) index_scores_kernel(const float* __restri
     for (int h = 0; h < H; ++h) {
         if (size_t(h) < heads) {
             // the term is rounded before it joins the sum: keep the multiply and the add apart
-            const float term = __fmul_rn(fmaxf(acc[h], 0.0f), weights[row * heads + h]);
-            total = __fadd_rn(total, term);
+            total = add_rounded_product(total, fmaxf(acc[h], 0.0f), weights[row * heads + h]);
         }
     }
-    scores[row * score_stride + place] = g < limit ? __fmul_rn(total, scale) : -INFINITY;
+    scores[row * score_stride + place] = g < limit ? rounded_product(total, scale) : -INFINITY;
 }
 
 // ---- top-k -------------------------------------------------------------------------------------------------

@@ -245,7 +245,7 @@ def test_the_two_level_indexer_matches_its_reference(gpu, oracle):
         weights = (rng.random((rows, heads)) * 2 - 1).astype(np.float32)
         kb, vb, qb, wb = gpu.upload(keys), gpu.upload(seen), gpu.upload(q), gpu.upload(weights)
         scores, out = gpu.buffer(rows * groups * 4), gpu.buffer(rows * k * 4)
-        gpu.index_select(qb.base(), kb.base(), wb.base(), vb.base(), rows, groups, heads, dim, scale, None, scores.base(), k, out.base())
+        gpu.index_select(qb.base(), kb.base(), wb.base(), vb.base(), rows, groups, heads, dim, scale, (0, vb.base(), None), scores.base(), k, out.base())
         cand = gpu.buffer(rows * blocks * 4)
         count = (groups + block - 1) // block
         scratch = gpu.buffer(rows * count * 4)
@@ -264,7 +264,7 @@ def test_the_two_level_indexer_matches_its_reference(gpu, oracle):
         masked = np.where(keep, every, -np.inf).astype(np.float32)
         for run in range(2):
             s3, o3 = gpu.buffer(rows * max(groups, blocks * block) * 4), gpu.buffer(rows * k * 4)
-            gpu.index_select(qb2.base(), kb.base(), wb2.base(), vb.base(), rows, groups, heads, dim, scale, None, s3.base(), k, o3.base(),
+            gpu.index_select(qb2.base(), kb.base(), wb2.base(), vb.base(), rows, groups, heads, dim, scale, (0, vb.base(), None), s3.base(), k, o3.base(),
                              (cand.base(), blocks, block))
             got = _read(gpu, o3, np.int32, rows * k).reshape(rows, k)
             assert np.array_equal(got, oracle.top_k(masked, k)), (rows, run)
