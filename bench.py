@@ -1,0 +1,177 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+A step is one pass of the Q8_0 paged grouped-query decode attention (sdx_paged_attention: split kernel + merge) over
+one batch of synthetic, HBM-resident inputs.  The default workload is BASELINE.json configs[1]: 32 sequences with
+lengths drawn uniformly from [1024, 32768], 32 query heads over 4 K/V heads, head_dim 128, 256-token pages behind a
+shuffled page table, FP16 queries and outputs.  The one JSON line also carries, under "also", the all-32768-token case
+of the same shape (the north-star target), config 0, the verify span of config 3 and the sparse path of config 4.
+
+    python bench.py --gpus 1 --steps 50 --warmup 10 [--workload config1|config1_32k|config0|config3|config4]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+
+
+def timed(gpu, step, steps, warmup):
+    """(ms per step over the whole stream, ms per launch of the dominant kernel) for `steps` steps after `warmup`."""
+    for _ in range(warmup):
+        step()
+    gpu.synchronize()
+    gpu.profile(True)
+    begin = gpu.event()
+    for _ in range(steps):
+        step()
+    end = gpu.event()
+    total = gpu.elapsed_ms(begin, end)
+    kernel_ms, launches = gpu.profile_read()
+    gpu.profile(False)
+    gpu.events_clear()
+    return total / steps, (kernel_ms / launches if launches else None)
+
+
+def copy_ceiling(gpu, size=1 << 30, repeats=10):
+    """Measured GB/s (read + write) of the library's plain copy kernel: the practical HBM ceiling on this box."""
+    a, b = gpu.buffer(size), gpu.buffer(size)
+    for _ in range(3):
+        gpu.copy(b.base(), a.base(), size)
+    gpu.synchronize()
+    begin = gpu.event()
+    for _ in range(repeats):
+        gpu.copy(b.base(), a.base(), size)
+    end = gpu.event()
+    ms = gpu.elapsed_ms(begin, end) / repeats
+    gpu.events_clear()
+    gpu.release(a); gpu.release(b)
+    return 2 * size / ms / 1e6
+
+
+def paged_result(gpu, work, steps, warmup):
+    ms, kernel_ms = timed(gpu, work.step, steps, warmup)
+    size = work.algorithmic_bytes()
+    return {
+        "ms_per_step": ms, "us_per_step": ms * 1e3, "kernel_us": None if kernel_ms is None else kernel_ms * 1e3,
+        "algorithmic_bytes": size, "gbps": size / ms / 1e6, "frac_of_hbm_peak": size / ms / 1e6 / HBM_PEAK_GBPS,
+        "kernel_gbps": None if kernel_ms is None else size / kernel_ms / 1e6,
+        "tokens_per_s": work.seqs * work.span / (ms * 1e-3), "tflops": work.flops() / ms / 1e9,
+    }
+
+
+def cpu_baseline_paged(work, sample_seqs, threads):
+    """The CPU oracle on a bounded sample of the same workload (the first `sample_seqs` sequences), timed on this host's
+    cores; also returns the GPU-vs-oracle error on that sample."""
+    import oracle
+    pool = work.read_pool()
+    q = work.read_queries()[:sample_seqs]
+    got = work.read_output()[:sample_seqs]
+    table, positions = work.table[:sample_seqs], work.positions[:sample_seqs]
+    start = time.perf_counter()
+    want = oracle.paged_attention(pool, work.row_bytes, work.page_tokens, work.kv_heads, work.dim, table, positions, q, work.scale,
+                                  threads=threads)
+    seconds = time.perf_counter() - start
+    rows = int(work.lengths[:sample_seqs].sum()) * work.kv_heads * 2 * work.row_bytes
+    error = float(np.abs(got - want).max())
+    return {"value": rows / seconds / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"first {sample_seqs} of {work.seqs} sequences of the same workload ({int(work.lengths[:sample_seqs].sum())} cached tokens), "
+                      f"{seconds:.2f} s, OpenMP over (sequence, K/V head)",
+            "tokens_per_s": sample_seqs * work.span / seconds}, error
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=50)
+    parser.add_argument("--warmup", type=int, default=10)
+    parser.add_argument("--workload", default="config1")
+    parser.add_argument("--no-also", action="store_true", help="measure only the named workload")
+    parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no second device); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    from straydog_amd.backend import Backend
+    from straydog_amd import workloads
+
+    gpu = Backend(0, 64 << 30)
+    lengths = workloads.config1_lengths()
+    builders = {
+        "config1": lambda: workloads.PagedWorkload(gpu, lengths, seed=1),
+        "config1_32k": lambda: workloads.PagedWorkload(gpu, [32768] * 32, seed=2),
+        "config0": lambda: workloads.PagedWorkload(gpu, [4096], heads=16, kv_heads=2, seed=3, q_f16=False, out_f16=False),
+        "config3": lambda: workloads.PagedWorkload(gpu, [65536 + 5] * 16, span=5, seed=5),
+    }
+    names = {
+        "config1": "configs[1]: 32 seqs, len~U[1024,32768], 32q/4kv heads, d128, Q8_0 pages of 256, fp16 q/out",
+        "config1_32k": "configs[1] shape with all 32 sequences at 32768 tokens",
+        "config0": "configs[0]: 1 seq, ctx 4096, 16q/2kv heads, d128, fp32 q/out",
+        "config3": "configs[3]: 16 seqs, ctx 65536 + span 5, 32q/4kv heads, d128, Q8_0 pages of 256",
+        "config4": "configs[4]: batch 8, ctx 131072, 64x128 bf16 indexer, top-2048, 64 heads over bf16 latents 576/512",
+    }
+    ceiling = copy_ceiling(gpu)
+
+    def run_paged(name, with_cpu):
+        work = builders[name]()
+        result = paged_result(gpu, work, args.steps, args.warmup)
+        baseline = None
+        if with_cpu:
+            threads = min(os.cpu_count() or 1, 16)
+            sample = {"config1": 8, "config1_32k": 4, "config0": 1, "config3": 1}[name]
+            baseline, error = cpu_baseline_paged(work, min(sample, work.seqs), threads)
+            result["max_abs_error_vs_oracle_on_sample"] = error
+        work.release()
+        return result, baseline
+
+    def run_sparse():
+        work = workloads.SparseWorkload(gpu)
+        ms_index, _ = timed(gpu, work.step_index, max(args.steps // 5, 3), 2)
+        ms_attention, _ = timed(gpu, work.step_attention, max(args.steps // 5, 3), 2)
+        size = work.algorithmic_bytes()
+        work.release()
+        total = ms_index + ms_attention
+        return {"us_per_step": total * 1e3, "index_topk_us": ms_index * 1e3, "gather_attention_us": ms_attention * 1e3,
+                "algorithmic_bytes": size, "gbps": size / total / 1e6, "frac_of_hbm_peak": size / total / 1e6 / HBM_PEAK_GBPS}
+
+    if args.workload == "config4":
+        main_result, baseline = run_sparse(), None
+    else:
+        main_result, baseline = run_paged(args.workload, not args.no_cpu)
+    also = {}
+    if not args.no_also:
+        for name in ("config1_32k", "config0", "config3"):
+            if name != args.workload:
+                also[name], _ = run_paged(name, False)
+                also[name]["workload"] = names[name]
+        if args.workload != "config4":
+            also["config4"] = run_sparse()
+            also["config4"]["workload"] = names["config4"]
+
+    kernel_us = main_result.get("kernel_us")
+    achieved = main_result["algorithmic_bytes"] / (kernel_us * 1e-6) / 1e9 if kernel_us else main_result["gbps"]
+    line = {
+        "metric": "Q8_0 decode-attn HBM GB/s", "value": main_result["gbps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": main_result.get("ms_per_step", main_result["us_per_step"] / 1e3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int8 K/V x fp16 MFMA, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": names[args.workload], "batch": 32 if args.workload.startswith("config1") else None},
+        "tokens_per_s": main_result.get("tokens_per_s"), "frac_of_hbm_peak": main_result["frac_of_hbm_peak"],
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": None, "kernel": "paged_attention_kernel<128,1,Q8_0>" if args.workload != "config4" else "index_scores_kernel",
+                     "kernel_us": kernel_us, "measured_copy_gbps": ceiling},
+        "cpu_baseline": baseline, "detail": main_result, "also": also,
+    }
+    print(json.dumps(line))
+    gpu.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -183,6 +183,15 @@ class Backend:
     def events_clear(self):
         self.check(self.lib.sdx_events_clear(self.handle))
 
+    def profile(self, enable):
+        self.check(self.lib.sdx_profile(self.handle, int(enable)))
+
+    def profile_read(self):
+        """(summed milliseconds of the ops' dominant kernels, launches) since profiling was enabled."""
+        ms, launches = ctypes.c_double(), abi.c_u64()
+        self.check(self.lib.sdx_profile_read(self.handle, ctypes.byref(ms), ctypes.byref(launches)))
+        return ms.value, launches.value
+
     def compute_units(self):
         return self.check(self.lib.sdx_device_compute_units(self.handle))
 

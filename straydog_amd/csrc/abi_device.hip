@@ -178,6 +178,7 @@ void sd_destroy(void* handle) {
     if (d->stream) (void)hipStreamSynchronize(d->stream);
     for (const auto& entry : d->allocations) (void)hipFree(const_cast<uint8_t*>(entry.first));
     for (auto& event : d->events) if (event) (void)hipEventDestroy(event);
+    for (auto& event : d->profile_events) (void)hipEventDestroy(event);
     if (d->arena) (void)hipHostFree(d->arena);
     if (d->stream) (void)hipStreamDestroy(d->stream);
     delete d;
@@ -333,6 +334,33 @@ int sdx_events_clear(void* handle) {
         Device& d = device(handle);
         SD_CHECK(hipStreamSynchronize(d.stream));
         while (d.events.size() > 2) { SD_CHECK(hipEventDestroy(d.events.back())); d.events.pop_back(); }
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sdx_profile(void* handle, int enable) {
+    try {
+        Device& d = device(handle);
+        SD_CHECK(hipStreamSynchronize(d.stream));
+        for (auto& event : d.profile_events) (void)hipEventDestroy(event);
+        d.profile_events.clear();
+        d.profile = enable != 0;
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sdx_profile_read(void* handle, double* milliseconds, uint64_t* launches) {
+    try {
+        Device& d = device(handle);
+        SD_CHECK(hipStreamSynchronize(d.stream));
+        double total = 0.0;
+        for (size_t i = 0; i + 1 < d.profile_events.size(); i += 2) {
+            float ms = 0.0f;
+            SD_CHECK(hipEventElapsedTime(&ms, d.profile_events[i], d.profile_events[i + 1]));
+            total += ms;
+        }
+        if (milliseconds) *milliseconds = total;
+        if (launches) *launches = d.profile_events.size() / 2;
         return 0;
     } catch (const std::exception& e) { last_error = e.what(); return -1; }
 }

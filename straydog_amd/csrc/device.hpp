@@ -52,6 +52,23 @@ struct Device {
     void* sequence_output = nullptr; size_t sequence_output_bytes = 0;
     void* workspace = nullptr; size_t workspace_bytes = 0;
     std::vector<hipEvent_t> events;
+    // Optional kernel timing for harnesses (sdx_profile): event pairs around the launches of the op's main kernel.
+    bool profile = false;
+    std::vector<hipEvent_t> profile_events;
+};
+
+// Brackets one kernel launch with events when the device's profiling is on.
+struct KernelTimer {
+    Device& d;
+    explicit KernelTimer(Device& device) : d(device) { mark(); }
+    ~KernelTimer() { mark(); }
+    void mark() {
+        if (!d.profile) return;
+        hipEvent_t event;
+        if (hipEventCreate(&event) != hipSuccess) return;
+        (void)hipEventRecord(event, d.stream);
+        d.profile_events.push_back(event);
+    }
 };
 
 Device& device(void* handle);                         // sets the HIP device of the handle; throws on null

@@ -409,8 +409,11 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
     args.partial = static_cast<float*>(scratch);
     const dim3 grid(args.chunks, pool->kv_heads, unsigned(seqs));
     const bool q8 = pool->row_bytes != 2 * pool->dim;
+    {
+    KernelTimer timer(value);
     if (pool->dim == 128) { if (q8) launch<128, true>(value, args, query_tiles, grid); else launch<128, false>(value, args, query_tiles, grid); }
     else { if (q8) launch<256, true>(value, args, query_tiles, grid); else launch<256, false>(value, args, query_tiles, grid); }
+    }
     SD_CHECK(hipGetLastError());
     const unsigned items = unsigned(checked_product({seqs, span, heads}));
     if (pool->dim == 128) {

@@ -1,0 +1,144 @@
+"""Synthetic workloads of the attention path, built on the GPU through the C ABI (no host-side arithmetic):
+the BASELINE configurations' shapes with seeded N(0,1) inputs, K/V quantised into the paged cache by the
+library's own writer.  Used by bench.py, __graft_entry__.smoke() and the full-size GPU tests."""
+import numpy as np
+
+ROW_Q8 = {128: 136, 256: 272}
+
+
+class PagedWorkload:
+    """A batch of sequences in a shuffled paged Q8_0 cache, with `span` query rows each."""
+
+    def __init__(self, gpu, lengths, span=1, heads=32, kv_heads=4, dim=128, page_tokens=256, seed=1, q_f16=True, out_f16=True,
+                 row_bytes=None):
+        self.gpu, self.span, self.heads, self.kv_heads, self.dim, self.page_tokens = gpu, span, heads, kv_heads, dim, page_tokens
+        self.lengths = np.asarray(lengths, dtype=np.int64)            # cached tokens per sequence, the span's rows included
+        self.seqs = len(lengths)
+        self.row_bytes = row_bytes or ROW_Q8[dim]
+        self.q_f16, self.out_f16 = q_f16, out_f16
+        rng = np.random.default_rng(seed)
+        pages_per = (self.lengths + page_tokens - 1) // page_tokens
+        self.page_count = int(pages_per.sum())
+        self.table_stride = int(pages_per.max())
+        order = rng.permutation(self.page_count).astype(np.int32)
+        self.table = np.zeros((self.seqs, self.table_stride), dtype=np.int32)
+        at = 0
+        for s in range(self.seqs):
+            self.table[s, :pages_per[s]] = order[at:at + pages_per[s]]
+            at += int(pages_per[s])
+        self.positions = (self.lengths - span).astype(np.int32)       # position of each sequence's first query row
+        self.max_context = int(self.lengths.max())
+        self.scale = float(1.0 / np.sqrt(np.float32(dim)))
+        self.pool, self.pool_buffer = gpu.kv_pool(self.page_count, page_tokens, kv_heads, dim, self.row_bytes)
+        self.table_buffer = gpu.upload(self.table)
+        self.position_buffer = gpu.upload(self.positions)
+        # K/V: N(0,1) generated on the device a sequence at a time, quantised by sdx_kv_write
+        longest = int(self.lengths.max())
+        stage_k = gpu.buffer(longest * kv_heads * dim * 4)
+        stage_v = gpu.buffer(longest * kv_heads * dim * 4)
+        zero = gpu.upload(np.zeros(1, dtype=np.int32))
+        for s in range(self.seqs):
+            n = int(self.lengths[s])
+            gpu.fill_normal(stage_k.base(), n * kv_heads * dim, seed * 1000003 + 2 * s, 0)
+            gpu.fill_normal(stage_v.base(), n * kv_heads * dim, seed * 1000003 + 2 * s + 1, 0)
+            gpu.kv_write(self.pool, self.table_buffer.at(s * self.table_stride * 4), self.table_stride, zero.base(), stage_k.base(),
+                         stage_v.base(), False, 1, n)
+        gpu.synchronize()
+        for b in (stage_k, stage_v, zero):
+            gpu.release(b)
+        count = self.seqs * span * heads * dim
+        self.q_buffer = gpu.buffer(count * (2 if q_f16 else 4))
+        gpu.fill_normal(self.q_buffer.base(), count, seed * 7919 + 5, 1 if q_f16 else 0)
+        self.out_buffer = gpu.buffer(count * (2 if out_f16 else 4))
+        self.scratch = gpu.buffer(max(gpu.paged_attention_scratch(self.seqs, span, heads, dim, self.max_context), 4))
+        gpu.synchronize()
+
+    def step(self):
+        g = self.gpu
+        g.paged_attention(self.pool, self.table_buffer.base(), self.table_stride, self.position_buffer.base(), self.max_context,
+                          self.q_buffer.base(), self.q_f16, self.seqs, self.span, self.heads, self.scale, self.out_buffer.base(),
+                          self.out_f16, self.scratch)
+
+    def algorithmic_bytes(self):
+        """Bytes one step must move: every cached row of every K/V head once (keys and values), the page-table entries,
+        the queries and the outputs."""
+        rows = int(self.lengths.sum()) * self.kv_heads * 2 * self.row_bytes
+        table = int(((self.lengths + self.page_tokens - 1) // self.page_tokens).sum()) * 4
+        io = self.seqs * self.span * self.heads * self.dim * ((2 if self.q_f16 else 4) + (2 if self.out_f16 else 4))
+        return rows + table + io
+
+    def flops(self):
+        # 2 products (QK^T and PV) x 2 flops per (query row, key, column)
+        visible = sum(int(self.lengths[s] - self.span + r + 1) for s in range(self.seqs) for r in range(self.span))
+        return 4 * self.heads * self.dim * visible
+
+    def read_output(self):
+        count = self.seqs * self.span * self.heads * self.dim
+        out = self.gpu.read_buffer(self.out_buffer, 0, np.float16 if self.out_f16 else np.float32, count)
+        return out.astype(np.float32).reshape(self.seqs, self.span, self.heads, self.dim)
+
+    def read_queries(self):
+        count = self.seqs * self.span * self.heads * self.dim
+        q = self.gpu.read_buffer(self.q_buffer, 0, np.float16 if self.q_f16 else np.float32, count)
+        return q.astype(np.float32).reshape(self.seqs, self.span, self.heads, self.dim)
+
+    def read_pool(self):
+        return self.gpu.read_buffer(self.pool_buffer, 0, np.uint8, self.pool_buffer.size)
+
+    def release(self):
+        for b in (self.pool_buffer, self.table_buffer, self.position_buffer, self.q_buffer, self.out_buffer, self.scratch):
+            self.gpu.release(b)
+
+
+class SparseWorkload:
+    """BASELINE config 4: per sequence, index scores over BF16 keys -> top-k -> gather attention over BF16 latents."""
+
+    def __init__(self, gpu, batch=8, context=131072, index_heads=64, index_dim=128, k=2048, heads=64, kdim=576, vdim=512, seed=4):
+        self.gpu, self.batch, self.context, self.index_heads, self.index_dim = gpu, batch, context, index_heads, index_dim
+        self.k, self.heads, self.kdim, self.vdim = k, heads, kdim, vdim
+        self.scale = float(1.0 / np.sqrt(np.float32(kdim)))
+        self.q_index = gpu.buffer(batch * index_heads * index_dim * 2)
+        self.keys = gpu.buffer(batch * context * index_dim * 2)
+        self.weights = gpu.buffer(batch * index_heads * 4)
+        self.visible = gpu.upload(np.full(batch, context, dtype=np.int32))
+        self.scores = gpu.buffer(batch * context * 4)
+        self.indices = gpu.buffer(batch * k * 4)
+        self.q = gpu.buffer(batch * heads * kdim * 2)
+        self.latents = gpu.buffer(batch * context * kdim * 2)
+        self.out = gpu.buffer(batch * heads * vdim * 4)
+        gpu.fill_normal(self.q_index.base(), batch * index_heads * index_dim, seed * 11 + 1, 2)
+        gpu.fill_normal(self.keys.base(), batch * context * index_dim, seed * 11 + 2, 2)
+        gpu.fill_uniform(self.weights.base(), batch * index_heads, seed * 11 + 3, 0.0, 1.0)
+        gpu.fill_normal(self.q.base(), batch * heads * kdim, seed * 11 + 4, 2)
+        gpu.fill_normal(self.latents.base(), batch * context * kdim, seed * 11 + 5, 2)
+        gpu.synchronize()
+
+    def step_index(self, keep_scores=True):
+        g = self.gpu
+        g.index_top_k(self.q_index.base(), self.keys.base(), self.weights.base(), self.visible.base(), self.batch, self.context,
+                      self.index_heads, self.index_dim, 1.0, self.scores.base() if keep_scores else None, self.k, self.indices.base())
+
+    def step_attention(self):
+        g = self.gpu
+        g.latent_attention(self.q.base(), self.latents.base(), self.indices.base(), self.batch, self.context, self.k, self.heads,
+                           self.kdim, self.vdim, self.scale, self.out.base())
+
+    def step(self):
+        self.step_index()
+        self.step_attention()
+
+    def algorithmic_bytes(self):
+        keys = self.batch * self.context * self.index_dim * 2
+        gather = self.batch * self.k * self.kdim * 2
+        small = self.batch * (self.index_heads * self.index_dim * 2 + self.index_heads * 4 + self.k * 4 + self.heads * self.kdim * 2 +
+                              self.heads * self.vdim * 4)
+        return keys + gather + small
+
+    def release(self):
+        for b in (self.q_index, self.keys, self.weights, self.visible, self.scores, self.indices, self.q, self.latents, self.out):
+            self.gpu.release(b)
+
+
+def config1_lengths(seed=0x9e3779b97f4a7c15 ^ 1, seqs=32, low=1024, high=32768):
+    rng = np.random.default_rng(seed & 0xffffffff)
+    return rng.integers(low, high + 1, size=seqs)
