@@ -17,6 +17,8 @@
 
 #include <hip/hip_fp16.h>
 
+#include <cstdlib>
+
 namespace sd { void validate_pool(Device& d, const sdx_kv_pool* pool); }
 using namespace sd;
 
@@ -45,45 +47,64 @@ struct PagedArgs {
 
 __device__ __forceinline__ half2v as_half2(uint32_t bits) { return __builtin_bit_cast(half2v, bits); }
 
-// Two int8 (already xor 0x80, in bits 0-7 and 16-23 of `pair`, zeros elsewhere) -> their values times `scale`, as two FP16:
-// 0x6400 | u is the FP16 1024 + u, exactly; minus 1152 leaves the signed byte; one rounding by the scale.
-__device__ __forceinline__ half2v bytes_to_half2(uint32_t pair, half2v scale) {
+// v_perm_b32: byte i of the result is byte sel[i] of the 8 bytes {high, low} (0-3 = low's bytes, 4-7 = high's, 0x0c = 0x00).
+__device__ __forceinline__ uint32_t byte_perm(uint32_t high, uint32_t low, uint32_t sel) { return __builtin_amdgcn_perm(high, low, sel); }
+
+// Two bytes u (an int8 xor 0x80) sitting in FP16 patterns 0x64uu: 0x6400 | u is the FP16 1024 + u exactly; minus 1152 leaves the
+// signed byte; one rounding by the block scale (the reference's qsa_q8_half16, gpu/qsa_prompt_attention.hpp:15-33).
+__device__ __forceinline__ half2v magic_to_half2(uint32_t pattern, half2v scale) {
     const half2v bias = {(_Float16)1152.0f, (_Float16)1152.0f};
-    return (as_half2(pair | 0x64006400u) - bias) * scale;
+    return (as_half2(pattern) - bias) * scale;
 }
+
+// Per-lane byte offsets of the rows a step reads, from the step's first row of the K (or V) plane.  They are the same for
+// every full step, so they are formed once; a last, partial step clamps its tokens to the last valid one.
+template<int DIM, bool Q8> struct LaneOffsets {
+    static constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, W = DIM / 16;
+    uint32_t k[2], ks[2], v[8], vs[8];
+    __device__ __forceinline__ void set(int valid, int li, int g) {
+        #pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint32_t row = uint32_t(min(16 * t + li, valid - 1)) * ROW;
+            k[t] = row + (Q8 ? 8 * g : 16 * g);
+            ks[t] = row + DIM;
+        }
+        #pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t row = uint32_t(min(e < 4 ? 4 * g + e : 16 + 4 * g + (e - 4), valid - 1)) * ROW;
+            v[e] = row + (Q8 ? W * li : 2 * W * li);
+            vs[e] = row + DIM + 2 * ((W * li) / 32);
+        }
+    }
+};
 
 template<int DIM, bool Q8> struct RowLoad;
 
 // What one step needs from HBM, as raw words.  Q8_0: K tile t (16 tokens, lane li = token) gives each lane 8 columns of
-// every 32-column block (blocks x uint2) and the row's scales; V gives lane (li, g) the columns [W*li, W*li + W) (W = DIM/16)
-// of its 8 tokens {4g..4g+3, 16+4g..16+4g+3} and those columns' block scale.
+// every 32-column block and the row's scales; V gives lane (li, g) the columns [W*li, W*li + W) (W = DIM/16) of its 8
+// tokens {4g..4g+3, 16+4g..16+4g+3} and those columns' block scale.
 template<int DIM> struct RowLoad<DIM, true> {
-    static constexpr int BLOCKS = DIM / 32, W = DIM / 16, VWORDS = W / 4;
+    static constexpr int BLOCKS = DIM / 32, W = DIM / 16;
     uint2 k[2][BLOCKS];
     uint32_t kscale[2][BLOCKS / 2];
-    uint32_t v[8][VWORDS];
+    uint32_t v[8][W / 4];
     uint16_t vscale[8];
 };
-
 template<int DIM>
-__device__ __forceinline__ void load_step(RowLoad<DIM, true>& r, const uint8_t* kplane, const uint8_t* vplane, int valid, int li, int g) {
-    constexpr int ROW = DIM + DIM / 16, BLOCKS = DIM / 32, W = DIM / 16;
+__device__ __forceinline__ void load_step(RowLoad<DIM, true>& r, const uint8_t* kplane, const uint8_t* vplane, const LaneOffsets<DIM, true>& o) {
+    constexpr int BLOCKS = DIM / 32, W = DIM / 16;
     #pragma unroll
     for (int t = 0; t < 2; ++t) {
-        const int token = min(16 * t + li, valid - 1);
-        const uint8_t* row = kplane + size_t(token) * ROW;
         #pragma unroll
-        for (int b = 0; b < BLOCKS; ++b) r.k[t][b] = *reinterpret_cast<const uint2*>(row + 32 * b + 8 * g);
+        for (int b = 0; b < BLOCKS; ++b) r.k[t][b] = *reinterpret_cast<const uint2*>(kplane + o.k[t] + 32 * b);
         #pragma unroll
-        for (int b = 0; b < BLOCKS / 2; ++b) r.kscale[t][b] = *reinterpret_cast<const uint32_t*>(row + DIM + 4 * b);
+        for (int b = 0; b < BLOCKS / 2; ++b) r.kscale[t][b] = *reinterpret_cast<const uint32_t*>(kplane + o.ks[t] + 4 * b);
     }
     #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        const int token = min((e < 4 ? 4 * g + e : 16 + 4 * g + (e - 4)), valid - 1);
-        const uint8_t* row = vplane + size_t(token) * ROW;
         #pragma unroll
-        for (int w = 0; w < W / 4; ++w) r.v[e][w] = *reinterpret_cast<const uint32_t*>(row + W * li + 4 * w);
-        r.vscale[e] = *reinterpret_cast<const uint16_t*>(row + DIM + 2 * ((W * li) / 32));
+        for (int w = 0; w < W / 4; ++w) r.v[e][w] = *reinterpret_cast<const uint32_t*>(vplane + o.v[e] + 4 * w);
+        r.vscale[e] = *reinterpret_cast<const uint16_t*>(vplane + o.vs[e]);
     }
 }
 
@@ -93,72 +114,72 @@ template<int DIM> struct RowLoad<DIM, false> {
     half8 k[2][BLOCKS];
     uint32_t v[8][W / 2];
 };
-
 template<int DIM>
-__device__ __forceinline__ void load_step(RowLoad<DIM, false>& r, const uint8_t* kplane, const uint8_t* vplane, int valid, int li, int g) {
-    constexpr int ROW = 2 * DIM, BLOCKS = DIM / 32, W = DIM / 16;
+__device__ __forceinline__ void load_step(RowLoad<DIM, false>& r, const uint8_t* kplane, const uint8_t* vplane, const LaneOffsets<DIM, false>& o) {
+    constexpr int BLOCKS = DIM / 32, W = DIM / 16;
     #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        const int token = min(16 * t + li, valid - 1);
-        const uint8_t* row = kplane + size_t(token) * ROW;
+    for (int t = 0; t < 2; ++t)
         #pragma unroll
-        for (int b = 0; b < BLOCKS; ++b) r.k[t][b] = *reinterpret_cast<const half8*>(row + 2 * (32 * b + 8 * g));
-    }
+        for (int b = 0; b < BLOCKS; ++b) r.k[t][b] = *reinterpret_cast<const half8*>(kplane + o.k[t] + 64 * b);
     #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const int token = min((e < 4 ? 4 * g + e : 16 + 4 * g + (e - 4)), valid - 1);
-        const uint8_t* row = vplane + size_t(token) * ROW;
+    for (int e = 0; e < 8; ++e)
         #pragma unroll
-        for (int w = 0; w < W / 2; ++w) r.v[e][w] = *reinterpret_cast<const uint32_t*>(row + 2 * W * li + 4 * w);
-    }
+        for (int w = 0; w < W / 2; ++w) r.v[e][w] = *reinterpret_cast<const uint32_t*>(vplane + o.v[e] + 4 * w);
 }
 
 // The A operand of S^T = K . Q^T for tile t, block b.
 template<int DIM>
 __device__ __forceinline__ half8 key_operand(const RowLoad<DIM, true>& r, int t, int b) {
     const uint32_t pairs = r.kscale[t][b / 2];
-    const uint32_t one = (b & 1) ? (pairs >> 16) : (pairs & 0xffffu);
-    const half2v scale = as_half2(one | (one << 16));
+    const half2v scale = as_half2((b & 1) ? byte_perm(pairs, pairs, 0x03020302u) : byte_perm(pairs, pairs, 0x01000100u));
+    const uint32_t magic = 0x64646464u;
     const uint32_t lo = r.k[t][b].x ^ 0x80808080u, hi = r.k[t][b].y ^ 0x80808080u;
-    const half2v a0 = bytes_to_half2((lo & 0xffu) | ((lo << 8) & 0xff0000u), scale);
-    const half2v a1 = bytes_to_half2(((lo >> 16) & 0xffu) | ((lo >> 8) & 0xff0000u), scale);
-    const half2v a2 = bytes_to_half2((hi & 0xffu) | ((hi << 8) & 0xff0000u), scale);
-    const half2v a3 = bytes_to_half2(((hi >> 16) & 0xffu) | ((hi >> 8) & 0xff0000u), scale);
+    const half2v a0 = magic_to_half2(byte_perm(magic, lo, 0x04010400u), scale);
+    const half2v a1 = magic_to_half2(byte_perm(magic, lo, 0x04030402u), scale);
+    const half2v a2 = magic_to_half2(byte_perm(magic, hi, 0x04010400u), scale);
+    const half2v a3 = magic_to_half2(byte_perm(magic, hi, 0x04030402u), scale);
     return half8{a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
 }
 template<int DIM>
 __device__ __forceinline__ half8 key_operand(const RowLoad<DIM, false>& r, int t, int b) { return r.k[t][b]; }
 
+// The scales of the lane's 8 tokens as 4 FP16 pairs (tokens e, e+1), formed once a step.
+template<int DIM> struct ValueScales { half2v pair[4]; };
+template<int DIM>
+__device__ __forceinline__ void value_scales(const RowLoad<DIM, true>& r, ValueScales<DIM>& s) {
+    #pragma unroll
+    for (int e = 0; e < 8; e += 2) s.pair[e / 2] = as_half2(uint32_t(r.vscale[e]) | (uint32_t(r.vscale[e + 1]) << 16));
+}
+template<int DIM>
+__device__ __forceinline__ void value_scales(const RowLoad<DIM, false>&, ValueScales<DIM>&) {}
+
 // The A operand of O^T += V^T . P^T for output tile jj: column W*li + jj of the lane's 8 tokens.
 template<int DIM>
-__device__ __forceinline__ half8 value_operand(const RowLoad<DIM, true>& r, int jj) {
+__device__ __forceinline__ half8 value_operand(const RowLoad<DIM, true>& r, const ValueScales<DIM>& s, int jj) {
     half2v out[4];
-    const int word = jj / 4, shift = 8 * (jj % 4);
+    const int word = jj / 4;
+    // bytes (jj % 4) of tokens e (low half) and e + 1 (high half), zero bytes between; the xor turns them into 0x64uu patterns
+    const uint32_t sel = 0x0c000c00u | uint32_t(jj % 4) | (uint32_t(4 + jj % 4) << 16);
     #pragma unroll
-    for (int e = 0; e < 8; e += 2) {
-        const uint32_t a = (r.v[e][word] >> shift) & 0xffu, b = (r.v[e + 1][word] >> shift) & 0xffu;
-        const half2v scale = as_half2(uint32_t(r.vscale[e]) | (uint32_t(r.vscale[e + 1]) << 16));
-        out[e / 2] = bytes_to_half2((a | (b << 16)) ^ 0x00800080u, scale);
-    }
+    for (int e = 0; e < 8; e += 2)
+        out[e / 2] = magic_to_half2(byte_perm(r.v[e + 1][word], r.v[e][word], sel) ^ 0x64806480u, s.pair[e / 2]);
     return half8{out[0].x, out[0].y, out[1].x, out[1].y, out[2].x, out[2].y, out[3].x, out[3].y};
 }
 template<int DIM>
-__device__ __forceinline__ half8 value_operand(const RowLoad<DIM, false>& r, int jj) {
+__device__ __forceinline__ half8 value_operand(const RowLoad<DIM, false>& r, const ValueScales<DIM>&, int jj) {
     half2v out[4];
-    const int word = jj / 2, shift = 16 * (jj % 2);
+    const int word = jj / 2;
+    const uint32_t sel = (jj & 1) ? 0x07060302u : 0x05040100u;
     #pragma unroll
-    for (int e = 0; e < 8; e += 2) {
-        const uint32_t a = (r.v[e][word] >> shift) & 0xffffu, b = (r.v[e + 1][word] >> shift) & 0xffffu;
-        out[e / 2] = as_half2(a | (b << 16));
-    }
+    for (int e = 0; e < 8; e += 2) out[e / 2] = as_half2(byte_perm(r.v[e + 1][word], r.v[e][word], sel));
     return half8{out[0].x, out[0].y, out[1].x, out[1].y, out[2].x, out[2].y, out[3].x, out[3].y};
 }
 
-template<int DIM, int QT, bool Q8>
+template<int DIM, int QT, bool Q8, bool PREFETCH>
 __global__ void __launch_bounds__(WAVES * 64) paged_attention_kernel(PagedArgs args) {
     constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, BLOCKS = DIM / 32, W = DIM / 16, TILES = DIM / 16;
     const int chunk = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, g = lane >> 4;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, g = lane >> 4;
     const int position = args.positions[seq], total = min(position + int(args.span), args.max_context);
     const int chunk_begin = chunk * int(args.chunk_tokens);
     if (chunk_begin >= total) return;
@@ -167,6 +188,7 @@ __global__ void __launch_bounds__(WAVES * 64) paged_attention_kernel(PagedArgs a
     const size_t plane_bytes = size_t(args.page_tokens) * ROW;
 
     // Query rows of this K/V head: row = span_row * group + head_in_group; a lane holds row qt*16 + li as B operands.
+    // A row past the last real one holds zeros (its scores are never stored).
     half8 qf[QT][BLOCKS];
     int limit[QT];
     #pragma unroll
@@ -174,7 +196,7 @@ __global__ void __launch_bounds__(WAVES * 64) paged_attention_kernel(PagedArgs a
         const int row = qt * 16 + li;
         const bool real = row < int(args.rows);
         const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
-        limit[qt] = real ? position + span_row : -1;
+        limit[qt] = real ? position + span_row : 0x7fffffff;
         const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
         #pragma unroll
         for (int b = 0; b < BLOCKS; ++b) {
@@ -200,84 +222,86 @@ __global__ void __launch_bounds__(WAVES * 64) paged_attention_kernel(PagedArgs a
         for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    const auto planes = [&](int token0, const uint8_t*& kplane, const uint8_t*& vplane) {
+    LaneOffsets<DIM, Q8> full;
+    full.set(STEP, li, g);
+    // A step's rows, requested from the (wave-uniform) first row of its K and V planes.
+    const auto request = [&](RowLoad<DIM, Q8>& rows, int token0) {
         const int page = __builtin_amdgcn_readfirstlane(table[token0 / int(args.page_tokens)]);
         const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads) * plane_bytes + size_t(token0 % int(args.page_tokens)) * ROW;
-        kplane = base + size_t(kvh) * plane_bytes;
-        vplane = base + size_t(args.kv_heads + kvh) * plane_bytes;
+        const uint8_t* kplane = base + size_t(kvh) * plane_bytes;
+        const uint8_t* vplane = base + size_t(args.kv_heads + kvh) * plane_bytes;
+        const int valid = total - token0;
+        if (valid >= STEP) load_step<DIM>(rows, kplane, vplane, full);
+        else { LaneOffsets<DIM, Q8> last; last.set(valid, li, g); load_step<DIM>(rows, kplane, vplane, last); }
     };
 
     int token0 = chunk_begin + STEP * wave;
     RowLoad<DIM, Q8> current, next;
-    if (token0 < chunk_end) {
-        const uint8_t *kplane, *vplane;
-        planes(token0, kplane, vplane);
-        load_step<DIM>(current, kplane, vplane, min(STEP, total - token0), li, g);
-    }
+    if (PREFETCH && token0 < chunk_end) request(current, token0);
     for (; token0 < chunk_end; token0 += STEP * WAVES) {
-        const int after = token0 + STEP * WAVES;
-        if (after < chunk_end) {
-            const uint8_t *kplane, *vplane;
-            planes(after, kplane, vplane);
-            load_step<DIM>(next, kplane, vplane, min(STEP, total - after), li, g);
-        }
+        if (PREFETCH) { if (token0 + STEP * WAVES < chunk_end) request(next, token0 + STEP * WAVES); }
+        else request(current, token0);
         // S^T tiles: tokens (rows, 4 per lane group) x query rows (lane li)
-        half8 ka[2][BLOCKS];
+        floatx4 s[QT][2];
         #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t) {
             #pragma unroll
-            for (int b = 0; b < BLOCKS; ++b) ka[t][b] = key_operand<DIM>(current, t, b);
+            for (int qt = 0; qt < QT; ++qt) s[qt][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            #pragma unroll
+            for (int b = 0; b < BLOCKS; ++b) {
+                const half8 ka = key_operand<DIM>(current, t, b);
+                #pragma unroll
+                for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qf[qt][b], s[qt][t], 0, 0, 0);
+            }
+        }
+        const bool edge = token0 + STEP - 1 > position;    // wave-uniform: some token of the step is past the first row's position
         half8 pb[QT];
         #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
-            floatx4 s[2];
-            #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                s[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-                #pragma unroll
-                for (int b = 0; b < BLOCKS; ++b) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][b], qf[qt][b], s[t], 0, 0, 0);
-            }
             float top = NEG_BIG;
-            const bool edge = token0 + STEP - 1 > limit[qt];    // some token of the step is past this row's position
             #pragma unroll
             for (int t = 0; t < 2; ++t)
                 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    float value = s[t][r] * args.scale_log2;
+                    float value = s[qt][t][r] * args.scale_log2;
                     if (edge && token0 + 16 * t + 4 * g + r > limit[qt]) value = -INFINITY;
-                    s[t][r] = value;
+                    s[qt][t][r] = value;
                     top = fmaxf(top, value);
                 }
             top = fmaxf(top, __shfl_xor(top, 16));
             top = fmaxf(top, __shfl_xor(top, 32));
-            const float m_new = fmaxf(m[qt], top);
-            const float alpha = __builtin_amdgcn_exp2f(m[qt] - m_new);
-            m[qt] = m_new;
+            // the running maximum rarely grows after the first steps: rescale only when some row's did
+            if (__any(top > m[qt])) {
+                const float m_new = fmaxf(m[qt], top);
+                const float alpha = __builtin_amdgcn_exp2f(m[qt] - m_new);
+                m[qt] = m_new;
+                l[qt] *= alpha;
+                #pragma unroll
+                for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] *= alpha;
+            }
             float sum = 0.0f;
             half8 p;
             #pragma unroll
             for (int t = 0; t < 2; ++t)
                 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float w = __builtin_amdgcn_exp2f(s[t][r] - m_new);
+                    const float w = __builtin_amdgcn_exp2f(s[qt][t][r] - m[qt]);
                     sum += w;
                     p[4 * t + r] = (_Float16)w;
                 }
             pb[qt] = p;
-            l[qt] = l[qt] * alpha + sum;
-            if (alpha != 1.0f) {
-                #pragma unroll
-                for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] *= alpha;
-            }
+            l[qt] += sum;
         }
         // O^T tiles: columns (rows of the tile, W*row + jj) x query rows
+        ValueScales<DIM> vs;
+        value_scales<DIM>(current, vs);
         #pragma unroll
         for (int jj = 0; jj < TILES; ++jj) {
-            const half8 va = value_operand<DIM>(current, jj);
+            const half8 va = value_operand<DIM>(current, vs, jj);
             #pragma unroll
             for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[qt], acc[qt][jj], 0, 0, 0);
         }
-        current = next;
+        if (PREFETCH) current = next;
     }
 
     // Merge the waves through LDS: per wave and query row the maximum, the sum and the unnormalised output.
@@ -306,11 +330,10 @@ __global__ void __launch_bounds__(WAVES * 64) paged_attention_kernel(PagedArgs a
         if (col == DIM) value = top;
         else {
             value = 0.0f;
-            const unsigned from = col == DIM + 1 ? DIM + 1 : col;
             #pragma unroll
             for (int w = 0; w < WAVES; ++w) {
                 const float* other = lds + (size_t(w) * QROWS + row) * STRIDE;
-                value += other[from] * __builtin_amdgcn_exp2f(other[DIM] - top);
+                value += other[col] * __builtin_amdgcn_exp2f(other[DIM] - top);
             }
         }
         out[i] = value;
@@ -342,11 +365,26 @@ __global__ void __launch_bounds__(DIM) paged_merge_kernel(PagedArgs args, void* 
     else static_cast<float*>(out)[at] = value;
 }
 
+// Tuning switches read once from the environment, as the reference reads its hot-path switches (STRAYDOG_QSA_MMA,
+// gpu/sparse_attention_compute.hpp:594): STRAYDOG_DECODE_CHUNK = tokens per workgroup (0: chosen from the shape),
+// STRAYDOG_DECODE_PREFETCH = 0 turns the register double buffering off.
+struct Tuning { unsigned chunk = 0; bool prefetch = true; };
+const Tuning& tuning() {
+    static const Tuning value = [] {
+        Tuning t;
+        if (const char* text = std::getenv("STRAYDOG_DECODE_CHUNK")) t.chunk = unsigned(std::strtoul(text, nullptr, 10));
+        if (const char* text = std::getenv("STRAYDOG_DECODE_PREFETCH")) t.prefetch = std::strtoul(text, nullptr, 10) != 0;
+        return t;
+    }();
+    return value;
+}
+
 unsigned pick_chunk(uint64_t seqs, uint64_t kv_heads, uint64_t max_context, unsigned page_tokens, unsigned compute_units) {
     // about eight workgroups per compute unit when every sequence is at max_context; a chunk is whole 128-token
     // rounds of the four waves and never smaller than 256 tokens
     const uint64_t want = uint64_t(compute_units) * 8;
     uint64_t chunk = (max_context * seqs * kv_heads + want - 1) / want;
+    if (tuning().chunk) chunk = tuning().chunk;
     chunk = (chunk + 127) / 128 * 128;
     if (chunk < 256) chunk = 256;
     if (chunk > 8192) chunk = 8192;
@@ -354,14 +392,14 @@ unsigned pick_chunk(uint64_t seqs, uint64_t kv_heads, uint64_t max_context, unsi
     return unsigned(chunk);
 }
 
-template<int DIM, bool Q8>
+template<int DIM, bool Q8, bool PF>
 void launch(Device& d, const PagedArgs& args, unsigned query_tiles, dim3 grid) {
     const size_t shared = size_t(WAVES) * query_tiles * 16 * (DIM + 2) * 4;
     if (shared > 160 * 1024) throw std::runtime_error("Straydog paged attention: too many query rows per K/V head for the decode kernel");
 #define SD_CASE(QT) case QT: { \
         static bool raised = false; \
-        if (!raised && shared > 64 * 1024) { SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_kernel<DIM, QT, Q8>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared))); raised = true; } \
-        paged_attention_kernel<DIM, QT, Q8><<<grid, WAVES * 64, shared, d.stream>>>(args); break; }
+        if (!raised && shared > 64 * 1024) { SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_kernel<DIM, QT, Q8, PF>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared))); raised = true; } \
+        paged_attention_kernel<DIM, QT, Q8, PF><<<grid, WAVES * 64, shared, d.stream>>>(args); break; }
     switch (query_tiles) {
         SD_CASE(1) SD_CASE(2) SD_CASE(3) SD_CASE(4)
         default: throw std::runtime_error("Straydog paged attention: too many query rows per K/V head for the decode kernel");
@@ -411,8 +449,14 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     {
     KernelTimer timer(value);
-    if (pool->dim == 128) { if (q8) launch<128, true>(value, args, query_tiles, grid); else launch<128, false>(value, args, query_tiles, grid); }
-    else { if (q8) launch<256, true>(value, args, query_tiles, grid); else launch<256, false>(value, args, query_tiles, grid); }
+    const bool prefetch = tuning().prefetch;
+    if (pool->dim == 128) {
+        if (q8) { if (prefetch) launch<128, true, true>(value, args, query_tiles, grid); else launch<128, true, false>(value, args, query_tiles, grid); }
+        else launch<128, false, true>(value, args, query_tiles, grid);
+    } else {
+        // 256 columns hold twice the accumulators: no register double buffering there
+        if (q8) launch<256, true, false>(value, args, query_tiles, grid); else launch<256, false, false>(value, args, query_tiles, grid);
+    }
     }
     SD_CHECK(hipGetLastError());
     const unsigned items = unsigned(checked_product({seqs, span, heads}));
