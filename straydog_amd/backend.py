@@ -201,5 +201,8 @@ class Backend:
     def fill_uniform(self, out, count, seed, lo=0.0, hi=1.0):
         self.check(self.lib.sdx_fill_uniform(self.handle, out, count, seed, lo, hi))
 
+    def read_probe(self, source, size, blocks_per_cu=8, unroll=4):
+        self.check(self.lib.sdx_read_probe(self.handle, source, size, blocks_per_cu, unroll))
+
     def copy(self, target, source, size):
         self.check(self.lib.sdx_copy(self.handle, target, source, size))

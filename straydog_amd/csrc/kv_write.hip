@@ -76,6 +76,23 @@ __global__ void __launch_bounds__(256) copy_kernel(uint4* target, const uint4* s
         target[i] = source[i];
 }
 
+// Read-only streaming probe: every lane reads UNROLL x 16 bytes per trip, block-contiguous, and folds them into one word
+// that is stored only if it is a value that cannot occur (keeps the loads alive).  The measured read ceiling of the box.
+typedef uint32_t probe_u4 __attribute__((ext_vector_type(4)));
+template<int UNROLL>
+__global__ void __launch_bounds__(256) read_probe_kernel(const probe_u4* __restrict__ source, size_t count, uint32_t* sink) {
+    uint32_t fold = 0;
+    const size_t stride = size_t(gridDim.x) * 256 * UNROLL;
+    for (size_t base = size_t(blockIdx.x) * 256 * UNROLL + threadIdx.x; base < count; base += stride) {
+        probe_u4 v[UNROLL];
+        #pragma unroll
+        for (int u = 0; u < UNROLL; ++u) v[u] = base + size_t(u) * 256 < count ? __builtin_nontemporal_load(source + base + size_t(u) * 256) : probe_u4{0, 0, 0, 0};
+        #pragma unroll
+        for (int u = 0; u < UNROLL; ++u) fold ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    if (fold == 0x9e3779b9u && sink) *sink = fold;
+}
+
 }  // namespace
 
 namespace sd {
@@ -123,6 +140,18 @@ int sdx_fill_uniform(void* handle, float* out, uint64_t count, uint64_t seed, fl
     if (!count) throw std::runtime_error("invalid Straydog fill");
     op_span(value, out, checked_floats({count}), "a filled buffer");
     fill_uniform_kernel<<<unsigned(std::min<size_t>(checked_blocks(size_t(count)), 65536)), 256, 0, value.stream>>>(out, size_t(count), seed, lo, hi);
+    SD_OP_END
+}
+
+int sdx_read_probe(void* handle, const void* source, uint64_t bytes, uint32_t blocks_per_cu, uint32_t unroll) {
+    SD_OP_BEGIN
+    if (!bytes || bytes % 16 || !blocks_per_cu || blocks_per_cu > 64) throw std::runtime_error("invalid Straydog read probe");
+    op_span(value, source, size_t(bytes), "a probe's source");
+    const unsigned grid = value.compute_units * blocks_per_cu;
+    uint32_t* sink = static_cast<uint32_t*>(workspace(value, 256));
+    if (unroll >= 8) read_probe_kernel<8><<<grid, 256, 0, value.stream>>>(static_cast<const probe_u4*>(source), size_t(bytes / 16), sink);
+    else if (unroll >= 4) read_probe_kernel<4><<<grid, 256, 0, value.stream>>>(static_cast<const probe_u4*>(source), size_t(bytes / 16), sink);
+    else read_probe_kernel<2><<<grid, 256, 0, value.stream>>>(static_cast<const probe_u4*>(source), size_t(bytes / 16), sink);
     SD_OP_END
 }
 

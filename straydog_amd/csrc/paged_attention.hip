@@ -27,6 +27,8 @@ namespace {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) const void* global_ptr;
+typedef __attribute__((address_space(3))) void* lds_ptr;
 
 constexpr int WAVES = 4, STEP = 32;
 constexpr float NEG_BIG = -1.0e30f;   // a finite "nothing seen yet" maximum: exp2(NEG_BIG - m) is 0, no inf - inf anywhere
@@ -175,8 +177,11 @@ __device__ __forceinline__ half8 value_operand(const RowLoad<DIM, false>& r, con
     return half8{out[0].x, out[0].y, out[1].x, out[1].y, out[2].x, out[2].y, out[3].x, out[3].y};
 }
 
-template<int DIM, int QT, bool Q8, bool PREFETCH>
-__global__ void __launch_bounds__(WAVES * 64) paged_attention_kernel(PagedArgs args) {
+// MODE: 0 = rows straight from HBM into operand registers, 1 = the same with the next step's rows requested before this
+// step is computed, 2 = a step's K and V slabs (32 contiguous rows each) copied by fully coalesced 16-byte global->LDS loads
+// into the wave's own LDS stage, operands then read from LDS in MFMA layout while the next step's copy is in flight.
+template<int DIM, int QT, bool Q8, int MODE, int OCC>
+__global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) paged_attention_kernel(PagedArgs args) {
     constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, BLOCKS = DIM / 32, W = DIM / 16, TILES = DIM / 16;
     const int chunk = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, g = lane >> 4;
@@ -224,23 +229,54 @@ __global__ void __launch_bounds__(WAVES * 64) paged_attention_kernel(PagedArgs a
 
     LaneOffsets<DIM, Q8> full;
     full.set(STEP, li, g);
-    // A step's rows, requested from the (wave-uniform) first row of its K and V planes.
-    const auto request = [&](RowLoad<DIM, Q8>& rows, int token0) {
+    extern __shared__ float lds[];
+    constexpr int SLAB = STEP * ROW;                       // one step's rows of one plane: contiguous in the page
+    uint8_t* stage = reinterpret_cast<uint8_t*>(lds) + wave * (2 * SLAB);
+    // The (wave-uniform) first row of a step in its K and V planes.
+    const auto planes = [&](int token0, const uint8_t*& kplane, const uint8_t*& vplane) {
         const int page = __builtin_amdgcn_readfirstlane(table[token0 / int(args.page_tokens)]);
         const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads) * plane_bytes + size_t(token0 % int(args.page_tokens)) * ROW;
-        const uint8_t* kplane = base + size_t(kvh) * plane_bytes;
-        const uint8_t* vplane = base + size_t(args.kv_heads + kvh) * plane_bytes;
+        kplane = base + size_t(kvh) * plane_bytes;
+        vplane = base + size_t(args.kv_heads + kvh) * plane_bytes;
+    };
+    // A step's rows into operand registers, from HBM (MODE 0/1) or from the wave's LDS stage (MODE 2).
+    const auto request = [&](RowLoad<DIM, Q8>& rows, int token0) {
+        const uint8_t *kplane, *vplane;
+        if (MODE >= 2) { kplane = stage; vplane = stage + SLAB; }
+        else planes(token0, kplane, vplane);
         const int valid = total - token0;
         if (valid >= STEP) load_step<DIM>(rows, kplane, vplane, full);
         else { LaneOffsets<DIM, Q8> last; last.set(valid, li, g); load_step<DIM>(rows, kplane, vplane, last); }
     };
+    // MODE 2: the step's two slabs copied into the stage, 1 KiB per instruction, lanes past a slab's end switched off.
+    const auto copy_in = [&](int token0) {
+        const uint8_t *kplane, *vplane;
+        planes(token0, kplane, vplane);
+        #pragma unroll
+        for (int part = 0; part < 2; ++part) {
+            const uint8_t* from = (part ? vplane : kplane) + 16 * lane;
+            #pragma unroll
+            for (int j = 0; j < (SLAB + 1023) / 1024; ++j)
+                if (1024 * j + 1024 <= SLAB || 16 * lane + 1024 * j < SLAB)
+                    __builtin_amdgcn_global_load_lds((global_ptr)(from + 1024 * j), (lds_ptr)(stage + part * SLAB + 1024 * j), 16, 0, 2 /* nt: streamed once */);
+        }
+    };
 
     int token0 = chunk_begin + STEP * wave;
     RowLoad<DIM, Q8> current, next;
-    if (PREFETCH && token0 < chunk_end) request(current, token0);
+    if (MODE == 1 && token0 < chunk_end) request(current, token0);
+    if (MODE >= 2 && token0 < chunk_end) copy_in(token0);
     for (; token0 < chunk_end; token0 += STEP * WAVES) {
-        if (PREFETCH) { if (token0 + STEP * WAVES < chunk_end) request(next, token0 + STEP * WAVES); }
-        else request(current, token0);
+        if (MODE == 1) { if (token0 + STEP * WAVES < chunk_end) request(next, token0 + STEP * WAVES); }
+        else if (MODE == 0) request(current, token0);
+        else {
+            __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0): the stage holds this step
+            request(current, token0);
+            __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): operands are in registers, the stage is free again
+            __builtin_amdgcn_sched_barrier(0);
+            if (token0 + STEP * WAVES < chunk_end) copy_in(token0 + STEP * WAVES);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         // S^T tiles: tokens (rows, 4 per lane group) x query rows (lane li)
         floatx4 s[QT][2];
         #pragma unroll
@@ -301,11 +337,11 @@ __global__ void __launch_bounds__(WAVES * 64) paged_attention_kernel(PagedArgs a
             #pragma unroll
             for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[qt], acc[qt][jj], 0, 0, 0);
         }
-        if (PREFETCH) current = next;
+        if (MODE == 1) current = next;
     }
 
     // Merge the waves through LDS: per wave and query row the maximum, the sum and the unnormalised output.
-    extern __shared__ float lds[];
+    if (MODE >= 2) __syncthreads();    // the merge area overlays the stages
     constexpr int STRIDE = DIM + 2, QROWS = QT * 16;
     #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
@@ -367,39 +403,42 @@ __global__ void __launch_bounds__(DIM) paged_merge_kernel(PagedArgs args, void* 
 
 // Tuning switches read once from the environment, as the reference reads its hot-path switches (STRAYDOG_QSA_MMA,
 // gpu/sparse_attention_compute.hpp:594): STRAYDOG_DECODE_CHUNK = tokens per workgroup (0: chosen from the shape),
-// STRAYDOG_DECODE_PREFETCH = 0 turns the register double buffering off.
-struct Tuning { unsigned chunk = 0; bool prefetch = true; };
+// STRAYDOG_DECODE_MODE = 0|1|2 picks how rows reach the operand registers (see the kernel), STRAYDOG_DECODE_OCCUPANCY the
+// waves per SIMD the decode variant is compiled for.
+struct Tuning { unsigned chunk = 0; unsigned mode = 2; unsigned occupancy = 4; };
 const Tuning& tuning() {
     static const Tuning value = [] {
         Tuning t;
         if (const char* text = std::getenv("STRAYDOG_DECODE_CHUNK")) t.chunk = unsigned(std::strtoul(text, nullptr, 10));
-        if (const char* text = std::getenv("STRAYDOG_DECODE_PREFETCH")) t.prefetch = std::strtoul(text, nullptr, 10) != 0;
+        if (const char* text = std::getenv("STRAYDOG_DECODE_OCCUPANCY")) t.occupancy = unsigned(std::strtoul(text, nullptr, 10));
+        if (const char* text = std::getenv("STRAYDOG_DECODE_MODE")) t.mode = unsigned(std::strtoul(text, nullptr, 10));
         return t;
     }();
     return value;
 }
 
 unsigned pick_chunk(uint64_t seqs, uint64_t kv_heads, uint64_t max_context, unsigned page_tokens, unsigned compute_units) {
-    // about eight workgroups per compute unit when every sequence is at max_context; a chunk is whole 128-token
+    // one resident round of workgroups when every sequence is at max_context; a chunk is whole 128-token
     // rounds of the four waves and never smaller than 256 tokens
-    const uint64_t want = uint64_t(compute_units) * 8;
+    const uint64_t want = uint64_t(compute_units) * 4;     // four workgroups (16 waves) are resident per compute unit
     uint64_t chunk = (max_context * seqs * kv_heads + want - 1) / want;
     if (tuning().chunk) chunk = tuning().chunk;
     chunk = (chunk + 127) / 128 * 128;
     if (chunk < 256) chunk = 256;
-    if (chunk > 8192) chunk = 8192;
+    if (chunk > 4096) chunk = 4096;
     (void)page_tokens;
     return unsigned(chunk);
 }
 
-template<int DIM, bool Q8, bool PF>
+template<int DIM, bool Q8, int PF, int OCC>
 void launch(Device& d, const PagedArgs& args, unsigned query_tiles, dim3 grid) {
-    const size_t shared = size_t(WAVES) * query_tiles * 16 * (DIM + 2) * 4;
+    size_t shared = size_t(WAVES) * query_tiles * 16 * (DIM + 2) * 4;
+    if (PF >= 2) shared = std::max(shared, size_t(WAVES) * 2 * STEP * (Q8 ? DIM + DIM / 16 : 2 * DIM));
     if (shared > 160 * 1024) throw std::runtime_error("Straydog paged attention: too many query rows per K/V head for the decode kernel");
 #define SD_CASE(QT) case QT: { \
         static bool raised = false; \
-        if (!raised && shared > 64 * 1024) { SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_kernel<DIM, QT, Q8, PF>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared))); raised = true; } \
-        paged_attention_kernel<DIM, QT, Q8, PF><<<grid, WAVES * 64, shared, d.stream>>>(args); break; }
+        if (!raised && shared > 64 * 1024) { SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_kernel<DIM, QT, Q8, PF, OCC>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared))); raised = true; } \
+        paged_attention_kernel<DIM, QT, Q8, PF, OCC><<<grid, WAVES * 64, shared, d.stream>>>(args); break; }
     switch (query_tiles) {
         SD_CASE(1) SD_CASE(2) SD_CASE(3) SD_CASE(4)
         default: throw std::runtime_error("Straydog paged attention: too many query rows per K/V head for the decode kernel");
@@ -449,13 +488,18 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     {
     KernelTimer timer(value);
-    const bool prefetch = tuning().prefetch;
+    const unsigned mode = tuning().mode, occupancy = tuning().occupancy;
     if (pool->dim == 128) {
-        if (q8) { if (prefetch) launch<128, true, true>(value, args, query_tiles, grid); else launch<128, true, false>(value, args, query_tiles, grid); }
-        else launch<128, false, true>(value, args, query_tiles, grid);
+        if (q8 && query_tiles == 1) {
+            // the decode shape: the variants differ in how rows reach the operand registers and in waves per SIMD
+            if (mode == 2) { if (occupancy >= 4) launch<128, true, 2, 4>(value, args, query_tiles, grid); else if (occupancy == 3) launch<128, true, 2, 3>(value, args, query_tiles, grid); else launch<128, true, 2, 2>(value, args, query_tiles, grid); }
+            else if (mode == 1) launch<128, true, 1, 2>(value, args, query_tiles, grid);
+            else launch<128, true, 0, 3>(value, args, query_tiles, grid);
+        }
+        else if (q8) launch<128, true, 2, 1>(value, args, query_tiles, grid);
+        else launch<128, false, 2, 1>(value, args, query_tiles, grid);
     } else {
-        // 256 columns hold twice the accumulators: no register double buffering there
-        if (q8) launch<256, true, false>(value, args, query_tiles, grid); else launch<256, false, false>(value, args, query_tiles, grid);
+        if (q8) launch<256, true, 2, 1>(value, args, query_tiles, grid); else launch<256, false, 2, 1>(value, args, query_tiles, grid);
     }
     }
     SD_CHECK(hipGetLastError());
