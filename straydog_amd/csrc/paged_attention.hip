@@ -29,6 +29,7 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) const void* global_ptr;
 typedef __attribute__((address_space(3))) void* lds_ptr;
+typedef __attribute__((address_space(4))) const int32_t* table_ptr;   // read through the scalar cache: a page number is wave-uniform
 
 constexpr int WAVES = 4, STEP = 32;
 constexpr float NEG_BIG = -1.0e30f;   // a finite "nothing seen yet" maximum: exp2(NEG_BIG - m) is 0, no inf - inf anywhere
@@ -43,9 +44,63 @@ struct PagedArgs {
     int q_f16;
     float scale_log2;      // softmax scale * log2(e): scores live in the base-2 domain
     float* partial;        // [seq][kv head][chunk][row][dim + 2]
-    unsigned chunk_tokens, chunks, rows;   // rows = span * group (query rows per K/V head)
+    unsigned chunks, rows;  // chunks = the most chunks a sequence can have; rows = span * group (query rows per K/V head)
+    unsigned chunk_min, chunk_max, seqs;   // tokens per chunk are chosen on the device between these (see chunk_tokens)
+    float slots, rounds;   // workgroups resident at once; workgroups per slot to cut the batch into (0: chosen from the batch)
     int max_context;       // positions[s] + span is clipped to this (the launch and the page table are sized for it)
 };
+
+// Tokens per chunk, the same for every workgroup of a launch and for the merge after it: the batch's cached tokens (all K/V
+// heads) cut into `rounds` workgroups per resident slot, in whole 128-token rounds of the four waves.  Workgroups are
+// dispatched in order as earlier ones finish: sequences of one length fill the device evenly in a single round, which has
+// the least start-up work; unequal ones even out over two rounds of smaller chunks.
+__device__ __forceinline__ unsigned chunk_tokens(const PagedArgs& args, int lane) {
+    if (args.chunk_min == args.chunk_max) return args.chunk_min;
+    float tokens = 0.0f;
+    int longest = 0;
+    for (unsigned s = lane; s < args.seqs; s += 64) {
+        const int total = min(args.positions[s] + int(args.span), args.max_context);
+        tokens += float(total);
+        longest = max(longest, total);
+    }
+    #pragma unroll
+    for (int d = 32; d; d >>= 1) { tokens += __shfl_xor(tokens, d); longest = max(longest, __shfl_xor(longest, d)); }
+    const float rounds = args.rounds > 0.0f ? args.rounds : tokens > 0.9f * float(args.seqs) * float(longest) ? 1.0f : 2.0f;
+    const float cut = tokens * float(args.kv_heads) / (args.slots * rounds);
+    const unsigned chunk = (unsigned(fminf(cut, 1.0e6f)) + 127u) / 128u * 128u;
+    return __builtin_amdgcn_readfirstlane(min(max(chunk, args.chunk_min), args.chunk_max));
+}
+
+// The work of workgroup `id`: the chunks that hold tokens are numbered sequence by sequence, then K/V head by K/V head, so
+// the workgroups with work are the first of the grid and the rest leave at once.  Every wave finds the same answer from
+// the positions alone (a running count over 64 sequences at a time).
+struct WorkItem { int seq, chunk, kvh, per_chunk, position, total; };
+__device__ __forceinline__ bool find_work(const PagedArgs& args, unsigned id, int lane, WorkItem& item) {
+    item.per_chunk = int(chunk_tokens(args, lane));
+    unsigned before = 0;
+    for (unsigned first = 0; first < args.seqs; first += 64) {
+        const unsigned s = first + lane;
+        const int position = s < args.seqs ? args.positions[s] : 0;
+        const int total = s < args.seqs ? min(position + int(args.span), args.max_context) : 0;
+        const unsigned used = unsigned(total + item.per_chunk - 1) / unsigned(item.per_chunk);
+        unsigned upto = used * args.kv_heads;      // workgroups of this and the earlier sequences of the 64
+        #pragma unroll
+        for (int d = 1; d < 64; d <<= 1) { const unsigned other = __shfl_up(upto, d); if (lane >= d) upto += other; }
+        const unsigned all = __shfl(upto, 63);
+        if (id < before + all) {
+            const int owner = __popcll(__ballot(before + upto <= id));
+            const unsigned chunks = __shfl(used, owner), within = id - before - __shfl(upto - used * args.kv_heads, owner);
+            item.seq = int(first) + owner;
+            item.total = __shfl(total, owner);
+            item.position = __shfl(position, owner);
+            item.kvh = int(within / chunks);
+            item.chunk = int(within % chunks);
+            return true;
+        }
+        before += all;
+    }
+    return false;
+}
 
 __device__ __forceinline__ half2v as_half2(uint32_t bits) { return __builtin_bit_cast(half2v, bits); }
 
@@ -59,27 +114,6 @@ __device__ __forceinline__ half2v magic_to_half2(uint32_t pattern, half2v scale)
     return (as_half2(pattern) - bias) * scale;
 }
 
-// Per-lane byte offsets of the rows a step reads, from the step's first row of the K (or V) plane.  They are the same for
-// every full step, so they are formed once; a last, partial step clamps its tokens to the last valid one.
-template<int DIM, bool Q8> struct LaneOffsets {
-    static constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, W = DIM / 16;
-    uint32_t k[2], ks[2], v[8], vs[8];
-    __device__ __forceinline__ void set(int valid, int li, int g) {
-        #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const uint32_t row = uint32_t(min(16 * t + li, valid - 1)) * ROW;
-            k[t] = row + (Q8 ? 8 * g : 16 * g);
-            ks[t] = row + DIM;
-        }
-        #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const uint32_t row = uint32_t(min(e < 4 ? 4 * g + e : 16 + 4 * g + (e - 4), valid - 1)) * ROW;
-            v[e] = row + (Q8 ? W * li : 2 * W * li);
-            vs[e] = row + DIM + 2 * ((W * li) / 32);
-        }
-    }
-};
-
 template<int DIM, bool Q8> struct RowLoad;
 
 // What one step needs from HBM, as raw words.  Q8_0: K tile t (16 tokens, lane li = token) gives each lane 8 columns of
@@ -92,21 +126,26 @@ template<int DIM> struct RowLoad<DIM, true> {
     uint32_t v[8][W / 4];
     uint16_t vscale[8];
 };
+// The rows lie in the wave's stage, 32 of each plane one after the other, so every piece is at a fixed distance from the
+// lane's first K row (li) and first V row (4g).
 template<int DIM>
-__device__ __forceinline__ void load_step(RowLoad<DIM, true>& r, const uint8_t* kplane, const uint8_t* vplane, const LaneOffsets<DIM, true>& o) {
-    constexpr int BLOCKS = DIM / 32, W = DIM / 16;
+__device__ __forceinline__ void load_step(RowLoad<DIM, true>& r, const uint8_t* kplane, const uint8_t* vplane, int li, int g) {
+    constexpr int BLOCKS = DIM / 32, W = DIM / 16, ROW = DIM + DIM / 16;
+    const uint8_t* krow = kplane + li * ROW;
+    const uint8_t* vrow = vplane + 4 * g * ROW;
     #pragma unroll
     for (int t = 0; t < 2; ++t) {
         #pragma unroll
-        for (int b = 0; b < BLOCKS; ++b) r.k[t][b] = *reinterpret_cast<const uint2*>(kplane + o.k[t] + 32 * b);
+        for (int b = 0; b < BLOCKS; ++b) r.k[t][b] = *reinterpret_cast<const uint2*>(krow + 16 * t * ROW + 8 * g + 32 * b);
         #pragma unroll
-        for (int b = 0; b < BLOCKS / 2; ++b) r.kscale[t][b] = *reinterpret_cast<const uint32_t*>(kplane + o.ks[t] + 4 * b);
+        for (int b = 0; b < BLOCKS / 2; ++b) r.kscale[t][b] = *reinterpret_cast<const uint32_t*>(krow + 16 * t * ROW + DIM + 4 * b);
     }
     #pragma unroll
     for (int e = 0; e < 8; ++e) {
+        const int token = e < 4 ? e : 12 + e;       // the lane's tokens are 4g + {0..3, 16..19}
         #pragma unroll
-        for (int w = 0; w < W / 4; ++w) r.v[e][w] = *reinterpret_cast<const uint32_t*>(vplane + o.v[e] + 4 * w);
-        r.vscale[e] = *reinterpret_cast<const uint16_t*>(vplane + o.vs[e]);
+        for (int w = 0; w < W / 4; ++w) r.v[e][w] = *reinterpret_cast<const uint32_t*>(vrow + token * ROW + W * li + 4 * w);
+        r.vscale[e] = *reinterpret_cast<const uint16_t*>(vrow + token * ROW + DIM + 2 * ((W * li) / 32));
     }
 }
 
@@ -117,16 +156,20 @@ template<int DIM> struct RowLoad<DIM, false> {
     uint32_t v[8][W / 2];
 };
 template<int DIM>
-__device__ __forceinline__ void load_step(RowLoad<DIM, false>& r, const uint8_t* kplane, const uint8_t* vplane, const LaneOffsets<DIM, false>& o) {
-    constexpr int BLOCKS = DIM / 32, W = DIM / 16;
+__device__ __forceinline__ void load_step(RowLoad<DIM, false>& r, const uint8_t* kplane, const uint8_t* vplane, int li, int g) {
+    constexpr int BLOCKS = DIM / 32, W = DIM / 16, ROW = 2 * DIM;
+    const uint8_t* krow = kplane + li * ROW;
+    const uint8_t* vrow = vplane + 4 * g * ROW;
     #pragma unroll
     for (int t = 0; t < 2; ++t)
         #pragma unroll
-        for (int b = 0; b < BLOCKS; ++b) r.k[t][b] = *reinterpret_cast<const half8*>(kplane + o.k[t] + 64 * b);
+        for (int b = 0; b < BLOCKS; ++b) r.k[t][b] = *reinterpret_cast<const half8*>(krow + 16 * t * ROW + 16 * g + 64 * b);
     #pragma unroll
-    for (int e = 0; e < 8; ++e)
+    for (int e = 0; e < 8; ++e) {
+        const int token = e < 4 ? e : 12 + e;
         #pragma unroll
-        for (int w = 0; w < W / 2; ++w) r.v[e][w] = *reinterpret_cast<const uint32_t*>(vplane + o.v[e] + 4 * w);
+        for (int w = 0; w < W / 2; ++w) r.v[e][w] = *reinterpret_cast<const uint32_t*>(vrow + token * ROW + 2 * W * li + 4 * w);
+    }
 }
 
 // The A operand of S^T = K . Q^T for tile t, block b.
@@ -177,19 +220,20 @@ __device__ __forceinline__ half8 value_operand(const RowLoad<DIM, false>& r, con
     return half8{out[0].x, out[0].y, out[1].x, out[1].y, out[2].x, out[2].y, out[3].x, out[3].y};
 }
 
-// MODE: 0 = rows straight from HBM into operand registers, 1 = the same with the next step's rows requested before this
-// step is computed, 2 = a step's K and V slabs (32 contiguous rows each) copied by fully coalesced 16-byte global->LDS loads
-// into the wave's own LDS stage, operands then read from LDS in MFMA layout while the next step's copy is in flight.
-template<int DIM, int QT, bool Q8, int MODE, int OCC>
+// A step's K and V slabs (32 contiguous rows each) are copied by fully coalesced 16-byte global->LDS loads into the wave's
+// own LDS stage; operands are then read from LDS in MFMA layout while the next step's copy is in flight.  OCC = the waves per
+// SIMD the variant is compiled for (its register budget).
+template<int DIM, int QT, bool Q8, int OCC>
 __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) paged_attention_kernel(PagedArgs args) {
     constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, BLOCKS = DIM / 32, W = DIM / 16, TILES = DIM / 16;
-    const int chunk = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, g = lane >> 4;
-    const int position = args.positions[seq], total = min(position + int(args.span), args.max_context);
-    const int chunk_begin = chunk * int(args.chunk_tokens);
-    if (chunk_begin >= total) return;
-    const int chunk_end = min(total, chunk_begin + int(args.chunk_tokens));
-    const int32_t* table = args.page_table + size_t(seq) * args.table_stride;
+    WorkItem item;
+    if (!find_work(args, blockIdx.x, lane, item)) return;
+    const int seq = __builtin_amdgcn_readfirstlane(item.seq), chunk = __builtin_amdgcn_readfirstlane(item.chunk);
+    const int kvh = __builtin_amdgcn_readfirstlane(item.kvh), total = __builtin_amdgcn_readfirstlane(item.total);
+    const int position = __builtin_amdgcn_readfirstlane(item.position);
+    const int chunk_begin = chunk * item.per_chunk, chunk_end = min(total, chunk_begin + item.per_chunk);
+    const table_ptr table = (table_ptr)(args.page_table + size_t(seq) * args.table_stride);
     const size_t plane_bytes = size_t(args.page_tokens) * ROW;
 
     // Query rows of this K/V head: row = span_row * group + head_in_group; a lane holds row qt*16 + li as B operands.
@@ -227,34 +271,25 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    LaneOffsets<DIM, Q8> full;
-    full.set(STEP, li, g);
     extern __shared__ float lds[];
     constexpr int SLAB = STEP * ROW;                       // one step's rows of one plane: contiguous in the page
     uint8_t* stage = reinterpret_cast<uint8_t*>(lds) + wave * (2 * SLAB);
-    // The (wave-uniform) first row of a step in its K and V planes.
-    const auto planes = [&](int token0, const uint8_t*& kplane, const uint8_t*& vplane) {
-        const int page = __builtin_amdgcn_readfirstlane(table[token0 / int(args.page_tokens)]);
-        const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads) * plane_bytes + size_t(token0 % int(args.page_tokens)) * ROW;
-        kplane = base + size_t(kvh) * plane_bytes;
-        vplane = base + size_t(args.kv_heads + kvh) * plane_bytes;
-    };
-    // A step's rows into operand registers, from HBM (MODE 0/1) or from the wave's LDS stage (MODE 2).
+    // A step's rows from the wave's stage into operand registers.  The rows past the sequence's end in its last step hold
+    // whatever the page held: they are cleared first (their scores are masked, but a stray scale must not meet a zero weight).
     const auto request = [&](RowLoad<DIM, Q8>& rows, int token0) {
-        const uint8_t *kplane, *vplane;
-        if (MODE >= 2) { kplane = stage; vplane = stage + SLAB; }
-        else planes(token0, kplane, vplane);
         const int valid = total - token0;
-        if (valid >= STEP) load_step<DIM>(rows, kplane, vplane, full);
-        else { LaneOffsets<DIM, Q8> last; last.set(valid, li, g); load_step<DIM>(rows, kplane, vplane, last); }
+        if (valid < STEP)
+            #pragma unroll
+            for (int part = 0; part < 2; ++part)
+                for (int at = valid * ROW + 4 * lane; at < SLAB; at += 256) *reinterpret_cast<uint32_t*>(stage + part * SLAB + at) = 0u;
+        load_step<DIM>(rows, stage, stage + SLAB, li, g);
     };
-    // MODE 2: the step's two slabs copied into the stage, 1 KiB per instruction, lanes past a slab's end switched off.
-    const auto copy_in = [&](int token0) {
-        const uint8_t *kplane, *vplane;
-        planes(token0, kplane, vplane);
+    // The step's two slabs copied into the stage, 1 KiB per instruction, lanes past a slab's end switched off.
+    const auto copy_in = [&](int page, int in_page) {
+        const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(in_page) * ROW + 16 * lane;
         #pragma unroll
         for (int part = 0; part < 2; ++part) {
-            const uint8_t* from = (part ? vplane : kplane) + 16 * lane;
+            const uint8_t* from = base + size_t(part ? args.kv_heads : 0) * plane_bytes;
             #pragma unroll
             for (int j = 0; j < (SLAB + 1023) / 1024; ++j)
                 if (1024 * j + 1024 <= SLAB || 16 * lane + 1024 * j < SLAB)
@@ -262,21 +297,24 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         }
     };
 
+    // Where the wave's step lies: page_index-th page of the sequence, in_page rows into it.  The page number of the step
+    // after the current one is fetched (a scalar load) before the current step is waited for, so it is there when its copy
+    // is issued.
     int token0 = chunk_begin + STEP * wave;
-    RowLoad<DIM, Q8> current, next;
-    if (MODE == 1 && token0 < chunk_end) request(current, token0);
-    if (MODE >= 2 && token0 < chunk_end) copy_in(token0);
+    const int last_page = (total - 1) / int(args.page_tokens);
+    int page_index = token0 / int(args.page_tokens), in_page = token0 % int(args.page_tokens);
+    if (token0 < chunk_end) copy_in(table[min(page_index, last_page)], in_page);
     for (; token0 < chunk_end; token0 += STEP * WAVES) {
-        if (MODE == 1) { if (token0 + STEP * WAVES < chunk_end) request(next, token0 + STEP * WAVES); }
-        else if (MODE == 0) request(current, token0);
-        else {
-            __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0): the stage holds this step
-            request(current, token0);
-            __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): operands are in registers, the stage is free again
-            __builtin_amdgcn_sched_barrier(0);
-            if (token0 + STEP * WAVES < chunk_end) copy_in(token0 + STEP * WAVES);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        in_page += STEP * WAVES;
+        while (in_page >= int(args.page_tokens)) { in_page -= int(args.page_tokens); ++page_index; }
+        const int page_ahead = table[min(page_index, last_page)];
+        RowLoad<DIM, Q8> current;
+        __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0): the stage holds this step
+        request(current, token0);
+        __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): operands are in registers, the stage is free again
+        __builtin_amdgcn_sched_barrier(0);
+        if (token0 + STEP * WAVES < chunk_end) copy_in(page_ahead, in_page);
+        __builtin_amdgcn_sched_barrier(0);
         // S^T tiles: tokens (rows, 4 per lane group) x query rows (lane li)
         floatx4 s[QT][2];
         #pragma unroll
@@ -337,11 +375,10 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
             #pragma unroll
             for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[qt], acc[qt][jj], 0, 0, 0);
         }
-        if (MODE == 1) current = next;
     }
 
     // Merge the waves through LDS: per wave and query row the maximum, the sum and the unnormalised output.
-    if (MODE >= 2) __syncthreads();    // the merge area overlays the stages
+    __syncthreads();    // the merge area overlays the stages
     constexpr int STRIDE = DIM + 2, QROWS = QT * 16;
     #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
@@ -376,74 +413,122 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
     }
 }
 
-// One block per (sequence, span row, head): the chunks' partial results merged and normalised
-// (the algebra of the reference's qsa_decode_merge, gpu/sparse_attention_compute.hpp:139-170).
+// One block per (sequence, span row, head): the chunks' partial results merged and normalised (the algebra of the
+// reference's qsa_decode_merge, gpu/sparse_attention_compute.hpp:139-170).  The block's 256 threads are GROUPS groups of
+// DIM/2 threads; a group takes every GROUPS-th chunk and a thread two columns, so all loads of a pass are in flight at
+// once; chunks are taken 256 at a time with a running maximum.
 template<int DIM, bool F16_OUT>
-__global__ void __launch_bounds__(DIM) paged_merge_kernel(PagedArgs args, void* out) {
-    constexpr int STRIDE = DIM + 2;
+__global__ void __launch_bounds__(256) paged_merge_kernel(PagedArgs args, void* out) {
+    constexpr int STRIDE = DIM + 2, LANES = DIM / 2, GROUPS = 256 / LANES;
     const unsigned item = blockIdx.x, head = item % args.heads, span_row = item / args.heads % args.span, seq = item / args.heads / args.span;
-    const unsigned kvh = head / args.group, row = span_row * args.group + head % args.group, col = threadIdx.x;
+    const unsigned kvh = head / args.group, row = span_row * args.group + head % args.group;
+    const unsigned tid = threadIdx.x, group = tid / LANES, col = 2 * (tid % LANES), wave = tid >> 6;
     const int total = min(args.positions[seq] + int(args.span), args.max_context);
-    const unsigned used = unsigned((total + int(args.chunk_tokens) - 1) / int(args.chunk_tokens));
+    const int per_chunk = int(chunk_tokens(args, int(tid & 63)));
+    const unsigned used = unsigned((total + per_chunk - 1) / per_chunk);
     const float* base = args.partial + ((size_t(seq) * args.kv_heads + kvh) * args.chunks) * args.rows * STRIDE + size_t(row) * STRIDE;
     const size_t step = size_t(args.rows) * STRIDE;
-    float top = NEG_BIG;
-    for (unsigned c = 0; c < used; ++c) top = fmaxf(top, base[c * step + DIM]);
-    float sum = 0.0f, value = 0.0f;
-    for (unsigned c = 0; c < used; ++c) {
-        const float w = __builtin_amdgcn_exp2f(base[c * step + DIM] - top);
-        sum += base[c * step + DIM + 1] * w;
-        value += base[c * step + col] * w;
+    __shared__ float weights[256];
+    __shared__ float reduce[2][4];
+    __shared__ float2 sums[GROUPS][LANES];
+    float top = NEG_BIG, sum = 0.0f;
+    float2 value = {0.0f, 0.0f};
+    for (unsigned first = 0; first < used; first += 256) {
+        const unsigned c = first + tid, count = min(used - first, 256u);
+        float m = NEG_BIG, l = 0.0f;
+        if (c < used) { const float2 pair = *reinterpret_cast<const float2*>(base + c * step + DIM); m = pair.x; l = pair.y; }
+        float tile_top = m;
+        #pragma unroll
+        for (int d = 32; d; d >>= 1) tile_top = fmaxf(tile_top, __shfl_xor(tile_top, d));
+        if ((tid & 63) == 0) reduce[0][wave] = tile_top;
+        __syncthreads();
+        tile_top = fmaxf(fmaxf(reduce[0][0], reduce[0][1]), fmaxf(reduce[0][2], reduce[0][3]));
+        const float top_new = fmaxf(top, tile_top), keep = __builtin_amdgcn_exp2f(top - top_new);
+        const float w = __builtin_amdgcn_exp2f(m - top_new);
+        weights[tid] = w;
+        float part = l * w;
+        #pragma unroll
+        for (int d = 32; d; d >>= 1) part += __shfl_xor(part, d);
+        if ((tid & 63) == 0) reduce[1][wave] = part;
+        __syncthreads();
+        sum = sum * keep + (reduce[1][0] + reduce[1][1]) + (reduce[1][2] + reduce[1][3]);
+        value.x *= keep; value.y *= keep;
+        top = top_new;
+        for (unsigned k = group; k < count; k += GROUPS) {
+            const float2 v = *reinterpret_cast<const float2*>(base + (first + k) * step + col);
+            value.x += v.x * weights[k]; value.y += v.y * weights[k];
+        }
+        __syncthreads();      // weights and reduce are rewritten by the next pass
     }
-    value /= sum;
-    const size_t at = size_t(item) * DIM + col;
-    if (F16_OUT) static_cast<__half*>(out)[at] = __float2half_rn(value);
-    else static_cast<float*>(out)[at] = value;
+    sums[group][tid % LANES] = value;
+    __syncthreads();
+    if (group == 0) {
+        #pragma unroll
+        for (int g = 1; g < GROUPS; ++g) { value.x += sums[g][tid].x; value.y += sums[g][tid].y; }
+        value.x /= sum; value.y /= sum;
+        const size_t at = size_t(item) * DIM + col;
+        if (F16_OUT) *reinterpret_cast<__half2*>(static_cast<__half*>(out) + at) = __floats2half2_rn(value.x, value.y);
+        else *reinterpret_cast<float2*>(static_cast<float*>(out) + at) = value;
+    }
 }
 
 // Tuning switches read once from the environment, as the reference reads its hot-path switches (STRAYDOG_QSA_MMA,
-// gpu/sparse_attention_compute.hpp:594): STRAYDOG_DECODE_CHUNK = tokens per workgroup (0: chosen from the shape),
-// STRAYDOG_DECODE_MODE = 0|1|2 picks how rows reach the operand registers (see the kernel), STRAYDOG_DECODE_OCCUPANCY the
-// waves per SIMD the decode variant is compiled for.
-struct Tuning { unsigned chunk = 0; unsigned mode = 2; unsigned occupancy = 4; };
+// gpu/sparse_attention_compute.hpp:594): STRAYDOG_DECODE_CHUNK = tokens per workgroup (0: chosen on the device from the
+// batch), STRAYDOG_DECODE_ROUNDS = workgroups per resident slot the batch is cut into (0: chosen from the batch too).
+struct Tuning { unsigned chunk = 0; float rounds = 0.0f; };
 const Tuning& tuning() {
     static const Tuning value = [] {
         Tuning t;
         if (const char* text = std::getenv("STRAYDOG_DECODE_CHUNK")) t.chunk = unsigned(std::strtoul(text, nullptr, 10));
-        if (const char* text = std::getenv("STRAYDOG_DECODE_OCCUPANCY")) t.occupancy = unsigned(std::strtoul(text, nullptr, 10));
-        if (const char* text = std::getenv("STRAYDOG_DECODE_MODE")) t.mode = unsigned(std::strtoul(text, nullptr, 10));
+        if (const char* text = std::getenv("STRAYDOG_DECODE_ROUNDS")) t.rounds = std::max(0.0f, std::strtof(text, nullptr));
         return t;
     }();
     return value;
 }
 
-unsigned pick_chunk(uint64_t seqs, uint64_t kv_heads, uint64_t max_context, unsigned page_tokens, unsigned compute_units) {
-    // one resident round of workgroups when every sequence is at max_context; a chunk is whole 128-token
-    // rounds of the four waves and never smaller than 256 tokens
-    const uint64_t want = uint64_t(compute_units) * 4;     // four workgroups (16 waves) are resident per compute unit
-    uint64_t chunk = (max_context * seqs * kv_heads + want - 1) / want;
-    if (tuning().chunk) chunk = tuning().chunk;
-    chunk = (chunk + 127) / 128 * 128;
-    if (chunk < 256) chunk = 256;
-    if (chunk > 4096) chunk = 4096;
-    (void)page_tokens;
-    return unsigned(chunk);
+constexpr unsigned smallest_chunk = 256, largest_chunk = 4096;
+
+// The host knows only max_context: it bounds the device's choice above by the chunk of a batch with every sequence full,
+// and sizes the grid for an eighth of that (the workgroups past the batch's last chunk leave at once).
+void plan_chunks(PagedArgs& args, uint64_t seqs, uint64_t kv_heads, uint64_t max_context, unsigned compute_units) {
+    args.slots = float(compute_units) * 4.0f;
+    args.rounds = tuning().rounds;
+    if (tuning().chunk) {
+        const unsigned chunk = std::min(std::max((tuning().chunk + 127u) / 128u * 128u, smallest_chunk), 1u << 20);
+        args.chunk_min = args.chunk_max = chunk;
+    } else {
+        const double full = double(max_context) * double(seqs) * double(kv_heads) / double(args.slots * (args.rounds > 0.0f ? args.rounds : 1.0f));
+        const unsigned chunk = unsigned(std::min(full, 1.0e6) + 127.0) / 128u * 128u;
+        args.chunk_max = std::min(std::max(chunk, smallest_chunk), largest_chunk);
+        args.chunk_min = std::max(smallest_chunk, args.chunk_max / 8 / 128u * 128u);
+    }
+    args.chunks = unsigned((max_context + args.chunk_min - 1) / args.chunk_min);
 }
 
-template<int DIM, bool Q8, int PF, int OCC>
-void launch(Device& d, const PagedArgs& args, unsigned query_tiles, dim3 grid) {
-    size_t shared = size_t(WAVES) * query_tiles * 16 * (DIM + 2) * 4;
-    if (PF >= 2) shared = std::max(shared, size_t(WAVES) * 2 * STEP * (Q8 ? DIM + DIM / 16 : 2 * DIM));
+template<int DIM, int QT, bool Q8, int OCC>
+void launch(Device& d, const PagedArgs& args, dim3 grid) {
+    const size_t shared = std::max(size_t(WAVES) * QT * 16 * (DIM + 2) * 4, size_t(WAVES) * 2 * STEP * (Q8 ? DIM + DIM / 16 : 2 * DIM));
     if (shared > 160 * 1024) throw std::runtime_error("Straydog paged attention: too many query rows per K/V head for the decode kernel");
-#define SD_CASE(QT) case QT: { \
-        static bool raised = false; \
-        if (!raised && shared > 64 * 1024) { SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_kernel<DIM, QT, Q8, PF, OCC>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared))); raised = true; } \
-        paged_attention_kernel<DIM, QT, Q8, PF, OCC><<<grid, WAVES * 64, shared, d.stream>>>(args); break; }
+    static bool raised = false;
+    if (!raised && shared > 64 * 1024) {
+        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_kernel<DIM, QT, Q8, OCC>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
+        raised = true;
+    }
+    paged_attention_kernel<DIM, QT, Q8, OCC><<<grid, WAVES * 64, shared, d.stream>>>(args);
+}
+
+// The variants that exist: (columns, query tiles, format) -> waves per SIMD the kernel is compiled for.  One query tile is
+// the decode shape (4 waves/SIMD at 128 columns of Q8_0); more tiles hold more accumulators.
+template<int DIM, bool Q8>
+void launch_tiles(Device& d, const PagedArgs& args, unsigned query_tiles, dim3 grid) {
+    constexpr bool small = DIM == 128;
     switch (query_tiles) {
-        SD_CASE(1) SD_CASE(2) SD_CASE(3) SD_CASE(4)
+        case 1: launch<DIM, 1, Q8, (small && Q8 ? 4 : small ? 2 : 1)>(d, args, grid); break;
+        case 2: launch<DIM, 2, Q8, (small ? 2 : 1)>(d, args, grid); break;
+        case 3: launch<DIM, 3, Q8, (small && Q8 ? 2 : 1)>(d, args, grid); break;
+        case 4: launch<DIM, 4, Q8, 1>(d, args, grid); break;
         default: throw std::runtime_error("Straydog paged attention: too many query rows per K/V head for the decode kernel");
     }
-#undef SD_CASE
 }
 
 }  // namespace
@@ -451,8 +536,8 @@ void launch(Device& d, const PagedArgs& args, unsigned query_tiles, dim3 grid) {
 extern "C" {
 
 uint64_t sdx_paged_attention_scratch(uint64_t seqs, uint64_t span, uint64_t heads, uint64_t dim, uint64_t max_context) {
-    // the smallest chunk the launch may pick is 256 tokens
-    const uint64_t chunks = (max_context + 255) / 256;
+    // the smallest chunk a launch may use
+    const uint64_t chunks = (max_context + smallest_chunk - 1) / smallest_chunk;
     return seqs * span * heads * chunks * (dim + 2) * 4;
 }
 
@@ -476,37 +561,27 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
     args.page_tokens = pool->page_tokens; args.kv_heads = pool->kv_heads; args.heads = unsigned(heads); args.group = unsigned(group);
     args.span = unsigned(span); args.page_table = page_table; args.table_stride = size_t(table_stride); args.positions = positions;
     args.q = q; args.q_f16 = q_f16; args.scale_log2 = scale * 1.44269504088896341f;
-    args.chunk_tokens = pick_chunk(seqs, pool->kv_heads, max_context, pool->page_tokens, value.compute_units);
-    args.chunks = unsigned((max_context + args.chunk_tokens - 1) / args.chunk_tokens);
-    args.rows = unsigned(rows);
+    args.rows = unsigned(rows); args.seqs = unsigned(seqs);
     args.max_context = int(max_context);
+    plan_chunks(args, seqs, pool->kv_heads, max_context, value.compute_units);
+    if (args.chunks > 65535) throw std::runtime_error("invalid Straydog paged attention shape");
     const size_t need = checked_floats({seqs, pool->kv_heads, args.chunks, rows, uint64_t(pool->dim) + 2});
     if (!scratch || scratch_bytes < need) throw std::runtime_error("Straydog paged attention scratch too small");
     op_span(value, scratch, need, "attention scratch");
     args.partial = static_cast<float*>(scratch);
-    const dim3 grid(args.chunks, pool->kv_heads, unsigned(seqs));
+    if (checked_product({seqs, args.chunks, pool->kv_heads}) > 0x7fffffffu) throw std::runtime_error("invalid Straydog paged attention shape");
+    const dim3 grid(unsigned(seqs * args.chunks * pool->kv_heads));
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     {
-    KernelTimer timer(value);
-    const unsigned mode = tuning().mode, occupancy = tuning().occupancy;
-    if (pool->dim == 128) {
-        if (q8 && query_tiles == 1) {
-            // the decode shape: the variants differ in how rows reach the operand registers and in waves per SIMD
-            if (mode == 2) { if (occupancy >= 4) launch<128, true, 2, 4>(value, args, query_tiles, grid); else if (occupancy == 3) launch<128, true, 2, 3>(value, args, query_tiles, grid); else launch<128, true, 2, 2>(value, args, query_tiles, grid); }
-            else if (mode == 1) launch<128, true, 1, 2>(value, args, query_tiles, grid);
-            else launch<128, true, 0, 3>(value, args, query_tiles, grid);
-        }
-        else if (q8) launch<128, true, 2, 1>(value, args, query_tiles, grid);
-        else launch<128, false, 2, 1>(value, args, query_tiles, grid);
-    } else {
-        if (q8) launch<256, true, 2, 1>(value, args, query_tiles, grid); else launch<256, false, 2, 1>(value, args, query_tiles, grid);
-    }
+        KernelTimer timer(value);
+        if (pool->dim == 128) { if (q8) launch_tiles<128, true>(value, args, query_tiles, grid); else launch_tiles<128, false>(value, args, query_tiles, grid); }
+        else { if (q8) launch_tiles<256, true>(value, args, query_tiles, grid); else launch_tiles<256, false>(value, args, query_tiles, grid); }
     }
     SD_CHECK(hipGetLastError());
     const unsigned items = unsigned(checked_product({seqs, span, heads}));
     if (pool->dim == 128) {
-        if (out_f16) paged_merge_kernel<128, true><<<items, 128, 0, value.stream>>>(args, out);
-        else paged_merge_kernel<128, false><<<items, 128, 0, value.stream>>>(args, out);
+        if (out_f16) paged_merge_kernel<128, true><<<items, 256, 0, value.stream>>>(args, out);
+        else paged_merge_kernel<128, false><<<items, 256, 0, value.stream>>>(args, out);
     } else {
         if (out_f16) paged_merge_kernel<256, true><<<items, 256, 0, value.stream>>>(args, out);
         else paged_merge_kernel<256, false><<<items, 256, 0, value.stream>>>(args, out);

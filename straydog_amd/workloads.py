@@ -1,8 +1,6 @@
 """Synthetic workloads of the attention path, built on the GPU through the C ABI (no host-side arithmetic):
 the BASELINE configurations' shapes with seeded N(0,1) inputs, K/V quantised into the paged cache by the
 library's own writer.  Used by bench.py, __graft_entry__.smoke() and the full-size GPU tests."""
-import os
-
 import numpy as np
 
 ROW_Q8 = {128: 136, 256: 272}
@@ -23,8 +21,6 @@ class PagedWorkload:
         self.page_count = int(pages_per.sum())
         self.table_stride = int(pages_per.max())
         order = rng.permutation(self.page_count).astype(np.int32)
-        if os.environ.get("STRAYDOG_BENCH_IDENTITY_PAGES"):      # experiment: physical pages in logical order
-            order = np.arange(self.page_count, dtype=np.int32)
         self.table = np.zeros((self.seqs, self.table_stride), dtype=np.int32)
         at = 0
         for s in range(self.seqs):
