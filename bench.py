@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the attention hot path on one MI355X.
 
-A step is one pass of the Q8_0 paged grouped-query decode attention (sdx_paged_attention: split kernel + merge) over
+A step is one pass of the Q8_0 paged grouped-query decode attention (sdx_paged_attention: chunk kernel + merge) over
 one batch of synthetic, HBM-resident inputs.  The default workload is BASELINE.json configs[1]: 32 sequences with
 lengths drawn uniformly from [1024, 32768], 32 query heads over 4 K/V heads, head_dim 128, 256-token pages behind a
 shuffled page table, FP16 queries and outputs.  The one JSON line also carries, under "also", the all-32768-token case
@@ -22,6 +22,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 
+# HBM bytes per launch of the dominant kernel as rocprofv3's FETCH_SIZE (x 2.000) + WRITE_SIZE (x 1.000) counted them, the
+# scale factors being what the same counters read for the library's 1 GiB copy kernel.
+MEASURED_TRAFFIC = {"config1": 630.7e6, "config1_32k": 1147.4e6}
+
 
 def timed(gpu, step, steps, warmup):
     """(ms per step over the whole stream, ms per launch of the dominant kernel) for `steps` steps after `warmup`."""
@@ -40,20 +44,23 @@ def timed(gpu, step, steps, warmup):
     return total / steps, (kernel_ms / launches if launches else None)
 
 
-def copy_ceiling(gpu, size=1 << 30, repeats=10):
-    """Measured GB/s (read + write) of the library's plain copy kernel: the practical HBM ceiling on this box."""
+def measured_ceilings(gpu, size=1 << 30, repeats=10):
+    """Measured GB/s of the library's plain copy kernel (read + write) and of its read-only streaming probe (coalesced
+    16-byte non-temporal loads): what this box's HBM delivers to the simplest kernels."""
     a, b = gpu.buffer(size), gpu.buffer(size)
-    for _ in range(3):
-        gpu.copy(b.base(), a.base(), size)
-    gpu.synchronize()
-    begin = gpu.event()
-    for _ in range(repeats):
-        gpu.copy(b.base(), a.base(), size)
-    end = gpu.event()
-    ms = gpu.elapsed_ms(begin, end) / repeats
-    gpu.events_clear()
+    rates = []
+    for run, moved in ((lambda: gpu.copy(b.base(), a.base(), size), 2 * size), (lambda: gpu.read_probe(a.base(), size), size)):
+        for _ in range(3):
+            run()
+        gpu.synchronize()
+        begin = gpu.event()
+        for _ in range(repeats):
+            run()
+        end = gpu.event()
+        rates.append(moved / (gpu.elapsed_ms(begin, end) / repeats) / 1e6)
+        gpu.events_clear()
     gpu.release(a); gpu.release(b)
-    return 2 * size / ms / 1e6
+    return rates
 
 
 def paged_result(gpu, work, steps, warmup):
@@ -67,24 +74,30 @@ def paged_result(gpu, work, steps, warmup):
     }
 
 
-def cpu_baseline_paged(work, sample_seqs, threads):
-    """The CPU oracle on a bounded sample of the same workload (the first `sample_seqs` sequences), timed on this host's
-    cores; also returns the GPU-vs-oracle error on that sample."""
+def cpu_baseline_paged(work, sample_seqs, threads, budget_seconds=12.0):
+    """The CPU oracle on the first `sample_seqs` sequences of the same workload, timed on this host's cores: passes are
+    repeated until about `budget_seconds` of wall time are spent and the fastest one counts.  Also returns the GPU-vs-oracle
+    error on those sequences."""
     import oracle
     pool = work.read_pool()
     q = work.read_queries()[:sample_seqs]
     got = work.read_output()[:sample_seqs]
     table, positions = work.table[:sample_seqs], work.positions[:sample_seqs]
-    start = time.perf_counter()
-    want = oracle.paged_attention(pool, work.row_bytes, work.page_tokens, work.kv_heads, work.dim, table, positions, q, work.scale,
-                                  threads=threads)
-    seconds = time.perf_counter() - start
+    best, spent, passes = None, 0.0, 0
+    while passes < 2 or (spent < budget_seconds and passes < 200):
+        start = time.perf_counter()
+        want = oracle.paged_attention(pool, work.row_bytes, work.page_tokens, work.kv_heads, work.dim, table, positions, q, work.scale,
+                                      threads=threads)
+        seconds = time.perf_counter() - start
+        best = seconds if best is None else min(best, seconds)
+        spent += seconds
+        passes += 1
     rows = int(work.lengths[:sample_seqs].sum()) * work.kv_heads * 2 * work.row_bytes
     error = float(np.abs(got - want).max())
-    return {"value": rows / seconds / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": f"first {sample_seqs} of {work.seqs} sequences of the same workload ({int(work.lengths[:sample_seqs].sum())} cached tokens), "
-                      f"{seconds:.2f} s, OpenMP over (sequence, K/V head)",
-            "tokens_per_s": sample_seqs * work.span / seconds}, error
+    return {"value": rows / best / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{sample_seqs} of {work.seqs} sequences of the same workload ({int(work.lengths[:sample_seqs].sum())} cached tokens, "
+                      f"{rows / 1e6:.0f} MB of K/V rows), fastest of {passes} passes in {spent:.1f} s, OpenMP over (sequence, K/V head)",
+            "tokens_per_s": sample_seqs * work.span / best}, error
 
 
 def main():
@@ -118,7 +131,7 @@ def main():
         "config3": "configs[3]: 16 seqs, ctx 65536 + span 5, 32q/4kv heads, d128, Q8_0 pages of 256",
         "config4": "configs[4]: batch 8, ctx 131072, 64x128 bf16 indexer, top-2048, 64 heads over bf16 latents 576/512",
     }
-    ceiling = copy_ceiling(gpu)
+    copy_rate, read_rate = measured_ceilings(gpu)
 
     def run_paged(name, with_cpu):
         work = builders[name]()
@@ -126,7 +139,7 @@ def main():
         baseline = None
         if with_cpu:
             threads = min(os.cpu_count() or 1, 16)
-            sample = {"config1": 8, "config1_32k": 4, "config0": 1, "config3": 1}[name]
+            sample = {"config1": 32, "config1_32k": 32, "config0": 1, "config3": 4}[name]
             baseline, error = cpu_baseline_paged(work, min(sample, work.seqs), threads)
             result["max_abs_error_vs_oracle_on_sample"] = error
         work.release()
@@ -165,8 +178,9 @@ def main():
         "config": {"workload": names[args.workload], "batch": 32 if args.workload.startswith("config1") else None},
         "tokens_per_s": main_result.get("tokens_per_s"), "frac_of_hbm_peak": main_result["frac_of_hbm_peak"],
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": None, "kernel": "paged_attention_kernel<128,1,Q8_0>" if args.workload != "config4" else "index_scores_kernel",
-                     "kernel_us": kernel_us, "measured_copy_gbps": ceiling},
+                     "traffic": MEASURED_TRAFFIC.get(args.workload),
+                     "kernel": "paged_attention_kernel<128,1,Q8_0>" if args.workload != "config4" else "index_scores_kernel",
+                     "kernel_us": kernel_us, "measured_copy_gbps": copy_rate, "measured_read_gbps": read_rate},
         "cpu_baseline": baseline, "detail": main_result, "also": also,
     }
     print(json.dumps(line))
