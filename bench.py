@@ -5,9 +5,10 @@ A step is one pass of the Q8_0 paged grouped-query decode attention (sdx_paged_a
 one batch of synthetic, HBM-resident inputs.  The default workload is BASELINE.json configs[1]: 32 sequences with
 lengths drawn uniformly from [1024, 32768], 32 query heads over 4 K/V heads, head_dim 128, 256-token pages behind a
 shuffled page table, FP16 queries and outputs.  The one JSON line also carries, under "also", the all-32768-token case
-of the same shape (the north-star target), config 0, the verify span of config 3 and the sparse path of config 4.
+of the same shape (the north-star target), config 0, the chunked prefill of config 2 (MFMA-bound: TFLOP/s against the
+dense FP16 peak), the verify span of config 3 and the sparse path of config 4.
 
-    python bench.py --gpus 1 --steps 50 --warmup 10 [--workload config1|config1_32k|config0|config3|config4]
+    python bench.py --gpus 1 --steps 50 --warmup 10 [--workload config1|config1_32k|config0|config2|config3|config4]
 """
 import argparse
 import json
@@ -21,6 +22,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense FP16/BF16 MFMA, published
 
 # HBM bytes per launch of the dominant kernel as rocprofv3's FETCH_SIZE (x 2.000) + WRITE_SIZE (x 1.000) counted them, the
 # scale factors being what the same counters read for the library's 1 GiB copy kernel.
@@ -129,6 +131,7 @@ def main():
         "config1_32k": "configs[1] shape with all 32 sequences at 32768 tokens",
         "config0": "configs[0]: 1 seq, ctx 4096, 16q/2kv heads, d128, fp32 q/out",
         "config3": "configs[3]: 16 seqs, ctx 65536 + span 5, 32q/4kv heads, d128, Q8_0 pages of 256",
+        "config2": "configs[2]: 1 prompt of 8192 tokens prefilled in 4 chunks of 2048 (fp16 K/V appended as Q8_0, causal attention), 32q/4kv heads, d128",
         "config4": "configs[4]: batch 8, ctx 131072, 64x128 bf16 indexer, top-2048, 64 heads over bf16 latents 576/512",
     }
     copy_rate, read_rate = measured_ceilings(gpu)
@@ -155,8 +158,23 @@ def main():
         return {"us_per_step": total * 1e3, "index_topk_us": ms_index * 1e3, "gather_attention_us": ms_attention * 1e3,
                 "algorithmic_bytes": size, "gbps": size / total / 1e6, "frac_of_hbm_peak": size / total / 1e6 / HBM_PEAK_GBPS}
 
+    def run_prefill():
+        work = workloads.PrefillWorkload(gpu)
+        steps = max(args.steps // 5, 3)
+        ms, kernel_ms = timed(gpu, work.step, steps, 2)
+        flops, size = work.flops(), work.algorithmic_bytes()
+        work.release()
+        # the timed kernel launches are the 4 attention launches of a step (the K/V writer is not bracketed)
+        return {"ms_per_step": ms, "us_per_step": ms * 1e3, "kernel_us": None if kernel_ms is None else kernel_ms * 4e3, "flops": flops,
+                "tflops": flops / ms / 1e9, "frac_of_mfma_peak": flops / ms / 1e9 / MFMA_PEAK_TFLOPS,
+                "kernel_tflops": None if kernel_ms is None else flops / (4 * kernel_ms) / 1e9,
+                "algorithmic_bytes": size, "gbps": size / ms / 1e6, "frac_of_hbm_peak": size / ms / 1e6 / HBM_PEAK_GBPS,
+                "tokens_per_s": work.tokens / (ms * 1e-3)}
+
     if args.workload == "config4":
         main_result, baseline = run_sparse(), None
+    elif args.workload == "config2":
+        main_result, baseline = run_prefill(), None
     else:
         main_result, baseline = run_paged(args.workload, not args.no_cpu)
     also = {}
@@ -165,22 +183,30 @@ def main():
             if name != args.workload:
                 also[name], _ = run_paged(name, False)
                 also[name]["workload"] = names[name]
+        if args.workload != "config2":
+            also["config2"] = run_prefill()
+            also["config2"]["workload"] = names["config2"]
         if args.workload != "config4":
             also["config4"] = run_sparse()
             also["config4"]["workload"] = names["config4"]
 
     kernel_us = main_result.get("kernel_us")
     achieved = main_result["algorithmic_bytes"] / (kernel_us * 1e-6) / 1e9 if kernel_us else main_result["gbps"]
+    roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                "traffic": MEASURED_TRAFFIC.get(args.workload),
+                "kernel": "paged_attention_kernel<128,1,Q8_0>" if args.workload != "config4" else "index_scores_kernel",
+                "kernel_us": kernel_us, "measured_copy_gbps": copy_rate, "measured_read_gbps": read_rate}
+    if args.workload == "config2":
+        achieved = main_result["kernel_tflops"] or main_result["tflops"]
+        roofline = {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
+                    "traffic": None, "kernel": "prefill_attention_kernel<128,4,Q8_0>", "kernel_us": kernel_us}
     line = {
         "metric": "Q8_0 decode-attn HBM GB/s", "value": main_result["gbps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": main_result.get("ms_per_step", main_result["us_per_step"] / 1e3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "int8 K/V x fp16 MFMA, fp32 accumulate", "data": "synthetic",
         "config": {"workload": names[args.workload], "batch": 32 if args.workload.startswith("config1") else None},
         "tokens_per_s": main_result.get("tokens_per_s"), "frac_of_hbm_peak": main_result["frac_of_hbm_peak"],
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC.get(args.workload),
-                     "kernel": "paged_attention_kernel<128,1,Q8_0>" if args.workload != "config4" else "index_scores_kernel",
-                     "kernel_us": kernel_us, "measured_copy_gbps": copy_rate, "measured_read_gbps": read_rate},
+        "roofline": roofline,
         "cpu_baseline": baseline, "detail": main_result, "also": also,
     }
     print(json.dumps(line))

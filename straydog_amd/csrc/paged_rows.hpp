@@ -1,0 +1,160 @@
+// Rows of the paged K/V cache as MFMA operands: the pieces shared by the decode kernel and the prefill kernel.
+//
+// Layouts (v_mfma_f32_16x16x32_f16 on gfx950, wave64): an A or B operand gives lane (l % 16, l / 16 = g) eight k-slots;
+// a C tile gives lane column l % 16 and rows 4g..4g+3.  S^T = K . Q^T takes K rows as A operands (lane = token, eight
+// consecutive columns per lane group), so the C layout (lane = query row, four tokens per lane group) is already the
+// B-operand layout of O^T += V^T . P^T: probabilities never move between lanes.  A 32-token step is two such tiles; the
+// eight k-slots of the second product are the lane's tokens {4g..4g+3, 16+4g..16+4g+3}.
+#pragma once
+#include "device.hpp"
+#include "../../include/straydog_gpu_ext.h"
+
+#include <hip/hip_fp16.h>
+
+namespace sd { namespace paged {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) const void* global_ptr;
+typedef __attribute__((address_space(3))) void* lds_ptr;
+typedef __attribute__((address_space(4))) const int32_t* table_ptr;   // read through the scalar cache: a page number is wave-uniform
+
+constexpr int WAVES = 4, STEP = 32;
+constexpr float NEG_BIG = -1.0e30f;   // a finite "nothing seen yet" maximum: exp2(NEG_BIG - m) is 0, no inf - inf anywhere
+
+struct PagedArgs {
+    const uint8_t* pages;
+    unsigned page_tokens, kv_heads, heads, group, span;
+    const int32_t* page_table;
+    size_t table_stride;
+    const int32_t* positions;
+    const void* q;
+    int q_f16;
+    float scale_log2;      // softmax scale * log2(e): scores live in the base-2 domain
+    float* partial;        // [seq][kv head][chunk][row][dim + 2]
+    unsigned chunks, rows;  // chunks = the most chunks a sequence can have; rows = span * group (query rows per K/V head)
+    unsigned chunk_min, chunk_max, seqs;   // tokens per chunk are chosen on the device between these (see chunk_tokens)
+    float slots, rounds;   // workgroups resident at once; workgroups per slot to cut the batch into (0: chosen from the batch)
+    int max_context;       // positions[s] + span is clipped to this (the launch and the page table are sized for it)
+};
+
+__device__ __forceinline__ half2v as_half2(uint32_t bits) { return __builtin_bit_cast(half2v, bits); }
+
+// v_perm_b32: byte i of the result is byte sel[i] of the 8 bytes {high, low} (0-3 = low's bytes, 4-7 = high's, 0x0c = 0x00).
+__device__ __forceinline__ uint32_t byte_perm(uint32_t high, uint32_t low, uint32_t sel) { return __builtin_amdgcn_perm(high, low, sel); }
+
+// Two bytes u (an int8 xor 0x80) sitting in FP16 patterns 0x64uu: 0x6400 | u is the FP16 1024 + u exactly; minus 1152 leaves the
+// signed byte; one rounding by the block scale (the reference's qsa_q8_half16, gpu/qsa_prompt_attention.hpp:15-33).
+__device__ __forceinline__ half2v magic_to_half2(uint32_t pattern, half2v scale) {
+    const half2v bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+    return (as_half2(pattern) - bias) * scale;
+}
+
+template<int DIM, bool Q8> struct RowLoad;
+
+// What one step needs from HBM, as raw words.  Q8_0: K tile t (16 tokens, lane li = token) gives each lane 8 columns of
+// every 32-column block and the row's scales; V gives lane (li, g) the columns [W*li, W*li + W) (W = DIM/16) of its 8
+// tokens {4g..4g+3, 16+4g..16+4g+3} and those columns' block scale.
+template<int DIM> struct RowLoad<DIM, true> {
+    static constexpr int BLOCKS = DIM / 32, W = DIM / 16;
+    uint2 k[2][BLOCKS];
+    uint32_t kscale[2][BLOCKS / 2];
+    uint32_t v[8][W / 4];
+    uint16_t vscale[8];
+};
+// The rows lie in the wave's stage, 32 of each plane one after the other, so every piece is at a fixed distance from the
+// lane's first K row (li) and first V row (4g).
+template<int DIM>
+__device__ __forceinline__ void load_step(RowLoad<DIM, true>& r, const uint8_t* kplane, const uint8_t* vplane, int li, int g) {
+    constexpr int BLOCKS = DIM / 32, W = DIM / 16, ROW = DIM + DIM / 16;
+    const uint8_t* krow = kplane + li * ROW;
+    const uint8_t* vrow = vplane + 4 * g * ROW;
+    #pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        #pragma unroll
+        for (int b = 0; b < BLOCKS; ++b) r.k[t][b] = *reinterpret_cast<const uint2*>(krow + 16 * t * ROW + 8 * g + 32 * b);
+        #pragma unroll
+        for (int b = 0; b < BLOCKS / 2; ++b) r.kscale[t][b] = *reinterpret_cast<const uint32_t*>(krow + 16 * t * ROW + DIM + 4 * b);
+    }
+    #pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int token = e < 4 ? e : 12 + e;       // the lane's tokens are 4g + {0..3, 16..19}
+        #pragma unroll
+        for (int w = 0; w < W / 4; ++w) r.v[e][w] = *reinterpret_cast<const uint32_t*>(vrow + token * ROW + W * li + 4 * w);
+        r.vscale[e] = *reinterpret_cast<const uint16_t*>(vrow + token * ROW + DIM + 2 * ((W * li) / 32));
+    }
+}
+
+// FP16 rows: the same pieces, two bytes a value.
+template<int DIM> struct RowLoad<DIM, false> {
+    static constexpr int BLOCKS = DIM / 32, W = DIM / 16;
+    half8 k[2][BLOCKS];
+    uint32_t v[8][W / 2];
+};
+template<int DIM>
+__device__ __forceinline__ void load_step(RowLoad<DIM, false>& r, const uint8_t* kplane, const uint8_t* vplane, int li, int g) {
+    constexpr int BLOCKS = DIM / 32, W = DIM / 16, ROW = 2 * DIM;
+    const uint8_t* krow = kplane + li * ROW;
+    const uint8_t* vrow = vplane + 4 * g * ROW;
+    #pragma unroll
+    for (int t = 0; t < 2; ++t)
+        #pragma unroll
+        for (int b = 0; b < BLOCKS; ++b) r.k[t][b] = *reinterpret_cast<const half8*>(krow + 16 * t * ROW + 16 * g + 64 * b);
+    #pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int token = e < 4 ? e : 12 + e;
+        #pragma unroll
+        for (int w = 0; w < W / 2; ++w) r.v[e][w] = *reinterpret_cast<const uint32_t*>(vrow + token * ROW + 2 * W * li + 4 * w);
+    }
+}
+
+// The A operand of S^T = K . Q^T for tile t, block b.
+template<int DIM>
+__device__ __forceinline__ half8 key_operand(const RowLoad<DIM, true>& r, int t, int b) {
+    const uint32_t pairs = r.kscale[t][b / 2];
+    const half2v scale = as_half2((b & 1) ? byte_perm(pairs, pairs, 0x03020302u) : byte_perm(pairs, pairs, 0x01000100u));
+    const uint32_t magic = 0x64646464u;
+    const uint32_t lo = r.k[t][b].x ^ 0x80808080u, hi = r.k[t][b].y ^ 0x80808080u;
+    const half2v a0 = magic_to_half2(byte_perm(magic, lo, 0x04010400u), scale);
+    const half2v a1 = magic_to_half2(byte_perm(magic, lo, 0x04030402u), scale);
+    const half2v a2 = magic_to_half2(byte_perm(magic, hi, 0x04010400u), scale);
+    const half2v a3 = magic_to_half2(byte_perm(magic, hi, 0x04030402u), scale);
+    return half8{a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+}
+template<int DIM>
+__device__ __forceinline__ half8 key_operand(const RowLoad<DIM, false>& r, int t, int b) { return r.k[t][b]; }
+
+// The scales of the lane's 8 tokens as 4 FP16 pairs (tokens e, e+1), formed once a step.
+template<int DIM> struct ValueScales { half2v pair[4]; };
+template<int DIM>
+__device__ __forceinline__ void value_scales(const RowLoad<DIM, true>& r, ValueScales<DIM>& s) {
+    #pragma unroll
+    for (int e = 0; e < 8; e += 2) s.pair[e / 2] = as_half2(uint32_t(r.vscale[e]) | (uint32_t(r.vscale[e + 1]) << 16));
+}
+template<int DIM>
+__device__ __forceinline__ void value_scales(const RowLoad<DIM, false>&, ValueScales<DIM>&) {}
+
+// The A operand of O^T += V^T . P^T for output tile jj: column W*li + jj of the lane's 8 tokens.
+template<int DIM>
+__device__ __forceinline__ half8 value_operand(const RowLoad<DIM, true>& r, const ValueScales<DIM>& s, int jj) {
+    half2v out[4];
+    const int word = jj / 4;
+    // bytes (jj % 4) of tokens e (low half) and e + 1 (high half), zero bytes between; the xor turns them into 0x64uu patterns
+    const uint32_t sel = 0x0c000c00u | uint32_t(jj % 4) | (uint32_t(4 + jj % 4) << 16);
+    #pragma unroll
+    for (int e = 0; e < 8; e += 2)
+        out[e / 2] = magic_to_half2(byte_perm(r.v[e + 1][word], r.v[e][word], sel) ^ 0x64806480u, s.pair[e / 2]);
+    return half8{out[0].x, out[0].y, out[1].x, out[1].y, out[2].x, out[2].y, out[3].x, out[3].y};
+}
+template<int DIM>
+__device__ __forceinline__ half8 value_operand(const RowLoad<DIM, false>& r, const ValueScales<DIM>&, int jj) {
+    half2v out[4];
+    const int word = jj / 2;
+    const uint32_t sel = (jj & 1) ? 0x07060302u : 0x05040100u;
+    #pragma unroll
+    for (int e = 0; e < 8; e += 2) out[e / 2] = as_half2(byte_perm(r.v[e + 1][word], r.v[e][word], sel));
+    return half8{out[0].x, out[0].y, out[1].x, out[1].y, out[2].x, out[2].y, out[3].x, out[3].y};
+}
+
+}}  // namespace sd::paged

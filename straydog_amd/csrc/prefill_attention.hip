@@ -1,0 +1,259 @@
+// Causal grouped-query attention over the paged Q8_0 / FP16 K/V cache for many query rows per sequence: chunked
+// prefill (a span of new tokens attends the cache, which already holds the span's own K/V rows, and is causal within
+// the span).  Stands in for the reference's per-token prompt attention qsa_prompt_attention
+// (gpu/qsa_prompt_attention.hpp:47-213: S^T = K . Q^T and O^T += V^T . P^T on matrix cores, Q8_0 -> FP16 operands,
+// base-2 online softmax in FP32) and its multi-token qsa_flash (gpu/sparse_attention_compute.hpp:176-279) with the
+// dense selection 0..position.
+//
+// Shape of the work on gfx950 (wave64, v_mfma_f32_16x16x32_f16):
+//   * a workgroup (4 waves) owns 4 x QT x 16 consecutive query rows of one (sequence, K/V head): rows are ordered
+//     (span row, head in group), so a workgroup is a run of consecutive tokens with all their grouped heads and
+//     every K/V row it reads serves all of them; a wave owns QT x 16 of those rows with their own online softmax, so
+//     no merge is needed and the output is written once, normalised;
+//   * the workgroup walks the keys 32 at a time: the step's K and V slabs (32 contiguous rows of a page plane) are
+//     copied by coalesced 16-byte global->LDS loads, a quarter by each wave, into one of two stages, so the next
+//     step's copy is in flight while this one is computed; one barrier per step;
+//   * every wave builds its MFMA operands from the stage (paged_rows.hpp) and skips steps that lie wholly after
+//     its rows' positions; the workgroups with the longest walks are dispatched first.
+#include "paged_rows.hpp"
+
+#include <cstdlib>
+
+using namespace sd;
+using namespace sd::paged;
+
+namespace {
+
+struct PrefillArgs {
+    const uint8_t* pages;
+    unsigned page_tokens, kv_heads, heads, group, span;
+    const int32_t* page_table;
+    size_t table_stride;
+    const int32_t* positions;
+    const void* q;
+    int q_f16;
+    float scale_log2;      // softmax scale * log2(e): scores live in the base-2 domain
+    unsigned rows;         // span * group: query rows per K/V head
+    int max_context;       // positions[s] + span is clipped to this
+    void* out;
+    int out_f16;
+};
+
+template<int DIM, int QT, bool Q8, int OCC>
+__global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) prefill_attention_kernel(PrefillArgs args) {
+    constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, BLOCKS = DIM / 32, W = DIM / 16, TILES = DIM / 16;
+    constexpr int SLAB = STEP * ROW, UNITS = (SLAB + 1023) / 1024;     // a slab is copied 1 KiB (one instruction of a wave) at a time
+    constexpr int WAVE_ROWS = QT * 16, GROUP_ROWS = WAVES * WAVE_ROWS;
+    const int tile = int(gridDim.x) - 1 - int(blockIdx.x), kvh = blockIdx.y, seq = blockIdx.z;   // later rows walk further: first
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, g = lane >> 4;
+    const int position = args.positions[seq];
+    const int cached = min(position + int(args.span), args.max_context);          // rows of the sequence the cache holds
+    const int row0 = tile * GROUP_ROWS + wave * WAVE_ROWS;                        // the wave's first query row
+    const int group_last = min(int(args.rows), (tile + 1) * GROUP_ROWS) - 1;
+    const int keys = min(position + group_last / int(args.group) + 1, cached);    // the workgroup walks keys 0..keys-1
+    const bool idle = row0 >= int(args.rows);                                     // a wave past the last row only helps copying
+    const int wave_first = position + row0 / int(args.group);                      // the smallest and largest position of
+    const int wave_last = position + (min(int(args.rows), row0 + WAVE_ROWS) - 1) / int(args.group);   // the wave's rows
+    const table_ptr table = (table_ptr)(args.page_table + size_t(seq) * args.table_stride);
+    const size_t plane_bytes = size_t(args.page_tokens) * ROW;
+    extern __shared__ uint8_t stages[];                                           // [2][K slab | V slab]
+
+    // The step's two slabs into a stage: 2 * UNITS pieces of 1 KiB, every fourth one by this wave.
+    const auto copy_in = [&](int buffer, int token0) {
+        const int page = table[token0 / int(args.page_tokens)];
+        const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(token0 % int(args.page_tokens)) * ROW + 16 * lane;
+        uint8_t* stage = stages + buffer * (2 * SLAB);
+        #pragma unroll
+        for (int k = 0; k < (2 * UNITS + WAVES - 1) / WAVES; ++k) {
+            const int unit = wave + WAVES * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS;
+            if (unit < 2 * UNITS && 16 * lane + 1024 * j < SLAB)
+                __builtin_amdgcn_global_load_lds((global_ptr)(base + size_t(part ? args.kv_heads : 0) * plane_bytes + 1024 * j),
+                                                 (lds_ptr)(stage + part * SLAB + 1024 * j), 16, 0, 0);
+        }
+    };
+    copy_in(0, 0);
+
+    // Query rows: row = span_row * group + head_in_group; a lane holds row row0 + qt*16 + li as B operands.  A row past the
+    // last real one holds zeros and is never stored.
+    half8 qf[QT][BLOCKS];
+    int limit[QT];
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int row = row0 + qt * 16 + li;
+        const bool real = row < int(args.rows);
+        const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
+        limit[qt] = real ? position + span_row : 0x7fffffff;
+        const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
+        #pragma unroll
+        for (int b = 0; b < BLOCKS; ++b) {
+            half8 value = {};
+            if (real) {
+                if (args.q_f16) value = *reinterpret_cast<const half8*>(static_cast<const _Float16*>(args.q) + at + 32 * b + 8 * g);
+                else {
+                    const float* from = static_cast<const float*>(args.q) + at + 32 * b + 8 * g;
+                    #pragma unroll
+                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)from[i];
+                }
+            }
+            qf[qt][b] = value;
+        }
+    }
+    floatx4 acc[QT][TILES];
+    float m[QT], l[QT];
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        m[qt] = NEG_BIG; l[qt] = 0.0f;
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    for (int token0 = 0, buffer = 0; token0 < keys; token0 += STEP, buffer ^= 1) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0): this wave's pieces of the step have landed
+        __syncthreads();                             // ... and everybody's; the other stage is no longer being read
+        if (token0 + STEP < keys) copy_in(buffer ^ 1, token0 + STEP);
+        uint8_t* stage = stages + buffer * (2 * SLAB);
+        if (cached - token0 < STEP) {
+            // the sequence's last rows: the stage's tail holds whatever the page held.  It is cleared (those scores are masked,
+            // but a stray scale must not meet a zero weight).
+            #pragma unroll
+            for (int part = 0; part < 2; ++part)
+                for (int at = (cached - token0) * ROW + 4 * int(threadIdx.x); at < SLAB; at += 4 * WAVES * 64)
+                    *reinterpret_cast<uint32_t*>(stage + part * SLAB + at) = 0u;
+            __syncthreads();
+        }
+        if (idle || token0 > wave_last) continue;    // nothing of this step is visible to the wave's rows
+        RowLoad<DIM, Q8> current;
+        load_step<DIM>(current, stage, stage + SLAB, li, g);
+        // S^T tiles: tokens (rows, 4 per lane group) x query rows (lane li)
+        floatx4 s[QT][2];
+        #pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt) s[qt][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            #pragma unroll
+            for (int b = 0; b < BLOCKS; ++b) {
+                const half8 ka = key_operand<DIM>(current, t, b);
+                #pragma unroll
+                for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qf[qt][b], s[qt][t], 0, 0, 0);
+            }
+        }
+        const bool edge = token0 + STEP - 1 > wave_first;    // wave-uniform: some token of the step is past some row's position
+        half8 pb[QT];
+        #pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            float top = NEG_BIG;
+            #pragma unroll
+            for (int t = 0; t < 2; ++t)
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float value = s[qt][t][r] * args.scale_log2;
+                    if (edge && token0 + 16 * t + 4 * g + r > limit[qt]) value = -INFINITY;
+                    s[qt][t][r] = value;
+                    top = fmaxf(top, value);
+                }
+            top = fmaxf(top, __shfl_xor(top, 16));
+            top = fmaxf(top, __shfl_xor(top, 32));
+            // the running maximum rarely grows after the first steps: rescale only when some row's did
+            if (__any(top > m[qt])) {
+                const float m_new = fmaxf(m[qt], top);
+                const float alpha = __builtin_amdgcn_exp2f(m[qt] - m_new);
+                m[qt] = m_new;
+                l[qt] *= alpha;
+                #pragma unroll
+                for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] *= alpha;
+            }
+            float sum = 0.0f;
+            half8 p;
+            #pragma unroll
+            for (int t = 0; t < 2; ++t)
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float w = __builtin_amdgcn_exp2f(s[qt][t][r] - m[qt]);
+                    sum += w;
+                    p[4 * t + r] = (_Float16)w;
+                }
+            pb[qt] = p;
+            l[qt] += sum;
+        }
+        // O^T tiles: columns (rows of the tile, W*row + jj) x query rows
+        ValueScales<DIM> vs;
+        value_scales<DIM>(current, vs);
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj) {
+            const half8 va = value_operand<DIM>(current, vs, jj);
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[qt], acc[qt][jj], 0, 0, 0);
+        }
+    }
+
+    // A lane holds, of its query row, the columns W*(4g + r) + jj: for each r a run of W consecutive ones.
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int row = row0 + qt * 16 + li;
+        float sum = l[qt];
+        sum += __shfl_xor(sum, 16);
+        sum += __shfl_xor(sum, 32);
+        if (row >= int(args.rows)) continue;
+        const float inverse = 1.0f / sum;
+        const int span_row = row / int(args.group), head = kvh * int(args.group) + row % int(args.group);
+        const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
+        #pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const size_t first = at + W * (4 * g + r);
+            if (args.out_f16) {
+                #pragma unroll
+                for (int part = 0; part < TILES / 8; ++part) {
+                    half8 packed;
+                    #pragma unroll
+                    for (int jj = 0; jj < 8; ++jj) packed[jj] = (_Float16)(acc[qt][8 * part + jj][r] * inverse);
+                    *reinterpret_cast<half8*>(static_cast<_Float16*>(args.out) + first + 8 * part) = packed;
+                }
+            } else {
+                #pragma unroll
+                for (int part = 0; part < TILES / 4; ++part) {
+                    floatx4 packed;
+                    #pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) packed[jj] = acc[qt][4 * part + jj][r] * inverse;
+                    *reinterpret_cast<floatx4*>(static_cast<float*>(args.out) + first + 4 * part) = packed;
+                }
+            }
+        }
+    }
+}
+
+template<int DIM, int QT, bool Q8, int OCC>
+void launch(Device& d, const PrefillArgs& args, unsigned seqs) {
+    constexpr size_t shared = size_t(2) * 2 * STEP * (Q8 ? DIM + DIM / 16 : 2 * DIM);
+    static bool raised = false;
+    if (!raised && shared > 64 * 1024) {
+        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attention_kernel<DIM, QT, Q8, OCC>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
+        raised = true;
+    }
+    const unsigned tiles = (args.rows + WAVES * QT * 16 - 1) / (WAVES * QT * 16);
+    prefill_attention_kernel<DIM, QT, Q8, OCC><<<dim3(tiles, args.kv_heads, seqs), WAVES * 64, shared, d.stream>>>(args);
+}
+
+}  // namespace
+
+namespace sd {
+
+// Called by sdx_paged_attention (which has validated the arguments) when a sequence has more query rows per K/V head than
+// the decode kernel's workgroup takes.
+void prefill_attention(Device& d, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
+                       uint64_t max_context, const void* q, int q_f16, uint64_t seqs, uint64_t span, uint64_t heads, float scale, void* out,
+                       int out_f16) {
+    PrefillArgs args{};
+    args.pages = static_cast<const uint8_t*>(pool->pages);
+    args.page_tokens = pool->page_tokens; args.kv_heads = pool->kv_heads; args.heads = unsigned(heads);
+    args.group = unsigned(heads / pool->kv_heads); args.span = unsigned(span);
+    args.page_table = page_table; args.table_stride = size_t(table_stride); args.positions = positions;
+    args.q = q; args.q_f16 = q_f16; args.scale_log2 = scale * 1.44269504088896341f;
+    args.rows = unsigned(span * args.group); args.max_context = int(max_context);
+    args.out = out; args.out_f16 = out_f16;
+    const bool q8 = pool->row_bytes != 2 * pool->dim;
+    KernelTimer timer(d);
+    if (pool->dim == 128) { if (q8) launch<128, 4, true, 1>(d, args, unsigned(seqs)); else launch<128, 4, false, 1>(d, args, unsigned(seqs)); }
+    else { if (q8) launch<256, 2, true, 1>(d, args, unsigned(seqs)); else launch<256, 2, false, 1>(d, args, unsigned(seqs)); }
+}
+
+}  // namespace sd

@@ -90,6 +90,58 @@ class PagedWorkload:
             self.gpu.release(b)
 
 
+class PrefillWorkload:
+    """BASELINE config 2: one prompt prefilled in chunks.  A step appends each chunk's FP16 K/V rows to the Q8_0 cache and
+    runs causal attention of the chunk's queries over the cache so far."""
+
+    def __init__(self, gpu, tokens=8192, chunk=2048, heads=32, kv_heads=4, dim=128, page_tokens=256, seed=2):
+        self.gpu, self.tokens, self.chunk, self.heads, self.kv_heads, self.dim, self.page_tokens = gpu, tokens, chunk, heads, kv_heads, dim, page_tokens
+        self.row_bytes = ROW_Q8[dim]
+        rng = np.random.default_rng(seed)
+        self.page_count = (tokens + page_tokens - 1) // page_tokens
+        self.table = rng.permutation(self.page_count).astype(np.int32).reshape(1, -1)
+        self.scale = float(1.0 / np.sqrt(np.float32(dim)))
+        self.pool, self.pool_buffer = gpu.kv_pool(self.page_count, page_tokens, kv_heads, dim, self.row_bytes)
+        self.table_buffer = gpu.upload(self.table)
+        self.starts = gpu.upload(np.arange(0, tokens, chunk, dtype=np.int32))          # position of each chunk's first token
+        self.k = gpu.buffer(tokens * kv_heads * dim * 2)
+        self.v = gpu.buffer(tokens * kv_heads * dim * 2)
+        self.q = gpu.buffer(tokens * heads * dim * 2)
+        self.out = gpu.buffer(tokens * heads * dim * 2)
+        gpu.fill_normal(self.k.base(), tokens * kv_heads * dim, seed * 13 + 1, 1)
+        gpu.fill_normal(self.v.base(), tokens * kv_heads * dim, seed * 13 + 2, 1)
+        gpu.fill_normal(self.q.base(), tokens * heads * dim, seed * 13 + 3, 1)
+        self.scratch = gpu.buffer(max(gpu.paged_attention_scratch(1, chunk, heads, dim, tokens), 4))
+        gpu.synchronize()
+
+    def step(self):
+        g = self.gpu
+        for c in range(self.tokens // self.chunk):
+            kv_at, q_at = c * self.chunk * self.kv_heads * self.dim * 2, c * self.chunk * self.heads * self.dim * 2
+            g.kv_write(self.pool, self.table_buffer.base(), self.table.shape[1], self.starts.at(4 * c), self.k.at(kv_at), self.v.at(kv_at),
+                       True, 1, self.chunk)
+            g.paged_attention(self.pool, self.table_buffer.base(), self.table.shape[1], self.starts.at(4 * c), self.tokens,
+                              self.q.at(q_at), True, 1, self.chunk, self.heads, self.scale, self.out.at(q_at), True, self.scratch)
+
+    def flops(self):
+        # causal only: 2 products x 2 flops per (query row, visible key, column)
+        return 4 * self.heads * self.dim * (self.tokens * (self.tokens + 1) // 2)
+
+    def algorithmic_bytes(self):
+        # queries and outputs once, the chunk's K/V rows in and out, and the cache read once per chunk
+        chunks = self.tokens // self.chunk
+        cache = sum((c + 1) * self.chunk for c in range(chunks)) * self.kv_heads * 2 * self.row_bytes
+        io = self.tokens * self.heads * self.dim * 4 + self.tokens * self.kv_heads * self.dim * 2 * 2 + self.tokens * self.kv_heads * 2 * self.row_bytes
+        return cache + io
+
+    def read(self, buffer, count):
+        return self.gpu.read_buffer(buffer, 0, np.float16, count).astype(np.float32)
+
+    def release(self):
+        for b in (self.pool_buffer, self.table_buffer, self.starts, self.k, self.v, self.q, self.out, self.scratch):
+            self.gpu.release(b)
+
+
 class SparseWorkload:
     """BASELINE config 4: per sequence, index scores over BF16 keys -> top-k -> gather attention over BF16 latents."""
 

@@ -136,6 +136,53 @@ def test_verify_span_rows(gpu, oracle, span, heads, kv_heads):
     gpu.release(buffer); gpu.release(tb)
 
 
+@pytest.mark.parametrize("dim,fmt,span,heads,kv_heads", [(128, "q8", 40, 32, 4), (128, "q8", 100, 8, 1), (128, "f16", 33, 16, 2),
+                                                         (256, "q8", 24, 24, 2), (256, "f16", 9, 24, 2), (128, "q8", 9, 4, 4)])
+def test_prefill_span_rows(gpu, oracle, dim, fmt, span, heads, kv_heads):
+    # BASELINE config 2 in small: a chunk of new tokens attends the cache (which holds the chunk's own rows) causally.
+    # Rows per K/V head = span * group exceed what the decode kernel's workgroup takes, so this is the many-rows kernel.
+    rng = np.random.default_rng(77 + span + dim)
+    row_bytes = (dim + dim // 16) if fmt == "q8" else 2 * dim
+    page_tokens = 64
+    contexts = [0, 31, 200, 517]
+    lengths = [c + span for c in contexts]
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, lengths, kv_heads, dim, page_tokens, row_bytes,
+                                              dtype=np.float32 if fmt == "q8" else np.float16)
+    seqs = len(lengths)
+    q = rng.standard_normal((seqs, span, heads, dim)).astype(np.float16).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array(contexts, np.int32), q, scale)
+    for q_f16, out_f16 in ((True, False), (False, False), (True, True)):
+        got = _run(gpu, pool, table, tb, contexts, q, span, heads, scale, q_f16, out_f16)
+        if out_f16:
+            assert np.abs(got - want).max() <= 2e-3 + 2.0 ** -11 * np.abs(want).max()
+        else:
+            close_enough(got, want, f"prefill span {span} dim {dim} {fmt}")
+    # the span's last row is the single-token decode at the last position
+    single = _run(gpu, pool, table, tb, [c + span - 1 for c in contexts], q[:, span - 1:], 1, heads, scale, True, False)
+    got = _run(gpu, pool, table, tb, contexts, q, span, heads, scale, True, False)
+    close_enough(single[:, 0], want[:, span - 1], "last row alone")
+    assert np.abs(single[:, 0] - got[:, span - 1]).max() < 2e-4
+    gpu.release(buffer); gpu.release(tb)
+
+
+def test_prefill_in_chunks_equals_prefill_at_once(gpu, oracle):
+    # a prompt prefilled in 4 chunks (each chunk attends the cache so far) gives the rows of one whole-prompt pass
+    rng = np.random.default_rng(5)
+    dim, row_bytes, page_tokens, heads, kv_heads, tokens, chunk = 128, 136, 64, 16, 2, 512, 128
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, [tokens], kv_heads, dim, page_tokens, row_bytes)
+    q = rng.standard_normal((1, tokens, heads, dim)).astype(np.float16).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    whole = _run(gpu, pool, table, tb, [0], q, tokens, heads, scale, True, False)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.zeros(1, np.int32), q, scale)
+    close_enough(whole, want, "whole prompt")
+    for c in range(tokens // chunk):
+        part = _run(gpu, pool, table, tb, [c * chunk], q[:, c * chunk:(c + 1) * chunk], chunk, heads, scale, True, False,
+                    max_context=tokens)
+        assert np.array_equal(part, whole[:, c * chunk:(c + 1) * chunk])     # the same keys in the same order: the same bits
+    gpu.release(buffer); gpu.release(tb)
+
+
 def test_zero_queries_give_the_mean_of_the_values(gpu, oracle):
     rng = np.random.default_rng(5)
     heads, kv_heads, dim, row_bytes, page_tokens = 8, 2, 128, 136, 32
