@@ -6,13 +6,14 @@
 // dense selection 0..position.
 //
 // Shape of the work on gfx950 (wave64, v_mfma_f32_16x16x32_f16):
-//   * a workgroup (4 waves) owns 4 x QT x 16 consecutive query rows of one (sequence, K/V head): rows are ordered
-//     (span row, head in group), so a workgroup is a run of consecutive tokens with all their grouped heads and
-//     every K/V row it reads serves all of them; a wave owns QT x 16 of those rows with their own online softmax, so
-//     no merge is needed and the output is written once, normalised;
-//   * the workgroup walks the keys 32 at a time: the step's K and V slabs (32 contiguous rows of a page plane) are
-//     copied by coalesced 16-byte global->LDS loads, a quarter by each wave, into one of two stages, so the next
-//     step's copy is in flight while this one is computed; one barrier per step;
+//   * a workgroup (8 waves, two per SIMD) owns 4 x QT x 16 consecutive query rows of one (sequence, K/V head): rows
+//     are ordered (span row, head in group), so a workgroup is a run of consecutive tokens with all their grouped
+//     heads and every K/V row it reads serves all of them; a quarter of the rows belongs to a pair of waves, one
+//     taking the first 32 keys of every 64-key step and one the last 32, each with its own online softmax; the pair
+//     merges through LDS at the end and the output is written once, normalised;
+//   * the workgroup walks the keys 64 at a time: the step's K and V slabs (64 contiguous rows of a page plane) are
+//     copied by coalesced 16-byte global->LDS loads, an eighth by each wave, into a ring of stages, so the copies of
+//     the next steps are in flight while this one is computed; one barrier per step;
 //   * every wave builds its MFMA operands from the stage (paged_rows.hpp) and skips steps that lie wholly after
 //     its rows' positions; the workgroups with the longest walks are dispatched first.
 #include "paged_rows.hpp"
@@ -23,6 +24,15 @@ using namespace sd;
 using namespace sd::paged;
 
 namespace {
+
+constexpr float SLACK = 8.0f;     // how far (base-2 exponent) a row's true maximum may run ahead of its reference maximum
+// The ring of K/V stages: the copies of STAGES - 1 steps are in flight or landed; as many as fit beside nothing else, at most 4.
+constexpr int stages_for(int stage_bytes) { return 150 * 1024 / stage_bytes < 4 ? 150 * 1024 / stage_bytes : 4; }
+constexpr int GROUPS = 4, HALVES = 2, TEAM = GROUPS * HALVES;   // row quarters x key halves = waves of a workgroup
+constexpr int WALK = HALVES * STEP;                            // keys per step of the workgroup
+
+// s_waitcnt for the vector-memory counter alone: wait until at most N of the wave's loads are outstanding.
+template<int N> __device__ __forceinline__ void wait_loads() { __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14)); }
 
 struct PrefillArgs {
     const uint8_t* pages;
@@ -40,15 +50,17 @@ struct PrefillArgs {
 };
 
 template<int DIM, int QT, bool Q8, int OCC>
-__global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) prefill_attention_kernel(PrefillArgs args) {
+__global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) prefill_attention_kernel(PrefillArgs args) {
     constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, BLOCKS = DIM / 32, W = DIM / 16, TILES = DIM / 16;
-    constexpr int SLAB = STEP * ROW, UNITS = (SLAB + 1023) / 1024;     // a slab is copied 1 KiB (one instruction of a wave) at a time
-    constexpr int WAVE_ROWS = QT * 16, GROUP_ROWS = WAVES * WAVE_ROWS;
+    constexpr int SLAB = WALK * ROW, UNITS = (SLAB + 1023) / 1024;     // a slab is copied 1 KiB (one instruction of a wave) at a time
+    constexpr int WAVE_ROWS = QT * 16, GROUP_ROWS = GROUPS * WAVE_ROWS, STAGES = stages_for(2 * SLAB);
+    static_assert(STAGES >= 2, "a step is copied while the one before is computed");
     const int tile = int(gridDim.x) - 1 - int(blockIdx.x), kvh = blockIdx.y, seq = blockIdx.z;   // later rows walk further: first
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, g = lane >> 4;
     const int position = args.positions[seq];
     const int cached = min(position + int(args.span), args.max_context);          // rows of the sequence the cache holds
-    const int row0 = tile * GROUP_ROWS + wave * WAVE_ROWS;                        // the wave's first query row
+    const int quarter = wave % GROUPS, half = wave / GROUPS;                      // waves w and w + 4 share a SIMD and the rows
+    const int row0 = tile * GROUP_ROWS + quarter * WAVE_ROWS;                     // the wave's first query row
     const int group_last = min(int(args.rows), (tile + 1) * GROUP_ROWS) - 1;
     const int keys = min(position + group_last / int(args.group) + 1, cached);    // the workgroup walks keys 0..keys-1
     const bool idle = row0 >= int(args.rows);                                     // a wave past the last row only helps copying
@@ -56,7 +68,9 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
     const int wave_last = position + (min(int(args.rows), row0 + WAVE_ROWS) - 1) / int(args.group);   // the wave's rows
     const table_ptr table = (table_ptr)(args.page_table + size_t(seq) * args.table_stride);
     const size_t plane_bytes = size_t(args.page_tokens) * ROW;
-    extern __shared__ uint8_t stages[];                                           // [2][K slab | V slab]
+    extern __shared__ uint8_t stages[];                                           // [STAGES][K slab | V slab]
+    constexpr int MOST = (2 * UNITS + TEAM - 1) / TEAM, LEAST = 2 * UNITS / TEAM;   // copy instructions a wave issues per step
+    const bool most = wave < 2 * UNITS - LEAST * TEAM;
 
     // The step's two slabs into a stage: 2 * UNITS pieces of 1 KiB, every fourth one by this wave.
     const auto copy_in = [&](int buffer, int token0) {
@@ -64,14 +78,18 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(token0 % int(args.page_tokens)) * ROW + 16 * lane;
         uint8_t* stage = stages + buffer * (2 * SLAB);
         #pragma unroll
-        for (int k = 0; k < (2 * UNITS + WAVES - 1) / WAVES; ++k) {
-            const int unit = wave + WAVES * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS;
+        for (int k = 0; k < MOST; ++k) {
+            const int unit = wave + TEAM * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS;
             if (unit < 2 * UNITS && 16 * lane + 1024 * j < SLAB)
                 __builtin_amdgcn_global_load_lds((global_ptr)(base + size_t(part ? args.kv_heads : 0) * plane_bytes + 1024 * j),
                                                  (lds_ptr)(stage + part * SLAB + 1024 * j), 16, 0, 0);
         }
     };
-    copy_in(0, 0);
+    // Steps past the last one are copied again from the last one's rows (and never read), so that the count of loads in flight
+    // is the same at every step.
+    const int last_step = (keys - 1) / WALK * WALK;
+    #pragma unroll
+    for (int ahead = 0; ahead < STAGES - 1; ++ahead) copy_in(ahead, min(ahead * WALK, last_step));
 
     // Query rows: row = span_row * group + head_in_group; a lane holds row row0 + qt*16 + li as B operands.  A row past the
     // last real one holds zeros and is never stored.
@@ -107,23 +125,25 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    for (int token0 = 0, buffer = 0; token0 < keys; token0 += STEP, buffer ^= 1) {
-        __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0): this wave's pieces of the step have landed
-        __syncthreads();                             // ... and everybody's; the other stage is no longer being read
-        if (token0 + STEP < keys) copy_in(buffer ^ 1, token0 + STEP);
+    for (int walk0 = 0, buffer = 0; walk0 < keys; walk0 += WALK, buffer = buffer + 1 == STAGES ? 0 : buffer + 1) {
+        // this wave's pieces of the step have landed when only the later steps' are outstanding
+        if (most) wait_loads<MOST * (STAGES - 2)>(); else wait_loads<LEAST * (STAGES - 2)>();
+        __syncthreads();                             // ... and everybody's; the stage of the step before is no longer being read
+        copy_in(buffer == 0 ? STAGES - 1 : buffer - 1, min(walk0 + (STAGES - 1) * WALK, last_step));
         uint8_t* stage = stages + buffer * (2 * SLAB);
-        if (cached - token0 < STEP) {
+        if (cached - walk0 < WALK) {
             // the sequence's last rows: the stage's tail holds whatever the page held.  It is cleared (those scores are masked,
             // but a stray scale must not meet a zero weight).
             #pragma unroll
             for (int part = 0; part < 2; ++part)
-                for (int at = (cached - token0) * ROW + 4 * int(threadIdx.x); at < SLAB; at += 4 * WAVES * 64)
+                for (int at = (cached - walk0) * ROW + 4 * int(threadIdx.x); at < SLAB; at += 4 * TEAM * 64)
                     *reinterpret_cast<uint32_t*>(stage + part * SLAB + at) = 0u;
             __syncthreads();
         }
-        if (idle || token0 > wave_last) continue;    // nothing of this step is visible to the wave's rows
+        const int token0 = walk0 + half * STEP;      // the wave's 32 keys of the step
+        if (idle || token0 > wave_last || token0 >= keys) continue;    // none of them is visible to the wave's rows
         RowLoad<DIM, Q8> current;
-        load_step<DIM>(current, stage, stage + SLAB, li, g);
+        load_step<DIM>(current, stage + half * STEP * ROW, stage + SLAB + half * STEP * ROW, li, g);
         // S^T tiles: tokens (rows, 4 per lane group) x query rows (lane li)
         floatx4 s[QT][2];
         #pragma unroll
@@ -137,38 +157,42 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
                 for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qf[qt][b], s[qt][t], 0, 0, 0);
             }
         }
-        const bool edge = token0 + STEP - 1 > wave_first;    // wave-uniform: some token of the step is past some row's position
+        // Scores stay unscaled; the scale goes into the exponent's multiply-add.  m is a row's reference maximum in unscaled units.
+        if (token0 + STEP - 1 > wave_first) {          // wave-uniform: some token of the step is past some row's position
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt)
+                #pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    #pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (token0 + 16 * t + 4 * g + r > limit[qt]) s[qt][t][r] = -INFINITY;
+        }
         half8 pb[QT];
         #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
-            float top = NEG_BIG;
-            #pragma unroll
-            for (int t = 0; t < 2; ++t)
-                #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float value = s[qt][t][r] * args.scale_log2;
-                    if (edge && token0 + 16 * t + 4 * g + r > limit[qt]) value = -INFINITY;
-                    s[qt][t][r] = value;
-                    top = fmaxf(top, value);
-                }
+            float top = fmaxf(fmaxf(fmaxf(s[qt][0][0], s[qt][0][1]), fmaxf(s[qt][0][2], s[qt][0][3])),
+                              fmaxf(fmaxf(s[qt][1][0], s[qt][1][1]), fmaxf(s[qt][1][2], s[qt][1][3])));
             top = fmaxf(top, __shfl_xor(top, 16));
             top = fmaxf(top, __shfl_xor(top, 32));
-            // the running maximum rarely grows after the first steps: rescale only when some row's did
-            if (__any(top > m[qt])) {
+            // The reference maximum follows the true one only when that has grown by more than SLACK (in base-2 exponent
+            // units): weights then stay below 2^SLACK, far inside FP16 and FP32 range, and the accumulators are rescaled
+            // a few times per row instead of at every new maximum.  The quotient sum/acc does not depend on the reference.
+            if (__any((top - m[qt]) * args.scale_log2 > SLACK)) {
                 const float m_new = fmaxf(m[qt], top);
-                const float alpha = __builtin_amdgcn_exp2f(m[qt] - m_new);
+                const float alpha = __builtin_amdgcn_exp2f((m[qt] - m_new) * args.scale_log2);
                 m[qt] = m_new;
                 l[qt] *= alpha;
                 #pragma unroll
                 for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] *= alpha;
             }
+            const float offset = -m[qt] * args.scale_log2;
             float sum = 0.0f;
             half8 p;
             #pragma unroll
             for (int t = 0; t < 2; ++t)
                 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float w = __builtin_amdgcn_exp2f(s[qt][t][r] - m[qt]);
+                    const float w = __builtin_amdgcn_exp2f(fmaf(s[qt][t][r], args.scale_log2, offset));
                     sum += w;
                     p[4 * t + r] = (_Float16)w;
                 }
@@ -186,15 +210,46 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         }
     }
 
+    // The pair of waves that shares rows merges: the second half's wave leaves its state in LDS (the stages are done with),
+    // register by register with the lane innermost, and the first half's wave adds it in under the common reference maximum.
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        l[qt] += __shfl_xor(l[qt], 16);
+        l[qt] += __shfl_xor(l[qt], 32);
+    }
+    __syncthreads();
+    float* mine = reinterpret_cast<float*>(stages) + size_t(quarter) * (QT * (TILES * 4 + 2)) * 64 + lane;
+    if (half == 1) {
+        #pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            float* at = mine + size_t(qt) * (TILES * 4 + 2) * 64;
+            at[0] = m[qt]; at[64] = l[qt];
+            #pragma unroll
+            for (int jj = 0; jj < TILES; ++jj)
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) at[(2 + 4 * jj + r) * 64] = acc[qt][jj][r];
+        }
+    }
+    __syncthreads();
+    if (half == 1) return;
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const float* at = mine + size_t(qt) * (TILES * 4 + 2) * 64;
+        const float other = at[0], top = fmaxf(m[qt], other);
+        const float keep = __builtin_amdgcn_exp2f((m[qt] - top) * args.scale_log2), add = __builtin_amdgcn_exp2f((other - top) * args.scale_log2);
+        l[qt] = l[qt] * keep + at[64] * add;
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj)
+            #pragma unroll
+            for (int r = 0; r < 4; ++r) acc[qt][jj][r] = acc[qt][jj][r] * keep + at[(2 + 4 * jj + r) * 64] * add;
+    }
+
     // A lane holds, of its query row, the columns W*(4g + r) + jj: for each r a run of W consecutive ones.
     #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
         const int row = row0 + qt * 16 + li;
-        float sum = l[qt];
-        sum += __shfl_xor(sum, 16);
-        sum += __shfl_xor(sum, 32);
         if (row >= int(args.rows)) continue;
-        const float inverse = 1.0f / sum;
+        const float inverse = 1.0f / l[qt];
         const int span_row = row / int(args.group), head = kvh * int(args.group) + row % int(args.group);
         const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
         #pragma unroll
@@ -223,14 +278,17 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
 
 template<int DIM, int QT, bool Q8, int OCC>
 void launch(Device& d, const PrefillArgs& args, unsigned seqs) {
-    constexpr size_t shared = size_t(2) * 2 * STEP * (Q8 ? DIM + DIM / 16 : 2 * DIM);
+    constexpr size_t merge = size_t(GROUPS) * QT * (DIM / 16 * 4 + 2) * 64 * 4;
+    constexpr size_t stage = size_t(2) * WALK * (Q8 ? DIM + DIM / 16 : 2 * DIM), ring = stages_for(int(stage)) * stage;
+    constexpr size_t shared = ring > merge ? ring : merge;
+    static_assert(shared <= 160 * 1024, "the stages and the merge area share the compute unit's LDS");
     static bool raised = false;
     if (!raised && shared > 64 * 1024) {
         SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attention_kernel<DIM, QT, Q8, OCC>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
         raised = true;
     }
-    const unsigned tiles = (args.rows + WAVES * QT * 16 - 1) / (WAVES * QT * 16);
-    prefill_attention_kernel<DIM, QT, Q8, OCC><<<dim3(tiles, args.kv_heads, seqs), WAVES * 64, shared, d.stream>>>(args);
+    const unsigned tiles = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
+    prefill_attention_kernel<DIM, QT, Q8, OCC><<<dim3(tiles, args.kv_heads, seqs), TEAM * 64, shared, d.stream>>>(args);
 }
 
 }  // namespace
@@ -252,8 +310,8 @@ void prefill_attention(Device& d, const sdx_kv_pool* pool, const int32_t* page_t
     args.out = out; args.out_f16 = out_f16;
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     KernelTimer timer(d);
-    if (pool->dim == 128) { if (q8) launch<128, 4, true, 1>(d, args, unsigned(seqs)); else launch<128, 4, false, 1>(d, args, unsigned(seqs)); }
-    else { if (q8) launch<256, 2, true, 1>(d, args, unsigned(seqs)); else launch<256, 2, false, 1>(d, args, unsigned(seqs)); }
+    if (pool->dim == 128) { if (q8) launch<128, 3, true, 2>(d, args, unsigned(seqs)); else launch<128, 3, false, 2>(d, args, unsigned(seqs)); }
+    else { if (q8) launch<256, 1, true, 2>(d, args, unsigned(seqs)); else launch<256, 1, false, 2>(d, args, unsigned(seqs)); }
 }
 
 }  // namespace sd

@@ -162,7 +162,7 @@ def test_prefill_span_rows(gpu, oracle, dim, fmt, span, heads, kv_heads):
     single = _run(gpu, pool, table, tb, [c + span - 1 for c in contexts], q[:, span - 1:], 1, heads, scale, True, False)
     got = _run(gpu, pool, table, tb, contexts, q, span, heads, scale, True, False)
     close_enough(single[:, 0], want[:, span - 1], "last row alone")
-    assert np.abs(single[:, 0] - got[:, span - 1]).max() < 2e-4
+    assert np.abs(single[:, 0] - got[:, span - 1]).max() < 1e-3      # two kernels, two roundings of the FP16 weights
     gpu.release(buffer); gpu.release(tb)
 
 
