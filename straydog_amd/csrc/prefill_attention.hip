@@ -27,6 +27,8 @@ namespace {
 
 constexpr float SLACK = 8.0f;     // how far (base-2 exponent) a row's true maximum may run ahead of its reference maximum
 // The ring of K/V stages: the copies of STAGES - 1 steps are in flight or landed; as many as fit beside nothing else, at most 4.
+// The same for the kernel that also keeps two pairs of FP16 tiles, at most 3.
+constexpr int tiles_ring(int stage_bytes, int tiles_bytes) { return (158 * 1024 - tiles_bytes) / stage_bytes < 3 ? (158 * 1024 - tiles_bytes) / stage_bytes : 3; }
 constexpr int stages_for(int stage_bytes) { return 150 * 1024 / stage_bytes < 4 ? 150 * 1024 / stage_bytes : 4; }
 constexpr int GROUPS = 4, HALVES = 2, TEAM = GROUPS * HALVES;   // row quarters x key halves = waves of a workgroup
 constexpr int WALK = HALVES * STEP;                            // keys per step of the workgroup
@@ -276,6 +278,300 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     }
 }
 
+// The second form of the kernel, for 128 columns: the workgroup converts every step's rows once into FP16 tiles in LDS (K
+// as rows with a 16-byte pad, V transposed with an 8-byte pad: both read without bank conflicts as MFMA operands), so the
+// Q8_0 -> FP16 work is shared by the eight waves instead of being done by each.  While a step is computed from one pair
+// of tiles the next step's raw rows (already landed) are converted into the other pair; one barrier per step.
+// Columns of an output tile jj are 16 jj + (0..15), a lane holding 16 jj + 4 g + r.
+template<int DIM, int QT, bool Q8>
+__global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) prefill_tiles_kernel(PrefillArgs args) {
+    constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, BLOCKS = DIM / 32, TILES = DIM / 16;
+    constexpr int SLAB = WALK * ROW, UNITS = (SLAB + 1023) / 1024;
+    constexpr int WAVE_ROWS = QT * 16, GROUP_ROWS = GROUPS * WAVE_ROWS;
+    constexpr int KP = 2 * DIM + 16, VP = 2 * WALK + 8, KT = WALK * KP, VT = DIM * VP;     // pitches and sizes of the FP16 tiles
+    constexpr int RING = tiles_ring(2 * SLAB, 2 * (KT + VT));
+    static_assert(RING >= 2 && WALK == 64 && TEAM == 8, "512 threads convert a step of 64 rows, one piece each");
+    const int tile = int(gridDim.x) - 1 - int(blockIdx.x), kvh = blockIdx.y, seq = blockIdx.z;
+    const int thread = threadIdx.x, lane = thread & 63, wave = __builtin_amdgcn_readfirstlane(thread >> 6), li = lane & 15, g = lane >> 4;
+    const int position = args.positions[seq];
+    const int cached = min(position + int(args.span), args.max_context);
+    const int quarter = wave % GROUPS, half = wave / GROUPS;
+    const int row0 = tile * GROUP_ROWS + quarter * WAVE_ROWS;
+    const int group_last = min(int(args.rows), (tile + 1) * GROUP_ROWS) - 1;
+    const int keys = min(position + group_last / int(args.group) + 1, cached);
+    const bool idle = row0 >= int(args.rows);
+    const int wave_first = position + row0 / int(args.group);
+    const int wave_last = position + (min(int(args.rows), row0 + WAVE_ROWS) - 1) / int(args.group);
+    const table_ptr table = (table_ptr)(args.page_table + size_t(seq) * args.table_stride);
+    const size_t plane_bytes = size_t(args.page_tokens) * ROW;
+    extern __shared__ uint8_t stages[];                        // [RING][K slab | V slab] raw rows, then [2][K tile | V tile]
+    uint8_t* const tiles = stages + RING * (2 * SLAB);
+    constexpr int MOST = (2 * UNITS + TEAM - 1) / TEAM, LEAST = 2 * UNITS / TEAM;
+    const bool most = wave < 2 * UNITS - LEAST * TEAM;
+
+    const auto copy_in = [&](int buffer, int token0) {
+        const int page = table[token0 / int(args.page_tokens)];
+        const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(token0 % int(args.page_tokens)) * ROW + 16 * lane;
+        uint8_t* stage = stages + buffer * (2 * SLAB);
+        #pragma unroll
+        for (int k = 0; k < MOST; ++k) {
+            const int unit = wave + TEAM * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS;
+            if (unit < 2 * UNITS && 16 * lane + 1024 * j < SLAB)
+                __builtin_amdgcn_global_load_lds((global_ptr)(base + size_t(part ? args.kv_heads : 0) * plane_bytes + 1024 * j),
+                                                 (lds_ptr)(stage + part * SLAB + 1024 * j), 16, 0, 0);
+        }
+    };
+    // One step's raw rows into FP16 tiles; rows past the sequence's end become zeros (the page holds anything there).
+    const auto convert = [&](int buffer, int into, int walk0) {
+        const uint8_t* raw = stages + buffer * (2 * SLAB);
+        uint8_t* ktile = tiles + into * (KT + VT);
+        uint8_t* vtile = ktile + KT;
+        const int valid = cached - walk0;                      // rows of the step the cache holds
+        if (Q8) {
+            {   // K: 16 columns of one row
+                const int key = thread >> 3, piece = thread & 7;
+                const uint8_t* from = raw + key * ROW;
+                const uint2 a = *reinterpret_cast<const uint2*>(from + 16 * piece), b = *reinterpret_cast<const uint2*>(from + 16 * piece + 8);
+                uint32_t scale_bits = *reinterpret_cast<const uint16_t*>(from + DIM + 2 * (piece >> 1));
+                if (key >= valid) scale_bits = 0;
+                const half2v scale = as_half2(scale_bits | (scale_bits << 16));
+                const uint32_t words[4] = {a.x, a.y, b.x, b.y};
+                half2v out[8];
+                #pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t bits = words[w] ^ 0x80808080u;
+                    out[2 * w] = magic_to_half2(byte_perm(0x64646464u, bits, 0x04010400u), scale);
+                    out[2 * w + 1] = magic_to_half2(byte_perm(0x64646464u, bits, 0x04030402u), scale);
+                }
+                half8* to = reinterpret_cast<half8*>(ktile + key * KP + 32 * piece);
+                to[0] = half8{out[0].x, out[0].y, out[1].x, out[1].y, out[2].x, out[2].y, out[3].x, out[3].y};
+                to[1] = half8{out[4].x, out[4].y, out[5].x, out[5].y, out[6].x, out[6].y, out[7].x, out[7].y};
+            }
+            {   // V: 4 rows x 4 columns, transposed
+                const int rows4 = thread & 15, cols4 = thread >> 4;
+                const uint8_t* from = raw + SLAB + 4 * rows4 * ROW;
+                uint32_t words[4], scales[4];
+                #pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    words[e] = *reinterpret_cast<const uint32_t*>(from + e * ROW + 4 * cols4);
+                    scales[e] = 4 * rows4 + e < valid ? uint32_t(*reinterpret_cast<const uint16_t*>(from + e * ROW + DIM + 2 * (cols4 >> 3))) : 0u;
+                    if (4 * rows4 + e >= valid) words[e] = 0x80808080u ^ 0x80808080u;
+                }
+                const half2v first = as_half2(scales[0] | (scales[1] << 16)), second = as_half2(scales[2] | (scales[3] << 16));
+                #pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const uint32_t sel = 0x0c000c00u | uint32_t(c) | (uint32_t(4 + c) << 16);
+                    const half2v lo = magic_to_half2(byte_perm(words[1], words[0], sel) ^ 0x64806480u, first);
+                    const half2v hi = magic_to_half2(byte_perm(words[3], words[2], sel) ^ 0x64806480u, second);
+                    uint2 packed;
+                    packed.x = __builtin_bit_cast(uint32_t, lo); packed.y = __builtin_bit_cast(uint32_t, hi);
+                    *reinterpret_cast<uint2*>(vtile + (4 * cols4 + c) * VP + 8 * rows4) = packed;
+                }
+            }
+        } else {
+            // K: the slab is 16-byte pieces one after the other; piece c goes to its row's place in the padded tile
+            #pragma unroll
+            for (int k = 0; k < SLAB / 16 / (TEAM * 64); ++k) {
+                const int c = thread + TEAM * 64 * k, key = c / (ROW / 16), at = (c % (ROW / 16)) * 16;
+                uint4 piece = *reinterpret_cast<const uint4*>(raw + 16 * c);
+                if (key >= valid) piece = uint4{0u, 0u, 0u, 0u};
+                *reinterpret_cast<uint4*>(ktile + key * KP + at) = piece;
+            }
+            // V: 4 rows x 4 columns, transposed
+            #pragma unroll
+            for (int k = 0; k < (WALK / 4) * (DIM / 4) / (TEAM * 64); ++k) {
+                const int block = thread + TEAM * 64 * k, rows4 = block & 15, cols4 = block >> 4;
+                const uint8_t* from = raw + SLAB + 4 * rows4 * ROW + 8 * cols4;
+                uint2 words[4];
+                #pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    words[e] = *reinterpret_cast<const uint2*>(from + e * ROW);
+                    if (4 * rows4 + e >= valid) words[e] = uint2{0u, 0u};
+                }
+                #pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+                    uint2 packed;
+                    packed.x = byte_perm(c < 2 ? words[1].x : words[1].y, c < 2 ? words[0].x : words[0].y, sel);
+                    packed.y = byte_perm(c < 2 ? words[3].x : words[3].y, c < 2 ? words[2].x : words[2].y, sel);
+                    *reinterpret_cast<uint2*>(vtile + (4 * cols4 + c) * VP + 8 * rows4) = packed;
+                }
+            }
+        }
+    };
+
+    const int last_step = (keys - 1) / WALK * WALK;
+    #pragma unroll
+    for (int ahead = 0; ahead < RING; ++ahead) copy_in(ahead, min(ahead * WALK, last_step));
+
+    half8 qf[QT][BLOCKS];
+    int limit[QT];
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int row = row0 + qt * 16 + li;
+        const bool real = row < int(args.rows);
+        const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
+        limit[qt] = real ? position + span_row : 0x7fffffff;
+        const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
+        #pragma unroll
+        for (int b = 0; b < BLOCKS; ++b) {
+            half8 value = {};
+            if (real) {
+                if (args.q_f16) value = *reinterpret_cast<const half8*>(static_cast<const _Float16*>(args.q) + at + 32 * b + 8 * g);
+                else {
+                    const float* from = static_cast<const float*>(args.q) + at + 32 * b + 8 * g;
+                    #pragma unroll
+                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)from[i];
+                }
+            }
+            qf[qt][b] = value;
+        }
+    }
+    floatx4 acc[QT][TILES];
+    float m[QT], l[QT];
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        m[qt] = NEG_BIG; l[qt] = 0.0f;
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    // the first step's tiles
+    if (most) wait_loads<MOST * (RING - 1)>(); else wait_loads<LEAST * (RING - 1)>();
+    __syncthreads();
+    convert(0, 0, 0);
+
+    for (int walk0 = 0, step = 0; walk0 < keys; walk0 += WALK, ++step) {
+        // the next step's raw rows have landed when only the later steps' copies are outstanding
+        if (most) wait_loads<MOST * (RING - 2)>(); else wait_loads<LEAST * (RING - 2)>();
+        __syncthreads();      // everybody's pieces have; this step's tiles are written; the other tiles and the raw stage of this step are free
+        copy_in(step % RING, min(walk0 + RING * WALK, last_step));
+        if (walk0 + WALK < keys) convert((step + 1) % RING, (step + 1) & 1, walk0 + WALK);
+        const int token0 = walk0 + half * STEP;
+        if (idle || token0 > wave_last || token0 >= keys) continue;
+        const uint8_t* ktile = tiles + (step & 1) * (KT + VT) + half * STEP * KP;
+        const uint8_t* vtile = tiles + (step & 1) * (KT + VT) + KT + half * STEP * 2;
+        floatx4 s[QT][2];
+        #pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt) s[qt][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            #pragma unroll
+            for (int b = 0; b < BLOCKS; ++b) {
+                const half8 ka = *reinterpret_cast<const half8*>(ktile + (16 * t + li) * KP + 64 * b + 16 * g);
+                #pragma unroll
+                for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qf[qt][b], s[qt][t], 0, 0, 0);
+            }
+        }
+        if (token0 + STEP - 1 > wave_first) {
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt)
+                #pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    #pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (token0 + 16 * t + 4 * g + r > limit[qt]) s[qt][t][r] = -INFINITY;
+        }
+        half8 pb[QT];
+        #pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            float top = fmaxf(fmaxf(fmaxf(s[qt][0][0], s[qt][0][1]), fmaxf(s[qt][0][2], s[qt][0][3])),
+                              fmaxf(fmaxf(s[qt][1][0], s[qt][1][1]), fmaxf(s[qt][1][2], s[qt][1][3])));
+            top = fmaxf(top, __shfl_xor(top, 16));
+            top = fmaxf(top, __shfl_xor(top, 32));
+            if (__any((top - m[qt]) * args.scale_log2 > SLACK)) {
+                const float m_new = fmaxf(m[qt], top);
+                const float alpha = __builtin_amdgcn_exp2f((m[qt] - m_new) * args.scale_log2);
+                m[qt] = m_new;
+                l[qt] *= alpha;
+                #pragma unroll
+                for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] *= alpha;
+            }
+            const float offset = -m[qt] * args.scale_log2;
+            float sum = 0.0f;
+            half8 p;
+            #pragma unroll
+            for (int t = 0; t < 2; ++t)
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float w = __builtin_amdgcn_exp2f(fmaf(s[qt][t][r], args.scale_log2, offset));
+                    sum += w;
+                    p[4 * t + r] = (_Float16)w;
+                }
+            pb[qt] = p;
+            l[qt] += sum;
+        }
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj) {
+            const uint8_t* from = vtile + (16 * jj + li) * VP + 8 * g;
+            const uint2 near = *reinterpret_cast<const uint2*>(from), far = *reinterpret_cast<const uint2*>(from + 32);
+            const uint4 both = {near.x, near.y, far.x, far.y};
+            const half8 va = __builtin_bit_cast(half8, both);
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[qt], acc[qt][jj], 0, 0, 0);
+        }
+    }
+
+    // The pair of waves that shares rows merges through LDS (the stages and tiles are done with).
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        l[qt] += __shfl_xor(l[qt], 16);
+        l[qt] += __shfl_xor(l[qt], 32);
+    }
+    __syncthreads();
+    float* mine = reinterpret_cast<float*>(stages) + size_t(quarter) * (QT * (TILES * 4 + 2)) * 64 + lane;
+    if (half == 1) {
+        #pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            float* at = mine + size_t(qt) * (TILES * 4 + 2) * 64;
+            at[0] = m[qt]; at[64] = l[qt];
+            #pragma unroll
+            for (int jj = 0; jj < TILES; ++jj)
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) at[(2 + 4 * jj + r) * 64] = acc[qt][jj][r];
+        }
+    }
+    __syncthreads();
+    if (half == 1) return;
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int row = row0 + qt * 16 + li;
+        const float* at = mine + size_t(qt) * (TILES * 4 + 2) * 64;
+        const float other = at[0], top = fmaxf(m[qt], other);
+        const float keep = __builtin_amdgcn_exp2f((m[qt] - top) * args.scale_log2), add = __builtin_amdgcn_exp2f((other - top) * args.scale_log2);
+        const float inverse = 1.0f / (l[qt] * keep + at[64] * add);
+        if (row >= int(args.rows)) continue;
+        const int span_row = row / int(args.group), head = kvh * int(args.group) + row % int(args.group);
+        const size_t first = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM + 4 * g;
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj) {
+            floatx4 value;
+            #pragma unroll
+            for (int r = 0; r < 4; ++r) value[r] = (acc[qt][jj][r] * keep + at[(2 + 4 * jj + r) * 64] * add) * inverse;
+            if (args.out_f16) {
+                typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+                *reinterpret_cast<half4*>(static_cast<_Float16*>(args.out) + first + 16 * jj) = half4{(_Float16)value[0], (_Float16)value[1], (_Float16)value[2], (_Float16)value[3]};
+            } else *reinterpret_cast<floatx4*>(static_cast<float*>(args.out) + first + 16 * jj) = value;
+        }
+    }
+}
+
+template<int DIM, int QT, bool Q8>
+void launch_tiles(Device& d, const PrefillArgs& args, unsigned seqs) {
+    constexpr size_t merge = size_t(GROUPS) * QT * (DIM / 16 * 4 + 2) * 64 * 4;
+    constexpr size_t stage = size_t(2) * WALK * (Q8 ? DIM + DIM / 16 : 2 * DIM), pair = size_t(2) * (WALK * (2 * DIM + 16) + DIM * (2 * WALK + 8));
+    constexpr size_t ring = tiles_ring(int(stage), int(pair)) * stage + pair;
+    constexpr size_t shared = ring > merge ? ring : merge;
+    static_assert(shared <= 160 * 1024, "the stages, the tiles and the merge area share the compute unit's LDS");
+    static bool raised = false;
+    if (!raised && shared > 64 * 1024) {
+        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_tiles_kernel<DIM, QT, Q8>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
+        raised = true;
+    }
+    const unsigned tiles = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
+    prefill_tiles_kernel<DIM, QT, Q8><<<dim3(tiles, args.kv_heads, seqs), TEAM * 64, shared, d.stream>>>(args);
+}
+
 template<int DIM, int QT, bool Q8, int OCC>
 void launch(Device& d, const PrefillArgs& args, unsigned seqs) {
     constexpr size_t merge = size_t(GROUPS) * QT * (DIM / 16 * 4 + 2) * 64 * 4;
@@ -310,7 +606,7 @@ void prefill_attention(Device& d, const sdx_kv_pool* pool, const int32_t* page_t
     args.out = out; args.out_f16 = out_f16;
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     KernelTimer timer(d);
-    if (pool->dim == 128) { if (q8) launch<128, 3, true, 2>(d, args, unsigned(seqs)); else launch<128, 3, false, 2>(d, args, unsigned(seqs)); }
+    if (pool->dim == 128) { if (q8) launch_tiles<128, 4, true>(d, args, unsigned(seqs)); else launch_tiles<128, 4, false>(d, args, unsigned(seqs)); }
     else { if (q8) launch<256, 1, true, 2>(d, args, unsigned(seqs)); else launch<256, 1, false, 2>(d, args, unsigned(seqs)); }
 }
 
