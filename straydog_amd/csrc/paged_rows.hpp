@@ -39,6 +39,29 @@ struct PagedArgs {
     int max_context;       // positions[s] + span is clipped to this (the launch and the page table are sized for it)
 };
 
+// The maximum / the sum over the four lanes li, li + 16, li + 32, li + 48 (one query row's four lane groups), in all four.
+// v_permlane16_swap exchanges the odd 16-lane rows of its first register with the even rows of its second, v_permlane32_swap
+// the upper half of the first with the lower half of the second: with both registers holding the same values, each lane
+// then finds its own value in one and its partner's in the other.  (Written as instructions: the compiler's builtin folds
+// the two results into one when both operands are the same value.  The swap may not follow the write of its operands
+// at once, hence the wait states.)
+__device__ __forceinline__ void swap_rows(float& a, float& b) { asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ void swap_halves(float& a, float& b) { asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ float row_max(float x) {
+    float a = x, b = x;
+    swap_rows(a, b);
+    a = fmaxf(a, b); b = a;
+    swap_halves(a, b);
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float row_sum(float x) {
+    float a = x, b = x;
+    swap_rows(a, b);
+    a += b; b = a;
+    swap_halves(a, b);
+    return a + b;
+}
+
 __device__ __forceinline__ half2v as_half2(uint32_t bits) { return __builtin_bit_cast(half2v, bits); }
 
 // v_perm_b32: byte i of the result is byte sel[i] of the 8 bytes {high, low} (0-3 = low's bytes, 4-7 = high's, 0x0c = 0x00).

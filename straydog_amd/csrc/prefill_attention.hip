@@ -19,6 +19,7 @@
 #include "paged_rows.hpp"
 
 #include <cstdlib>
+#include <type_traits>
 
 using namespace sd;
 using namespace sd::paged;
@@ -323,6 +324,8 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     };
     // One step's raw rows into FP16 tiles; rows past the sequence's end become zeros (the page holds anything there).
     const auto convert = [&](int buffer, int into, int walk0) {
+        int thread = threadIdx.x;
+        asm volatile("" : "+v"(thread));                       // the piece's addresses are formed here, not kept across the walk
         const uint8_t* raw = stages + buffer * (2 * SLAB);
         uint8_t* ktile = tiles + into * (KT + VT);
         uint8_t* vtile = ktile + KT;
@@ -355,7 +358,6 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
                 for (int e = 0; e < 4; ++e) {
                     words[e] = *reinterpret_cast<const uint32_t*>(from + e * ROW + 4 * cols4);
                     scales[e] = 4 * rows4 + e < valid ? uint32_t(*reinterpret_cast<const uint16_t*>(from + e * ROW + DIM + 2 * (cols4 >> 3))) : 0u;
-                    if (4 * rows4 + e >= valid) words[e] = 0x80808080u ^ 0x80808080u;
                 }
                 const half2v first = as_half2(scales[0] | (scales[1] << 16)), second = as_half2(scales[2] | (scales[3] << 16));
                 #pragma unroll
@@ -405,13 +407,11 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     for (int ahead = 0; ahead < RING; ++ahead) copy_in(ahead, min(ahead * WALK, last_step));
 
     half8 qf[QT][BLOCKS];
-    int limit[QT];
     #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
         const int row = row0 + qt * 16 + li;
         const bool real = row < int(args.rows);
         const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
-        limit[qt] = real ? position + span_row : 0x7fffffff;
         const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
         #pragma unroll
         for (int b = 0; b < BLOCKS; ++b) {
@@ -441,14 +441,18 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     __syncthreads();
     convert(0, 0, 0);
 
+    // The two waves of a SIMD walk in different orders: the first half's converts its piece of the next step and then computes,
+    // the second half's computes and then converts, so that one's MFMA phases meet the other's VALU phases.  (Two loops: the
+    // order is fixed at compile time in each.)
+    const auto walk = [&](auto convert_first) {
     for (int walk0 = 0, step = 0; walk0 < keys; walk0 += WALK, ++step) {
         // the next step's raw rows have landed when only the later steps' copies are outstanding
         if (most) wait_loads<MOST * (RING - 2)>(); else wait_loads<LEAST * (RING - 2)>();
         __syncthreads();      // everybody's pieces have; this step's tiles are written; the other tiles and the raw stage of this step are free
         copy_in(step % RING, min(walk0 + RING * WALK, last_step));
-        if (walk0 + WALK < keys) convert((step + 1) % RING, (step + 1) & 1, walk0 + WALK);
+        if (decltype(convert_first)::value && walk0 + WALK < keys) convert((step + 1) % RING, (step + 1) & 1, walk0 + WALK);
         const int token0 = walk0 + half * STEP;
-        if (idle || token0 > wave_last || token0 >= keys) continue;
+        if (!(idle || token0 > wave_last || token0 >= keys)) {
         const uint8_t* ktile = tiles + (step & 1) * (KT + VT) + half * STEP * KP;
         const uint8_t* vtile = tiles + (step & 1) * (KT + VT) + KT + half * STEP * 2;
         floatx4 s[QT][2];
@@ -463,30 +467,47 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
                 for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qf[qt][b], s[qt][t], 0, 0, 0);
             }
         }
-        if (token0 + STEP - 1 > wave_first) {
+        if (token0 + STEP - 1 > wave_first) {          // wave-uniform: some token of the step is past some row's position
+            asm volatile("; the step crosses the diagonal" ::: "memory");      // keeps the block a branch: it is rare
             #pragma unroll
-            for (int qt = 0; qt < QT; ++qt)
+            for (int qt = 0; qt < QT; ++qt) {
+                const int row = row0 + qt * 16 + li;
+                const int limit = row < int(args.rows) ? position + row / int(args.group) : 0x7fffffff;   // a padding row masks nothing
                 #pragma unroll
                 for (int t = 0; t < 2; ++t)
                     #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        if (token0 + 16 * t + 4 * g + r > limit[qt]) s[qt][t][r] = -INFINITY;
+                        if (token0 + 16 * t + 4 * g + r > limit) s[qt][t][r] = -INFINITY;
+            }
         }
-        half8 pb[QT];
+        // Every row's new maximum first; one rare block moves the reference maxima of the rows that need it; then the weights.
+        // Scores stay unscaled (the scale goes into the exponent's multiply-add); m is a row's reference maximum in unscaled
+        // units.  It follows the true maximum only when that has grown by more than SLACK (in base-2 exponent units): weights
+        // then stay below 2^SLACK, far inside FP16 and FP32 range, and the accumulators are rescaled a few times per row
+        // instead of at every new maximum.  The quotient acc/sum does not depend on the reference.
+        float top[QT];
+        bool grown = false;
         #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
-            float top = fmaxf(fmaxf(fmaxf(s[qt][0][0], s[qt][0][1]), fmaxf(s[qt][0][2], s[qt][0][3])),
-                              fmaxf(fmaxf(s[qt][1][0], s[qt][1][1]), fmaxf(s[qt][1][2], s[qt][1][3])));
-            top = fmaxf(top, __shfl_xor(top, 16));
-            top = fmaxf(top, __shfl_xor(top, 32));
-            if (__any((top - m[qt]) * args.scale_log2 > SLACK)) {
-                const float m_new = fmaxf(m[qt], top);
+            top[qt] = row_max(fmaxf(fmaxf(fmaxf(s[qt][0][0], s[qt][0][1]), fmaxf(s[qt][0][2], s[qt][0][3])),
+                                    fmaxf(fmaxf(s[qt][1][0], s[qt][1][1]), fmaxf(s[qt][1][2], s[qt][1][3]))));
+            grown |= (top[qt] - m[qt]) * args.scale_log2 > SLACK;
+        }
+        if (__any(grown)) {
+            asm volatile("; new reference maxima" ::: "memory");          // keeps the block a branch: it is rare
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt) {
+                const float m_new = fmaxf(m[qt], top[qt]);
                 const float alpha = __builtin_amdgcn_exp2f((m[qt] - m_new) * args.scale_log2);
                 m[qt] = m_new;
                 l[qt] *= alpha;
                 #pragma unroll
                 for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] *= alpha;
             }
+        }
+        half8 pb[QT];
+        #pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
             const float offset = -m[qt] * args.scale_log2;
             float sum = 0.0f;
             half8 p;
@@ -510,14 +531,15 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
             #pragma unroll
             for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[qt], acc[qt][jj], 0, 0, 0);
         }
+        }
+        if (!decltype(convert_first)::value && walk0 + WALK < keys) convert((step + 1) % RING, (step + 1) & 1, walk0 + WALK);
     }
+    };
+    if (half == 0) walk(std::true_type{}); else walk(std::false_type{});
 
     // The pair of waves that shares rows merges through LDS (the stages and tiles are done with).
     #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-        l[qt] += __shfl_xor(l[qt], 16);
-        l[qt] += __shfl_xor(l[qt], 32);
-    }
+    for (int qt = 0; qt < QT; ++qt) l[qt] = row_sum(l[qt]);
     __syncthreads();
     float* mine = reinterpret_cast<float*>(stages) + size_t(quarter) * (QT * (TILES * 4 + 2)) * 64 + lane;
     if (half == 1) {
