@@ -357,7 +357,8 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
                 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     words[e] = *reinterpret_cast<const uint32_t*>(from + e * ROW + 4 * cols4);
-                    scales[e] = 4 * rows4 + e < valid ? uint32_t(*reinterpret_cast<const uint16_t*>(from + e * ROW + DIM + 2 * (cols4 >> 3))) : 0u;
+                    scales[e] = *reinterpret_cast<const uint16_t*>(from + e * ROW + DIM + 2 * (cols4 >> 3));
+                    if (4 * rows4 + e >= valid) scales[e] = 0u;
                 }
                 const half2v first = as_half2(scales[0] | (scales[1] << 16)), second = as_half2(scales[2] | (scales[3] << 16));
                 #pragma unroll
