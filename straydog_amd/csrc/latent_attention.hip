@@ -12,6 +12,13 @@
 
 using namespace sd;
 
+namespace sd {
+bool latent_gather_supported(uint64_t kdim, uint64_t vdim);
+uint64_t latent_gather_scratch(uint64_t batch, uint64_t k, uint64_t heads, uint64_t vdim);
+void latent_gather(Device& d, const void* q, const void* latents, const int32_t* selected, uint64_t batch, uint64_t groups, uint64_t k,
+                   uint64_t heads, float scale, float* out, float* partial);
+}
+
 namespace {
 
 constexpr int HB = 8, THREADS = 256, PAD = 4, MAX_COLS = 4;
@@ -205,6 +212,13 @@ int sdx_latent_attention(void* handle, const void* q, const void* latents, const
     op_span(value, latents, checked_product({batch, groups, kdim, 2}), "latent rows");
     op_span(value, selected, checked_floats({batch, k}), "selected rows");
     op_span(value, out, checked_floats({batch, heads, vdim}), "an attention output");
+    if (latent_gather_supported(kdim, vdim) && groups < (uint64_t(1) << 31) && k < (uint64_t(1) << 31)) {
+        // the matrix-core path; its chunk partials live in the device's workspace (grown outside graph capture)
+        float* partial = static_cast<float*>(workspace(value, latent_gather_scratch(batch, k, heads, vdim)));
+        latent_gather(value, q, latents, selected, batch, groups, k, heads, scale, out, partial);
+        SD_CHECK(hipGetLastError());
+        return 0;
+    }
     LatentArgs args{};
     args.q_bf16 = static_cast<const uint16_t*>(q); args.compressed = latents; args.compressed_batch_stride = size_t(groups * kdim);
     args.selected = selected; args.selections = size_t(k); args.heads = size_t(heads); args.kdim = size_t(kdim); args.vdim = size_t(vdim);

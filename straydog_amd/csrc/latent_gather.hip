@@ -1,0 +1,208 @@
+// The batched gather attention of the sparse top-k path on matrix cores: every sequence's query heads attend the BF16
+// latent rows its selection lists, keys being a row's kdim columns and values its first vdim columns.  The arithmetic is
+// op_sparse_attention_kernel's (reference gpu/ops.hpp:1240-1297) without window or sink, with BF16 operands and FP32
+// sums, as the reference's WMMA prompt path does it (gpu/ds_attention_wmma.hpp:26-340).
+//
+// Shape of the work on gfx950 (wave64, v_mfma_f32_16x16x32_bf16):
+//   * a workgroup (4 waves) owns one sequence, 128 of its selected rows and 64 heads, a wave 16 of the heads;
+//   * 32 rows at a time are gathered (16-byte pieces, every row whole) into a padded K tile in LDS and from there
+//     transposed into a V tile, both read without bank conflicts as MFMA operands by all four waves;
+//   * S^T = K . Q^T (rows x heads) leaves the weights in the B-operand layout of O^T += V^T . P^T, so they never move
+//     between lanes (the layout notes of paged_rows.hpp apply);
+//   * the chunks' (maximum, sum, unnormalised output) are merged by a second kernel.
+#include "paged_rows.hpp"
+
+using namespace sd;
+using namespace sd::paged;
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int CHUNK = 128;          // selected rows per workgroup
+
+struct GatherArgs {
+    const uint16_t* q;              // [batch][heads][kdim] BF16
+    const uint16_t* latents;        // [batch][groups][kdim] BF16
+    const int32_t* selected;        // [batch][k], entries outside 0..groups-1 are skipped
+    unsigned groups, k, heads, chunks;
+    float scale_log2;
+    float* partial;                 // [batch][chunk][heads][vdim + 2]
+    float* out;                     // [batch][heads][vdim]
+};
+
+__device__ __forceinline__ uint32_t bf16_pair(float low, float high) {
+    // round to nearest even, as the reference's to_bf16 (gpu/token_mixing.hpp:729-735) does for finite values
+    const uint32_t a = __float_as_uint(low), b = __float_as_uint(high);
+    return ((a + 0x7fffu + ((a >> 16) & 1u)) >> 16) | ((b + 0x7fffu + ((b >> 16) & 1u)) & 0xffff0000u);
+}
+
+template<int KDIM, int VDIM>
+__global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
+    constexpr int KSTEPS = KDIM / 32, TILES = VDIM / 16, KP = 2 * KDIM + 16, VP = 2 * STEP + 8, PIECES = KDIM / 8;
+    const int chunk = blockIdx.x, batch = blockIdx.z, thread = threadIdx.x;
+    const int lane = thread & 63, wave = __builtin_amdgcn_readfirstlane(thread >> 6), li = lane & 15, g = lane >> 4;
+    const int head = int(blockIdx.y) * 64 + wave * 16 + li;
+    const bool real = head < int(a.heads);
+    extern __shared__ uint8_t lds[];
+    uint8_t* ktile = lds;                                     // [32 rows][KP]
+    uint8_t* vtile = ktile + STEP * KP;                       // [VDIM columns][VP]
+    uint32_t* seen = reinterpret_cast<uint32_t*>(vtile + VDIM * VP);   // [32]: 1 where the step's row exists
+
+    bf16x8 qf[KSTEPS];
+    #pragma unroll
+    for (int b = 0; b < KSTEPS; ++b) {
+        uint4 bits = {0u, 0u, 0u, 0u};
+        if (real) bits = *reinterpret_cast<const uint4*>(a.q + (size_t(batch) * a.heads + head) * KDIM + 32 * b + 8 * g);
+        qf[b] = __builtin_bit_cast(bf16x8, bits);
+    }
+    floatx4 acc[TILES];
+    #pragma unroll
+    for (int jj = 0; jj < TILES; ++jj) acc[jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    float m = NEG_BIG, l = 0.0f;
+
+    const int first = chunk * CHUNK, last = min(int(a.k), first + CHUNK);
+    for (int key0 = first; key0 < last; key0 += STEP) {
+        __syncthreads();                                      // the tiles of the step before are done with
+        // gather: a row is PIECES pieces of 16 bytes; a missing row is read from row 0 and masked
+        for (int piece = thread; piece < STEP * PIECES; piece += 256) {
+            const int row = piece / PIECES, part = piece % PIECES;
+            const int index = key0 + row < last ? a.selected[size_t(batch) * a.k + key0 + row] : -1;
+            const bool exists = index >= 0 && index < int(a.groups);
+            const uint4 bits = *reinterpret_cast<const uint4*>(a.latents + (size_t(batch) * a.groups + (exists ? index : 0)) * KDIM + 8 * part);
+            *reinterpret_cast<uint4*>(ktile + row * KP + 16 * part) = bits;
+            if (part == 0) seen[row] = exists ? 1u : 0u;
+        }
+        __syncthreads();
+        // V tile: 4 rows x 4 columns at a time, transposed
+        for (int block = thread; block < (STEP / 4) * (VDIM / 4); block += 256) {
+            const int rows4 = block % (STEP / 4), cols4 = block / (STEP / 4);
+            uint2 words[4];
+            #pragma unroll
+            for (int e = 0; e < 4; ++e) words[e] = *reinterpret_cast<const uint2*>(ktile + (4 * rows4 + e) * KP + 8 * cols4);
+            #pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+                uint2 packed;
+                packed.x = byte_perm(c < 2 ? words[1].x : words[1].y, c < 2 ? words[0].x : words[0].y, sel);
+                packed.y = byte_perm(c < 2 ? words[3].x : words[3].y, c < 2 ? words[2].x : words[2].y, sel);
+                *reinterpret_cast<uint2*>(vtile + (4 * cols4 + c) * VP + 8 * rows4) = packed;
+            }
+        }
+        __syncthreads();
+        // S^T tiles: rows of the step (4 per lane group) x heads (lane li)
+        floatx4 s[2] = {floatx4{0.0f, 0.0f, 0.0f, 0.0f}, floatx4{0.0f, 0.0f, 0.0f, 0.0f}};
+        #pragma unroll
+        for (int b = 0; b < KSTEPS; ++b)
+            #pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const bf16x8 ka = *reinterpret_cast<const bf16x8*>(ktile + (16 * t + li) * KP + 64 * b + 16 * g);
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[b], s[t], 0, 0, 0);
+            }
+        float top = NEG_BIG;
+        #pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint4 flags = *reinterpret_cast<const uint4*>(seen + 16 * t + 4 * g);
+            const uint32_t flag[4] = {flags.x, flags.y, flags.z, flags.w};
+            #pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if (!flag[r]) s[t][r] = -INFINITY;
+                top = fmaxf(top, s[t][r]);
+            }
+        }
+        top = row_max(top);
+        if (__any(top > m)) {
+            const float m_new = fmaxf(m, top), alpha = __builtin_amdgcn_exp2f((m - m_new) * a.scale_log2);
+            m = m_new;
+            l *= alpha;
+            #pragma unroll
+            for (int jj = 0; jj < TILES; ++jj) acc[jj] *= alpha;
+        }
+        const float offset = -m * a.scale_log2;
+        float w[8], sum = 0.0f;
+        #pragma unroll
+        for (int t = 0; t < 2; ++t)
+            #pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                w[4 * t + r] = __builtin_amdgcn_exp2f(fmaf(s[t][r], a.scale_log2, offset));
+                sum += w[4 * t + r];
+            }
+        l += sum;
+        // The weights as two BF16 terms (the value and what its rounding left), so the products keep 16 bits of each weight.
+        float rest[8];
+        #pragma unroll
+        for (int i = 0; i < 8; ++i) rest[i] = w[i] - __uint_as_float(bf16_pair(0.0f, w[i]) & 0xffff0000u);
+        const uint4 high = {bf16_pair(w[0], w[1]), bf16_pair(w[2], w[3]), bf16_pair(w[4], w[5]), bf16_pair(w[6], w[7])};
+        const uint4 low = {bf16_pair(rest[0], rest[1]), bf16_pair(rest[2], rest[3]), bf16_pair(rest[4], rest[5]), bf16_pair(rest[6], rest[7])};
+        const bf16x8 pb = __builtin_bit_cast(bf16x8, high), pl = __builtin_bit_cast(bf16x8, low);
+        // O^T tiles: columns (16 jj + 4 g + r) x heads
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj) {
+            const uint8_t* from = vtile + (16 * jj + li) * VP + 8 * g;
+            const uint2 near = *reinterpret_cast<const uint2*>(from), far = *reinterpret_cast<const uint2*>(from + 32);
+            const uint4 both = {near.x, near.y, far.x, far.y};
+            acc[jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb, acc[jj], 0, 0, 0);
+            acc[jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pl, acc[jj], 0, 0, 0);
+        }
+    }
+    l = row_sum(l);
+    if (!real) return;
+    float* to = a.partial + ((size_t(batch) * a.chunks + chunk) * a.heads + head) * (VDIM + 2);
+    #pragma unroll
+    for (int jj = 0; jj < TILES; ++jj) *reinterpret_cast<floatx4*>(to + 16 * jj + 4 * g) = acc[jj];
+    if (g == 0) { to[VDIM] = m; to[VDIM + 1] = l; }
+}
+
+// One block per (sequence, head): the chunks merged under their common maximum and normalised; a head none of whose
+// rows exists gives zeros.
+template<int VDIM>
+__global__ void __launch_bounds__(VDIM / 4) latent_merge_kernel(GatherArgs a) {
+    const size_t item = blockIdx.x, batch = item / a.heads, head = item % a.heads;
+    const float* base = a.partial + (batch * a.chunks * a.heads + head) * (VDIM + 2);
+    const size_t step = size_t(a.heads) * (VDIM + 2);
+    float top = NEG_BIG;
+    for (unsigned c = 0; c < a.chunks; ++c) top = fmaxf(top, base[c * step + VDIM]);
+    floatx4 value = {0.0f, 0.0f, 0.0f, 0.0f};
+    float sum = 0.0f;
+    for (unsigned c = 0; c < a.chunks; ++c) {
+        const float weight = __builtin_amdgcn_exp2f((base[c * step + VDIM] - top) * a.scale_log2);
+        sum += base[c * step + VDIM + 1] * weight;
+        value += *reinterpret_cast<const floatx4*>(base + c * step + 4 * threadIdx.x) * weight;
+    }
+    if (sum > 0.0f) value *= 1.0f / sum; else value = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    *reinterpret_cast<floatx4*>(a.out + item * VDIM + 4 * threadIdx.x) = value;
+}
+
+}  // namespace
+
+namespace sd {
+
+// The shapes the matrix-core path takes (the batched entry falls back to the general kernel otherwise).
+bool latent_gather_supported(uint64_t kdim, uint64_t vdim) { return kdim == 576 && vdim == 512; }
+
+uint64_t latent_gather_scratch(uint64_t batch, uint64_t k, uint64_t heads, uint64_t vdim) {
+    return batch * ((k + CHUNK - 1) / CHUNK) * heads * (vdim + 2) * 4;
+}
+
+void latent_gather(Device& d, const void* q, const void* latents, const int32_t* selected, uint64_t batch, uint64_t groups, uint64_t k,
+                   uint64_t heads, float scale, float* out, float* partial) {
+    constexpr int KDIM = 576, VDIM = 512;
+    GatherArgs args{};
+    args.q = static_cast<const uint16_t*>(q); args.latents = static_cast<const uint16_t*>(latents); args.selected = selected;
+    args.groups = unsigned(groups); args.k = unsigned(k); args.heads = unsigned(heads); args.chunks = unsigned((k + CHUNK - 1) / CHUNK);
+    args.scale_log2 = scale * 1.44269504088896341f; args.partial = partial; args.out = out;
+    constexpr size_t shared = size_t(STEP) * (2 * KDIM + 16) + size_t(VDIM) * (2 * STEP + 8) + STEP * 4;
+    static bool raised = false;
+    if (!raised) {
+        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_gather_kernel<KDIM, VDIM>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
+        raised = true;
+    }
+    {
+        KernelTimer timer(d);
+        latent_gather_kernel<KDIM, VDIM><<<dim3(args.chunks, unsigned((heads + 63) / 64), unsigned(batch)), 256, shared, d.stream>>>(args);
+    }
+    SD_CHECK(hipGetLastError());
+    latent_merge_kernel<VDIM><<<unsigned(batch * heads), VDIM / 4, 0, d.stream>>>(args);
+}
+
+}  // namespace sd
