@@ -59,6 +59,12 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
  * ties to the lowest index, -1 padding: bit-exact. */
 int sdx_index_top_k(void* handle, const void* q_index, const void* keys, const float* weights, const int32_t* visible, uint64_t batch,
                     uint64_t groups, uint64_t heads, uint64_t dim, float scale, float* scores, uint64_t k, int32_t* indices);
+/* The bracket the matrix cores put around every canonical score of stage 1 (dim 128, heads a multiple of 16 up to 64):
+ * lower[b][g] <= score <= upper[b][g], -inf for groups that are not visible.  sdx_index_top_k without a scores buffer
+ * scores canonically only the groups whose upper bound reaches the k-th highest lower bound (the approach of the
+ * reference's interval indexer, gpu/qsa_interval.hpp:152-419); this entry exposes the brackets for inspection. */
+int sdx_index_score_bounds(void* handle, const void* q_index, const void* keys, const float* weights, const int32_t* visible, uint64_t batch,
+                           uint64_t groups, uint64_t heads, uint64_t dim, float scale, float* lower, float* upper);
 /* stage 3 = op_sparse_attention_kernel's arithmetic (gpu/ops.hpp:1240-1297) without window or sink, keys = the
  * selected rows' kdim columns, values = their first vdim columns: q [batch][heads][kdim] BF16, latents
  * [batch][groups][kdim] BF16, selected [batch][k] (-1 skipped), out [batch][heads][vdim] FP32. */

@@ -168,6 +168,10 @@ class Backend:
         self.check(self.lib.sdx_index_top_k(self.handle, q_index, keys, weights, visible, batch, groups, heads, dim, scale, scores,
                                             k, indices))
 
+    def index_score_bounds(self, q_index, keys, weights, visible, batch, groups, heads, dim, scale, lower, upper):
+        self.check(self.lib.sdx_index_score_bounds(self.handle, q_index, keys, weights, visible, batch, groups, heads, dim, scale, lower,
+                                                   upper))
+
     def latent_attention(self, q, latents, selected, batch, groups, k, heads, kdim, vdim, scale, out):
         self.check(self.lib.sdx_latent_attention(self.handle, q, latents, selected, batch, groups, k, heads, kdim, vdim, scale, out))
 

@@ -27,6 +27,10 @@ __device__ __forceinline__ float rounded_product(float a, float b) {
     #pragma clang fp contract(off)
     return a * b;
 }
+__device__ __forceinline__ float rounded_sum(float a, float b) {
+    #pragma clang fp contract(off)
+    return a + b;
+}
 
 __global__ void to_bf16_kernel(const float* x, size_t count, uint16_t* out) {
     for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) {
@@ -283,6 +287,272 @@ __global__ void __launch_bounds__(256) block_tops_kernel(const float* scores, co
     tops[row * count + b] = top;
 }
 
+// ---- the sparse path's indexer on matrix cores --------------------------------------------------------------
+//
+// The canonical score (one fmaf chain per head, heads added in order) fixes every bit, and a matrix-core sum does not
+// follow that order.  So the matrix cores only bracket each score: s~ from BF16 MFMAs with FP32 sums, and a margin e that
+// bounds |s~ - s| for the canonical s (the reference takes the same road for its long contexts: approximate scores, a
+// threshold, exact work near it only -- gpu/qsa_interval.hpp:152-419).  With L the k-th highest lower bound s~ - e, at least
+// k groups score L or more, so a group whose upper bound s~ + e is below L cannot be among the top k, ties included.  The
+// others (k and a few) are listed in index order, scored canonically, and the exact top-k runs over that list: the
+// result is the canonical one, bit for bit.
+//
+// Margin: each head's MFMA dot and its canonical chain both differ from the real dot by at most 128 roundings of
+// sum|q_d k_d| <= |q_h| |k|; the 1-Lipschitz max(.,0), the weights and the 64-term head sum add at most 130 roundings of
+// sum_h |w_h| |dot_h|.  With unit roundoff 2^-23 (safe for truncating accumulators too) that is below 2^-14 |scale| |k| W,
+// W = sum_h |w_h| |q_h| (3.8e-5 against 6.1e-5); the norms' own rounding is covered by a further percent.
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int RADIX_BINS = 2048, RADIX_LEVELS = 3, INTERVAL_KEYS = 1024;   // digits of 11, 11 and 10 bits; groups per workgroup
+__device__ __forceinline__ uint32_t radix_digit(uint32_t key, int level) { return level == 0 ? key >> 21 : level == 1 ? (key >> 10) & 2047u : key & 1023u; }
+
+// The sum over the four lanes li, li + 16, li + 32, li + 48 in all of them (see paged_rows.hpp for the instructions).
+__device__ __forceinline__ float quad_sum(float x) {
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    a += b; b = a;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    return a + b;
+}
+
+// W of the margin for every row: sum_h |w_h| |q_h| * |scale| * 2^-14, rounded up a little.
+__global__ void __launch_bounds__(64) index_margin_kernel(const uint16_t* q, const float* weights, size_t heads, size_t dim, float scale, float* margin) {
+    const size_t row = blockIdx.x;
+    float total = 0.0f;
+    for (size_t h = threadIdx.x; h < heads; h += 64) {
+        float square = 0.0f;
+        for (size_t d = 0; d < dim; ++d) { const float v = bf16_value(q[(row * heads + h) * dim + d]); square += v * v; }
+        total += fabsf(weights[row * heads + h]) * sqrtf(square);
+    }
+    #pragma unroll
+    for (int d = 32; d; d >>= 1) total += __shfl_xor(total, d);
+    if (threadIdx.x == 0) margin[row] = total * fabsf(scale) * (1.0f / 16384.0f) * 1.01f;
+}
+
+// Bounds of the scores of INTERVAL_KEYS groups per workgroup, 16 groups per MFMA tile and wave, and the first radix
+// histogram of the lower bounds.  S = Q . K^T with Q (heads x dim) as A operands from registers and K rows straight from
+// memory as B operands; K . K^T from the same registers gives |k|^2 on its diagonal.
+template<int HEADS>
+__global__ void __launch_bounds__(256) index_interval_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
+                                                             const int32_t* __restrict__ visible, const float* __restrict__ margin, size_t groups, float scale,
+                                                             float* __restrict__ lower, float* __restrict__ upper, uint32_t* __restrict__ histogram) {
+    constexpr int DIM = 128, HT = HEADS / 16, KS = DIM / 32;
+    const size_t row = blockIdx.y;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, g = lane >> 4;
+    __shared__ uint32_t bins[RADIX_BINS];
+    for (int i = threadIdx.x; i < RADIX_BINS; i += 256) bins[i] = 0;
+    bf16x8 qa[HT][KS];
+    float w[HT][4];
+    #pragma unroll
+    for (int t = 0; t < HT; ++t) {
+        #pragma unroll
+        for (int b = 0; b < KS; ++b)
+            qa[t][b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(q + (row * HEADS + 16 * t + li) * DIM + 32 * b + 8 * g));
+        #pragma unroll
+        for (int r = 0; r < 4; ++r) w[t][r] = weights[row * HEADS + 16 * t + 4 * g + r];
+    }
+    const int32_t seen = visible[row];
+    const size_t limit = min(groups, size_t(seen > 0 ? seen : 0));
+    const float bound = margin[row];
+    const uint16_t* row_keys = keys + row * groups * DIM;
+    __syncthreads();
+    const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS;
+    for (size_t tile = first + 16 * wave; tile < min(first + INTERVAL_KEYS, groups); tile += 64) {
+        const size_t group = tile + li;
+        const uint16_t* from = row_keys + min(group, groups - 1) * DIM + 8 * g;
+        bf16x8 kb[KS];
+        #pragma unroll
+        for (int b = 0; b < KS; ++b) kb[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(from + 32 * b));
+        floatx4 norms = {0.0f, 0.0f, 0.0f, 0.0f};
+        #pragma unroll
+        for (int b = 0; b < KS; ++b) norms = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[b], kb[b], norms, 0, 0, 0);
+        float total = 0.0f;
+        #pragma unroll
+        for (int t = 0; t < HT; ++t) {
+            floatx4 dots = {0.0f, 0.0f, 0.0f, 0.0f};
+            #pragma unroll
+            for (int b = 0; b < KS; ++b) dots = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[t][b], kb[b], dots, 0, 0, 0);
+            #pragma unroll
+            for (int r = 0; r < 4; ++r) total = fmaf(fmaxf(dots[r], 0.0f), w[t][r], total);
+        }
+        total = quad_sum(total) * scale;
+        // the diagonal of K . K^T: row 4g + r = column li
+        const int r = li & 3;
+        const float square = r == 0 ? norms[0] : r == 1 ? norms[1] : r == 2 ? norms[2] : norms[3];
+        if (g == (li >> 2) && group < groups) {
+            const float e = bound * sqrtf(square);
+            const bool live = group < limit;
+            const float low = live ? total - e : -INFINITY, high = live ? total + e : -INFINITY;
+            lower[row * groups + group] = low;
+            upper[row * groups + group] = high;
+            const uint32_t key = top_k_key(low);
+            if (key > top_k_key(-INFINITY)) atomicAdd(&bins[radix_digit(key, 0)], 1u);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < RADIX_BINS; i += 256)
+        if (bins[i]) atomicAdd(&histogram[row * RADIX_BINS + i], bins[i]);
+}
+
+// Where the rank-th highest key lies, one digit at a time, from the levels' histograms (256 threads, every workgroup
+// that needs it finds it anew).  After `levels` digits: the key's leading digits and the rank among the keys that share
+// them; `everything` when fewer than rank keys are live at all.
+struct RadixPick { uint32_t prefix, rank; bool everything; };
+__device__ RadixPick radix_pick(const uint32_t* histogram /* [level][rows][RADIX_BINS] */, size_t rows, size_t row, int levels, uint32_t k) {
+    __shared__ uint32_t sums[256], found[3];
+    RadixPick pick{0u, k, false};
+    const unsigned t = threadIdx.x;
+    for (int level = 0; level < levels; ++level) {
+        const uint32_t* bins = histogram + (size_t(level) * rows + row) * RADIX_BINS;
+        // thread t owns the 8 bins below 2048 - 8t, highest first
+        uint32_t mine[8], sum = 0;
+        #pragma unroll
+        for (int i = 0; i < 8; ++i) { mine[i] = bins[RADIX_BINS - 1 - (8 * t + i)]; sum += mine[i]; }
+        __syncthreads();
+        sums[t] = sum;
+        __syncthreads();
+        uint32_t above = 0, every = 0;
+        for (unsigned i = 0; i < 256; ++i) { const uint32_t c = sums[i]; above += i < t ? c : 0u; every += c; }
+        if (level == 0 && every < pick.rank) { pick.everything = true; return pick; }
+        if (above < pick.rank && above + sum >= pick.rank) {
+            uint32_t before = above;
+            #pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (before < pick.rank && before + mine[i] >= pick.rank) { found[0] = RADIX_BINS - 1 - (8 * t + i); found[1] = pick.rank - before; }
+                before += mine[i];
+            }
+        }
+        __syncthreads();
+        pick.prefix = level == 0 ? found[0] << 21 : level == 1 ? pick.prefix | (found[0] << 10) : pick.prefix | found[0];
+        pick.rank = found[1];
+    }
+    return pick;
+}
+
+// The histogram of digit `level` over the keys that share the digits found so far.
+__global__ void __launch_bounds__(256) radix_histogram_kernel(const float* values, size_t groups, size_t rows, int level, uint32_t k, uint32_t* histogram) {
+    const size_t row = blockIdx.y;
+    __shared__ uint32_t bins[RADIX_BINS];
+    for (int i = threadIdx.x; i < RADIX_BINS; i += 256) bins[i] = 0;
+    const RadixPick pick = radix_pick(histogram, rows, row, level, k);
+    __syncthreads();
+    if (pick.everything) return;
+    const uint32_t mask = level == 1 ? 0xffe00000u : 0xfffffc00u;
+    const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS;
+    for (size_t group = first + threadIdx.x; group < min(first + INTERVAL_KEYS, groups); group += 256) {
+        const uint32_t key = top_k_key(values[row * groups + group]);
+        if ((key & mask) == pick.prefix) atomicAdd(&bins[radix_digit(key, level)], 1u);
+    }
+    __syncthreads();
+    uint32_t* to = histogram + (size_t(level) * rows + row) * RADIX_BINS;
+    for (int i = threadIdx.x; i < RADIX_BINS; i += 256)
+        if (bins[i]) atomicAdd(&to[i], bins[i]);
+}
+
+// Candidates: groups whose upper bound reaches the k-th highest lower bound (every live group when fewer than k are live).
+__device__ __forceinline__ bool is_candidate(float high, const RadixPick& pick) {
+    const uint32_t key = top_k_key(high);
+    return pick.everything ? key > top_k_key(-INFINITY) : key >= pick.prefix;
+}
+__global__ void __launch_bounds__(256) candidate_count_kernel(const float* upper, size_t groups, size_t rows, uint32_t k, const uint32_t* histogram,
+                                                              uint32_t* counts) {
+    const size_t row = blockIdx.y;
+    const RadixPick pick = radix_pick(histogram, rows, row, RADIX_LEVELS, k);
+    __shared__ uint32_t total;
+    if (threadIdx.x == 0) total = 0;
+    __syncthreads();
+    const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS;
+    uint32_t mine = 0;
+    for (size_t group = first + threadIdx.x; group < min(first + INTERVAL_KEYS, groups); group += 256) mine += is_candidate(upper[row * groups + group], pick);
+    #pragma unroll
+    for (int d = 32; d; d >>= 1) mine += __shfl_xor(mine, d);
+    if ((threadIdx.x & 63) == 0) atomicAdd(&total, mine);
+    __syncthreads();
+    if (threadIdx.x == 0) counts[row * gridDim.x + blockIdx.x] = total;
+}
+// ... listed in index order: a workgroup's candidates follow those of the workgroups before it.
+__global__ void __launch_bounds__(256) candidate_list_kernel(const float* upper, size_t groups, size_t rows, uint32_t k, const uint32_t* histogram,
+                                                             const uint32_t* counts, int32_t* list, uint32_t* totals) {
+    const size_t row = blockIdx.y;
+    const RadixPick pick = radix_pick(histogram, rows, row, RADIX_LEVELS, k);
+    __shared__ uint32_t wave_sums[4], base;
+    uint32_t before = 0;
+    for (unsigned b = threadIdx.x; b < gridDim.x; b += 256) before += b < blockIdx.x ? counts[row * gridDim.x + b] : 0u;
+    #pragma unroll
+    for (int d = 32; d; d >>= 1) before += __shfl_xor(before, d);
+    if (threadIdx.x == 0) base = 0;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) atomicAdd(&base, before);
+    __syncthreads();
+    // thread t owns 4 consecutive groups
+    const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS + 4 * threadIdx.x;
+    bool keep[4];
+    uint32_t mine = 0;
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) { keep[i] = first + i < groups && is_candidate(upper[row * groups + first + i], pick); mine += keep[i]; }
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t inclusive = mine;
+    #pragma unroll
+    for (unsigned offset = 1; offset < 64; offset *= 2) { const uint32_t other = __shfl_up(inclusive, offset); if (lane >= offset) inclusive += other; }
+    if (lane == 63) wave_sums[wave] = inclusive;
+    __syncthreads();
+    uint32_t at = base + inclusive - mine;
+    for (unsigned v = 0; v < wave; ++v) at += wave_sums[v];
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) if (keep[i]) list[row * groups + at++] = int32_t(first + i);
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 255) totals[row] = at;
+}
+
+// The canonical score of every listed group: a wave per group, a lane per head (its query row in registers, the key row
+// in scalar registers), then the heads' terms added in head order.
+template<int HEADS>
+__global__ void __launch_bounds__(256) candidate_score_kernel(const float* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
+                                                              size_t groups, float scale, const int32_t* __restrict__ list, const uint32_t* __restrict__ totals,
+                                                              float* __restrict__ scores) {
+    constexpr int DIM = 128;
+    const size_t row = blockIdx.y;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int head = min(lane, HEADS - 1);
+    float query[DIM];
+    #pragma unroll
+    for (int d = 0; d < DIM; d += 4) {
+        const float4 v = *reinterpret_cast<const float4*>(q + (row * HEADS + head) * DIM + d);
+        query[d] = v.x; query[d + 1] = v.y; query[d + 2] = v.z; query[d + 3] = v.w;
+    }
+    const float weight = weights[row * HEADS + head];
+    const uint32_t total = totals[row];
+    for (uint32_t at = blockIdx.x * 4 + wave; at < total; at += gridDim.x * 4) {
+        const int32_t group = __builtin_amdgcn_readfirstlane(list[row * groups + at]);
+        const uint32_t* key = reinterpret_cast<const uint32_t*>(keys + (row * groups + size_t(group)) * DIM);
+        float dot = 0.0f;
+        #pragma unroll
+        for (int d = 0; d < DIM; d += 2) {
+            const uint32_t pair = __builtin_amdgcn_readfirstlane(key[d / 2]);
+            dot = __builtin_fmaf(query[d], __uint_as_float(pair << 16), dot);
+            dot = __builtin_fmaf(query[d + 1], __uint_as_float(pair & 0xffff0000u), dot);
+        }
+        const float term = rounded_product(fmaxf(dot, 0.0f), weight);
+        float sum = 0.0f;
+        #pragma unroll
+        for (int h = 0; h < HEADS; ++h) sum = rounded_sum(sum, __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(term), h)));
+        if (lane == 0) scores[row * groups + at] = rounded_product(sum, scale);
+    }
+}
+
+// The exact top-k over a row's listed groups (scores in list order, which is index order).
+__global__ void __launch_bounds__(TOPK_THREADS) top_k_listed_kernel(const float* scores, const int32_t* list, const uint32_t* totals, size_t groups, size_t k,
+                                                                    int32_t* out) {
+    const float* s = scores + size_t(blockIdx.x) * groups;
+    const int32_t* c = list + size_t(blockIdx.x) * groups;
+    top_k_row([=](size_t v) { return s[v]; }, [=](size_t v) { return c[v]; }, totals[blockIdx.x], k, out + size_t(blockIdx.x) * k);
+}
+
+__global__ void fill_words_kernel(uint32_t* to, size_t count) {
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) to[i] = 0u;
+}
+
 __global__ void widen_bf16_kernel(const uint16_t* from, float* to, size_t count) {
     for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) to[i] = bf16_value(from[i]);
 }
@@ -302,6 +572,58 @@ void launch_scores(Device& d, const float* q, const void* keys, bool bf16, size_
     if (heads <= 32) { if (bf16) SD_SCORES(32, true); else SD_SCORES(32, false); }
     else { if (bf16) SD_SCORES(64, true); else SD_SCORES(64, false); }
 #undef SD_SCORES
+    SD_CHECK(hipGetLastError());
+}
+
+
+// The matrix-core indexer of the batched sparse path (scores are not returned by it): see the kernels above.
+bool index_fast_supported(uint64_t heads, uint64_t dim) { return dim == 128 && heads % 16 == 0 && heads >= 16 && heads <= 64; }
+
+struct FastIndexSpace { float *wide_q, *margin, *lower, *upper, *scores; uint32_t *histogram, *counts, *totals; int32_t* list; size_t blocks; };
+size_t fast_index_bytes(size_t batch, size_t groups, size_t heads, size_t dim) {
+    const size_t blocks = (groups + INTERVAL_KEYS - 1) / INTERVAL_KEYS;
+    return 4 * (batch * heads * dim + batch + 4 * batch * groups + RADIX_LEVELS * batch * RADIX_BINS + batch * blocks + batch) + 9 * 256;
+}
+FastIndexSpace fast_index_space(void* base, size_t batch, size_t groups, size_t heads, size_t dim) {
+    uint8_t* at = static_cast<uint8_t*>(base);
+    const auto take = [&](size_t words) { void* p = at; at += (4 * words + 255) & ~size_t(255); return p; };
+    FastIndexSpace s{};
+    s.blocks = (groups + INTERVAL_KEYS - 1) / INTERVAL_KEYS;
+    s.wide_q = static_cast<float*>(take(batch * heads * dim)); s.margin = static_cast<float*>(take(batch));
+    s.lower = static_cast<float*>(take(batch * groups)); s.upper = static_cast<float*>(take(batch * groups));
+    s.scores = static_cast<float*>(take(batch * groups)); s.list = static_cast<int32_t*>(take(batch * groups));
+    s.histogram = static_cast<uint32_t*>(take(RADIX_LEVELS * batch * RADIX_BINS)); s.counts = static_cast<uint32_t*>(take(batch * s.blocks));
+    s.totals = static_cast<uint32_t*>(take(batch));
+    return s;
+}
+
+template<int HEADS>
+void fast_index_bounds(Device& d, const FastIndexSpace& s, const void* q_index, const void* keys, const float* weights, const int32_t* visible, size_t batch,
+                       size_t groups, float scale) {
+    fill_words_kernel<<<unsigned(std::min<size_t>(checked_blocks(RADIX_LEVELS * batch * RADIX_BINS), 1024)), 256, 0, d.stream>>>(s.histogram, RADIX_LEVELS * batch * RADIX_BINS);
+    index_margin_kernel<<<unsigned(batch), 64, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), weights, HEADS, 128, scale, s.margin);
+    index_interval_kernel<HEADS><<<dim3(unsigned(s.blocks), unsigned(batch)), 256, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys),
+                                                                                                   weights, visible, s.margin, groups, scale, s.lower, s.upper, s.histogram);
+    SD_CHECK(hipGetLastError());
+}
+
+template<int HEADS>
+void fast_index_top_k(Device& d, const FastIndexSpace& s, const void* q_index, const void* keys, const float* weights, const int32_t* visible, size_t batch,
+                      size_t groups, float scale, size_t k, int32_t* indices) {
+    const dim3 grid(unsigned(s.blocks), unsigned(batch));
+    widen_bf16(d, q_index, s.wide_q, batch * HEADS * 128);
+    {
+        KernelTimer timer(d);
+        fast_index_bounds<HEADS>(d, s, q_index, keys, weights, visible, batch, groups, scale);
+    }
+    const uint32_t rank = uint32_t(std::min<size_t>(k, 0xffffffffu));
+    radix_histogram_kernel<<<grid, 256, 0, d.stream>>>(s.lower, groups, batch, 1, rank, s.histogram);
+    radix_histogram_kernel<<<grid, 256, 0, d.stream>>>(s.lower, groups, batch, 2, rank, s.histogram);
+    candidate_count_kernel<<<grid, 256, 0, d.stream>>>(s.upper, groups, batch, rank, s.histogram, s.counts);
+    candidate_list_kernel<<<grid, 256, 0, d.stream>>>(s.upper, groups, batch, rank, s.histogram, s.counts, s.list, s.totals);
+    candidate_score_kernel<HEADS><<<dim3(64, unsigned(batch)), 256, 0, d.stream>>>(s.wide_q, static_cast<const uint16_t*>(keys), weights, groups, scale, s.list, s.totals,
+                                                                                   s.scores);
+    top_k_listed_kernel<<<unsigned(batch), TOPK_THREADS, 0, d.stream>>>(s.scores, s.list, s.totals, groups, k, indices);
     SD_CHECK(hipGetLastError());
 }
 
@@ -437,6 +759,17 @@ int sdx_index_top_k(void* handle, const void* q_index, const void* keys, const f
     op_span(value, weights, checked_floats({batch, heads}), "index weights");
     op_span(value, visible, checked_floats({batch}), "visible counts");
     op_span(value, indices, checked_floats({batch, k}), "top-k indices");
+    if (!scores && index_fast_supported(heads, dim)) {
+        // the matrix cores bracket the scores; the canonical arithmetic runs on the few groups near the k-th only
+        const FastIndexSpace space = fast_index_space(workspace(value, fast_index_bytes(batch, groups, heads, dim)), batch, groups, heads, dim);
+        switch (heads) {
+            case 16: fast_index_top_k<16>(value, space, q_index, keys, weights, visible, batch, groups, scale, k, indices); break;
+            case 32: fast_index_top_k<32>(value, space, q_index, keys, weights, visible, batch, groups, scale, k, indices); break;
+            case 48: fast_index_top_k<48>(value, space, q_index, keys, weights, visible, batch, groups, scale, k, indices); break;
+            default: fast_index_top_k<64>(value, space, q_index, keys, weights, visible, batch, groups, scale, k, indices); break;
+        }
+        return 0;
+    }
     // workspace: the queries widened to FP32 (exact), and the scores when the caller does not want them
     const size_t q_bytes = checked_floats({batch, heads, dim}), score_bytes = checked_floats({batch, groups});
     uint8_t* space = static_cast<uint8_t*>(workspace(value, q_bytes + 256 + (scores ? 0 : score_bytes)));
@@ -447,6 +780,28 @@ int sdx_index_top_k(void* handle, const void* q_index, const void* keys, const f
     launch_scores(value, wide_q, keys, true, size_t(groups * dim), weights, visible, size_t(batch), size_t(groups), size_t(heads), size_t(dim), scale,
                   row_scores, size_t(groups), nullptr, 0, 1);
     top_k_kernel<<<unsigned(batch), TOPK_THREADS, 0, value.stream>>>(row_scores, size_t(groups), size_t(groups), size_t(k), indices);
+    SD_OP_END
+}
+
+int sdx_index_score_bounds(void* handle, const void* q_index, const void* keys, const float* weights, const int32_t* visible, uint64_t batch,
+                           uint64_t groups, uint64_t heads, uint64_t dim, float scale, float* lower, float* upper) {
+    SD_OP_BEGIN
+    if (!batch || batch > 65535 || !groups || groups > (uint64_t(1) << 31) || !index_fast_supported(heads, dim))
+        throw std::runtime_error("invalid Straydog index shape");
+    op_span(value, q_index, checked_product({batch, heads, dim, 2}), "index queries");
+    op_span(value, keys, checked_product({batch, groups, dim, 2}), "index keys");
+    op_span(value, weights, checked_floats({batch, heads}), "index weights");
+    op_span(value, visible, checked_floats({batch}), "visible counts");
+    op_span(value, lower, checked_floats({batch, groups}), "score bounds");
+    op_span(value, upper, checked_floats({batch, groups}), "score bounds");
+    FastIndexSpace space = fast_index_space(workspace(value, fast_index_bytes(batch, groups, heads, dim)), batch, groups, heads, dim);
+    space.lower = lower; space.upper = upper;
+    switch (heads) {
+        case 16: fast_index_bounds<16>(value, space, q_index, keys, weights, visible, batch, groups, scale); break;
+        case 32: fast_index_bounds<32>(value, space, q_index, keys, weights, visible, batch, groups, scale); break;
+        case 48: fast_index_bounds<48>(value, space, q_index, keys, weights, visible, batch, groups, scale); break;
+        default: fast_index_bounds<64>(value, space, q_index, keys, weights, visible, batch, groups, scale); break;
+    }
     SD_OP_END
 }
 

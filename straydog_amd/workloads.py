@@ -165,7 +165,7 @@ class SparseWorkload:
         gpu.fill_normal(self.latents.base(), batch * context * kdim, seed * 11 + 5, 2)
         gpu.synchronize()
 
-    def step_index(self, keep_scores=True):
+    def step_index(self, keep_scores=False):
         g = self.gpu
         g.index_top_k(self.q_index.base(), self.keys.base(), self.weights.base(), self.visible.base(), self.batch, self.context,
                       self.index_heads, self.index_dim, 1.0, self.scores.base() if keep_scores else None, self.k, self.indices.base())

@@ -303,6 +303,43 @@ def test_sparse_attention_matches_the_oracle_and_bf16_rows_match_f32(gpu, oracle
             gpu.release(b)
 
 
+@pytest.mark.parametrize("heads,groups,k", [(64, 5000, 256), (32, 3000, 2048), (16, 777, 100), (48, 20000, 512)])
+def test_matrix_core_indexer_brackets_and_selects_exactly(gpu, oracle, heads, groups, k):
+    # the fast indexer of the batched sparse path: every canonical score lies inside its bracket, and the indices chosen
+    # from the brackets and the exact rescoring are those of the exact path, bit for bit (ties and short rows included)
+    rng = np.random.default_rng(heads * 1000 + k)
+    batch, dim = 4, 128
+    q_bits, q_vals = _bf16_round(oracle, rng.standard_normal((batch, heads, dim)).astype(np.float32))
+    keys = rng.standard_normal((batch, groups, dim)).astype(np.float32)
+    keys[1, 100:400] = keys[1, 50]                  # a run of identical keys: equal scores, the tie rule decides
+    keys[2] *= (rng.random((groups, 1)) * 4).astype(np.float32)     # rows of very different norms
+    keys[3, ::7] = 0.0
+    key_bits, key_vals = _bf16_round(oracle, keys)
+    weights = rng.random((batch, heads)).astype(np.float32)
+    weights[3, ::2] = 0.0
+    visible = np.array([groups, groups - 37, groups, min(groups, k // 2)], dtype=np.int32)   # the last row: fewer visible than k
+    qb, kb, wb, vb = gpu.upload(q_bits), gpu.upload(key_bits), gpu.upload(weights), gpu.upload(visible)
+    lower, upper = gpu.buffer(batch * groups * 4), gpu.buffer(batch * groups * 4)
+    for scale in (1.0, 0.37):
+        gpu.index_score_bounds(qb.base(), kb.base(), wb.base(), vb.base(), batch, groups, heads, dim, scale, lower.base(), upper.base())
+        low = _read(gpu, lower, np.float32, batch * groups).reshape(batch, groups)
+        high = _read(gpu, upper, np.float32, batch * groups).reshape(batch, groups)
+        indices = gpu.buffer(batch * k * 4)
+        gpu.index_top_k(qb.base(), kb.base(), wb.base(), vb.base(), batch, groups, heads, dim, scale, None, k, indices.base())
+        got = _read(gpu, indices, np.int32, batch * k).reshape(batch, k)
+        for b in range(batch):
+            want = oracle.index_scores(q_vals[b:b + 1], key_vals[b], weights[b:b + 1], visible[b:b + 1], scale)[0]
+            seen = np.arange(groups) < visible[b]
+            assert np.all(low[b][seen] <= want[seen]) and np.all(want[seen] <= high[b][seen])
+            assert np.all(np.isneginf(low[b][~seen])) and np.all(np.isneginf(high[b][~seen]))
+            width = (high[b][seen] - low[b][seen]).max()
+            assert width < 1e-2 * max(1.0, np.abs(want[seen]).max())            # the brackets are tight, not vacuous
+            assert np.array_equal(got[b], oracle.top_k(want[None, :], k)[0])
+        gpu.release(indices)
+    for b in (qb, kb, wb, vb, lower, upper):
+        gpu.release(b)
+
+
 def test_batched_sparse_path_small(gpu, oracle):
     # BASELINE config 4 in small: index scores -> top-k (bit-exact) -> gather attention over BF16 latents, per sequence
     rng = np.random.default_rng(12)
