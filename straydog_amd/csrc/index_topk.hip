@@ -318,17 +318,27 @@ __device__ __forceinline__ float quad_sum(float x) {
 }
 
 // W of the margin for every row: sum_h |w_h| |q_h| * |scale| * 2^-14, rounded up a little.
-__global__ void __launch_bounds__(64) index_margin_kernel(const uint16_t* q, const float* weights, size_t heads, size_t dim, float scale, float* margin) {
+__global__ void __launch_bounds__(256) index_margin_kernel(const uint16_t* q, const float* weights, size_t heads, size_t dim, float scale, float* margin) {
+    // four lanes per head, 8 values a load
     const size_t row = blockIdx.x;
-    float total = 0.0f;
-    for (size_t h = threadIdx.x; h < heads; h += 64) {
-        float square = 0.0f;
-        for (size_t d = 0; d < dim; ++d) { const float v = bf16_value(q[(row * heads + h) * dim + d]); square += v * v; }
-        total += fabsf(weights[row * heads + h]) * sqrtf(square);
-    }
+    const unsigned t = threadIdx.x, h = t / 4, part = t % 4;
+    float square = 0.0f;
+    if (h < heads)
+        for (size_t d = 8 * part; d < dim; d += 32) {
+            const uint4 bits = *reinterpret_cast<const uint4*>(q + (row * heads + h) * dim + d);
+            const uint32_t words[4] = {bits.x, bits.y, bits.z, bits.w};
+            #pragma unroll
+            for (int i = 0; i < 4; ++i) { const float a = __uint_as_float(words[i] << 16), b = __uint_as_float(words[i] & 0xffff0000u); square += a * a + b * b; }
+        }
+    square += __shfl_xor(square, 1);
+    square += __shfl_xor(square, 2);
+    float total = h < heads && part == 0 ? fabsf(weights[row * heads + h]) * sqrtf(square) : 0.0f;
     #pragma unroll
     for (int d = 32; d; d >>= 1) total += __shfl_xor(total, d);
-    if (threadIdx.x == 0) margin[row] = total * fabsf(scale) * (1.0f / 16384.0f) * 1.01f;
+    __shared__ float waves[4];
+    if ((t & 63) == 0) waves[t >> 6] = total;
+    __syncthreads();
+    if (t == 0) margin[row] = (waves[0] + waves[1] + waves[2] + waves[3]) * fabsf(scale) * (1.0f / 16384.0f) * 1.01f;
 }
 
 // Bounds of the scores of INTERVAL_KEYS groups per workgroup, 16 groups per MFMA tile and wave, and the first radix
@@ -401,20 +411,26 @@ __global__ void __launch_bounds__(256) index_interval_kernel(const uint16_t* __r
 // them; `everything` when fewer than rank keys are live at all.
 struct RadixPick { uint32_t prefix, rank; bool everything; };
 __device__ RadixPick radix_pick(const uint32_t* histogram /* [level][rows][RADIX_BINS] */, size_t rows, size_t row, int levels, uint32_t k) {
-    __shared__ uint32_t sums[256], found[3];
+    __shared__ uint32_t wave_sums[4], found[2];
     RadixPick pick{0u, k, false};
-    const unsigned t = threadIdx.x;
+    const unsigned t = threadIdx.x, lane = t & 63, wave = t >> 6;
     for (int level = 0; level < levels; ++level) {
         const uint32_t* bins = histogram + (size_t(level) * rows + row) * RADIX_BINS;
-        // thread t owns the 8 bins below 2048 - 8t, highest first
+        // thread t owns the 8 bins below 2048 - 8t, highest first; a scan in thread order counts the keys in higher bins
         uint32_t mine[8], sum = 0;
+        const uint4 a = *reinterpret_cast<const uint4*>(bins + RADIX_BINS - 8 - 8 * t), b = *reinterpret_cast<const uint4*>(bins + RADIX_BINS - 4 - 8 * t);
+        mine[0] = b.w; mine[1] = b.z; mine[2] = b.y; mine[3] = b.x; mine[4] = a.w; mine[5] = a.z; mine[6] = a.y; mine[7] = a.x;
         #pragma unroll
-        for (int i = 0; i < 8; ++i) { mine[i] = bins[RADIX_BINS - 1 - (8 * t + i)]; sum += mine[i]; }
+        for (int i = 0; i < 8; ++i) sum += mine[i];
+        uint32_t inclusive = sum;
+        #pragma unroll
+        for (unsigned offset = 1; offset < 64; offset *= 2) { const uint32_t other = __shfl_up(inclusive, offset); if (lane >= offset) inclusive += other; }
+        __syncthreads();                              // the shared words of the level before are read
+        if (lane == 63) wave_sums[wave] = inclusive;
         __syncthreads();
-        sums[t] = sum;
-        __syncthreads();
-        uint32_t above = 0, every = 0;
-        for (unsigned i = 0; i < 256; ++i) { const uint32_t c = sums[i]; above += i < t ? c : 0u; every += c; }
+        uint32_t above = inclusive - sum, every = 0;
+        #pragma unroll
+        for (unsigned v = 0; v < 4; ++v) { const uint32_t c = wave_sums[v]; above += v < wave ? c : 0u; every += c; }
         if (level == 0 && every < pick.rank) { pick.everything = true; return pick; }
         if (above < pick.rank && above + sum >= pick.rank) {
             uint32_t before = above;
@@ -505,33 +521,35 @@ __global__ void __launch_bounds__(256) candidate_list_kernel(const float* upper,
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 255) totals[row] = at;
 }
 
-// The canonical score of every listed group: a wave per group, a lane per head (its query row in registers, the key row
-// in scalar registers), then the heads' terms added in head order.
+// The canonical score of every listed group: a wave per group, a lane per head (the key row in scalar registers), then
+// the heads' terms added in head order.  The workgroup's eight waves share one copy of the row's queries in LDS,
+// transposed so that the lanes of a wave read neighbouring words; few registers, so many waves hide the loads' latency.
 template<int HEADS>
-__global__ void __launch_bounds__(256) candidate_score_kernel(const float* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
+__global__ void __launch_bounds__(512) candidate_score_kernel(const float* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
                                                               size_t groups, float scale, const int32_t* __restrict__ list, const uint32_t* __restrict__ totals,
                                                               float* __restrict__ scores) {
     constexpr int DIM = 128;
     const size_t row = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int head = min(lane, HEADS - 1);
-    float query[DIM];
-    #pragma unroll
-    for (int d = 0; d < DIM; d += 4) {
-        const float4 v = *reinterpret_cast<const float4*>(q + (row * HEADS + head) * DIM + d);
-        query[d] = v.x; query[d + 1] = v.y; query[d + 2] = v.z; query[d + 3] = v.w;
-    }
-    const float weight = weights[row * HEADS + head];
     const uint32_t total = totals[row];
-    for (uint32_t at = blockIdx.x * 4 + wave; at < total; at += gridDim.x * 4) {
+    if (blockIdx.x * 8 >= total) return;
+    __shared__ float shared_q[DIM][HEADS + 1];
+    for (int i = threadIdx.x; i < HEADS * DIM; i += 512) shared_q[i % DIM][i / DIM] = q[row * HEADS * DIM + i];
+    __syncthreads();
+    const float weight = weights[row * HEADS + head];
+    for (uint32_t at = blockIdx.x * 8 + wave; at < total; at += gridDim.x * 8) {
         const int32_t group = __builtin_amdgcn_readfirstlane(list[row * groups + at]);
-        const uint32_t* key = reinterpret_cast<const uint32_t*>(keys + (row * groups + size_t(group)) * DIM);
+        typedef __attribute__((address_space(4))) const uint32_t* uniform_words;     // the row is the wave's: scalar loads
+        const uniform_words key = (uniform_words)(keys + (row * groups + size_t(group)) * DIM);
+        const float* mine = &shared_q[0][head];
+        asm volatile("" : "+v"(mine));               // read anew for every group: the values are not kept in registers
         float dot = 0.0f;
         #pragma unroll
         for (int d = 0; d < DIM; d += 2) {
-            const uint32_t pair = __builtin_amdgcn_readfirstlane(key[d / 2]);
-            dot = __builtin_fmaf(query[d], __uint_as_float(pair << 16), dot);
-            dot = __builtin_fmaf(query[d + 1], __uint_as_float(pair & 0xffff0000u), dot);
+            const uint32_t pair = key[d / 2];
+            dot = __builtin_fmaf(mine[d * (HEADS + 1)], __uint_as_float(pair << 16), dot);
+            dot = __builtin_fmaf(mine[(d + 1) * (HEADS + 1)], __uint_as_float(pair & 0xffff0000u), dot);
         }
         const float term = rounded_product(fmaxf(dot, 0.0f), weight);
         float sum = 0.0f;
@@ -601,7 +619,7 @@ template<int HEADS>
 void fast_index_bounds(Device& d, const FastIndexSpace& s, const void* q_index, const void* keys, const float* weights, const int32_t* visible, size_t batch,
                        size_t groups, float scale) {
     fill_words_kernel<<<unsigned(std::min<size_t>(checked_blocks(RADIX_LEVELS * batch * RADIX_BINS), 1024)), 256, 0, d.stream>>>(s.histogram, RADIX_LEVELS * batch * RADIX_BINS);
-    index_margin_kernel<<<unsigned(batch), 64, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), weights, HEADS, 128, scale, s.margin);
+    index_margin_kernel<<<unsigned(batch), 256, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), weights, HEADS, 128, scale, s.margin);
     index_interval_kernel<HEADS><<<dim3(unsigned(s.blocks), unsigned(batch)), 256, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys),
                                                                                                    weights, visible, s.margin, groups, scale, s.lower, s.upper, s.histogram);
     SD_CHECK(hipGetLastError());
@@ -621,7 +639,7 @@ void fast_index_top_k(Device& d, const FastIndexSpace& s, const void* q_index, c
     radix_histogram_kernel<<<grid, 256, 0, d.stream>>>(s.lower, groups, batch, 2, rank, s.histogram);
     candidate_count_kernel<<<grid, 256, 0, d.stream>>>(s.upper, groups, batch, rank, s.histogram, s.counts);
     candidate_list_kernel<<<grid, 256, 0, d.stream>>>(s.upper, groups, batch, rank, s.histogram, s.counts, s.list, s.totals);
-    candidate_score_kernel<HEADS><<<dim3(64, unsigned(batch)), 256, 0, d.stream>>>(s.wide_q, static_cast<const uint16_t*>(keys), weights, groups, scale, s.list, s.totals,
+    candidate_score_kernel<HEADS><<<dim3(128, unsigned(batch)), 512, 0, d.stream>>>(s.wide_q, static_cast<const uint16_t*>(keys), weights, groups, scale, s.list, s.totals,
                                                                                    s.scores);
     top_k_listed_kernel<<<unsigned(batch), TOPK_THREADS, 0, d.stream>>>(s.scores, s.list, s.totals, groups, k, indices);
     SD_CHECK(hipGetLastError());
