@@ -80,6 +80,11 @@ __device__ __forceinline__ bool find_work(const PagedArgs& args, unsigned id, in
     return false;
 }
 
+constexpr float SLACK = 8.0f;     // how far (base-2 exponent) a row's true maximum may run ahead of its reference maximum
+constexpr int stages_per_wave(int slab, int occupancy) { return occupancy <= 2 && WAVES * 2 * 2 * slab * occupancy <= 160 * 1024 ? 2 : 1; }
+// s_waitcnt for the vector-memory counter alone: wait until at most N of the wave's loads are outstanding.
+template<int N> __device__ __forceinline__ void wait_loads() { __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14)); }
+
 // A step's K and V slabs (32 contiguous rows each) are copied by fully coalesced 16-byte global->LDS loads into the wave's
 // own LDS stage; operands are then read from LDS in MFMA layout while the next step's copy is in flight.  OCC = the waves per
 // SIMD the variant is compiled for (its register budget).
@@ -133,10 +138,13 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
 
     extern __shared__ float lds[];
     constexpr int SLAB = STEP * ROW;                       // one step's rows of one plane: contiguous in the page
-    uint8_t* stage = reinterpret_cast<uint8_t*>(lds) + wave * (2 * SLAB);
+    // Stages per wave: with few waves per SIMD one step in flight per wave does not cover the memory latency, so a wave then
+    // keeps two (where the workgroups resident at once still fit the 160 KiB of LDS).
+    constexpr int DEPTH = stages_per_wave(SLAB, OCC), LOADS = 2 * ((SLAB + 1023) / 1024);
+    uint8_t* const stages = reinterpret_cast<uint8_t*>(lds) + wave * (DEPTH * 2 * SLAB);
     // A step's rows from the wave's stage into operand registers.  The rows past the sequence's end in its last step hold
     // whatever the page held: they are cleared first (their scores are masked, but a stray scale must not meet a zero weight).
-    const auto request = [&](RowLoad<DIM, Q8>& rows, int token0) {
+    const auto request = [&](RowLoad<DIM, Q8>& rows, uint8_t* stage, int token0) {
         const int valid = total - token0;
         if (valid < STEP)
             #pragma unroll
@@ -145,7 +153,7 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         load_step<DIM>(rows, stage, stage + SLAB, li, g);
     };
     // The step's two slabs copied into the stage, 1 KiB per instruction, lanes past a slab's end switched off.
-    const auto copy_in = [&](int page, int in_page) {
+    const auto copy_in = [&](uint8_t* stage, int page, int in_page) {
         const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(in_page) * ROW + 16 * lane;
         #pragma unroll
         for (int part = 0; part < 2; ++part) {
@@ -157,23 +165,34 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         }
     };
 
-    // Where the wave's step lies: page_index-th page of the sequence, in_page rows into it.  The page number of the step
-    // after the current one is fetched (a scalar load) before the current step is waited for, so it is there when its copy
-    // is issued.
+    // Where the step to copy next lies: page_index-th page of the sequence, in_page rows into it.  Its page number is fetched
+    // (a scalar load) a step before its copy is issued.
     int token0 = chunk_begin + STEP * wave;
     const int last_page = (total - 1) / int(args.page_tokens);
     int page_index = token0 / int(args.page_tokens), in_page = token0 % int(args.page_tokens);
-    if (token0 < chunk_end) copy_in(table[min(page_index, last_page)], in_page);
-    for (; token0 < chunk_end; token0 += STEP * WAVES) {
+    const auto advance = [&] {
         in_page += STEP * WAVES;
         while (in_page >= int(args.page_tokens)) { in_page -= int(args.page_tokens); ++page_index; }
-        const int page_ahead = table[min(page_index, last_page)];
+    };
+    #pragma unroll
+    for (int ahead = 0; ahead < DEPTH; ++ahead) {
+        if (token0 + ahead * STEP * WAVES < chunk_end) copy_in(stages + ahead * (2 * SLAB), table[min(page_index, last_page)], in_page);
+        advance();
+    }
+    int page_ahead = table[min(page_index, last_page)];
+    for (int buffer = 0; token0 < chunk_end; token0 += STEP * WAVES, buffer = DEPTH == 2 ? buffer ^ 1 : 0) {
+        uint8_t* const stage = stages + buffer * (2 * SLAB);
+        const bool more = token0 + DEPTH * STEP * WAVES < chunk_end;      // a step to copy into this stage once it is read
+        const int page_now = page_ahead, in_page_now = in_page;
+        advance();
+        page_ahead = table[min(page_index, last_page)];
         RowLoad<DIM, Q8> current;
-        __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0): the stage holds this step
-        request(current, token0);
+        // the stage holds this step when only the step after it is still on its way
+        if (DEPTH == 2 && token0 + STEP * WAVES < chunk_end) wait_loads<LOADS>(); else wait_loads<0>();
+        request(current, stage, token0);
         __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): operands are in registers, the stage is free again
         __builtin_amdgcn_sched_barrier(0);
-        if (token0 + STEP * WAVES < chunk_end) copy_in(page_ahead, in_page);
+        if (more) copy_in(stage, page_now, in_page_now);
         __builtin_amdgcn_sched_barrier(0);
         // S^T tiles: tokens (rows, 4 per lane group) x query rows (lane li)
         floatx4 s[QT][2];
@@ -188,38 +207,49 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
                 for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qf[qt][b], s[qt][t], 0, 0, 0);
             }
         }
-        const bool edge = token0 + STEP - 1 > position;    // wave-uniform: some token of the step is past the first row's position
-        half8 pb[QT];
+        // Scores stay unscaled (the scale goes into the exponent's multiply-add); m is a row's reference maximum in unscaled
+        // units.  It follows the true maximum only when that has grown by more than SLACK (in base-2 exponent units): weights
+        // then stay below 2^SLACK, far inside FP16 and FP32 range, and the accumulators are rescaled a few times per row
+        // instead of at every new maximum.  The quotient acc/sum does not depend on the reference.
+        if (token0 + STEP - 1 > position) {          // wave-uniform: some token of the step is past the first row's position
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt)
+                #pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    #pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (token0 + 16 * t + 4 * g + r > limit[qt]) s[qt][t][r] = -INFINITY;
+        }
+        float top[QT];
+        bool grown = false;
         #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
-            float top = NEG_BIG;
+            top[qt] = row_max(fmaxf(fmaxf(fmaxf(s[qt][0][0], s[qt][0][1]), fmaxf(s[qt][0][2], s[qt][0][3])),
+                                    fmaxf(fmaxf(s[qt][1][0], s[qt][1][1]), fmaxf(s[qt][1][2], s[qt][1][3]))));
+            grown |= (top[qt] - m[qt]) * args.scale_log2 > SLACK;
+        }
+        if (__any(grown)) {
             #pragma unroll
-            for (int t = 0; t < 2; ++t)
-                #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float value = s[qt][t][r] * args.scale_log2;
-                    if (edge && token0 + 16 * t + 4 * g + r > limit[qt]) value = -INFINITY;
-                    s[qt][t][r] = value;
-                    top = fmaxf(top, value);
-                }
-            top = fmaxf(top, __shfl_xor(top, 16));
-            top = fmaxf(top, __shfl_xor(top, 32));
-            // the running maximum rarely grows after the first steps: rescale only when some row's did
-            if (__any(top > m[qt])) {
-                const float m_new = fmaxf(m[qt], top);
-                const float alpha = __builtin_amdgcn_exp2f(m[qt] - m_new);
+            for (int qt = 0; qt < QT; ++qt) {
+                const float m_new = fmaxf(m[qt], top[qt]);
+                const float alpha = __builtin_amdgcn_exp2f((m[qt] - m_new) * args.scale_log2);
                 m[qt] = m_new;
                 l[qt] *= alpha;
                 #pragma unroll
                 for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] *= alpha;
             }
+        }
+        half8 pb[QT];
+        #pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            const float offset = -m[qt] * args.scale_log2;
             float sum = 0.0f;
             half8 p;
             #pragma unroll
             for (int t = 0; t < 2; ++t)
                 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float w = __builtin_amdgcn_exp2f(s[qt][t][r] - m[qt]);
+                    const float w = __builtin_amdgcn_exp2f(fmaf(s[qt][t][r], args.scale_log2, offset));
                     sum += w;
                     p[4 * t + r] = (_Float16)w;
                 }
@@ -242,11 +272,9 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
     constexpr int STRIDE = DIM + 2, QROWS = QT * 16;
     #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
-        float sum = l[qt];
-        sum += __shfl_xor(sum, 16);
-        sum += __shfl_xor(sum, 32);
+        const float sum = row_sum(l[qt]);
         float* row = lds + (size_t(wave) * QROWS + qt * 16 + li) * STRIDE;
-        if (g == 0) { row[DIM] = m[qt]; row[DIM + 1] = sum; }
+        if (g == 0) { row[DIM] = m[qt] * args.scale_log2; row[DIM + 1] = sum; }      // maxima leave in exponent units
         #pragma unroll
         for (int jj = 0; jj < TILES; ++jj)
             #pragma unroll
@@ -367,7 +395,8 @@ void plan_chunks(PagedArgs& args, uint64_t seqs, uint64_t kv_heads, uint64_t max
 
 template<int DIM, int QT, bool Q8, int OCC>
 void launch(Device& d, const PagedArgs& args, dim3 grid) {
-    const size_t shared = std::max(size_t(WAVES) * QT * 16 * (DIM + 2) * 4, size_t(WAVES) * 2 * STEP * (Q8 ? DIM + DIM / 16 : 2 * DIM));
+    constexpr int slab = STEP * (Q8 ? DIM + DIM / 16 : 2 * DIM);
+    const size_t shared = std::max(size_t(WAVES) * QT * 16 * (DIM + 2) * 4, size_t(WAVES) * stages_per_wave(slab, OCC) * 2 * slab);
     if (shared > 160 * 1024) throw std::runtime_error("Straydog paged attention: too many query rows per K/V head for the decode kernel");
     static bool raised = false;
     if (!raised && shared > 64 * 1024) {
@@ -406,7 +435,7 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
                         uint64_t heads, float scale, void* out, int out_f16, void* scratch, uint64_t scratch_bytes) {
     SD_OP_BEGIN
     validate_pool(value, pool);
-    if (!seqs || seqs > 65535 || !span || !heads || heads % pool->kv_heads || !max_context || max_context > (uint64_t(1) << 30) ||
+    if (!(scale > 0.0f) || !seqs || seqs > 65535 || !span || !heads || heads % pool->kv_heads || !max_context || max_context > (uint64_t(1) << 30) ||
         !table_stride || max_context > table_stride * pool->page_tokens)
         throw std::runtime_error("invalid Straydog paged attention shape");
     const uint64_t group = heads / pool->kv_heads, rows = span * group;
