@@ -43,7 +43,7 @@ __device__ __forceinline__ unsigned chunk_tokens(const PagedArgs& args, int lane
     }
     #pragma unroll
     for (int d = 32; d; d >>= 1) { tokens += __shfl_xor(tokens, d); longest = max(longest, __shfl_xor(longest, d)); }
-    const float rounds = args.rounds > 0.0f ? args.rounds : tokens > 0.9f * float(args.seqs) * float(longest) ? 1.0f : 2.0f;
+    const float rounds = tokens > 0.9f * float(args.seqs) * float(longest) ? args.rounds_even : args.rounds;
     const float cut = tokens * float(args.kv_heads) / (args.slots * rounds);
     const unsigned chunk = (unsigned(fminf(cut, 1.0e6f)) + 127u) / 128u * 128u;
     return __builtin_amdgcn_readfirstlane(min(max(chunk, args.chunk_min), args.chunk_max));
@@ -374,21 +374,26 @@ const Tuning& tuning() {
     return value;
 }
 
-constexpr unsigned smallest_chunk = 256, largest_chunk = 4096;
+constexpr unsigned smallest_chunk = 256, largest_chunk = 16384;
 
 // The host knows only max_context: it bounds the device's choice above by the chunk of a batch with every sequence full,
 // and sizes the grid for an eighth of that (the workgroups past the batch's last chunk leave at once).
-void plan_chunks(PagedArgs& args, uint64_t seqs, uint64_t kv_heads, uint64_t max_context, unsigned compute_units) {
-    args.slots = float(compute_units) * 4.0f;
-    args.rounds = tuning().rounds;
+void plan_chunks(PagedArgs& args, uint64_t seqs, uint64_t kv_heads, uint64_t max_context, unsigned slots) {
+    args.slots = float(slots);
+    // One query tile (decode, 4 workgroups per compute unit): one round for even batches, two for uneven ones; the heavier
+    // variants (1-2 workgroups per compute unit) even out better over three, and their idle trailing workgroups cost more, so
+    // their grid allows less room below the largest chunk.
+    const bool decode = args.rows <= 16;
+    args.rounds = tuning().rounds > 0.0f ? tuning().rounds : decode ? 2.0f : 3.0f;
+    args.rounds_even = tuning().rounds > 0.0f ? tuning().rounds : decode ? 1.0f : 3.0f;
     if (tuning().chunk) {
         const unsigned chunk = std::min(std::max((tuning().chunk + 127u) / 128u * 128u, smallest_chunk), 1u << 20);
         args.chunk_min = args.chunk_max = chunk;
     } else {
-        const double full = double(max_context) * double(seqs) * double(kv_heads) / double(args.slots * (args.rounds > 0.0f ? args.rounds : 1.0f));
+        const double full = double(max_context) * double(seqs) * double(kv_heads) / double(args.slots * args.rounds_even);
         const unsigned chunk = unsigned(std::min(full, 1.0e6) + 127.0) / 128u * 128u;
         args.chunk_max = std::min(std::max(chunk, smallest_chunk), largest_chunk);
-        args.chunk_min = std::max(smallest_chunk, args.chunk_max / 8 / 128u * 128u);
+        args.chunk_min = std::max(smallest_chunk, args.chunk_max / (decode ? 4 : 2) / 128u * 128u);
     }
     args.chunks = unsigned((max_context + args.chunk_min - 1) / args.chunk_min);
 }
@@ -408,16 +413,26 @@ void launch(Device& d, const PagedArgs& args, dim3 grid) {
 
 // The variants that exist: (columns, query tiles, format) -> waves per SIMD the kernel is compiled for.  One query tile is
 // the decode shape (4 waves/SIMD at 128 columns of Q8_0); more tiles hold more accumulators.
+constexpr int variant_occupancy(int dim, bool q8, unsigned query_tiles) {
+    const bool small = dim == 128;
+    return query_tiles == 1 ? (small && q8 ? 4 : small ? 2 : 1) : query_tiles == 2 ? (small ? 2 : 1) : query_tiles == 3 ? (small && q8 ? 2 : 1) : 1;
+}
 template<int DIM, bool Q8>
 void launch_tiles(Device& d, const PagedArgs& args, unsigned query_tiles, dim3 grid) {
     constexpr bool small = DIM == 128;
     switch (query_tiles) {
-        case 1: launch<DIM, 1, Q8, (small && Q8 ? 4 : small ? 2 : 1)>(d, args, grid); break;
-        case 2: launch<DIM, 2, Q8, (small ? 2 : 1)>(d, args, grid); break;
-        case 3: if constexpr (small) { launch<DIM, 3, Q8, (Q8 ? 2 : 1)>(d, args, grid); break; }
-        case 4: if constexpr (small) { launch<DIM, 4, Q8, 1>(d, args, grid); break; }
+        case 1: launch<DIM, 1, Q8, variant_occupancy(DIM, Q8, 1)>(d, args, grid); break;
+        case 2: launch<DIM, 2, Q8, variant_occupancy(DIM, Q8, 2)>(d, args, grid); break;
+        case 3: if constexpr (small) { launch<DIM, 3, Q8, variant_occupancy(DIM, Q8, 3)>(d, args, grid); break; }
+        case 4: if constexpr (small) { launch<DIM, 4, Q8, variant_occupancy(DIM, Q8, 4)>(d, args, grid); break; }
         default: throw std::runtime_error("Straydog paged attention: too many query rows per K/V head for the decode kernel");
     }
+}
+// Workgroups resident at once: as many per compute unit as the variant's waves per SIMD and its LDS allow.
+unsigned resident_slots(const Device& d, unsigned dim, bool q8, unsigned query_tiles) {
+    const int occupancy = variant_occupancy(int(dim), q8, query_tiles), slab = STEP * int(q8 ? dim + dim / 16 : 2 * dim);
+    const size_t shared = std::max(size_t(WAVES) * query_tiles * 16 * (dim + 2) * 4, size_t(WAVES) * stages_per_wave(slab, occupancy) * 2 * slab);
+    return d.compute_units * unsigned(std::max<size_t>(1, std::min<size_t>(size_t(occupancy), (160 * 1024) / shared)));
 }
 
 }  // namespace
@@ -457,7 +472,7 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
     args.q = q; args.q_f16 = q_f16; args.scale_log2 = scale * 1.44269504088896341f;
     args.rows = unsigned(rows); args.seqs = unsigned(seqs);
     args.max_context = int(max_context);
-    plan_chunks(args, seqs, pool->kv_heads, max_context, value.compute_units);
+    plan_chunks(args, seqs, pool->kv_heads, max_context, resident_slots(value, pool->dim, pool->row_bytes != 2 * pool->dim, query_tiles));
     if (args.chunks > 65535) throw std::runtime_error("invalid Straydog paged attention shape");
     const size_t need = checked_floats({seqs, pool->kv_heads, args.chunks, rows, uint64_t(pool->dim) + 2});
     if (!scratch || scratch_bytes < need) throw std::runtime_error("Straydog paged attention scratch too small");

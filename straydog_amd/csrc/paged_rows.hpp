@@ -35,7 +35,7 @@ struct PagedArgs {
     float* partial;        // [seq][kv head][chunk][row][dim + 2]
     unsigned chunks, rows;  // chunks = the most chunks a sequence can have; rows = span * group (query rows per K/V head)
     unsigned chunk_min, chunk_max, seqs;   // tokens per chunk are chosen on the device between these (see chunk_tokens)
-    float slots, rounds;   // workgroups resident at once; workgroups per slot to cut the batch into (0: chosen from the batch)
+    float slots, rounds, rounds_even;   // workgroups resident at once; workgroups per slot to cut an uneven / an even batch into
     int max_context;       // positions[s] + span is clipped to this (the launch and the page table are sized for it)
 };
 
