@@ -10,13 +10,13 @@ class PagedWorkload:
     """A batch of sequences in a shuffled paged Q8_0 cache, with `span` query rows each."""
 
     def __init__(self, gpu, lengths, span=1, heads=32, kv_heads=4, dim=128, page_tokens=256, seed=1, q_f16=True, out_f16=True,
-                 row_bytes=None):
+                 row_bytes=None, page_seed=None):
         self.gpu, self.span, self.heads, self.kv_heads, self.dim, self.page_tokens = gpu, span, heads, kv_heads, dim, page_tokens
         self.lengths = np.asarray(lengths, dtype=np.int64)            # cached tokens per sequence, the span's rows included
         self.seqs = len(lengths)
         self.row_bytes = row_bytes or ROW_Q8[dim]
         self.q_f16, self.out_f16 = q_f16, out_f16
-        rng = np.random.default_rng(seed)
+        rng = np.random.default_rng(seed if page_seed is None else page_seed)     # where the pages lie; the rows are `seed`'s
         pages_per = (self.lengths + page_tokens - 1) // page_tokens
         self.page_count = int(pages_per.sum())
         self.table_stride = int(pages_per.max())
