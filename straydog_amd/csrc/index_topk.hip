@@ -306,6 +306,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int RADIX_BINS = 2048, RADIX_LEVELS = 3, INTERVAL_KEYS = 1024;   // digits of 11, 11 and 10 bits; groups per workgroup
+constexpr int BRACKET_WAVES = 8, BRACKET_KEYS = 2048, BRACKET_RING = 4;     // the bracket kernel: waves, groups per workgroup, stages per wave
 __device__ __forceinline__ uint32_t radix_digit(uint32_t key, int level) { return level == 0 ? key >> 21 : level == 1 ? (key >> 10) & 2047u : key & 1023u; }
 
 // The sum over the four lanes li, li + 16, li + 32, li + 48 in all of them (see paged_rows.hpp for the instructions).
@@ -342,17 +343,21 @@ __global__ void __launch_bounds__(256) index_margin_kernel(const uint16_t* q, co
 }
 
 // Bounds of the scores of INTERVAL_KEYS groups per workgroup, 16 groups per MFMA tile and wave, and the first radix
-// histogram of the lower bounds.  S = Q . K^T with Q (heads x dim) as A operands from registers and K rows straight from
-// memory as B operands; K . K^T from the same registers gives |k|^2 on its diagonal.
+// histogram of the lower bounds.  S = Q . K^T with Q (heads x dim) as A operands from registers and K rows as B operands;
+// K . K^T from the same registers gives |k|^2 on its diagonal.  A tile's 16 rows are 4 KiB in one piece: they come HBM -> LDS
+// by four coalesced 1 KiB global->LDS loads into the wave's ring of stages, three tiles ahead of the one being computed
+// (two waves per SIMD leave room for that much in flight).  The loads place piece c of row r at position c ^ r of the row, so that the 16 lanes of an operand read (one
+// row each, the same piece) touch 16 different banks.
 template<int HEADS>
-__global__ void __launch_bounds__(256) index_interval_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
+__global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
                                                              const int32_t* __restrict__ visible, const float* __restrict__ margin, size_t groups, float scale,
                                                              float* __restrict__ lower, float* __restrict__ upper, uint32_t* __restrict__ histogram) {
     constexpr int DIM = 128, HT = HEADS / 16, KS = DIM / 32;
     const size_t row = blockIdx.y;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, li = lane & 15, g = lane >> 4;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, g = lane >> 4;
     __shared__ uint32_t bins[RADIX_BINS];
-    for (int i = threadIdx.x; i < RADIX_BINS; i += 256) bins[i] = 0;
+    __shared__ __attribute__((aligned(16))) uint8_t stages[BRACKET_WAVES][BRACKET_RING][4096];
+    for (int i = threadIdx.x; i < RADIX_BINS; i += BRACKET_WAVES * 64) bins[i] = 0;
     bf16x8 qa[HT][KS];
     float w[HT][4];
     #pragma unroll
@@ -368,13 +373,33 @@ __global__ void __launch_bounds__(256) index_interval_kernel(const uint16_t* __r
     const float bound = margin[row];
     const uint16_t* row_keys = keys + row * groups * DIM;
     __syncthreads();
-    const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS;
-    for (size_t tile = first + 16 * wave; tile < min(first + INTERVAL_KEYS, groups); tile += 64) {
+    const size_t first = size_t(blockIdx.x) * BRACKET_KEYS, end = min(first + BRACKET_KEYS, groups);
+    typedef __attribute__((address_space(1))) const void* global_ptr;
+    typedef __attribute__((address_space(3))) void* lds_ptr;
+    const auto copy_in = [&](int buffer, size_t tile) {
+        #pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int r = 4 * j + (lane >> 4), c = (lane & 15) ^ r;
+            const uint16_t* from = row_keys + min(tile + r, groups - 1) * DIM + 8 * c;
+            __builtin_amdgcn_global_load_lds((global_ptr)from, (lds_ptr)(stages[wave][buffer] + 1024 * j), 16, 0, 2 /* nt: read once */);
+        }
+    };
+    constexpr size_t stride = 16 * BRACKET_WAVES;
+    size_t tile = first + 16 * wave;
+    #pragma unroll
+    for (int ahead = 0; ahead < BRACKET_RING - 1; ++ahead)
+        if (tile + ahead * stride < end) copy_in(ahead, tile + ahead * stride);
+    for (int buffer = 0; tile < end; tile += stride, buffer = (buffer + 1) % BRACKET_RING) {
         const size_t group = tile + li;
-        const uint16_t* from = row_keys + min(group, groups - 1) * DIM + 8 * g;
+        if (tile + (BRACKET_RING - 1) * stride < end) copy_in((buffer + BRACKET_RING - 1) % BRACKET_RING, tile + (BRACKET_RING - 1) * stride);
+        // this tile has landed when only the tiles after it (at most three, four loads each) are outstanding
+        const size_t after = (end - tile - 1) / stride;
+        if (after >= 3) __builtin_amdgcn_s_waitcnt(0x0f70 | 12); else if (after == 2) __builtin_amdgcn_s_waitcnt(0x0f70 | 8);
+        else if (after == 1) __builtin_amdgcn_s_waitcnt(0x0f70 | 4); else __builtin_amdgcn_s_waitcnt(0x0f70);
         bf16x8 kb[KS];
         #pragma unroll
-        for (int b = 0; b < KS; ++b) kb[b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(from + 32 * b));
+        for (int b = 0; b < KS; ++b) kb[b] = *reinterpret_cast<const bf16x8*>(stages[wave][buffer] + li * 256 + 16 * ((4 * b + g) ^ li));
+        __builtin_amdgcn_s_waitcnt(0xc07f);          // the operands are in registers: the stage is free for the copy issued next
         floatx4 norms = {0.0f, 0.0f, 0.0f, 0.0f};
         #pragma unroll
         for (int b = 0; b < KS; ++b) norms = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[b], kb[b], norms, 0, 0, 0);
@@ -402,7 +427,7 @@ __global__ void __launch_bounds__(256) index_interval_kernel(const uint16_t* __r
         }
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < RADIX_BINS; i += 256)
+    for (int i = threadIdx.x; i < RADIX_BINS; i += BRACKET_WAVES * 64)
         if (bins[i]) atomicAdd(&histogram[row * RADIX_BINS + i], bins[i]);
 }
 
@@ -620,7 +645,7 @@ void fast_index_bounds(Device& d, const FastIndexSpace& s, const void* q_index, 
                        size_t groups, float scale) {
     fill_words_kernel<<<unsigned(std::min<size_t>(checked_blocks(RADIX_LEVELS * batch * RADIX_BINS), 1024)), 256, 0, d.stream>>>(s.histogram, RADIX_LEVELS * batch * RADIX_BINS);
     index_margin_kernel<<<unsigned(batch), 256, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), weights, HEADS, 128, scale, s.margin);
-    index_interval_kernel<HEADS><<<dim3(unsigned(s.blocks), unsigned(batch)), 256, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys),
+    index_interval_kernel<HEADS><<<dim3(unsigned((groups + BRACKET_KEYS - 1) / BRACKET_KEYS), unsigned(batch)), BRACKET_WAVES * 64, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys),
                                                                                                    weights, visible, s.margin, groups, scale, s.lower, s.upper, s.histogram);
     SD_CHECK(hipGetLastError());
 }
