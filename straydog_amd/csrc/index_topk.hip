@@ -306,6 +306,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int RADIX_BINS = 2048, RADIX_LEVELS = 3, INTERVAL_KEYS = 1024;   // digits of 11, 11 and 10 bits; groups per workgroup
+constexpr int SCORE_WAVES = 4, SCORE_BATCH = 4;                             // the rescoring kernel: waves per workgroup, groups a wave takes at a time
 constexpr int BRACKET_WAVES = 8, BRACKET_KEYS = 2048, BRACKET_RING = 4;     // the bracket kernel: waves, groups per workgroup, stages per wave
 __device__ __forceinline__ uint32_t radix_digit(uint32_t key, int level) { return level == 0 ? key >> 21 : level == 1 ? (key >> 10) & 2047u : key & 1023u; }
 
@@ -546,41 +547,52 @@ __global__ void __launch_bounds__(256) candidate_list_kernel(const float* upper,
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 255) totals[row] = at;
 }
 
-// The canonical score of every listed group: a wave per group, a lane per head (the key row in scalar registers), then
-// the heads' terms added in head order.  The workgroup's eight waves share one copy of the row's queries in LDS,
-// transposed so that the lanes of a wave read neighbouring words; few registers, so many waves hide the loads' latency.
+// The canonical score of every listed group: a wave takes a few groups at a time, a lane per head (the key rows in scalar
+// registers), and then adds each group's 64 terms in head order -- lane c the terms of group c, read from LDS, so the
+// ordered sums run side by side.  The workgroup's waves share one copy of the row's queries in LDS, transposed so
+// that the lanes of a wave read neighbouring words; few registers, so many waves hide the loads' latency.
 template<int HEADS>
-__global__ void __launch_bounds__(512) candidate_score_kernel(const float* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
+__global__ void __launch_bounds__(SCORE_WAVES * 64) candidate_score_kernel(const float* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
                                                               size_t groups, float scale, const int32_t* __restrict__ list, const uint32_t* __restrict__ totals,
                                                               float* __restrict__ scores) {
-    constexpr int DIM = 128;
+    constexpr int DIM = 128, BATCH = SCORE_BATCH;
     const size_t row = blockIdx.y;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int head = min(lane, HEADS - 1);
     const uint32_t total = totals[row];
-    if (blockIdx.x * 8 >= total) return;
+    if (blockIdx.x * SCORE_WAVES * BATCH >= total) return;
     __shared__ float shared_q[DIM][HEADS + 1];
-    for (int i = threadIdx.x; i < HEADS * DIM; i += 512) shared_q[i % DIM][i / DIM] = q[row * HEADS * DIM + i];
+    __shared__ float terms[SCORE_WAVES][BATCH][HEADS + 1];
+    for (int i = threadIdx.x; i < HEADS * DIM; i += SCORE_WAVES * 64) shared_q[i % DIM][i / DIM] = q[row * HEADS * DIM + i];
     __syncthreads();
     const float weight = weights[row * HEADS + head];
-    for (uint32_t at = blockIdx.x * 8 + wave; at < total; at += gridDim.x * 8) {
-        const int32_t group = __builtin_amdgcn_readfirstlane(list[row * groups + at]);
-        typedef __attribute__((address_space(4))) const uint32_t* uniform_words;     // the row is the wave's: scalar loads
-        const uniform_words key = (uniform_words)(keys + (row * groups + size_t(group)) * DIM);
-        const float* mine = &shared_q[0][head];
-        asm volatile("" : "+v"(mine));               // read anew for every group: the values are not kept in registers
-        float dot = 0.0f;
-        #pragma unroll
-        for (int d = 0; d < DIM; d += 2) {
-            const uint32_t pair = key[d / 2];
-            dot = __builtin_fmaf(mine[d * (HEADS + 1)], __uint_as_float(pair << 16), dot);
-            dot = __builtin_fmaf(mine[(d + 1) * (HEADS + 1)], __uint_as_float(pair & 0xffff0000u), dot);
+    const uint32_t* row_keys = reinterpret_cast<const uint32_t*>(keys + row * groups * DIM);
+    for (uint32_t first = (blockIdx.x * SCORE_WAVES + wave) * BATCH; first < total; first += gridDim.x * SCORE_WAVES * BATCH) {
+        const int count = int(min(uint32_t(BATCH), total - first));
+        // A key row is 64 words: lane i fetches word i (one coalesced load), the words then go round by v_readlane.  The next
+        // group's row is on its way while this one is used.
+        uint32_t words = row_keys[size_t(list[row * groups + first]) * (DIM / 2) + lane];
+        for (int c = 0; c < count; ++c) {
+            const uint32_t current = words;
+            if (c + 1 < count) words = row_keys[size_t(list[row * groups + first + c + 1]) * (DIM / 2) + lane];
+            const float* mine = &shared_q[0][head];
+            asm volatile("" : "+v"(mine));               // read anew for every group: the values are not kept in registers
+            float dot = 0.0f;
+            #pragma unroll
+            for (int d = 0; d < DIM; d += 2) {
+                const uint32_t pair = __builtin_amdgcn_readlane(current, d / 2);
+                dot = __builtin_fmaf(mine[d * (HEADS + 1)], __uint_as_float(pair << 16), dot);
+                dot = __builtin_fmaf(mine[(d + 1) * (HEADS + 1)], __uint_as_float(pair & 0xffff0000u), dot);
+            }
+            if (lane < HEADS) terms[wave][c][lane] = rounded_product(fmaxf(dot, 0.0f), weight);
         }
-        const float term = rounded_product(fmaxf(dot, 0.0f), weight);
-        float sum = 0.0f;
-        #pragma unroll
-        for (int h = 0; h < HEADS; ++h) sum = rounded_sum(sum, __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(term), h)));
-        if (lane == 0) scores[row * groups + at] = rounded_product(sum, scale);
+        // the wave's own writes, read back by the wave: LDS keeps a wave's accesses in order
+        if (lane < count) {
+            float sum = 0.0f;
+            #pragma unroll
+            for (int h = 0; h < HEADS; ++h) sum = rounded_sum(sum, terms[wave][lane][h]);
+            scores[row * groups + first + lane] = rounded_product(sum, scale);
+        }
     }
 }
 
@@ -664,7 +676,7 @@ void fast_index_top_k(Device& d, const FastIndexSpace& s, const void* q_index, c
     radix_histogram_kernel<<<grid, 256, 0, d.stream>>>(s.lower, groups, batch, 2, rank, s.histogram);
     candidate_count_kernel<<<grid, 256, 0, d.stream>>>(s.upper, groups, batch, rank, s.histogram, s.counts);
     candidate_list_kernel<<<grid, 256, 0, d.stream>>>(s.upper, groups, batch, rank, s.histogram, s.counts, s.list, s.totals);
-    candidate_score_kernel<HEADS><<<dim3(128, unsigned(batch)), 512, 0, d.stream>>>(s.wide_q, static_cast<const uint16_t*>(keys), weights, groups, scale, s.list, s.totals,
+    candidate_score_kernel<HEADS><<<dim3(unsigned((k + k / 8 + 64 + SCORE_WAVES * SCORE_BATCH - 1) / (SCORE_WAVES * SCORE_BATCH)), unsigned(batch)), SCORE_WAVES * 64, 0, d.stream>>>(s.wide_q, static_cast<const uint16_t*>(keys), weights, groups, scale, s.list, s.totals,
                                                                                    s.scores);
     top_k_listed_kernel<<<unsigned(batch), TOPK_THREADS, 0, d.stream>>>(s.scores, s.list, s.totals, groups, k, indices);
     SD_CHECK(hipGetLastError());
