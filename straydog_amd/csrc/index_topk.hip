@@ -319,6 +319,16 @@ __device__ __forceinline__ float quad_sum(float x) {
     return a + b;
 }
 
+// One global->LDS load: every lane's 16 bytes from its own address to LDS at to + 16 * lane (to is the wave's), marked as
+// read once.  Written as instructions so that the compiler does not know of it: it would guard every later LDS read against
+// all such loads in flight, and the ring of stages below is there to keep several in flight; the waits are explicit.
+__device__ __forceinline__ void load_to_lds(const void* from, const void* to) {
+    typedef __attribute__((address_space(3))) const uint8_t* lds_bytes;
+    const uint32_t base = __builtin_amdgcn_readfirstlane(uint32_t(uintptr_t((lds_bytes)to)));
+    uint32_t keep;      // M0 names the LDS address; it is put back for whatever else the compiler keeps there
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt\n\ts_mov_b32 m0, %0" : "=&s"(keep) : "v"(from), "s"(base) : "memory");
+}
+
 // W of the margin for every row: sum_h |w_h| |q_h| * |scale| * 2^-14, rounded up a little.
 __global__ void __launch_bounds__(256) index_margin_kernel(const uint16_t* q, const float* weights, size_t heads, size_t dim, float scale, float* margin) {
     // four lanes per head, 8 values a load
@@ -375,18 +385,17 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
     const uint16_t* row_keys = keys + row * groups * DIM;
     __syncthreads();
     const size_t first = size_t(blockIdx.x) * BRACKET_KEYS, end = min(first + BRACKET_KEYS, groups);
-    typedef __attribute__((address_space(1))) const void* global_ptr;
-    typedef __attribute__((address_space(3))) void* lds_ptr;
     const auto copy_in = [&](int buffer, size_t tile) {
         #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int r = 4 * j + (lane >> 4), c = (lane & 15) ^ r;
             const uint16_t* from = row_keys + min(tile + r, groups - 1) * DIM + 8 * c;
-            __builtin_amdgcn_global_load_lds((global_ptr)from, (lds_ptr)(stages[wave][buffer] + 1024 * j), 16, 0, 2 /* nt: read once */);
+            load_to_lds(from, stages[wave][buffer] + 1024 * j);
         }
     };
     constexpr size_t stride = 16 * BRACKET_WAVES;
     size_t tile = first + 16 * wave;
+    __builtin_amdgcn_s_waitcnt(0x0f70);      // the queries and weights are in: the compiler's wait for them stays out of the loop
     #pragma unroll
     for (int ahead = 0; ahead < BRACKET_RING - 1; ++ahead)
         if (tile + ahead * stride < end) copy_in(ahead, tile + ahead * stride);

@@ -161,7 +161,7 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
             #pragma unroll
             for (int j = 0; j < (SLAB + 1023) / 1024; ++j)
                 if (1024 * j + 1024 <= SLAB || 16 * lane + 1024 * j < SLAB)
-                    __builtin_amdgcn_global_load_lds((global_ptr)(from + 1024 * j), (lds_ptr)(stage + part * SLAB + 1024 * j), 16, 0, 2 /* nt: streamed once */);
+                    load_to_lds<true>(from + 1024 * j, stage + part * SLAB + 1024 * j);
         }
     };
 
@@ -174,6 +174,7 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         in_page += STEP * WAVES;
         while (in_page >= int(args.page_tokens)) { in_page -= int(args.page_tokens); ++page_index; }
     };
+    settle_loads();
     #pragma unroll
     for (int ahead = 0; ahead < DEPTH; ++ahead) {
         if (token0 + ahead * STEP * WAVES < chunk_end) copy_in(stages + ahead * (2 * SLAB), table[min(page_index, last_page)], in_page);

@@ -62,6 +62,30 @@ __device__ __forceinline__ float row_sum(float x) {
     return a + b;
 }
 
+// LDS that global->LDS loads fill, read back and synchronised by hand.  The compiler guards every LDS read it can see
+// against *all* outstanding global->LDS loads (a full vector-memory wait), and a __syncthreads() is a fence that waits for
+// them too -- either would drain the ring of stages the loads are meant to keep full.  So the reads of such a stage are
+// written as instructions (the caller has waited for exactly the loads it needs), and the barrier of a loop over the ring
+// waits for the wave's LDS operations only.
+typedef __attribute__((address_space(3))) const uint8_t* lds_bytes;
+__device__ __forceinline__ uint32_t lds_address(const void* p) { return uint32_t(uintptr_t((lds_bytes)p)); }
+__device__ __forceinline__ void ring_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// One global->LDS load: every lane's 16 bytes from its own address to LDS at to + 16 * lane (to is the wave's).  Written as
+// instructions so that the compiler does not know of it -- the waits are the caller's (see above).  STREAM marks data
+// that is read once (non-temporal).
+template<bool STREAM>
+__device__ __forceinline__ void load_to_lds(const void* from, const void* to) {
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_address(to));
+    uint32_t keep;      // M0 names the LDS address; it is put back for whatever else the compiler keeps there
+    if (STREAM) asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt\n\ts_mov_b32 m0, %0" : "=&s"(keep) : "v"(from), "s"(base) : "memory");
+    else asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0" : "=&s"(keep) : "v"(from), "s"(base) : "memory");
+}
+// The loads the compiler knows of (queries and the like) are waited for once, before the first hidden load is issued:
+// its own wait for them would otherwise sit at their first use inside the loop and wait for the hidden loads as well.
+__device__ __forceinline__ void settle_loads() { __builtin_amdgcn_s_waitcnt(0x0f70); }
+typedef uint32_t words2 __attribute__((ext_vector_type(2)));
+typedef uint32_t words4 __attribute__((ext_vector_type(4)));
+
 __device__ __forceinline__ half2v as_half2(uint32_t bits) { return __builtin_bit_cast(half2v, bits); }
 
 // v_perm_b32: byte i of the result is byte sel[i] of the 8 bytes {high, low} (0-3 = low's bytes, 4-7 = high's, 0x0c = 0x00).

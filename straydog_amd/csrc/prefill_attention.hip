@@ -279,34 +279,42 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     }
 }
 
-// The second form of the kernel, for 128 columns: the workgroup converts every step's rows once into FP16 tiles in LDS (K
+// The second form of the kernel, for 128 columns.  The workgroup converts every step's rows once into FP16 tiles in LDS (K
 // as rows with a 16-byte pad, V transposed with an 8-byte pad: both read without bank conflicts as MFMA operands), so the
-// Q8_0 -> FP16 work is shared by the eight waves instead of being done by each.  While a step is computed from one pair
-// of tiles the next step's raw rows (already landed) are converted into the other pair; one barrier per step.
-// Columns of an output tile jj are 16 jj + (0..15), a lane holding 16 jj + 4 g + r.
+// Q8_0 -> FP16 work is shared by the eight waves instead of being done by each; while a step is computed from one pair of
+// tiles the next step's raw rows (already landed) are converted into the other pair; one barrier per step.  Columns of an
+// output tile jj are 16 jj + (0..15), a lane holding 16 jj + 4 g + r.  The causal triangle is evened out inside every
+// workgroup: it owns two runs of 4 x QT x 16 query rows: one from the end of the span (its rows see the most keys)
+// on waves 0-3 and its mirror image from the start of the span on waves 4-7, so every workgroup walks about the same number
+// of (row, key) pairs and every SIMD hosts one wave of each run -- when the short run's waves are done the long run's have
+// the SIMD to themselves.  A wave takes both 32-key halves of a step in turn, so nothing is merged at the end.
 template<int DIM, int QT, bool Q8>
-__global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) prefill_tiles_kernel(PrefillArgs args) {
+__global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) prefill_pairs_kernel(PrefillArgs args) {
     constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, BLOCKS = DIM / 32, TILES = DIM / 16;
     constexpr int SLAB = WALK * ROW, UNITS = (SLAB + 1023) / 1024;
     constexpr int WAVE_ROWS = QT * 16, GROUP_ROWS = GROUPS * WAVE_ROWS;
     constexpr int KP = 2 * DIM + 16, VP = 2 * WALK + 8, KT = WALK * KP, VT = DIM * VP;     // pitches and sizes of the FP16 tiles
     constexpr int RING = tiles_ring(2 * SLAB, 2 * (KT + VT));
     static_assert(RING >= 2 && WALK == 64 && TEAM == 8, "512 threads convert a step of 64 rows, one piece each");
-    const int tile = int(gridDim.x) - 1 - int(blockIdx.x), kvh = blockIdx.y, seq = blockIdx.z;
+    const int kvh = blockIdx.y, seq = blockIdx.z;
     const int thread = threadIdx.x, lane = thread & 63, wave = __builtin_amdgcn_readfirstlane(thread >> 6), li = lane & 15, g = lane >> 4;
     const int position = args.positions[seq];
     const int cached = min(position + int(args.span), args.max_context);
-    const int quarter = wave % GROUPS, half = wave / GROUPS;
+    const int quarter = wave % GROUPS, half = wave / GROUPS;       // half 0: the run from the end of the span, half 1: its mirror
+    const int runs = (int(args.rows) + GROUP_ROWS - 1) / GROUP_ROWS;
+    const int late = runs - 1 - int(blockIdx.x), early = int(blockIdx.x), tile = half == 0 ? late : early;
     const int row0 = tile * GROUP_ROWS + quarter * WAVE_ROWS;
-    const int group_last = min(int(args.rows), (tile + 1) * GROUP_ROWS) - 1;
-    const int keys = min(position + group_last / int(args.group) + 1, cached);
-    const bool idle = row0 >= int(args.rows);
+    const int group_last = min(int(args.rows), (late + 1) * GROUP_ROWS) - 1;
+    const int keys = min(position + group_last / int(args.group) + 1, cached);     // the walk is the late run's
+    const bool idle = row0 >= int(args.rows) || (half == 1 && early == late);      // an odd number of runs: the middle one is alone
     const int wave_first = position + row0 / int(args.group);
     const int wave_last = position + (min(int(args.rows), row0 + WAVE_ROWS) - 1) / int(args.group);
     const table_ptr table = (table_ptr)(args.page_table + size_t(seq) * args.table_stride);
     const size_t plane_bytes = size_t(args.page_tokens) * ROW;
-    extern __shared__ uint8_t stages[];                        // [RING][K slab | V slab] raw rows, then [2][K tile | V tile]
-    uint8_t* const tiles = stages + RING * (2 * SLAB);
+    // Two objects, so that the compiler knows the tiles apart from the stages the global->LDS loads fill (it would otherwise
+    // guard every access to the tiles against those loads).
+    __shared__ __attribute__((aligned(16))) uint8_t stages[RING * 2 * SLAB];     // [RING][K slab | V slab] raw rows
+    extern __shared__ __attribute__((aligned(16))) uint8_t tiles[];              // [2][K tile | V tile]
     constexpr int MOST = (2 * UNITS + TEAM - 1) / TEAM, LEAST = 2 * UNITS / TEAM;
     const bool most = wave < 2 * UNITS - LEAST * TEAM;
 
@@ -318,8 +326,7 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
         for (int k = 0; k < MOST; ++k) {
             const int unit = wave + TEAM * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS;
             if (unit < 2 * UNITS && 16 * lane + 1024 * j < SLAB)
-                __builtin_amdgcn_global_load_lds((global_ptr)(base + size_t(part ? args.kv_heads : 0) * plane_bytes + 1024 * j),
-                                                 (lds_ptr)(stage + part * SLAB + 1024 * j), 16, 0, 0);
+                load_to_lds<false>(base + size_t(part ? args.kv_heads : 0) * plane_bytes + 1024 * j, stage + part * SLAB + 1024 * j);
         }
     };
     // One step's raw rows into FP16 tiles; rows past the sequence's end become zeros (the page holds anything there).
@@ -333,9 +340,11 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
         if (Q8) {
             {   // K: 16 columns of one row
                 const int key = thread >> 3, piece = thread & 7;
-                const uint8_t* from = raw + key * ROW;
-                const uint2 a = *reinterpret_cast<const uint2*>(from + 16 * piece), b = *reinterpret_cast<const uint2*>(from + 16 * piece + 8);
-                uint32_t scale_bits = *reinterpret_cast<const uint16_t*>(from + DIM + 2 * (piece >> 1));
+                const uint32_t from = lds_address(raw + key * ROW);
+                words2 a, b;
+                uint32_t scale_bits;
+                asm volatile("ds_read_b64 %0, %3\n\tds_read_b64 %1, %3 offset:8\n\tds_read_u16 %2, %4\n\ts_waitcnt lgkmcnt(0)"
+                             : "=&v"(a), "=&v"(b), "=&v"(scale_bits) : "v"(from + 16 * piece), "v"(from + DIM + 2 * (piece >> 1)) : "memory");
                 if (key >= valid) scale_bits = 0;
                 const half2v scale = as_half2(scale_bits | (scale_bits << 16));
                 const uint32_t words[4] = {a.x, a.y, b.x, b.y};
@@ -352,14 +361,16 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
             }
             {   // V: 4 rows x 4 columns, transposed
                 const int rows4 = thread & 15, cols4 = thread >> 4;
-                const uint8_t* from = raw + SLAB + 4 * rows4 * ROW;
+                const uint32_t from = lds_address(raw + SLAB + 4 * rows4 * ROW);
                 uint32_t words[4], scales[4];
+                asm volatile("ds_read_b32 %0, %8\n\tds_read_b32 %1, %8 offset:%c10\n\tds_read_b32 %2, %8 offset:%c11\n\tds_read_b32 %3, %8 offset:%c12\n\t"
+                             "ds_read_u16 %4, %9\n\tds_read_u16 %5, %9 offset:%c10\n\tds_read_u16 %6, %9 offset:%c11\n\tds_read_u16 %7, %9 offset:%c12\n\t"
+                             "s_waitcnt lgkmcnt(0)"
+                             : "=&v"(words[0]), "=&v"(words[1]), "=&v"(words[2]), "=&v"(words[3]), "=&v"(scales[0]), "=&v"(scales[1]), "=&v"(scales[2]), "=&v"(scales[3])
+                             : "v"(from + 4 * cols4), "v"(from + DIM + 2 * (cols4 >> 3)), "n"(ROW), "n"(2 * ROW), "n"(3 * ROW) : "memory");
                 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    words[e] = *reinterpret_cast<const uint32_t*>(from + e * ROW + 4 * cols4);
-                    scales[e] = *reinterpret_cast<const uint16_t*>(from + e * ROW + DIM + 2 * (cols4 >> 3));
+                for (int e = 0; e < 4; ++e)
                     if (4 * rows4 + e >= valid) scales[e] = 0u;
-                }
                 const half2v first = as_half2(scales[0] | (scales[1] << 16)), second = as_half2(scales[2] | (scales[3] << 16));
                 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
@@ -376,21 +387,22 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
             #pragma unroll
             for (int k = 0; k < SLAB / 16 / (TEAM * 64); ++k) {
                 const int c = thread + TEAM * 64 * k, key = c / (ROW / 16), at = (c % (ROW / 16)) * 16;
-                uint4 piece = *reinterpret_cast<const uint4*>(raw + 16 * c);
-                if (key >= valid) piece = uint4{0u, 0u, 0u, 0u};
-                *reinterpret_cast<uint4*>(ktile + key * KP + at) = piece;
+                words4 piece;
+                asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(piece) : "v"(lds_address(raw + 16 * c)) : "memory");
+                if (key >= valid) piece = words4{0u, 0u, 0u, 0u};
+                *reinterpret_cast<words4*>(ktile + key * KP + at) = piece;
             }
             // V: 4 rows x 4 columns, transposed
             #pragma unroll
             for (int k = 0; k < (WALK / 4) * (DIM / 4) / (TEAM * 64); ++k) {
                 const int block = thread + TEAM * 64 * k, rows4 = block & 15, cols4 = block >> 4;
-                const uint8_t* from = raw + SLAB + 4 * rows4 * ROW + 8 * cols4;
-                uint2 words[4];
+                const uint32_t from = lds_address(raw + SLAB + 4 * rows4 * ROW + 8 * cols4);
+                words2 words[4];
+                asm volatile("ds_read_b64 %0, %4\n\tds_read_b64 %1, %4 offset:%c5\n\tds_read_b64 %2, %4 offset:%c6\n\tds_read_b64 %3, %4 offset:%c7\n\ts_waitcnt lgkmcnt(0)"
+                             : "=&v"(words[0]), "=&v"(words[1]), "=&v"(words[2]), "=&v"(words[3]) : "v"(from), "n"(ROW), "n"(2 * ROW), "n"(3 * ROW) : "memory");
                 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    words[e] = *reinterpret_cast<const uint2*>(from + e * ROW);
-                    if (4 * rows4 + e >= valid) words[e] = uint2{0u, 0u};
-                }
+                for (int e = 0; e < 4; ++e)
+                    if (4 * rows4 + e >= valid) words[e] = words2{0u, 0u};
                 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
@@ -403,9 +415,6 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
         }
     };
 
-    const int last_step = (keys - 1) / WALK * WALK;
-    #pragma unroll
-    for (int ahead = 0; ahead < RING; ++ahead) copy_in(ahead, min(ahead * WALK, last_step));
 
     half8 qf[QT][BLOCKS];
     #pragma unroll
@@ -437,9 +446,13 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
         for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
+    settle_loads();
+    const int last_step = (keys - 1) / WALK * WALK;
+    #pragma unroll
+    for (int ahead = 0; ahead < RING; ++ahead) copy_in(ahead, min(ahead * WALK, last_step));
     // the first step's tiles
     if (most) wait_loads<MOST * (RING - 1)>(); else wait_loads<LEAST * (RING - 1)>();
-    __syncthreads();
+    ring_barrier();
     convert(0, 0, 0);
 
     // The two waves of a SIMD walk in different orders: the first half's converts its piece of the next step and then computes,
@@ -449,13 +462,15 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     for (int walk0 = 0, step = 0; walk0 < keys; walk0 += WALK, ++step) {
         // the next step's raw rows have landed when only the later steps' copies are outstanding
         if (most) wait_loads<MOST * (RING - 2)>(); else wait_loads<LEAST * (RING - 2)>();
-        __syncthreads();      // everybody's pieces have; this step's tiles are written; the other tiles and the raw stage of this step are free
+        ring_barrier();       // everybody's pieces have; this step's tiles are written; the other tiles and the raw stage of this step are free
         copy_in(step % RING, min(walk0 + RING * WALK, last_step));
         if (decltype(convert_first)::value && walk0 + WALK < keys) convert((step + 1) % RING, (step + 1) & 1, walk0 + WALK);
-        const int token0 = walk0 + half * STEP;
+        #pragma unroll 1
+        for (int part = 0; part < WALK / STEP; ++part) {
+        const int token0 = walk0 + part * STEP;
         if (!(idle || token0 > wave_last || token0 >= keys)) {
-        const uint8_t* ktile = tiles + (step & 1) * (KT + VT) + half * STEP * KP;
-        const uint8_t* vtile = tiles + (step & 1) * (KT + VT) + KT + half * STEP * 2;
+        const uint8_t* ktile = tiles + (step & 1) * (KT + VT) + part * STEP * KP;
+        const uint8_t* vtile = tiles + (step & 1) * (KT + VT) + KT + part * STEP * 2;
         floatx4 s[QT][2];
         #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -533,44 +548,23 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
             for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[qt], acc[qt][jj], 0, 0, 0);
         }
         }
+        }
         if (!decltype(convert_first)::value && walk0 + WALK < keys) convert((step + 1) % RING, (step + 1) & 1, walk0 + WALK);
     }
     };
     if (half == 0) walk(std::true_type{}); else walk(std::false_type{});
 
-    // The pair of waves that shares rows merges through LDS (the stages and tiles are done with).
-    #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) l[qt] = row_sum(l[qt]);
-    __syncthreads();
-    float* mine = reinterpret_cast<float*>(stages) + size_t(quarter) * (QT * (TILES * 4 + 2)) * 64 + lane;
-    if (half == 1) {
-        #pragma unroll
-        for (int qt = 0; qt < QT; ++qt) {
-            float* at = mine + size_t(qt) * (TILES * 4 + 2) * 64;
-            at[0] = m[qt]; at[64] = l[qt];
-            #pragma unroll
-            for (int jj = 0; jj < TILES; ++jj)
-                #pragma unroll
-                for (int r = 0; r < 4; ++r) at[(2 + 4 * jj + r) * 64] = acc[qt][jj][r];
-        }
-    }
-    __syncthreads();
-    if (half == 1) return;
+    if (idle) return;
     #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
         const int row = row0 + qt * 16 + li;
-        const float* at = mine + size_t(qt) * (TILES * 4 + 2) * 64;
-        const float other = at[0], top = fmaxf(m[qt], other);
-        const float keep = __builtin_amdgcn_exp2f((m[qt] - top) * args.scale_log2), add = __builtin_amdgcn_exp2f((other - top) * args.scale_log2);
-        const float inverse = 1.0f / (l[qt] * keep + at[64] * add);
+        const float inverse = 1.0f / row_sum(l[qt]);
         if (row >= int(args.rows)) continue;
         const int span_row = row / int(args.group), head = kvh * int(args.group) + row % int(args.group);
         const size_t first = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM + 4 * g;
         #pragma unroll
         for (int jj = 0; jj < TILES; ++jj) {
-            floatx4 value;
-            #pragma unroll
-            for (int r = 0; r < 4; ++r) value[r] = (acc[qt][jj][r] * keep + at[(2 + 4 * jj + r) * 64] * add) * inverse;
+            const floatx4 value = acc[qt][jj] * inverse;
             if (args.out_f16) {
                 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
                 *reinterpret_cast<half4*>(static_cast<_Float16*>(args.out) + first + 16 * jj) = half4{(_Float16)value[0], (_Float16)value[1], (_Float16)value[2], (_Float16)value[3]};
@@ -580,19 +574,16 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
 }
 
 template<int DIM, int QT, bool Q8>
-void launch_tiles(Device& d, const PrefillArgs& args, unsigned seqs) {
-    constexpr size_t merge = size_t(GROUPS) * QT * (DIM / 16 * 4 + 2) * 64 * 4;
-    constexpr size_t stage = size_t(2) * WALK * (Q8 ? DIM + DIM / 16 : 2 * DIM), pair = size_t(2) * (WALK * (2 * DIM + 16) + DIM * (2 * WALK + 8));
-    constexpr size_t ring = tiles_ring(int(stage), int(pair)) * stage + pair;
-    constexpr size_t shared = ring > merge ? ring : merge;
-    static_assert(shared <= 160 * 1024, "the stages, the tiles and the merge area share the compute unit's LDS");
+void launch_pairs(Device& d, const PrefillArgs& args, unsigned seqs) {
+    constexpr size_t stage = size_t(2) * WALK * (Q8 ? DIM + DIM / 16 : 2 * DIM), shared = size_t(2) * (WALK * (2 * DIM + 16) + DIM * (2 * WALK + 8));
+    static_assert(tiles_ring(int(stage), int(shared)) * stage + shared <= 160 * 1024, "the stages and the tiles share the compute unit's LDS");
     static bool raised = false;
     if (!raised && shared > 64 * 1024) {
-        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_tiles_kernel<DIM, QT, Q8>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
+        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_pairs_kernel<DIM, QT, Q8>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
         raised = true;
     }
-    const unsigned tiles = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
-    prefill_tiles_kernel<DIM, QT, Q8><<<dim3(tiles, args.kv_heads, seqs), TEAM * 64, shared, d.stream>>>(args);
+    const unsigned runs = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
+    prefill_pairs_kernel<DIM, QT, Q8><<<dim3((runs + 1) / 2, args.kv_heads, seqs), TEAM * 64, shared, d.stream>>>(args);
 }
 
 template<int DIM, int QT, bool Q8, int OCC>
@@ -629,7 +620,7 @@ void prefill_attention(Device& d, const sdx_kv_pool* pool, const int32_t* page_t
     args.out = out; args.out_f16 = out_f16;
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     KernelTimer timer(d);
-    if (pool->dim == 128) { if (q8) launch_tiles<128, 4, true>(d, args, unsigned(seqs)); else launch_tiles<128, 4, false>(d, args, unsigned(seqs)); }
+    if (pool->dim == 128) { if (q8) launch_pairs<128, 2, true>(d, args, unsigned(seqs)); else launch_pairs<128, 2, false>(d, args, unsigned(seqs)); }
     else { if (q8) launch<256, 1, true, 2>(d, args, unsigned(seqs)); else launch<256, 1, false, 2>(d, args, unsigned(seqs)); }
 }
 
