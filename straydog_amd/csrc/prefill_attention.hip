@@ -318,8 +318,7 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     constexpr int MOST = (2 * UNITS + TEAM - 1) / TEAM, LEAST = 2 * UNITS / TEAM;
     const bool most = wave < 2 * UNITS - LEAST * TEAM;
 
-    const auto copy_in = [&](int buffer, int token0) {
-        const int page = table[token0 / int(args.page_tokens)];
+    const auto copy_in = [&](int buffer, int token0, int page) {
         const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(token0 % int(args.page_tokens)) * ROW + 16 * lane;
         uint8_t* stage = stages + buffer * (2 * SLAB);
         #pragma unroll
@@ -338,20 +337,27 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
         uint8_t* vtile = ktile + KT;
         const int valid = cached - walk0;                      // rows of the step the cache holds
         if (Q8) {
-            {   // K: 16 columns of one row
-                const int key = thread >> 3, piece = thread & 7;
-                const uint32_t from = lds_address(raw + key * ROW);
-                words2 a, b;
-                uint32_t scale_bits;
-                asm volatile("ds_read_b64 %0, %3\n\tds_read_b64 %1, %3 offset:8\n\tds_read_u16 %2, %4\n\ts_waitcnt lgkmcnt(0)"
-                             : "=&v"(a), "=&v"(b), "=&v"(scale_bits) : "v"(from + 16 * piece), "v"(from + DIM + 2 * (piece >> 1)) : "memory");
+            // K: 16 columns of one row; V: 4 rows x 4 columns, transposed.  All of the thread's raw reads are asked for at once.
+            const int key = thread >> 3, piece = thread & 7, rows4 = thread & 15, cols4 = thread >> 4;
+            const uint32_t from_k = lds_address(raw + key * ROW), from_v = lds_address(raw + SLAB + 4 * rows4 * ROW);
+            words2 a, b;
+            uint32_t scale_bits, words[4], scales[4];
+            asm volatile("ds_read_b64 %0, %11\n\tds_read_b64 %1, %11 offset:8\n\tds_read_u16 %2, %12\n\t"
+                         "ds_read_b32 %3, %13\n\tds_read_b32 %4, %13 offset:%c15\n\tds_read_b32 %5, %13 offset:%c16\n\tds_read_b32 %6, %13 offset:%c17\n\t"
+                         "ds_read_u16 %7, %14\n\tds_read_u16 %8, %14 offset:%c15\n\tds_read_u16 %9, %14 offset:%c16\n\tds_read_u16 %10, %14 offset:%c17\n\t"
+                         "s_waitcnt lgkmcnt(0)"
+                         : "=&v"(a), "=&v"(b), "=&v"(scale_bits), "=&v"(words[0]), "=&v"(words[1]), "=&v"(words[2]), "=&v"(words[3]),
+                           "=&v"(scales[0]), "=&v"(scales[1]), "=&v"(scales[2]), "=&v"(scales[3])
+                         : "v"(from_k + 16 * piece), "v"(from_k + DIM + 2 * (piece >> 1)), "v"(from_v + 4 * cols4), "v"(from_v + DIM + 2 * (cols4 >> 3)),
+                           "n"(ROW), "n"(2 * ROW), "n"(3 * ROW) : "memory");
+            {
                 if (key >= valid) scale_bits = 0;
                 const half2v scale = as_half2(scale_bits | (scale_bits << 16));
-                const uint32_t words[4] = {a.x, a.y, b.x, b.y};
+                const uint32_t pieces[4] = {a.x, a.y, b.x, b.y};
                 half2v out[8];
                 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    const uint32_t bits = words[w] ^ 0x80808080u;
+                    const uint32_t bits = pieces[w] ^ 0x80808080u;
                     out[2 * w] = magic_to_half2(byte_perm(0x64646464u, bits, 0x04010400u), scale);
                     out[2 * w + 1] = magic_to_half2(byte_perm(0x64646464u, bits, 0x04030402u), scale);
                 }
@@ -359,15 +365,7 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
                 to[0] = half8{out[0].x, out[0].y, out[1].x, out[1].y, out[2].x, out[2].y, out[3].x, out[3].y};
                 to[1] = half8{out[4].x, out[4].y, out[5].x, out[5].y, out[6].x, out[6].y, out[7].x, out[7].y};
             }
-            {   // V: 4 rows x 4 columns, transposed
-                const int rows4 = thread & 15, cols4 = thread >> 4;
-                const uint32_t from = lds_address(raw + SLAB + 4 * rows4 * ROW);
-                uint32_t words[4], scales[4];
-                asm volatile("ds_read_b32 %0, %8\n\tds_read_b32 %1, %8 offset:%c10\n\tds_read_b32 %2, %8 offset:%c11\n\tds_read_b32 %3, %8 offset:%c12\n\t"
-                             "ds_read_u16 %4, %9\n\tds_read_u16 %5, %9 offset:%c10\n\tds_read_u16 %6, %9 offset:%c11\n\tds_read_u16 %7, %9 offset:%c12\n\t"
-                             "s_waitcnt lgkmcnt(0)"
-                             : "=&v"(words[0]), "=&v"(words[1]), "=&v"(words[2]), "=&v"(words[3]), "=&v"(scales[0]), "=&v"(scales[1]), "=&v"(scales[2]), "=&v"(scales[3])
-                             : "v"(from + 4 * cols4), "v"(from + DIM + 2 * (cols4 >> 3)), "n"(ROW), "n"(2 * ROW), "n"(3 * ROW) : "memory");
+            {
                 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     if (4 * rows4 + e >= valid) scales[e] = 0u;
@@ -449,7 +447,8 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     settle_loads();
     const int last_step = (keys - 1) / WALK * WALK;
     #pragma unroll
-    for (int ahead = 0; ahead < RING; ++ahead) copy_in(ahead, min(ahead * WALK, last_step));
+    for (int ahead = 0; ahead < RING; ++ahead) copy_in(ahead, min(ahead * WALK, last_step), table[min(ahead * WALK, last_step) / int(args.page_tokens)]);
+    int page_ahead = table[min(RING * WALK, last_step) / int(args.page_tokens)];      // of the step the walk's first copy brings in
     // the first step's tiles
     if (most) wait_loads<MOST * (RING - 1)>(); else wait_loads<LEAST * (RING - 1)>();
     ring_barrier();
@@ -463,7 +462,8 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
         // the next step's raw rows have landed when only the later steps' copies are outstanding
         if (most) wait_loads<MOST * (RING - 2)>(); else wait_loads<LEAST * (RING - 2)>();
         ring_barrier();       // everybody's pieces have; this step's tiles are written; the other tiles and the raw stage of this step are free
-        copy_in(step % RING, min(walk0 + RING * WALK, last_step));
+        copy_in(step % RING, min(walk0 + RING * WALK, last_step), page_ahead);
+        page_ahead = table[min(walk0 + (RING + 1) * WALK, last_step) / int(args.page_tokens)];     // a scalar load, back long before the next step
         if (decltype(convert_first)::value && walk0 + WALK < keys) convert((step + 1) % RING, (step + 1) & 1, walk0 + WALK);
         #pragma unroll 1
         for (int part = 0; part < WALK / STEP; ++part) {
@@ -471,17 +471,28 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
         if (!(idle || token0 > wave_last || token0 >= keys)) {
         const uint8_t* ktile = tiles + (step & 1) * (KT + VT) + part * STEP * KP;
         const uint8_t* vtile = tiles + (step & 1) * (KT + VT) + KT + part * STEP * 2;
+        // all of the step's operands are asked for at once: one LDS round trip for K, and V's is hidden behind the softmax
+        half8 ka[2][BLOCKS];
+        #pragma unroll
+        for (int t = 0; t < 2; ++t)
+            #pragma unroll
+            for (int b = 0; b < BLOCKS; ++b) ka[t][b] = *reinterpret_cast<const half8*>(ktile + (16 * t + li) * KP + 64 * b + 16 * g);
+        uint2 va[TILES][2];
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj) {
+            const uint8_t* from = vtile + (16 * jj + li) * VP + 8 * g;
+            va[jj][0] = *reinterpret_cast<const uint2*>(from); va[jj][1] = *reinterpret_cast<const uint2*>(from + 32);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         floatx4 s[QT][2];
         #pragma unroll
         for (int t = 0; t < 2; ++t) {
             #pragma unroll
             for (int qt = 0; qt < QT; ++qt) s[qt][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
             #pragma unroll
-            for (int b = 0; b < BLOCKS; ++b) {
-                const half8 ka = *reinterpret_cast<const half8*>(ktile + (16 * t + li) * KP + 64 * b + 16 * g);
+            for (int b = 0; b < BLOCKS; ++b)
                 #pragma unroll
-                for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qf[qt][b], s[qt][t], 0, 0, 0);
-            }
+                for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][b], qf[qt][b], s[qt][t], 0, 0, 0);
         }
         if (token0 + STEP - 1 > wave_first) {          // wave-uniform: some token of the step is past some row's position
             asm volatile("; the step crosses the diagonal" ::: "memory");      // keeps the block a branch: it is rare
@@ -540,12 +551,9 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
         }
         #pragma unroll
         for (int jj = 0; jj < TILES; ++jj) {
-            const uint8_t* from = vtile + (16 * jj + li) * VP + 8 * g;
-            const uint2 near = *reinterpret_cast<const uint2*>(from), far = *reinterpret_cast<const uint2*>(from + 32);
-            const uint4 both = {near.x, near.y, far.x, far.y};
-            const half8 va = __builtin_bit_cast(half8, both);
+            const uint4 both = {va[jj][0].x, va[jj][0].y, va[jj][1].x, va[jj][1].y};
             #pragma unroll
-            for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[qt], acc[qt][jj], 0, 0, 0);
+            for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, both), pb[qt], acc[qt][jj], 0, 0, 0);
         }
         }
         }
