@@ -183,6 +183,24 @@ def test_prefill_in_chunks_equals_prefill_at_once(gpu, oracle):
     gpu.release(buffer); gpu.release(tb)
 
 
+def test_many_short_sequences(gpu, oracle):
+    # more sequences than a wave has lanes: the device's numbering of the work runs over several groups of 64 sequences;
+    # some sequences hold a single token, some exactly a page
+    rng = np.random.default_rng(404)
+    dim, row_bytes, page_tokens, heads, kv_heads = 128, 136, 32, 8, 2
+    lengths = [int(n) for n in rng.integers(1, 200, size=150)]
+    lengths[3], lengths[64], lengths[149] = 1, 32, 64
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, lengths, kv_heads, dim, page_tokens, row_bytes)
+    seqs = len(lengths)
+    q = rng.standard_normal((seqs, 1, heads, dim)).astype(np.float16).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    positions = [n - 1 for n in lengths]
+    got = _run(gpu, pool, table, tb, positions, q, 1, heads, scale, True, False)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array(positions, np.int32), q, scale)
+    close_enough(got, want, "150 sequences")
+    gpu.release(buffer); gpu.release(tb)
+
+
 def test_zero_queries_give_the_mean_of_the_values(gpu, oracle):
     rng = np.random.default_rng(5)
     heads, kv_heads, dim, row_bytes, page_tokens = 8, 2, 128, 136, 32
@@ -205,6 +223,8 @@ def test_refusals(gpu):
         table = gpu.upload(np.zeros(4, np.int32))
         q = gpu.buffer(8 * 128 * 4)
         gpu.paged_attention(pool, table.base(), 1, table.base(), 32, q.base(), 0, 1, 1, 8, 0.1, q.base(), 0, small)
+    with pytest.raises(StraydogError, match="invalid Straydog paged attention shape"):      # the scale must be positive
+        gpu.paged_attention(pool, table.base(), 1, table.base(), 32, q.base(), 0, 1, 1, 8, 0.0, q.base(), 0, small)
     bad = type(pool)(buffer.pointer, 2, 33, 1, 128, 136)
     with pytest.raises(StraydogError, match="invalid Straydog K/V pool"):
         gpu.kv_write(bad, small.base(), 1, small.base(), small.base(), small.base(), False, 1, 1)
