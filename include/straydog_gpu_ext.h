@@ -52,6 +52,30 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
                         const int32_t* positions, uint64_t max_context, const void* q, int q_f16, uint64_t seqs, uint64_t span,
                         uint64_t heads, float scale, void* out, int out_f16, void* scratch, uint64_t scratch_bytes);
 
+/* Qwen's block indexer (the reference runs it inside sd_qsa_sequence / sd_decode_span / sd_prefill_span; here its stages are
+ * callable on their own).  All buffers are device memory of the handle.
+ *
+ * sdx_qsa_normalize = qsa_normalize (gpu/sparse_attention.hpp:8-23, rope :2-6): rows x heads vectors of `width` (128 or 256)
+ * floats, `stride` floats apart, RMS-normalised with the weight `norm` and turned for position + row; target [rows*heads][width]
+ * (may be the source when stride == width). */
+int sdx_qsa_normalize(void* handle, const float* source, const float* norm, uint64_t rows, uint64_t heads, uint64_t width, uint64_t stride,
+                      uint64_t position, float* target);
+/* sdx_qsa_pool = qsa_pool + qsa_save_history (gpu/sparse_attention.hpp:87-108, 132-139; call site :497-501): the blocks of four
+ * positions completed by rows base .. base + steps are pooled from `incoming` [steps][128] and the ring `history` [16][128] into
+ * blocks[column * pool + block]; the ring then takes the span's last four rows. */
+int sdx_qsa_pool(void* handle, const float* incoming, float* history, const float* norm, uint64_t pool, uint64_t base, uint64_t steps,
+                 float* blocks);
+/* sdx_qsa_index = qsa_index_exact (gpu/sparse_attention.hpp:403-414: qsa_block_scores :141-155 / qsa_block_scores_tiled
+ * :247-298, then qsa_select :172-241 / qsa_select_rows :314-400) for rows at positions base .. base + steps - 1.
+ * queries: [steps][query_stride], the 4 x 128 normalised index queries at each row's start; blocks: [128][pool] pooled keys;
+ * scores: steps x pool floats of scratch (holds the scores of rows with more than 512 complete blocks afterwards);
+ * indices: [steps][selected] positions as floats, counts: [steps] as floats -- the two tails of the reference's packed
+ * buffer (gpu/sparse_attention.hpp:177-178, 240).  dynamic_base, if not null, is a device-resident position that replaces
+ * `base` (the decode and verification passes' replayable form, gpu/qsa_decode.hpp:36-38, 125-127; up to 8 rows).
+ * The same bits as the reference's kernels: scores by fused chains in column order, ties to the earliest blocks. */
+int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, const float* blocks, uint64_t pool, uint64_t base,
+                  const uint32_t* dynamic_base, uint64_t steps, uint64_t selected, float* scores, float* indices, float* counts);
+
 /* Top-k indexed sparse attention over BF16 latent K/V for a batch of sequences (one decode row each):
  * stage 1+2 = sd_op_index_scores + sd_op_top_k per sequence (gpu/ops.hpp:1700-1739, 1766-1941) with each sequence's own
  * keys [batch][groups][dim] BF16; q_index [batch][heads][dim] BF16; weights [batch][heads] FP32; visible [batch].

@@ -73,6 +73,9 @@ _latent = _sig("sdo_latent_attention", None, _vp, _vp, _sz, _vp, _sz, _vp, ctype
                ctypes.c_float, _sz, _vp, _vp, _vp, ctypes.c_int)
 _compress = _sig("sdo_compress", None, _vp, _vp, _sz, _sz, _sz, _vp)
 _qsa_select = _sig("sdo_qsa_select", _sz, _vp, _sz, _sz, _vp)
+_qsa_normalize = _sig("sdo_qsa_normalize", None, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _vp)
+_qsa_pool = _sig("sdo_qsa_pool", None, _vp, _vp, _vp, _sz, _sz, _sz, _vp)
+_qsa_block_scores = _sig("sdo_qsa_block_scores", None, _vp, _sz, _vp, _sz, _sz, _sz, _vp)
 _fill_n = _sig("sdo_fill_normal", None, ctypes.c_uint64, _vp, _sz)
 _fill_u = _sig("sdo_fill_uniform", None, ctypes.c_uint64, _vp, _sz, ctypes.c_float, ctypes.c_float)
 max_threads = _sig("sdo_max_threads", ctypes.c_int)
@@ -279,6 +282,31 @@ def qsa_select(scores, position, keep_blocks=512):
     out = np.zeros(keep_blocks * 4 + 4 + max(0, position + 1), dtype=np.float32)
     count = _qsa_select(_ptr(scores), position, keep_blocks, _ptr(out))
     return out[:count].copy()
+
+
+def qsa_normalize(source, norm, rows, heads, width, stride, position):
+    """source: flat floats, row r head h at (r * heads + h) * stride; returns [rows * heads, width]."""
+    source, norm = _f32(source).reshape(-1), _f32(norm)
+    out = np.zeros((rows * heads, width), dtype=np.float32)
+    _qsa_normalize(_ptr(source), _ptr(norm), rows, heads, width, stride, position, _ptr(out))
+    return out
+
+
+def qsa_pool(incoming, history, norm, pool, base, blocks):
+    """Updates `blocks` ([128, pool]) and `history` ([16, 128]) in place for rows base .. base + len(incoming)."""
+    incoming, norm = _f32(incoming), _f32(norm)
+    assert history.dtype == np.float32 and blocks.dtype == np.float32 and history.flags.c_contiguous and blocks.flags.c_contiguous
+    _qsa_pool(_ptr(incoming), _ptr(history), _ptr(norm), pool, base, incoming.shape[0], _ptr(blocks))
+
+
+def qsa_block_scores(queries, blocks, base, scores=None):
+    """queries: [steps, stride >= 512]; blocks: [128, pool].  Returns [steps, pool] (zeros where the reference writes nothing)."""
+    queries, blocks = _f32(queries), _f32(blocks)
+    steps, pool = queries.shape[0], blocks.shape[1]
+    if scores is None:
+        scores = np.zeros((steps, pool), dtype=np.float32)
+    _qsa_block_scores(_ptr(queries), queries.shape[1], _ptr(blocks), pool, base, steps, _ptr(scores))
+    return scores
 
 
 def fill_normal(seed, count):

@@ -653,6 +653,92 @@ size_t sdo_qsa_select(const float* scores, size_t position, size_t keep_blocks, 
     return out;
 }
 
+/* ------------------------------------------------------------------ Qwen block indexer: norm, rope, pool, scores */
+
+/* sparse_attention.hpp:2-6: the first 64 columns turn in pairs (c, c + 32) by position / 1e7^(c % 32 / 32). */
+static float qsa_rope(float own, float partner, size_t column, size_t position) {
+    if (column >= 64) return own;
+    const float angle = (float)position / powf(1e7f, (float)(column % 32) / 32.0f);
+    return own * cosf(angle) + (column < 32 ? -partner : partner) * sinf(angle);
+}
+
+/* The sum of squares as the kernels' halving tree forms it (sparse_attention.hpp:14-17, 101-104): sums[c] += sums[c + offset]. */
+static float qsa_tree_sum(float* sums, size_t width) {
+    for (size_t offset = width / 2; offset; offset /= 2)
+        for (size_t c = 0; c < offset; ++c) sums[c] += sums[c + offset];
+    return sums[0];
+}
+
+/* sparse_attention.hpp:8-23 (qsa_normalize): rows x heads vectors of `width` (128 or 256) at `stride` floats apart, RMS-normalised
+ * with the weight `norm`, the first 64 columns turned for position + row. */
+void sdo_qsa_normalize(const float* source, const float* norm, size_t rows, size_t heads, size_t width, size_t stride,
+                       size_t position, float* target) {
+    float values[256], sums[256];
+    for (size_t head = 0; head < rows * heads; ++head) {
+        const size_t token = head / heads;
+        for (size_t c = 0; c < width; ++c) { const float x = source[head * stride + c]; values[c] = x * norm[c]; sums[c] = x * x; }
+        const float denominator = sqrtf(qsa_tree_sum(sums, width) / (float)width + 1e-6f);
+        for (size_t c = 0; c < width; ++c) {
+            const float own = values[c] / denominator;
+            const float partner = c < 64 ? values[(c + 32) % 64] / denominator : 0.0f;
+            target[head * width + c] = qsa_rope(own, partner, c, position + token);
+        }
+    }
+}
+
+/* sparse_attention.hpp:87-108 (qsa_pool) then :132-139 (qsa_save_history): every block of four positions completed by rows
+ * base .. base + steps is the mean of its four index-key inputs (earlier ones from the ring of sixteen), normalised and turned
+ * for the block's first position, stored column-major blocks[c * pool + block]; the ring then takes the span's last four rows. */
+void sdo_qsa_pool(const float* incoming, float* history, const float* norm, size_t pool, size_t base, size_t steps, float* blocks) {
+    float values[128], sums[128];
+    for (size_t block = base / 4; block < (base + steps) / 4; ++block) {
+        const size_t begin = block * 4;
+        for (size_t c = 0; c < 128; ++c) {
+            float x = 0.0f;
+            for (size_t tap = 0; tap < 4; ++tap) {
+                const size_t pos = begin + tap;
+                x += pos < base ? history[(pos % 16) * 128 + c] : incoming[(pos - base) * 128 + c];
+            }
+            x /= 4.0f;
+            values[c] = x * norm[c]; sums[c] = x * x;
+        }
+        const float denominator = sqrtf(qsa_tree_sum(sums, 128) / 128.0f + 1e-6f);
+        for (size_t c = 0; c < 128; ++c) {
+            const float own = values[c] / denominator;
+            const float partner = c < 64 ? values[(c + 32) % 64] / denominator : 0.0f;
+            blocks[c * pool + block] = qsa_rope(own, partner, c, begin);
+        }
+    }
+    const size_t kept = steps < 4 ? steps : 4;
+    for (size_t i = 0; i < kept * 128; ++i) {
+        const size_t token = steps - kept + i / 128;
+        history[((base + token) % 16) * 128 + i % 128] = incoming[token * 128 + i % 128];
+    }
+}
+
+/* sparse_attention.hpp:141-155 (qsa_block_scores; the same bits as the tiled form, :243-246): for every row with more than
+ * 512 complete blocks, score(block) = sum over the four heads, in order, of the positive part of the head's dot product, each
+ * dot product a chain of fused multiply-adds over the 128 columns in order.  Other entries of `scores` are left alone. */
+void sdo_qsa_block_scores(const float* queries, size_t query_stride, const float* blocks, size_t pool, size_t base, size_t steps,
+                          float* scores) {
+    #pragma omp parallel for schedule(dynamic, 1)
+    for (size_t token = 0; token < steps; ++token) {
+        const size_t complete = (base + token + 1) / 4;
+        if (complete <= 512) continue;
+        for (size_t block = 0; block < complete; ++block) {
+            float dot[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (size_t c = 0; c < 128; ++c) {
+                const float key = blocks[c * pool + block];
+                for (size_t h = 0; h < 4; ++h) dot[h] = fmaf(key, queries[token * query_stride + h * 128 + c], dot[h]);
+            }
+            float total = fmaxf(dot[0], 0.0f) + fmaxf(dot[1], 0.0f);
+            total += fmaxf(dot[2], 0.0f);
+            total += fmaxf(dot[3], 0.0f);
+            scores[token * pool + block] = total;
+        }
+    }
+}
+
 /* ------------------------------------------------------------------ seeded inputs */
 
 static inline uint64_t xorshift64(uint64_t* s) { *s ^= *s << 13; *s ^= *s >> 7; *s ^= *s << 17; return *s; }

@@ -16,7 +16,10 @@
  * sdo_op_attention (float64 numpy softmax + the derived bound of attention_gpu.rs:28-31),
  * sdo_index_scores (float64 closed form + scalar-vs-vector bit equality), sdo_top_k (brute-force
  * stable sort + the adversarial generator of fused_gpu.rs:370-379), sdo_latent_attention (float64
- * closed form + special cases), sdo_compress (float64 closed form), sdo_qsa_select (brute force).
+ * closed form + special cases), sdo_compress (float64 closed form), sdo_qsa_select (brute force),
+ * sdo_qsa_block_scores (exact rational arithmetic rounded once per fused step, in pure Python, + float64 closed form),
+ * sdo_qsa_normalize / sdo_qsa_pool (float64 closed form; rotation invariants: pair norms kept, position 0 and columns
+ * from 64 on unturned; the ring's contents).
  * PARITY UNPINNED: none of the above; bit-level agreement with the reference's device summation
  * order inside its flash kernels is not claimed anywhere (tolerance-based, see the tests).
  */
@@ -122,6 +125,16 @@ void sdo_compress(const float* kv, const float* gate, size_t groups, size_t rati
  * scores: [pool] non-negative block scores of one token at `position`; writes up to `selected` (2052) indices
  * as floats and returns the count. */
 size_t sdo_qsa_select(const float* scores, size_t position, size_t keep_blocks, float* indices);
+
+/* ---- Qwen block indexer inputs and scores: gpu/sparse_attention.hpp:2-23 (qsa_rope, qsa_normalize), :87-108 + :132-139
+ * (qsa_pool, qsa_save_history), :141-155 (qsa_block_scores).  blocks: [128][pool] column-major pooled keys; history: the ring
+ * of the last sixteen index-key inputs [16][128], updated by sdo_qsa_pool; scores: [steps][pool], written for rows with more
+ * than 512 complete blocks, blocks below the row's complete count. */
+void sdo_qsa_normalize(const float* source, const float* norm, size_t rows, size_t heads, size_t width, size_t stride,
+                       size_t position, float* target);
+void sdo_qsa_pool(const float* incoming, float* history, const float* norm, size_t pool, size_t base, size_t steps, float* blocks);
+void sdo_qsa_block_scores(const float* queries, size_t query_stride, const float* blocks, size_t pool, size_t base, size_t steps,
+                          float* scores);
 
 /* ---- Seeded inputs: xorshift64 (crates/straydog-engine/tests/fused_gpu.rs:39-53) -> Box-Muller
  *      (gpu/tests/qsa_interval_test.cpp:12-18). */

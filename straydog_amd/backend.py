@@ -172,6 +172,16 @@ class Backend:
         self.check(self.lib.sdx_index_score_bounds(self.handle, q_index, keys, weights, visible, batch, groups, heads, dim, scale, lower,
                                                    upper))
 
+    def qsa_normalize(self, source, norm, rows, heads, width, stride, position, target):
+        self.check(self.lib.sdx_qsa_normalize(self.handle, source, norm, rows, heads, width, stride, position, target))
+
+    def qsa_pool(self, incoming, history, norm, pool, base, steps, blocks):
+        self.check(self.lib.sdx_qsa_pool(self.handle, incoming, history, norm, pool, base, steps, blocks))
+
+    def qsa_index(self, queries, query_stride, blocks, pool, base, steps, selected, scores, indices, counts, dynamic_base=None):
+        self.check(self.lib.sdx_qsa_index(self.handle, queries, query_stride, blocks, pool, base, dynamic_base, steps, selected, scores,
+                                          indices, counts))
+
     def latent_attention(self, q, latents, selected, batch, groups, k, heads, kdim, vdim, scale, out):
         self.check(self.lib.sdx_latent_attention(self.handle, q, latents, selected, batch, groups, k, heads, kdim, vdim, scale, out))
 

@@ -1,0 +1,198 @@
+"""GPU parity of Qwen's block indexer (sdx_qsa_normalize, sdx_qsa_pool, sdx_qsa_index) against the CPU oracle.
+
+The cases follow the reference's own regression of this stage, gpu/tests/qsa_interval_test.cpp:58-118: gaussian keys and
+queries, topic-correlated ones, exact ties at the 512th best score, zero queries, small magnitudes; every row must select
+the blocks, in the order and with the ties, of the exact rule, and the block scores must be the same bits.
+"""
+import numpy as np
+import pytest
+
+from gpu_util import backend
+
+pytestmark = pytest.mark.gpu
+
+CANARY = np.float32(-77.5)
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    with backend(4 << 30) as handle:
+        yield handle
+
+
+def _read(gpu, buffer, dtype, count):
+    return gpu.read_buffer(buffer, 0, dtype, count)
+
+
+def _case(oracle, mode, base, steps, pool, stride, seed):
+    """Pooled keys [128, pool] and index queries [steps, stride] in the manner of qsa_interval_test.cpp:71-93."""
+    rng = np.random.default_rng(seed)
+    complete_all = (base + steps) // 4
+    topics = rng.standard_normal((64, 128)).astype(np.float32)
+    strength = {"g": 0.0, "t": 1.0, "d": 2.5, "z": 0.0, "s": 0.0}[mode]
+    scale = 1.0e-4 if mode == "s" else 1.0
+    weight_k = (0.4 + 1.2 * rng.random(128)).astype(np.float32)
+    weight_q = (0.4 + 1.2 * rng.random(128)).astype(np.float32)
+    x = rng.standard_normal((complete_all, 128)).astype(np.float32) + strength * 0.6 * topics[(np.arange(complete_all) // 48 * 2654435761 % 64)]
+    x = x / np.sqrt((x * x).mean(axis=1, keepdims=True) + 1e-6) * weight_k * scale
+    blocks = np.zeros((128, pool), dtype=np.float32)
+    blocks[:, :complete_all] = x.T
+    blocks[:, complete_all:] = np.nan                      # never read: a block past the last row's complete count
+    queries = np.zeros((steps, stride), dtype=np.float32)
+    for r in range(steps):
+        for h in range(4):
+            z = ((base + r) // 700 + h * 5) * 40503 % 64
+            v = rng.standard_normal(128).astype(np.float32) + strength * 0.6 * topics[z]
+            queries[r, h * 128:(h + 1) * 128] = v / np.sqrt((v * v).mean() + 1e-6) * weight_q * scale
+    queries[:, 512:] = 1.0e9                                # the rest of a row's stride belongs to others
+    if mode == "z":
+        queries[::2, :512] = 0.0
+    if mode == "d" and complete_all > 600:
+        # blocks around the 512th best of the last row given the same key: exact ties where the cut falls
+        scores = oracle.qsa_block_scores(queries[-1:], np.nan_to_num(blocks), base + steps - 1)[0][:complete_all]
+        order = sorted(range(complete_all), key=lambda b: (-float(scores[b]), b))
+        for k in range(6):
+            blocks[:, order[512 + 2 * k + (k & 1)]] = blocks[:, order[505 + 3 * k]]
+    return queries, blocks
+
+
+def _run_index(gpu, queries, blocks, base, selected, dynamic=False):
+    steps, stride = queries.shape
+    pool = blocks.shape[1]
+    qb, kb = gpu.upload(queries), gpu.upload(blocks)
+    scores = gpu.upload(np.full(steps * pool, CANARY, dtype=np.float32))
+    indices = gpu.upload(np.full(steps * selected + 8, CANARY, dtype=np.float32))
+    counts = gpu.upload(np.full(steps, CANARY, dtype=np.float32))
+    position = gpu.upload(np.array([base], dtype=np.uint32)) if dynamic else None
+    gpu.qsa_index(qb.base(), stride, kb.base(), pool, 0 if dynamic else base, steps, selected, scores.base(), indices.base(), counts.base(),
+                  dynamic_base=position.base() if dynamic else None)
+    out = (_read(gpu, scores, np.float32, steps * pool).reshape(steps, pool), _read(gpu, indices, np.float32, steps * selected + 8),
+           _read(gpu, counts, np.float32, steps))
+    for b in (qb, kb, scores, indices, counts) + ((position,) if dynamic else ()):
+        gpu.release(b)
+    return out
+
+
+def _check(oracle, queries, blocks, base, selected, got):
+    scores, indices, counts = got
+    steps, pool = queries.shape[0], blocks.shape[1]
+    want_scores = oracle.qsa_block_scores(queries, np.nan_to_num(blocks), base)
+    assert np.all(indices[steps * selected:] == CANARY), "nothing is written past the last row's selection"
+    for r in range(steps):
+        position = base + r
+        complete = (position + 1) // 4
+        if complete > 512:
+            assert np.array_equal(scores[r, :complete].view(np.uint32), want_scores[r, :complete].view(np.uint32)), f"row {r}: score bits"
+            want = oracle.qsa_select(want_scores[r], position)
+        else:
+            want = np.arange(position + 1, dtype=np.float32)
+        assert np.all(scores[r, max(complete, 0) if complete > 512 else 0:] == CANARY), f"row {r}: scores outside the row's blocks are not touched"
+        assert counts[r] == float(len(want)), f"row {r}: count {counts[r]} != {len(want)}"
+        row = indices[r * selected:(r + 1) * selected]
+        assert np.array_equal(row[:len(want)], want), f"row {r}: selection"
+        assert np.all(row[len(want):] == CANARY), f"row {r}: entries past the count are not touched"
+
+
+@pytest.mark.parametrize("mode,base,steps,context,stride", [
+    ("g", 30000, 1, 32768, 512),        # a decode row
+    ("t", 2044, 8, 4096, 512),          # a verification span across the 512-block line: rows that keep everything, rows that select
+    ("g", 9000, 5, 16384, 640),         # a verification span (a wider row stride)
+    ("t", 9001, 100, 16384, 512),       # a prefill chunk: the tiled form, rows of different complete counts
+    ("d", 20000, 37, 32768, 512),       # exact ties where the cut falls
+    ("z", 5000, 12, 8192, 512),         # zero queries: every score ties at zero, the earliest 512 blocks win
+    ("s", 7000, 3, 8192, 512),          # small magnitudes
+    ("g", 262100, 3, 262144, 512),      # the longest context: rows re-read per pass
+    ("g", 70000, 2, 131072, 512),       # 16 values a thread
+    ("g", 100, 20, 1024, 512),          # a short context: every row keeps every causal position
+])
+def test_block_scores_and_selection(gpu, oracle, mode, base, steps, context, stride):
+    pool = context // 4 + 1
+    selected = min(base + steps, 2052)
+    queries, blocks = _case(oracle, mode, base, steps, pool, stride, seed=base + steps)
+    _check(oracle, queries, blocks, base, selected, _run_index(gpu, queries, blocks, base, selected))
+
+
+def test_device_resident_position(gpu, oracle):
+    # the replayable form: the position is read on the device, the launch shape does not depend on it
+    base, steps, context = 12345, 4, 32768
+    pool = context // 4 + 1
+    queries, blocks = _case(oracle, "g", base, steps, pool, 512, seed=5)
+    blocks = np.nan_to_num(blocks)
+    _check(oracle, queries, blocks, base, 2052, _run_index(gpu, queries, blocks, base, 2052, dynamic=True))
+
+
+def _rope_slack(want, position):
+    """How far a turned value may move when the float32 angle lands one float32 step away (the power function's last bit)."""
+    slack = np.zeros(want.shape, dtype=np.float64)
+    c = np.arange(32)
+    angle = (np.float32(position) / np.power(np.float32(1e7), (c / 32.0).astype(np.float32))).astype(np.float32)
+    slack[..., :32] = slack[..., 32:64] = 2.0 * np.spacing(angle).astype(np.float64) * np.hypot(want[..., :32], want[..., 32:64])
+    return slack
+
+
+def _close(got, want, slack):
+    return np.all(np.abs(got.astype(np.float64) - want) <= 2e-5 + 2e-5 * np.abs(want) + slack)
+
+
+@pytest.mark.parametrize("width,heads,stride", [(256, 24, 512), (256, 2, 256), (128, 4, 128)])
+def test_normalize(gpu, oracle, width, heads, stride):
+    rng = np.random.default_rng(width + heads)
+    rows, position = 5, 123457
+    source = (rng.standard_normal(rows * heads * stride) * 3).astype(np.float32)
+    norm = (0.4 + 1.2 * rng.random(width)).astype(np.float32)
+    want = oracle.qsa_normalize(source, norm, rows, heads, width, stride, position)
+    sb, nb = gpu.upload(source), gpu.upload(norm)
+    target = sb if stride == width else gpu.buffer(rows * heads * width * 4)       # in place where the rows are dense, as the reference does
+    gpu.qsa_normalize(sb.base(), nb.base(), rows, heads, width, stride, position, target.base())
+    got = _read(gpu, target, np.float32, rows * heads * width).reshape(rows * heads, width)
+    for r in range(rows):
+        span = slice(r * heads, (r + 1) * heads)
+        assert _close(got[span], want[span].astype(np.float64), _rope_slack(want[span], position + r))
+    assert np.array_equal(got[:, 64:], want[:, 64:]), "columns that are not turned: the same bits (tree-ordered sum, exact division)"
+    for b in {sb, nb, target}:
+        gpu.release(b)
+
+
+def test_pool_over_spans(gpu, oracle):
+    # spans that start and end inside blocks; the ring of sixteen carries the inputs of a block across calls
+    rng = np.random.default_rng(8)
+    pool, base = 600, 2000
+    norm = (0.4 + 1.2 * rng.random(128)).astype(np.float32)
+    want_blocks, want_history = np.zeros((128, pool), np.float32), rng.standard_normal((16, 128)).astype(np.float32)
+    bb, hb, nb = gpu.upload(want_blocks), gpu.upload(want_history), gpu.upload(norm)
+    for steps in (1, 2, 5, 3, 1, 1, 1, 7, 4, 16, 9, 2, 45, 256):
+        incoming = rng.standard_normal((steps, 128)).astype(np.float32)
+        ib = gpu.upload(incoming)
+        gpu.qsa_pool(ib.base(), hb.base(), nb.base(), pool, base, steps, bb.base())
+        oracle.qsa_pool(incoming, want_history, norm, pool, base, want_blocks)
+        gpu.release(ib)
+        base += steps
+    assert np.array_equal(_read(gpu, hb, np.float32, 16 * 128).reshape(16, 128), want_history)
+    got = _read(gpu, bb, np.float32, 128 * pool).reshape(128, pool)
+    for block in range(2000 // 4, base // 4):
+        assert _close(got[:, block], want_blocks[:, block].astype(np.float64), _rope_slack(want_blocks[:, block], block * 4)), f"block {block}"
+    untouched = np.ones(pool, bool)
+    untouched[2000 // 4:base // 4] = False
+    assert np.all(got[:, untouched] == 0.0)
+    for b in (bb, hb, nb):
+        gpu.release(b)
+
+
+def test_refusals(gpu):
+    from straydog_amd.backend import StraydogError as GpuError
+    pool, steps = 1025, 2
+    q, k = gpu.buffer(steps * 512 * 4), gpu.buffer(128 * pool * 4)
+    scores, indices, counts = gpu.buffer(steps * pool * 4), gpu.buffer(steps * 2052 * 4), gpu.buffer(steps * 4)
+    args = dict(queries=q.base(), query_stride=512, blocks=k.base(), pool=pool, base=3000, steps=steps, selected=2052, scores=scores.base(),
+                indices=indices.base(), counts=counts.base())
+    gpu.qsa_index(**args)
+    for change, text in ((dict(base=4099), "fit the pool"), (dict(selected=2051), "selected"), (dict(query_stride=511), "stride"),
+                         (dict(pool=70000), "65537"), (dict(steps=0), "steps"), (dict(counts=counts.at(4)), "outside")):
+        with pytest.raises(GpuError, match=text):
+            gpu.qsa_index(**{**args, **change})
+    with pytest.raises(GpuError, match="width"):
+        gpu.qsa_normalize(q.base(), k.base(), 1, 4, 64, 64, 0, q.base())
+    with pytest.raises(GpuError, match="fit the pool"):
+        gpu.qsa_pool(q.base(), k.base(), k.base(), 10, 100, 4, k.base())
+    for b in (q, k, scores, indices, counts):
+        gpu.release(b)
