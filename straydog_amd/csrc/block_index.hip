@@ -13,8 +13,8 @@
 //
 // Wave64 forms: one lane per block and all of a span's rows per lane while the span is short (decode, verification: the keys
 // are read once from HBM, 512 bytes a block); a 32-row x 256-block tile per workgroup with operands staged through LDS for a
-// prefill chunk (FP32 FMA-bound); a 1024-thread workgroup per row for the selection, the row's scores held in registers, four
-// 8-bit radix passes over per-wave LDS histograms (the first, where nearly all values share a digit, counted by ballots), and
+// prefill chunk (FP32 FMA-bound); a 1024-thread workgroup per row for the selection, the row's scores read once and held in LDS (and registers,
+// beyond 32768 blocks), four 8-bit radix passes over per-wave LDS histograms (the first, where nearly all values share a digit, counted by ballots), and
 // one ordered pass whose slots come from 64-wide ballots and a scan over (run, wave) counts.
 #include "device.hpp"
 #include "../../include/straydog_gpu_ext.h"
@@ -242,73 +242,38 @@ __device__ __forceinline__ uint32_t group_scan(uint32_t value, uint32_t* wave_su
     return before + inclusive - value;
 }
 
-// body(i) for every run of 1024 blocks the row has: unrolled over the registers that hold the row, or a plain loop.
-template<int RUN, bool HELD, class Body>
-__device__ __forceinline__ void each_run(unsigned runs, Body body) {
-    if constexpr (HELD) {
-        #pragma unroll
-        for (int i = 0; i < RUN; ++i)
-            if (unsigned(i) < runs) body(i);
-    } else {
-        for (unsigned i = 0; i < runs; ++i) body(int(i));
-    }
-}
+// What the selection keeps between its steps, in LDS.
+struct SelectShared {
+    uint32_t bins[SELECT_WAVES * 256];      // a histogram per wave; at other times the (run, wave) counts or the sample's histogram
+    uint32_t wave_sums[SELECT_WAVES], threshold, remaining;
+};
 
-// One workgroup per row of up to RUN * 1024 complete blocks; block i * 1024 + t is thread t's value i.  HELD: the row is read
-// once into registers (a prefill chunk's many rows); otherwise every pass reads it again, from L2 (the longest rows, whose
-// 64 values a thread would not fit beside the rest at sixteen waves).
-template<int RUN, bool HELD>
-__global__ void __launch_bounds__(SELECT_THREADS) select_kernel(const float* __restrict__ scores, size_t pool, size_t base, const uint32_t* dynamic,
-                                                                size_t selected, float* __restrict__ indices, float* __restrict__ counts) {
-    __shared__ uint32_t bins[SELECT_WAVES * 256];            // a histogram per wave; later the (run, wave) counts
-    __shared__ uint32_t wave_sums[SELECT_WAVES], threshold, remaining;
-    if (dynamic) base = *dynamic;
-    const size_t token = blockIdx.x, position = base + token, complete = (position + 1) / 4;
+// The choice itself over values a thread holds as (run i, thread t) in ascending block order: each_run(body) calls
+// body(i, bits, valid) for the thread's value of every run, block_of(i) names its block.  Values below `guess` are known
+// not to be among the 512 highest; should fewer than 512 be left, the guess is dropped.  Four 8-bit radix passes find the 512th
+// highest value (a per-wave histogram; the first pass, where nearly all values share the digit, adds once per digit by a
+// ballot), then one ordered pass gives every kept value its slot: ballots rank the lanes of a wave, a scan over the (run, wave)
+// counts ranks the waves, and the values equal to the 512th are taken from the earliest blocks on.
+template<class Each, class BlockOf>
+__device__ __forceinline__ void choose_blocks(SelectShared& sh, Each each_run, BlockOf block_of, unsigned runs, unsigned most_runs, uint32_t guess,
+                                              float* out) {
     const unsigned t = threadIdx.x, lane = t % 64, wave = t / 64;
-    float* out = indices + token * selected;
-    if (position + 1 > 4 * pool || complete > size_t(RUN) * SELECT_THREADS) {   // a position this key pool (or this variant) cannot hold
-        if (t == 0) counts[token] = 0.0f;
-        return;
-    }
-    if (complete <= KEEP) {
-        for (size_t i = t; i <= position; i += SELECT_THREADS) out[i] = float(i);
-        if (t == 0) counts[token] = float(position + 1);
-        return;
-    }
-    const float* row = scores + token * pool;
-    const unsigned runs = unsigned((complete + SELECT_THREADS - 1) / SELECT_THREADS);
-    uint32_t values[HELD ? RUN : 1];
-    if constexpr (HELD) {
-        #pragma unroll
-        for (int i = 0; i < RUN; ++i) {
-            const size_t block = size_t(i) * SELECT_THREADS + t;
-            values[i] = block < complete ? __float_as_uint(row[block]) : 0u;
-        }
-    }
-    const auto value_of = [&](int i, bool valid) -> uint32_t {
-        if constexpr (HELD) return values[i];
-        else return valid ? __float_as_uint(row[size_t(i) * SELECT_THREADS + t]) : 0u;
-    };
-    // The 512th highest value, eight bits a pass.
     uint32_t prefix = 0, wanted = KEEP, mask = 0;
-    uint32_t* own = bins + wave * 256;
+    uint32_t* own = sh.bins + wave * 256;
     #pragma unroll 1
     for (int shift = 24; shift >= 0; shift -= 8) {
-        for (unsigned i = t; i < SELECT_WAVES * 256; i += SELECT_THREADS) bins[i] = 0;
+        for (unsigned i = t; i < SELECT_WAVES * 256; i += SELECT_THREADS) sh.bins[i] = 0;
         __syncthreads();
-        each_run<RUN, HELD>(runs, [&](int i) {
-            const bool valid = size_t(i) * SELECT_THREADS + t < complete;
-            const uint32_t bits = value_of(i, valid);
-            const bool live = valid && (bits & mask) == prefix;
+        each_run([&](unsigned, uint32_t bits, bool valid) {
+            const bool live = valid && bits >= guess && (bits & mask) == prefix;
             const uint32_t digit = (bits >> shift) & 255u;
             if (shift == 24) {
-                // nearly every score shares its top byte: the lanes of a digit add once, by a ballot
                 uint64_t todo = __ballot(live);
                 while (todo) {
                     const int leader = __ffsll(static_cast<long long>(todo)) - 1;
-                    const uint32_t d = __shfl(digit, leader);
+                    const uint32_t d = uint32_t(__builtin_amdgcn_readlane(int(digit), leader));
                     const uint64_t same = __ballot(live && digit == d);
-                    if (int(lane) == leader) own[d] += uint32_t(__popcll(same));
+                    if (int(lane) == leader) atomicAdd(own + d, uint32_t(__popcll(same)));
                     todo &= ~same;
                 }
             } else if (live) {
@@ -320,19 +285,22 @@ __global__ void __launch_bounds__(SELECT_THREADS) select_kernel(const float* __r
         const uint32_t bucket = 255u - (t & 255u);
         uint32_t count = 0, every;
         if (t < 256)
-            for (int w = 0; w < SELECT_WAVES; ++w) count += bins[w * 256 + bucket];
-        const uint32_t above = group_scan(count, wave_sums, every);
-        if (t < 256 && above < wanted && above + count >= wanted) { threshold = prefix | (bucket << shift); remaining = wanted - above; }
+            for (int w = 0; w < SELECT_WAVES; ++w) count += sh.bins[w * 256 + bucket];
+        const uint32_t above = group_scan(count, sh.wave_sums, every);
+        if (shift == 24 && every < KEEP) {                   // the guess was too high: once more, over every value
+            guess = 0;
+            shift += 8;
+            continue;
+        }
+        if (t < 256 && above < wanted && above + count >= wanted) { sh.threshold = prefix | (bucket << shift); sh.remaining = wanted - above; }
         __syncthreads();
-        prefix = threshold; wanted = remaining;
+        prefix = sh.threshold; wanted = sh.remaining;
         mask |= 255u << shift;
     }
     // Kept: every value above `prefix` and the first `wanted` equal to it, in block order.
-    uint32_t* greater = bins;
-    uint32_t* equal = bins + RUN * SELECT_WAVES;
-    each_run<RUN, HELD>(runs, [&](int i) {
-        const bool valid = size_t(i) * SELECT_THREADS + t < complete;
-        const uint32_t bits = value_of(i, valid);
+    uint32_t* greater = sh.bins;
+    uint32_t* equal = sh.bins + most_runs * SELECT_WAVES;
+    each_run([&](unsigned i, uint32_t bits, bool valid) {
         const uint64_t above = __ballot(valid && bits > prefix), same = __ballot(valid && bits == prefix);
         if (lane == 0) { greater[i * SELECT_WAVES + wave] = uint32_t(__popcll(above)); equal[i * SELECT_WAVES + wave] = uint32_t(__popcll(same)); }
     });
@@ -340,27 +308,174 @@ __global__ void __launch_bounds__(SELECT_THREADS) select_kernel(const float* __r
     const unsigned entries = runs * SELECT_WAVES;           // at most 1024: one per thread
     const uint32_t g = t < entries ? greater[t] : 0u, e = t < entries ? equal[t] : 0u;
     uint32_t every;
-    const uint32_t greater_before = group_scan(g, wave_sums, every);
-    const uint32_t equal_before = group_scan(e, wave_sums, every);
+    const uint32_t greater_before = group_scan(g, sh.wave_sums, every);
+    const uint32_t equal_before = group_scan(e, sh.wave_sums, every);
     if (t < entries) { greater[t] = greater_before; equal[t] = equal_before; }
     __syncthreads();
     const uint64_t below = (uint64_t(1) << lane) - 1;
-    each_run<RUN, HELD>(runs, [&](int i) {
-        const size_t block = size_t(i) * SELECT_THREADS + t;
-        const bool valid = block < complete;
-        const uint32_t bits = value_of(i, valid);
+    each_run([&](unsigned i, uint32_t bits, bool valid) {
         const bool above = valid && bits > prefix, same = valid && bits == prefix;
         const uint64_t above_mask = __ballot(above), same_mask = __ballot(same);
         if (!above && !same) return;
         const uint32_t equal_seen = equal[i * SELECT_WAVES + wave] + uint32_t(__popcll(same_mask & below));
         if (same && equal_seen >= wanted) return;
         const size_t at = size_t(greater[i * SELECT_WAVES + wave] + uint32_t(__popcll(above_mask & below)) + min(equal_seen, wanted)) * 4;
+        const size_t block = block_of(i);
         #pragma unroll
         for (size_t tap = 0; tap < 4; ++tap) out[at + tap] = float(block * 4 + tap);
     });
+}
+
+// One workgroup per row; block i * 1024 + t is thread t's value i.  The row is read once and stays on the chip: its first
+// LDS_RUNS runs of 1024 values in LDS (as many as the row has: the launch sizes the array), the runs beyond, for the longest
+// rows, in REGS registers a thread.
+//
+// A long row is thinned first, since every sweep over 64 values a thread costs about as much as all the rest: the R-th
+// highest of a sample of four values a thread (spread over the runs in LDS; R: one and a half times the sample's share of 512, and
+// a margin), found to 24 bits by two 4096-bin histograms, is a guess below the 512th highest value of the row.  Two light sweeps count and list, in block order, the values that reach the guess; when they are
+// at least 512 and fit the list, the choice runs over the list alone, otherwise over the whole row.
+constexpr int LDS_RUNS = 31, LIST_RUNS = 2, LIST = LIST_RUNS * SELECT_THREADS;
+template<int REGS>
+__global__ void __launch_bounds__(SELECT_THREADS) select_kernel(const float* __restrict__ scores, size_t pool, size_t base, const uint32_t* dynamic,
+                                                                size_t selected, unsigned held_runs, float* __restrict__ indices,
+                                                                float* __restrict__ counts) {
+    extern __shared__ uint32_t held[];                       // [run][1024]
+    __shared__ SelectShared sh;
+    __shared__ uint2 list[LIST];                             // (score bits, block) of the values that reach the guess
+    if (dynamic) base = *dynamic;
+    const size_t token = blockIdx.x, position = base + token, complete = (position + 1) / 4;
+    const unsigned t = threadIdx.x, lane = t % 64, wave = t / 64;
+    float* out = indices + token * selected;
+    if (position + 1 > 4 * pool || complete > size_t(held_runs + REGS) * SELECT_THREADS) {   // a position this key pool (or this launch) cannot hold
+        if (t == 0) counts[token] = 0.0f;
+        return;
+    }
+    if (complete <= KEEP) {
+        for (size_t i = t; i <= position; i += SELECT_THREADS) out[i] = float(i);
+        if (t == 0) counts[token] = float(position + 1);
+        return;
+    }
+    const float* row = scores + token * pool;
+    const unsigned runs = unsigned((complete + SELECT_THREADS - 1) / SELECT_THREADS), lds_runs = min(runs, held_runs);
+    uint32_t values[REGS ? REGS : 1];
+    #pragma unroll 8
+    for (unsigned i = 0; i < lds_runs; ++i) {
+        const size_t block = size_t(i) * SELECT_THREADS + t;
+        held[i * SELECT_THREADS + t] = block < complete ? __float_as_uint(row[block]) : 0u;
+    }
+    if constexpr (REGS > 0) {
+        #pragma unroll
+        for (int j = 0; j < REGS; ++j) {
+            const size_t block = size_t(LDS_RUNS + j) * SELECT_THREADS + t;
+            values[j] = block < complete ? __float_as_uint(row[block]) : 0u;
+        }
+    }
+    // body(run, bits, valid) for every run of the row, in run order (every thread reads back only what it wrote)
+    const auto each_run = [&](auto body) {
+        unsigned i = 0;
+        for (; i + 4 <= lds_runs; i += 4) {                  // four reads in flight at a time
+            uint32_t four[4];
+            #pragma unroll
+            for (unsigned j = 0; j < 4; ++j) four[j] = held[(i + j) * SELECT_THREADS + t];
+            #pragma unroll
+            for (unsigned j = 0; j < 4; ++j) body(i + j, four[j], size_t(i + j) * SELECT_THREADS + t < complete);
+        }
+        for (; i < lds_runs; ++i) body(i, held[i * SELECT_THREADS + t], size_t(i) * SELECT_THREADS + t < complete);
+        if constexpr (REGS > 0) {
+            #pragma unroll
+            for (int j = 0; j < REGS; ++j)
+                if (unsigned(LDS_RUNS + j) < runs) body(unsigned(LDS_RUNS + j), values[j], size_t(LDS_RUNS + j) * SELECT_THREADS + t < complete);
+        }
+    };
+    uint32_t guess = 0;
+    bool listed = false;
+    uint32_t list_count = 0;
+    if (runs >= 8) {
+        constexpr unsigned SAMPLES = 4;                      // values a thread gives to the sample
+        uint32_t sample[SAMPLES];
+        bool sampled[SAMPLES];
+        #pragma unroll
+        for (unsigned k = 0; k < SAMPLES; ++k) {
+            const unsigned run = (t + 7 * k) % lds_runs;
+            sampled[k] = size_t(run) * SELECT_THREADS + t < complete;
+            sample[k] = held[run * SELECT_THREADS + t];
+        }
+        uint32_t rank = uint32_t(3 * size_t(KEEP) * SAMPLES * SELECT_THREADS / (2 * complete)) + 16;
+        #pragma unroll 1
+        for (int shift = 20; shift >= 8; shift -= 12) {     // the sample's rank-th highest value to 24 bits: 12 bits a level
+            for (unsigned i = t; i < SELECT_WAVES * 256; i += SELECT_THREADS) sh.bins[i] = 0;
+            if (t == 0) { sh.threshold = guess; sh.remaining = rank; }
+            __syncthreads();
+            #pragma unroll
+            for (unsigned k = 0; k < SAMPLES; ++k)
+                if (sampled[k] && (shift == 20 || (sample[k] >> 20) == (guess >> 20))) atomicAdd(sh.bins + ((sample[k] >> shift) & 4095u), 1u);
+            __syncthreads();
+            uint32_t four[4], sum = 0, every;
+            #pragma unroll
+            for (unsigned j = 0; j < 4; ++j) { four[j] = sh.bins[4095 - 4 * t - j]; sum += four[j]; }
+            uint32_t above = group_scan(sum, sh.wave_sums, every);
+            #pragma unroll
+            for (unsigned j = 0; j < 4; ++j) {
+                if (above < rank && above + four[j] >= rank) { sh.threshold = guess | ((4095 - 4 * t - j) << shift); sh.remaining = rank - above; }
+                above += four[j];
+            }
+            __syncthreads();
+            guess = sh.threshold; rank = sh.remaining;
+            __syncthreads();
+        }
+        // how many values reach the guess, per (run, wave) in block order
+        uint32_t* reach = sh.bins;
+        each_run([&](unsigned i, uint32_t bits, bool valid) {
+            const uint64_t reaching = __ballot(valid && bits >= guess);
+            if (lane == 0) reach[i * SELECT_WAVES + wave] = uint32_t(__popcll(reaching));
+        });
+        __syncthreads();
+        const unsigned entries = runs * SELECT_WAVES;
+        const uint32_t mine = t < entries ? reach[t] : 0u;
+        const uint32_t before = group_scan(mine, sh.wave_sums, list_count);
+        if (t < entries) reach[t] = before;
+        __syncthreads();
+        if (list_count < KEEP) guess = 0;                    // too high a guess: the whole row, every value
+        listed = list_count >= KEEP && list_count <= LIST;
+        if (listed) {
+            const uint64_t below = (uint64_t(1) << lane) - 1;
+            each_run([&](unsigned i, uint32_t bits, bool valid) {
+                const bool reaches = valid && bits >= guess;
+                const uint64_t reaching = __ballot(reaches);
+                if (reaches) list[reach[i * SELECT_WAVES + wave] + uint32_t(__popcll(reaching & below))] = make_uint2(bits, i * SELECT_THREADS + t);
+            });
+        }
+        __syncthreads();
+    }
+    if (listed) {
+        uint2 mine[LIST_RUNS];
+        #pragma unroll
+        for (int j = 0; j < LIST_RUNS; ++j) mine[j] = unsigned(j) * SELECT_THREADS + t < list_count ? list[j * SELECT_THREADS + t] : make_uint2(0u, 0u);
+        const unsigned list_runs = (list_count + SELECT_THREADS - 1) / SELECT_THREADS;
+        choose_blocks(sh, [&](auto body) {
+            #pragma unroll
+            for (int j = 0; j < LIST_RUNS; ++j)
+                if (unsigned(j) < list_runs) body(unsigned(j), mine[j].x, unsigned(j) * SELECT_THREADS + t < list_count);
+        }, [&](unsigned j) { return size_t(j == 0 ? mine[0].y : mine[1].y); }, list_runs, LIST_RUNS, 0u, out);
+    } else {
+        choose_blocks(sh, each_run, [&](unsigned i) { return size_t(i) * SELECT_THREADS + t; }, runs, LDS_RUNS + REGS, guess, out);
+    }
     const size_t head = size_t(KEEP) * 4;
     for (size_t i = t; complete * 4 + i <= position; i += SELECT_THREADS) out[head + i] = float(complete * 4 + i);
     if (t == 0) counts[token] = float(head + position + 1 - complete * 4);
+}
+
+template<int REGS>
+void launch_select(Device& d, const float* scores, size_t pool, size_t base, const uint32_t* dynamic, size_t selected, size_t most, unsigned rows,
+                   float* indices, float* counts) {
+    const unsigned held_runs = unsigned(std::min<size_t>((most + SELECT_THREADS - 1) / SELECT_THREADS, LDS_RUNS));
+    const size_t shared = size_t(std::max(held_runs, 1u)) * SELECT_THREADS * 4;
+    static bool raised[2] = {false, false};
+    if (shared > 48 * 1024 && !raised[REGS ? 1 : 0]) {
+        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&select_kernel<REGS>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_RUNS * SELECT_THREADS * 4));
+        raised[REGS ? 1 : 0] = true;
+    }
+    select_kernel<REGS><<<rows, SELECT_THREADS, shared, d.stream>>>(scores, pool, base, dynamic, selected, held_runs, indices, counts);
 }
 
 template<int T>
@@ -430,9 +545,8 @@ int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, con
         }
     }
     const unsigned rows = checked_blocks(steps, 1);
-    if (most <= size_t(4) * SELECT_THREADS) select_kernel<4, true><<<rows, SELECT_THREADS, 0, value.stream>>>(scores, pool, base, dynamic_base, selected, indices, counts);
-    else if (most <= size_t(16) * SELECT_THREADS) select_kernel<16, true><<<rows, SELECT_THREADS, 0, value.stream>>>(scores, pool, base, dynamic_base, selected, indices, counts);
-    else select_kernel<64, false><<<rows, SELECT_THREADS, 0, value.stream>>>(scores, pool, base, dynamic_base, selected, indices, counts);
+    if (most <= size_t(LDS_RUNS) * SELECT_THREADS) launch_select<0>(value, scores, pool, base, dynamic_base, selected, most, rows, indices, counts);
+    else launch_select<33>(value, scores, pool, base, dynamic_base, selected, most, rows, indices, counts);
     SD_OP_END
 }
 
