@@ -5,17 +5,20 @@
 // base-2 online softmax in FP32) and its multi-token qsa_flash (gpu/sparse_attention_compute.hpp:176-279) with the
 // dense selection 0..position.
 //
-// Shape of the work on gfx950 (wave64, v_mfma_f32_16x16x32_f16):
-//   * a workgroup (8 waves, two per SIMD) owns 4 x QT x 16 consecutive query rows of one (sequence, K/V head): rows
-//     are ordered (span row, head in group), so a workgroup is a run of consecutive tokens with all their grouped
-//     heads and every K/V row it reads serves all of them; a quarter of the rows belongs to a pair of waves, one
-//     taking the first 32 keys of every 64-key step and one the last 32, each with its own online softmax; the pair
-//     merges through LDS at the end and the output is written once, normalised;
-//   * the workgroup walks the keys 64 at a time: the step's K and V slabs (64 contiguous rows of a page plane) are
-//     copied by coalesced 16-byte global->LDS loads, an eighth by each wave, into a ring of stages, so the copies of
-//     the next steps are in flight while this one is computed; one barrier per step;
-//   * every wave builds its MFMA operands from the stage (paged_rows.hpp) and skips steps that lie wholly after
-//     its rows' positions; the workgroups with the longest walks are dispatched first.
+// Shape of the work on gfx950 (wave64, v_mfma_f32_16x16x32_f16).  Query rows are ordered (span row, head in group), so a
+// run of consecutive rows is a run of consecutive tokens with all their grouped heads and every K/V row read serves all of
+// them.  A workgroup of 8 waves (two per SIMD) walks the keys 64 at a time; a step's K and V slabs (64 contiguous rows of a
+// page plane) arrive by coalesced 16-byte global->LDS loads, an eighth by each wave, into a ring of stages, so the copies
+// of the next steps are in flight while this one is computed; one barrier per step; steps that lie wholly after a wave's
+// rows are skipped.  Two kernels:
+//   * prefill_pairs_kernel (128 columns, the headline shape): the workgroup converts a step's raw rows once into FP16
+//     tiles in LDS which all eight waves read as MFMA operands; it owns two runs of 128 rows, one from the end of the span
+//     and its mirror image from the start, so every workgroup does about the same work, and writes its outputs normalised,
+//     with no merge (details at the kernel);
+//   * prefill_attention_kernel (256 columns): 4 x QT x 16 rows per workgroup; every wave builds its own operands from the
+//     stage (paged_rows.hpp); a quarter of the rows belongs to a pair of waves, one taking the first 32 keys of every step
+//     and one the last 32, each with its own online softmax, merged through LDS at the end; the workgroups with the
+//     longest walks are dispatched first.
 #include "paged_rows.hpp"
 
 #include <cstdlib>

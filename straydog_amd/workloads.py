@@ -191,6 +191,40 @@ class SparseWorkload:
             self.gpu.release(b)
 
 
+class BlockIndexWorkload:
+    """Qwen's block indexer at the reference's long-context point (gpu/sparse_attention.hpp:403-437 is quoted at 242K tokens):
+    `steps` rows at positions base.., 4 x 128 index queries each, pooled keys [128][context / 4 + 1] FP32."""
+
+    def __init__(self, gpu, steps, base=242000, context=262144, seed=6):
+        self.gpu, self.steps, self.base, self.pool = gpu, steps, base, context // 4 + 1
+        self.queries = gpu.buffer(steps * 512 * 4)
+        self.blocks = gpu.buffer(128 * self.pool * 4)
+        self.scores = gpu.buffer(steps * self.pool * 4)
+        self.indices = gpu.buffer(steps * 2052 * 4)
+        self.counts = gpu.buffer(steps * 4)
+        gpu.fill_normal(self.queries.base(), steps * 512, seed * 11 + 1, 0)
+        gpu.fill_normal(self.blocks.base(), 128 * self.pool, seed * 11 + 2, 0)
+        gpu.synchronize()
+
+    def step(self):
+        self.gpu.qsa_index(self.queries.base(), 512, self.blocks.base(), self.pool, self.base, self.steps, 2052, self.scores.base(),
+                           self.indices.base(), self.counts.base())
+
+    def complete(self):
+        return (self.base + self.steps) // 4
+
+    def algorithmic_bytes(self):
+        # the pooled keys of the complete blocks once, the scores out and in again, queries and the selection
+        return self.complete() * 128 * 4 + 2 * self.steps * self.complete() * 4 + self.steps * (512 + 2052 + 1) * 4
+
+    def flops(self):
+        return 2 * 512 * self.steps * self.complete()
+
+    def release(self):
+        for b in (self.queries, self.blocks, self.scores, self.indices, self.counts):
+            self.gpu.release(b)
+
+
 def config1_lengths(seed=0x9e3779b97f4a7c15 ^ 1, seqs=32, low=1024, high=32768):
     rng = np.random.default_rng(seed & 0xffffffff)
     return rng.integers(low, high + 1, size=seqs)
