@@ -76,6 +76,21 @@ int sdx_qsa_pool(void* handle, const float* incoming, float* history, const floa
 int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, const float* blocks, uint64_t pool, uint64_t base,
                   const uint32_t* dynamic_base, uint64_t steps, uint64_t selected, float* scores, float* indices, float* counts);
 
+/* Selection-list attention over K/V rows of 256 columns (Q8_0 or FP16): the reference's qsa_attention / qsa_attention_rows
+ * (gpu/sparse_attention_compute.hpp:609-647: qsa_decode_parts :41-135 + qsa_decode_merge :139-170) followed by qsa_gate
+ * (gpu/sparse_attention.hpp:439-442).  Row r, at position base + r (or *dynamic_base + r, a device-resident position),
+ * attends the positions its list names: indices [rows][selected] and counts [rows], both floats, as sdx_qsa_index and the
+ * reference's packed buffer hold them; an entry counts iff 0 <= raw <= position and raw < context (gpu/kernels.cpp:100-165).
+ * The rows come from `pool` through page_table ([ceil(context / page_tokens)] pages of the one sequence) or, with a null
+ * page_table, from a pool whose single page holds the context (which is the reference's state layout, planes x context).
+ * q and out are [rows][heads][256], FP32 or FP16 each; gate (optional) is read at gate[(r * heads + h) * gate_stride + c] and
+ * out *= sigmoid(gate).  heads / kv_heads <= 16.  scratch: sdx_selected_attention_scratch(rows, kv_heads, selected) bytes. */
+uint64_t sdx_selected_attention_scratch(uint64_t rows, uint64_t kv_heads, uint64_t selected);
+int sdx_selected_attention(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t context, uint64_t base,
+                           const uint32_t* dynamic_base, const float* indices, uint64_t selected, const float* counts, const void* q, int q_f16,
+                           uint64_t rows, uint64_t heads, float scale, const float* gate, uint64_t gate_stride, void* out, int out_f16,
+                           void* scratch, uint64_t scratch_bytes);
+
 /* Top-k indexed sparse attention over BF16 latent K/V for a batch of sequences (one decode row each):
  * stage 1+2 = sd_op_index_scores + sd_op_top_k per sequence (gpu/ops.hpp:1700-1739, 1766-1941) with each sequence's own
  * keys [batch][groups][dim] BF16; q_index [batch][heads][dim] BF16; weights [batch][heads] FP32; visible [batch].

@@ -63,6 +63,9 @@ SIGNATURES = {
     "sdx_qsa_normalize": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_u64, c_void_p]),
     "sdx_qsa_pool": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_void_p]),
     "sdx_qsa_index": (c_int, [c_void_p, c_void_p, c_u64, c_void_p, c_u64, c_u64, c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_void_p]),
+    "sdx_selected_attention_scratch": (c_u64, [c_u64, c_u64, c_u64]),
+    "sdx_selected_attention": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_u64, c_void_p, c_void_p, c_int,
+                                       c_u64, c_u64, c_float, c_void_p, c_u64, c_void_p, c_int, c_void_p, c_u64]),
     "sdx_index_score_bounds": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float, c_void_p, c_void_p]),
     "sdx_index_top_k": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float, c_void_p,
                                 c_u64, c_void_p]),

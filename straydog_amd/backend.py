@@ -164,6 +164,15 @@ class Backend:
                                                 q, int(q_f16), seqs, span, heads, scale, out, int(out_f16), scratch.pointer,
                                                 scratch.size))
 
+    def selected_attention_scratch(self, rows, kv_heads, selected):
+        return int(self.lib.sdx_selected_attention_scratch(rows, kv_heads, selected))
+
+    def selected_attention(self, pool, page_table, context, base, indices, selected, counts, q, q_f16, rows, heads, scale, out, out_f16,
+                           scratch, gate=None, gate_stride=0, dynamic_base=None):
+        self.check(self.lib.sdx_selected_attention(self.handle, ctypes.byref(pool), page_table, context, base, dynamic_base, indices, selected,
+                                                   counts, q, int(q_f16), rows, heads, scale, gate, gate_stride, out, int(out_f16),
+                                                   scratch.pointer, scratch.size))
+
     def index_top_k(self, q_index, keys, weights, visible, batch, groups, heads, dim, scale, scores, k, indices):
         self.check(self.lib.sdx_index_top_k(self.handle, q_index, keys, weights, visible, batch, groups, heads, dim, scale, scores,
                                             k, indices))

@@ -210,6 +210,33 @@ class BlockIndexWorkload:
         self.gpu.qsa_index(self.queries.base(), 512, self.blocks.base(), self.pool, self.base, self.steps, 2052, self.scores.base(),
                            self.indices.base(), self.counts.base())
 
+    def with_attention(self, heads=24, kv_heads=2, row_bytes=272, seed=7):
+        """Adds the attention over each row's selection: Q8_0 rows of 256 columns in the reference's state layout."""
+        gpu, context = self.gpu, (self.pool - 1) * 4
+        self.heads, self.kv_heads, self.row_bytes = heads, kv_heads, row_bytes
+        self.kv, self.kv_buffer = gpu.kv_pool(1, context, kv_heads, 256, row_bytes)
+        k, table = gpu.buffer(8192 * kv_heads * 256 * 2), gpu.upload(np.zeros(1, dtype=np.int32))
+        gpu.fill_normal(k.base(), 8192 * kv_heads * 256, seed * 11 + 3, 1)
+        for first in range(0, context, 8192):                # the cache is filled through the library's own writer
+            start = gpu.upload(np.array([first], dtype=np.int32))
+            gpu.kv_write(self.kv, table.base(), 1, start.base(), k.base(), k.base(), True, 1, 8192)
+            gpu.release(start)
+        self.q = gpu.buffer(self.steps * heads * 256 * 2)
+        gpu.fill_normal(self.q.base(), self.steps * heads * 256, seed * 11 + 4, 1)
+        self.out = gpu.buffer(self.steps * heads * 256 * 2)
+        self.scratch = gpu.buffer(gpu.selected_attention_scratch(self.steps, kv_heads, 2052))
+        gpu.synchronize()
+        gpu.release(k); gpu.release(table)
+        return self
+
+    def step_attention(self):
+        self.gpu.selected_attention(self.kv, None, (self.pool - 1) * 4, self.base, self.indices.base(), 2052, self.counts.base(), self.q.base(), True,
+                                    self.steps, self.heads, 0.0625, self.out.base(), True, self.scratch)
+
+    def attention_bytes(self):
+        # the selected rows of both planes of every K/V head, once per row
+        return self.steps * 2051 * self.kv_heads * 2 * self.row_bytes
+
     def complete(self):
         return (self.base + self.steps) // 4
 
@@ -223,6 +250,9 @@ class BlockIndexWorkload:
     def release(self):
         for b in (self.queries, self.blocks, self.scores, self.indices, self.counts):
             self.gpu.release(b)
+        if hasattr(self, "kv_buffer"):
+            for b in (self.kv_buffer, self.q, self.out, self.scratch):
+                self.gpu.release(b)
 
 
 def config1_lengths(seed=0x9e3779b97f4a7c15 ^ 1, seqs=32, low=1024, high=32768):

@@ -196,3 +196,111 @@ def test_refusals(gpu):
         gpu.qsa_pool(q.base(), k.base(), k.base(), 10, 100, 4, k.base())
     for b in (q, k, scores, indices, counts):
         gpu.release(b)
+
+
+def _qwen_case(oracle, rng, row_bytes, context, base, steps, selected=2052):
+    """The Qwen state (planes x context rows) with `base` cached positions, a span's packed input with realistic selection
+    lists (sdx_qsa_index's rule on random scores) and one adversarial list; the oracle's outputs and the state afterwards."""
+    state = np.zeros(context * 4 * row_bytes, dtype=np.uint8)
+    old_k = rng.standard_normal((1, base, 2, 256)).astype(np.float32)
+    old_v = rng.standard_normal((1, base, 2, 256)).astype(np.float32)
+    oracle.kv_write(state, row_bytes, context, 2, 256, np.zeros((1, 1), np.int32), np.zeros(1, np.int32), old_k, old_v)
+    q = rng.standard_normal((steps, 24, 256)).astype(np.float32)
+    k = rng.standard_normal((steps, 2, 256)).astype(np.float32)
+    v = rng.standard_normal((steps, 2, 256)).astype(np.float32)
+    indices = np.full((steps, selected), -1.0, dtype=np.float32)
+    counts = np.zeros(steps, dtype=np.float32)
+    for s in range(steps):
+        if s == steps - 1:
+            # entries that do not count: past the row's position, negative, past the context; and a short list
+            row = np.concatenate([np.sort(rng.permutation(base + s + 1)[:77]), [base + s + 3, -2.0, context + 1, base + s]]).astype(np.float32)
+        else:
+            row = oracle.qsa_select(rng.random(context // 4 + 1).astype(np.float32), base + s)
+        indices[s, :row.size] = row
+        counts[s] = row.size
+    packed = np.concatenate([q.ravel(), k.ravel(), v.ravel(), indices.ravel(), counts]).astype(np.float32)
+    want = oracle.attention_sequence(state, row_bytes, context, base, steps, selected, packed).reshape(steps, 24, 256)
+    return state, q, indices, counts, want
+
+
+@pytest.mark.parametrize("row_bytes", [272, 512])
+@pytest.mark.parametrize("paged", [False, True])
+def test_selected_attention(gpu, oracle, row_bytes, paged):
+    # the attention of a Qwen decode / verification pass over each row's selection: Q8_0 and FP16 rows, the reference's state
+    # layout and a shuffled page table, FP32 and FP16 queries and outputs, the sigmoid gate, a device-resident position
+    from gpu_util import close_enough
+    rng = np.random.default_rng(row_bytes + paged)
+    context, base, steps, selected = 4096, 3000, 5, 2052
+    state, q, indices, counts, want = _qwen_case(oracle, rng, row_bytes, context, base, steps, selected)
+    planes = state.reshape(4, context, row_bytes)
+    if paged:
+        page_tokens, pages = 256, context // 256
+        order = rng.permutation(pages + 3)[:pages].astype(np.int32)
+        host = np.zeros((pages + 3, 4, page_tokens, row_bytes), dtype=np.uint8)
+        for p in range(pages):
+            host[order[p]] = planes[:, p * page_tokens:(p + 1) * page_tokens]
+        pool, buffer = gpu.kv_pool(pages + 3, page_tokens, 2, 256, row_bytes)
+        table = gpu.upload(order)
+    else:
+        host = planes
+        pool, buffer = gpu.kv_pool(1, context, 2, 256, row_bytes)
+        table = None
+    gpu.write_buffer(buffer, 0, np.ascontiguousarray(host).reshape(-1))
+    gate = rng.standard_normal((steps, 24, 512)).astype(np.float32) * 2
+    ib, cb, gb = gpu.upload(indices), gpu.upload(counts), gpu.upload(gate)
+    scratch = gpu.buffer(gpu.selected_attention_scratch(steps, 2, selected))
+    position = gpu.upload(np.array([base], dtype=np.uint32))
+    for q_f16, out_f16, gated, dynamic in ((False, False, False, False), (True, True, True, False), (False, False, True, True)):
+        qb = gpu.upload(q.astype(np.float16) if q_f16 else q)
+        out = gpu.buffer(steps * 24 * 256 * (2 if out_f16 else 4))
+        gpu.selected_attention(pool, table.base() if paged else None, context, 0 if dynamic else base, ib.base(), selected, cb.base(), qb.base(),
+                               q_f16, steps, 24, 0.0625, out.base(), out_f16, scratch, gate=gb.at(256 * 4) if gated else None, gate_stride=512,
+                               dynamic_base=position.base() if dynamic else None)
+        got = _read(gpu, out, np.float16 if out_f16 else np.float32, steps * 24 * 256).astype(np.float32).reshape(steps, 24, 256)
+        expect = want * (1.0 / (1.0 + np.exp(-gate[:, :, 256:].astype(np.float64)))) if gated else want
+        close_enough(got, expect, f"selected attention f16={q_f16} gated={gated} dynamic={dynamic}")
+        gpu.release(qb); gpu.release(out)
+    for b in (ib, cb, gb, scratch, position, buffer) + ((table,) if paged else ()):
+        gpu.release(b)
+
+
+def test_index_then_attend_on_the_device(gpu, oracle):
+    # the two stages chained on the device, as a decode pass runs them: sdx_qsa_index's lists feed sdx_selected_attention unchanged
+    from gpu_util import close_enough
+    rng = np.random.default_rng(77)
+    context, base, steps, row_bytes = 8192, 6000, 3, 272
+    pool_blocks = context // 4 + 1
+    queries, blocks = _case(oracle, "t", base, steps, pool_blocks, 512, seed=9)
+    blocks = np.nan_to_num(blocks)
+    state = np.zeros(context * 4 * row_bytes, dtype=np.uint8)
+    k = rng.standard_normal((1, base + steps, 2, 256)).astype(np.float32)
+    v = rng.standard_normal((1, base + steps, 2, 256)).astype(np.float32)
+    oracle.kv_write(state, row_bytes, context, 2, 256, np.zeros((1, 1), np.int32), np.zeros(1, np.int32), k, v)
+    q = rng.standard_normal((steps, 24, 256)).astype(np.float32)
+    scores = oracle.qsa_block_scores(queries, blocks, base)
+    indices = np.full((steps, 2052), -1.0, dtype=np.float32)
+    counts = np.zeros(steps, dtype=np.float32)
+    for r in range(steps):
+        row = oracle.qsa_select(scores[r], base + r)
+        indices[r, :row.size] = row
+        counts[r] = row.size
+    # the oracle rewrites the span's K/V rows from its packed input: hand it the rows the state already holds (decoded values
+    # re-encode to the same bytes)
+    held_k = np.stack([oracle.kv_q8_values(state.reshape(4, context, row_bytes)[h, base:base + steps], 256) for h in range(2)], axis=1)
+    held_v = np.stack([oracle.kv_q8_values(state.reshape(4, context, row_bytes)[2 + h, base:base + steps], 256) for h in range(2)], axis=1)
+    packed = np.concatenate([q.ravel(), held_k.ravel(), held_v.ravel(), indices.ravel(), counts]).astype(np.float32)
+    before = state.copy()
+    want = oracle.attention_sequence(state, row_bytes, context, base, steps, 2052, packed).reshape(steps, 24, 256)
+    assert np.array_equal(before, state)
+    pool, buffer = gpu.kv_pool(1, context, 2, 256, row_bytes)
+    gpu.write_buffer(buffer, 0, state)
+    qb, kb, qq = gpu.upload(queries), gpu.upload(blocks), gpu.upload(q)
+    sb, ib, cb = gpu.buffer(steps * pool_blocks * 4), gpu.buffer(steps * 2052 * 4), gpu.buffer(steps * 4)
+    out = gpu.buffer(steps * 24 * 256 * 4)
+    scratch = gpu.buffer(gpu.selected_attention_scratch(steps, 2, 2052))
+    gpu.qsa_index(qb.base(), 512, kb.base(), pool_blocks, base, steps, 2052, sb.base(), ib.base(), cb.base())
+    gpu.selected_attention(pool, None, context, base, ib.base(), 2052, cb.base(), qq.base(), False, steps, 24, 0.0625, out.base(), False, scratch)
+    got = _read(gpu, out, np.float32, steps * 24 * 256).reshape(steps, 24, 256)
+    close_enough(got, want, "index then attend")
+    for b in (qb, kb, qq, sb, ib, cb, out, scratch, buffer):
+        gpu.release(b)
