@@ -109,6 +109,27 @@ int sd_op_index_select(void* handle, const float* q, const float* keys, const fl
                        uint64_t groups, uint64_t heads, uint64_t dim, float scale, uint64_t rope_dims, const int32_t* positions,
                        const float* frequencies, float* scores, uint64_t k, int32_t* out, const int32_t* candidates, uint64_t blocks,
                        uint64_t block);
+/* ---- The inputs of a dense attention step (its neighbours in a span) ---- */
+/* reference straydog_gpu.h:446 (gpu/token_mixing.hpp:246-252, :628-637): rows of [first | second], `width` each, apart. */
+int sd_op_split(void* handle, const float* x, uint64_t rows, uint64_t width, float* first, float* second);
+/* reference straydog_gpu.h:251 (gpu/kernels.cpp:4901-4913, gpu/ops.hpp:28-59): output = input * rsqrt(mean(input^2) + eps) * weight
+ * per row; the sum of squares in the order of the reference's 256-thread halving tree.  May run in place. */
+int sd_op_rms_norm(void* handle, const float* input, const float* weight, uint64_t rows, uint64_t width, float eps, float* output);
+/* reference straydog_gpu.h:452 (gpu/token_mixing.hpp:254-274, :639-650): the leading rope_dims values of each of a row's
+ * `vectors` vectors of `width` turned in pairs (i, i + rope_dims/2) by positions[row] * frequencies[i], angles in double. */
+int sd_op_rope_halves(void* handle, float* x, uint64_t rows, uint64_t vectors, uint64_t width, uint64_t rope_dims, const int32_t* positions,
+                      const float* frequencies);
+/* reference straydog_gpu.h:307 (gpu/kernels.cpp:5244-5252, gpu/ops.hpp:1171-1175): out[rows[i]] = x[i], `width` values a row.
+ * An index outside 0 .. out_rows - 1 writes nothing here (the reference leaves it undefined). */
+int sd_op_scatter(void* handle, const float* x, const int32_t* rows, uint64_t count, uint64_t width, float* out, uint64_t out_rows);
+/* reference straydog_gpu.h:447-451 (gpu/token_mixing.hpp:276-338, :601-626): an attention step's inputs in one launch:
+ * sd_op_split of q_full (rows x heads x [query | gate], each dim) into q and gate, sd_op_rms_norm of the queries (q_weight) and
+ * of k's heads (k_weight, in place), sd_op_rope_halves of both (rope_dims), and sd_op_scatter of k and v (rows x kv_heads x dim)
+ * to rows `positions` of keys and values (context rows each); the same bits as the separate ops.  A position outside the
+ * cache writes no row of it. */
+int sd_op_attention_prepare(void* handle, const float* q_full, float* k, const float* v, uint64_t rows, uint64_t heads, uint64_t kv_heads,
+                            uint64_t dim, const float* q_weight, const float* k_weight, float eps, uint64_t rope_dims, const int32_t* positions,
+                            const float* frequencies, float* q, float* gate, float* keys, float* values, uint64_t context);
 /* reference straydog_gpu.h:459 (gpu/token_mixing.hpp:728-744): out = x as BF16, nearest even, a NaN stays a NaN. */
 int sd_op_to_bf16(void* handle, const float* x, uint64_t count, void* out);
 

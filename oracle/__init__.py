@@ -73,6 +73,10 @@ _latent = _sig("sdo_latent_attention", None, _vp, _vp, _sz, _vp, _sz, _vp, ctype
                ctypes.c_float, _sz, _vp, _vp, _vp, ctypes.c_int)
 _compress = _sig("sdo_compress", None, _vp, _vp, _sz, _sz, _sz, _vp)
 _qsa_select = _sig("sdo_qsa_select", _sz, _vp, _sz, _sz, _vp)
+_rms_norm = _sig("sdo_rms_norm", None, _vp, _vp, _sz, _sz, ctypes.c_float, _vp)
+_rope_halves = _sig("sdo_rope_halves", None, _vp, _sz, _sz, _sz, _sz, _vp, _vp)
+_attention_prepare = _sig("sdo_attention_prepare", None, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp, ctypes.c_float, _sz, _vp, _vp, _vp, _vp,
+                          _vp, _vp, _sz)
 _qsa_normalize = _sig("sdo_qsa_normalize", None, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _vp)
 _qsa_pool = _sig("sdo_qsa_pool", None, _vp, _vp, _vp, _sz, _sz, _sz, _vp)
 _qsa_block_scores = _sig("sdo_qsa_block_scores", None, _vp, _sz, _vp, _sz, _sz, _sz, _vp)
@@ -282,6 +286,33 @@ def qsa_select(scores, position, keep_blocks=512):
     out = np.zeros(keep_blocks * 4 + 4 + max(0, position + 1), dtype=np.float32)
     count = _qsa_select(_ptr(scores), position, keep_blocks, _ptr(out))
     return out[:count].copy()
+
+
+def rms_norm(x, weight, eps):
+    x, weight = _f32(x), _f32(weight)
+    out = np.zeros_like(x)
+    _rms_norm(_ptr(x), _ptr(weight), x.shape[0], x.shape[1], ctypes.c_float(eps), _ptr(out))
+    return out
+
+
+def rope_halves(x, rope_dims, positions, frequencies):
+    """x: [rows, vectors, width]; returns the turned copy."""
+    out, positions, frequencies = _f32(x).copy(), _i32(positions), _f32(frequencies)
+    _rope_halves(_ptr(out), out.shape[0], out.shape[1], out.shape[2], rope_dims, _ptr(positions), _ptr(frequencies))
+    return out
+
+
+def attention_prepare(q_full, k, v, q_weight, k_weight, eps, rope_dims, positions, frequencies, keys, values):
+    """q_full [rows, heads, 2*dim], k/v [rows, kv_heads, dim]; keys/values [context, kv_heads*dim] are updated in place.
+    Returns (q, gate, k_after)."""
+    q_full, k, v = _f32(q_full), _f32(k).copy(), _f32(v)
+    rows, heads, dim = q_full.shape[0], q_full.shape[1], q_full.shape[2] // 2
+    q_weight, k_weight, positions, frequencies = _f32(q_weight), _f32(k_weight), _i32(positions), _f32(frequencies)
+    assert keys.dtype == np.float32 and values.dtype == np.float32 and keys.flags.c_contiguous and values.flags.c_contiguous
+    q, gate = np.zeros((rows, heads, dim), np.float32), np.zeros((rows, heads, dim), np.float32)
+    _attention_prepare(_ptr(q_full), _ptr(k), _ptr(v), rows, heads, k.shape[1], dim, _ptr(q_weight), _ptr(k_weight), ctypes.c_float(eps),
+                       rope_dims, _ptr(positions), _ptr(frequencies), _ptr(q), _ptr(gate), _ptr(keys), _ptr(values), keys.shape[0])
+    return q, gate, k
 
 
 def qsa_normalize(source, norm, rows, heads, width, stride, position):

@@ -739,6 +739,66 @@ void sdo_qsa_block_scores(const float* queries, size_t query_stride, const float
     }
 }
 
+/* ------------------------------------------------------------------ the inputs of a dense attention step */
+
+/* ops.hpp:28-55 (op_rms_norm_row with tree256_first_wave): thread t of 256 sums the squares of columns t, t + 256, ... (a fused
+ * multiply-add each, as the device compiler contracts it), the 256 partial sums are added in halving-tree order, and
+ * out = (x * rsqrt(mean + eps)) * weight. */
+void sdo_rms_norm(const float* input, const float* weight, size_t rows, size_t width, float eps, float* output) {
+    for (size_t r = 0; r < rows; ++r) {
+        const float* x = input + r * width;
+        float sums[256];
+        for (size_t t = 0; t < 256; ++t) {
+            float sum = 0.0f;
+            for (size_t c = t; c < width; c += 256) sum = fmaf(x[c], x[c], sum);
+            sums[t] = sum;
+        }
+        const float scale = 1.0f / sqrtf(qsa_tree_sum(sums, 256) / (float)width + eps);
+        for (size_t c = 0; c < width; ++c) output[r * width + c] = x[c] * scale * weight[c];
+    }
+}
+
+/* token_mixing.hpp:254-274: pair (i, i + pairs) of each vector's leading values turned by position * frequency, in double. */
+void sdo_rope_halves(float* x, size_t rows, size_t vectors, size_t width, size_t rope_dims, const int32_t* positions,
+                     const float* frequencies) {
+    const size_t pairs = rope_dims / 2;
+    for (size_t r = 0; r < rows; ++r)
+        for (size_t v = 0; v < vectors; ++v)
+            for (size_t i = 0; i < pairs; ++i) {
+                float* first = x + (r * vectors + v) * width + i;
+                float* second = first + pairs;
+                const double angle = (double)positions[r] * (double)frequencies[i];
+                const double s = sin(angle), c = cos(angle), a = *first, b = *second;
+                *first = (float)(a * c - b * s);
+                *second = (float)(a * s + b * c);
+            }
+}
+
+/* token_mixing.hpp:276-338 (tm_attention_prepare_kernel): q_full rows x heads x [query | gate] split, queries and keys normed
+ * and turned, keys (also back into k) and values written to row positions[row] of the caches when it lies inside them. */
+void sdo_attention_prepare(const float* q_full, float* k, const float* v, size_t rows, size_t heads, size_t kv_heads, size_t dim,
+                           const float* q_weight, const float* k_weight, float eps, size_t rope_dims, const int32_t* positions,
+                           const float* frequencies, float* q, float* gate, float* keys, float* values, size_t context) {
+    const size_t kv_width = kv_heads * dim;
+    for (size_t r = 0; r < rows; ++r) {
+        for (size_t h = 0; h < heads; ++h) {
+            const float* x = q_full + (r * heads + h) * 2 * dim;
+            memcpy(gate + (r * heads + h) * dim, x + dim, dim * sizeof(float));
+            sdo_rms_norm(x, q_weight, 1, dim, eps, q + (r * heads + h) * dim);
+        }
+        sdo_rms_norm(k + r * kv_width, k_weight, kv_heads, dim, eps, k + r * kv_width);
+    }
+    if (rope_dims) {
+        sdo_rope_halves(q, rows, heads, dim, rope_dims, positions, frequencies);
+        sdo_rope_halves(k, rows, kv_heads, dim, rope_dims, positions, frequencies);
+    }
+    for (size_t r = 0; r < rows; ++r) {
+        if (positions[r] < 0 || (size_t)positions[r] >= context) continue;
+        memcpy(keys + (size_t)positions[r] * kv_width, k + r * kv_width, kv_width * sizeof(float));
+        memcpy(values + (size_t)positions[r] * kv_width, v + r * kv_width, kv_width * sizeof(float));
+    }
+}
+
 /* ------------------------------------------------------------------ seeded inputs */
 
 static inline uint64_t xorshift64(uint64_t* s) { *s ^= *s << 13; *s ^= *s >> 7; *s ^= *s << 17; return *s; }

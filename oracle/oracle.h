@@ -19,7 +19,8 @@
  * closed form + special cases), sdo_compress (float64 closed form), sdo_qsa_select (brute force),
  * sdo_qsa_block_scores (exact rational arithmetic rounded once per fused step, in pure Python, + float64 closed form),
  * sdo_qsa_normalize / sdo_qsa_pool (float64 closed form; rotation invariants: pair norms kept, position 0 and columns
- * from 64 on unturned; the ring's contents).
+ * from 64 on unturned; the ring's contents), sdo_rms_norm / sdo_rope_halves / sdo_attention_prepare (float64 closed forms; a
+ * rotation keeps pair norms; the fused step equals its parts).
  * PARITY UNPINNED: none of the above; bit-level agreement with the reference's device summation
  * order inside its flash kernels is not claimed anywhere (tolerance-based, see the tests).
  */
@@ -135,6 +136,15 @@ void sdo_qsa_normalize(const float* source, const float* norm, size_t rows, size
 void sdo_qsa_pool(const float* incoming, float* history, const float* norm, size_t pool, size_t base, size_t steps, float* blocks);
 void sdo_qsa_block_scores(const float* queries, size_t query_stride, const float* blocks, size_t pool, size_t base, size_t steps,
                           float* scores);
+
+/* ---- The inputs of a dense attention step: gpu/ops.hpp:28-59 (rms norm, halving-tree sum of squares), gpu/token_mixing.hpp:254-274
+ * (rope of halves, double angles), :276-338 (the fused step: split, norm, rope, scatter into the caches). */
+void sdo_rms_norm(const float* input, const float* weight, size_t rows, size_t width, float eps, float* output);
+void sdo_rope_halves(float* x, size_t rows, size_t vectors, size_t width, size_t rope_dims, const int32_t* positions,
+                     const float* frequencies);
+void sdo_attention_prepare(const float* q_full, float* k, const float* v, size_t rows, size_t heads, size_t kv_heads, size_t dim,
+                           const float* q_weight, const float* k_weight, float eps, size_t rope_dims, const int32_t* positions,
+                           const float* frequencies, float* q, float* gate, float* keys, float* values, size_t context);
 
 /* ---- Seeded inputs: xorshift64 (crates/straydog-engine/tests/fused_gpu.rs:39-53) -> Box-Muller
  *      (gpu/tests/qsa_interval_test.cpp:12-18). */

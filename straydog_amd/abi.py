@@ -56,6 +56,12 @@ SIGNATURES = {
                                    c_void_p, c_void_p, c_void_p, c_u64, c_void_p, c_void_p, c_u64, c_u64]),
     "sd_op_to_bf16": (c_int, [c_void_p, c_void_p, c_u64, c_void_p]),
     # straydog_gpu_ext.h
+    "sd_op_split": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_void_p, c_void_p]),
+    "sd_op_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_float, c_void_p]),
+    "sd_op_rope_halves": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_void_p]),
+    "sd_op_scatter": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_void_p, c_u64]),
+    "sd_op_attention_prepare": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_void_p, c_float, c_u64,
+                                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64]),
     "sdx_kv_write": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_void_p, c_void_p, c_int, c_u64, c_u64]),
     "sdx_paged_attention_scratch": (c_u64, [c_u64, c_u64, c_u64, c_u64, c_u64]),
     "sdx_paged_attention": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_u64, c_void_p, c_int, c_u64, c_u64, c_u64,

@@ -146,6 +146,24 @@ class Backend:
         self.check(self.lib.sd_op_to_bf16(self.handle, x, count, out))
 
     # ---- paged cache extensions --------------------------------------------------------
+    # ---- the inputs of a dense attention step (ops.rs: split, rms_norm, rope_halves, scatter, attention_prepare) ----
+    def split(self, x, rows, width, first, second):
+        self.check(self.lib.sd_op_split(self.handle, x, rows, width, first, second))
+
+    def rms_norm(self, x, weight, rows, width, eps, out):
+        self.check(self.lib.sd_op_rms_norm(self.handle, x, weight, rows, width, eps, out))
+
+    def rope_halves(self, x, rows, vectors, width, rope_dims, positions, frequencies):
+        self.check(self.lib.sd_op_rope_halves(self.handle, x, rows, vectors, width, rope_dims, positions, frequencies))
+
+    def scatter(self, x, rows, count, width, out, out_rows):
+        self.check(self.lib.sd_op_scatter(self.handle, x, rows, count, width, out, out_rows))
+
+    def attention_prepare(self, q_full, k, v, rows, heads, kv_heads, dim, q_weight, k_weight, eps, rope_dims, positions, frequencies, q, gate,
+                          keys, values, context):
+        self.check(self.lib.sd_op_attention_prepare(self.handle, q_full, k, v, rows, heads, kv_heads, dim, q_weight, k_weight, eps, rope_dims,
+                                                    positions, frequencies, q, gate, keys, values, context))
+
     def kv_pool(self, pages, page_tokens, kv_heads, dim, row_bytes):
         size = pages * 2 * kv_heads * page_tokens * row_bytes
         buffer = self.buffer(size)

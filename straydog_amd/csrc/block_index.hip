@@ -17,6 +17,7 @@
 // beyond 32768 blocks), four 8-bit radix passes over per-wave LDS histograms (the first, where nearly all values share a digit, counted by ballots), and
 // one ordered pass whose slots come from 64-wide ballots and a scan over (run, wave) counts.
 #include "device.hpp"
+#include "tree_sum.hpp"
 #include "../../include/straydog_gpu_ext.h"
 
 using namespace sd;
@@ -29,26 +30,6 @@ __device__ __forceinline__ float turn(float own, float partner, unsigned column,
     if (column >= 64) return own;
     const float angle = float(position) / powf(1e7f, float(column % 32) / 32.0f);
     return own * cosf(angle) + (column < 32 ? -partner : partner) * sinf(angle);
-}
-
-// The sum over the workgroup's `width` threads in the order of a halving tree, sums[c] += sums[c + offset], which is the
-// reference's order; the last six levels are lane shifts inside the first wave.
-__device__ __forceinline__ float tree_sum(float mine, float* sums, unsigned width) {
-    const unsigned c = threadIdx.x;
-    sums[c] = mine;
-    __syncthreads();
-    for (unsigned offset = width / 2; offset >= 64; offset /= 2) {
-        if (c < offset) sums[c] += sums[c + offset];
-        __syncthreads();
-    }
-    if (c < 64) {
-        float v = sums[c];
-        #pragma unroll
-        for (unsigned offset = 32; offset; offset /= 2) v += __shfl_down(v, offset);
-        if (c == 0) sums[0] = v;
-    }
-    __syncthreads();
-    return sums[0];
 }
 
 // One workgroup of `width` threads per (row, head).

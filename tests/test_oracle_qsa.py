@@ -142,3 +142,54 @@ def test_pool_closed_form_and_ring(oracle):
         want, slack = _rope64(flat[None], block * 4)
         assert _close(blocks[:, block], want[0], slack[0])
     assert np.all(blocks[:, 97 // 4:] == 0.0), "an incomplete block is not pooled"
+
+
+def _prepare_case(rng, rows=3, heads=8, kv_heads=1, dim=256, rope_dims=64, context=16):
+    # the shapes and the out-of-order positions of crates/straydog-engine/tests/fused_gpu.rs:225-268
+    case = dict(q_full=(rng.standard_normal((rows, heads, 2 * dim)) * 4).astype(np.float32),
+                k=(rng.standard_normal((rows, kv_heads, dim)) * 4).astype(np.float32),
+                v=(rng.standard_normal((rows, kv_heads, dim)) * 4).astype(np.float32),
+                q_weight=(rng.standard_normal(dim) * 2).astype(np.float32), k_weight=(rng.standard_normal(dim) * 2).astype(np.float32),
+                frequencies=np.power(np.float32(1e7), -(2.0 * np.arange(rope_dims // 2, dtype=np.float32)) / np.float32(rope_dims)).astype(np.float32),
+                positions=np.array([9, 2, 13][:rows] + list(range(20, 20 + max(0, rows - 3))), dtype=np.int32)[:rows],
+                cache=rng.standard_normal((context, kv_heads * dim)).astype(np.float32))
+    return case
+
+
+def test_rms_norm_and_rope_halves_closed_forms(oracle):
+    rng = np.random.default_rng(6)
+    for width in (64, 256, 1000):
+        x = (rng.standard_normal((5, width)) * 3).astype(np.float32)
+        weight = (rng.standard_normal(width) * 2).astype(np.float32)
+        got = oracle.rms_norm(x, weight, 1e-6)
+        x64 = x.astype(np.float64)
+        want = x64 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + 1e-6) * weight
+        assert np.allclose(got, want, rtol=3e-6, atol=1e-7)
+    x = rng.standard_normal((3, 4, 96)).astype(np.float32)
+    positions = np.array([0, 70001, 5], dtype=np.int32)
+    frequencies = np.power(1e7, -np.arange(16) / 16.0).astype(np.float32)
+    got = oracle.rope_halves(x, 32, positions, frequencies)
+    angle = positions[:, None, None].astype(np.float64) * frequencies.astype(np.float64)
+    low, high = x[..., :16].astype(np.float64), x[..., 16:32].astype(np.float64)
+    assert np.allclose(got[..., :16], low * np.cos(angle) - high * np.sin(angle), rtol=1e-6, atol=1e-7)
+    assert np.allclose(got[..., 16:32], low * np.sin(angle) + high * np.cos(angle), rtol=1e-6, atol=1e-7)
+    assert np.array_equal(got[..., 32:], x[..., 32:]) and np.array_equal(got[0], x[0]), "columns past the rope and position 0 are not turned"
+    assert np.allclose(got[..., :16].astype(np.float64) ** 2 + got[..., 16:32].astype(np.float64) ** 2, low ** 2 + high ** 2, rtol=1e-5)
+
+
+def test_prepared_step_equals_its_parts(oracle):
+    case = _prepare_case(np.random.default_rng(7))
+    keys, values = case["cache"].copy(), case["cache"].copy()
+    q, gate, k_after = oracle.attention_prepare(case["q_full"], case["k"], case["v"], case["q_weight"], case["k_weight"], 1e-6, 64,
+                                                case["positions"], case["frequencies"], keys, values)
+    rows, heads, dim = 3, 8, 256
+    assert np.array_equal(gate, case["q_full"][:, :, dim:])
+    want_q = oracle.rope_halves(oracle.rms_norm(case["q_full"][:, :, :dim].reshape(-1, dim), case["q_weight"], 1e-6).reshape(rows, heads, dim), 64,
+                                case["positions"], case["frequencies"])
+    want_k = oracle.rope_halves(oracle.rms_norm(case["k"].reshape(-1, dim), case["k_weight"], 1e-6).reshape(rows, 1, dim), 64, case["positions"],
+                                case["frequencies"])
+    assert np.array_equal(q, want_q) and np.array_equal(k_after, want_k)
+    want_keys, want_values = case["cache"].copy(), case["cache"].copy()
+    for r, p in enumerate(case["positions"]):
+        want_keys[p], want_values[p] = want_k[r].reshape(-1), case["v"][r].reshape(-1)
+    assert np.array_equal(keys, want_keys) and np.array_equal(values, want_values)
