@@ -115,6 +115,17 @@ int sd_op_split(void* handle, const float* x, uint64_t rows, uint64_t width, flo
 /* reference straydog_gpu.h:251 (gpu/kernels.cpp:4901-4913, gpu/ops.hpp:28-59): output = input * rsqrt(mean(input^2) + eps) * weight
  * per row; the sum of squares in the order of the reference's 256-thread halving tree.  May run in place. */
 int sd_op_rms_norm(void* handle, const float* input, const float* weight, uint64_t rows, uint64_t width, float eps, float* output);
+/* reference straydog_gpu.h:252-254 (gpu/kernels.cpp:4915-4940, gpu/ops.hpp:60-106): sd_op_rms_norm, then the last rope_dims values
+ * of each row turned in adjacent pairs by positions[row] * frequencies[pair] (as sd_op_rope), the row stored at row out_rows[row]
+ * of `out` (out_count rows; the row itself when out_rows is null).  Fills an armed attention rope table of exactly `rows` rows. */
+int sd_op_norm_rope(void* handle, const float* input, const float* weight, uint64_t rows, uint64_t width, float eps, uint64_t rope_dims,
+                    const int32_t* positions, const float* frequencies, const int32_t* out_rows, float* out, uint64_t out_count);
+/* reference straydog_gpu.h:382-389 (gpu/kernels.cpp:558-616, :5288-5303): the attention rope table of a pass, rows x rope_dims/2 pairs
+ * of (cosine, sine) forward and inverse.  Reserve allocates it (outside a recorded graph; a larger request replaces it); arm makes
+ * the next sd_op_norm_rope of exactly `rows` rows (0 clears) write it, and the next sd_op_sparse_attention of those rows then reads
+ * it instead of forming the angles again: the same bits. */
+int sd_attention_turns_reserve(void* handle, uint64_t rows, uint64_t rope_dims);
+int sd_attention_turns_arm(void* handle, uint64_t rows);
 /* reference straydog_gpu.h:452 (gpu/token_mixing.hpp:254-274, :639-650): the leading rope_dims values of each of a row's
  * `vectors` vectors of `width` turned in pairs (i, i + rope_dims/2) by positions[row] * frequencies[i], angles in double. */
 int sd_op_rope_halves(void* handle, float* x, uint64_t rows, uint64_t vectors, uint64_t width, uint64_t rope_dims, const int32_t* positions,

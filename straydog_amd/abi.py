@@ -58,6 +58,9 @@ SIGNATURES = {
     # straydog_gpu_ext.h
     "sd_op_split": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_void_p, c_void_p]),
     "sd_op_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_float, c_void_p]),
+    "sd_op_norm_rope": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_float, c_u64, c_void_p, c_void_p, c_void_p, c_void_p, c_u64]),
+    "sd_attention_turns_reserve": (c_int, [c_void_p, c_u64, c_u64]),
+    "sd_attention_turns_arm": (c_int, [c_void_p, c_u64]),
     "sd_op_rope_halves": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_void_p]),
     "sd_op_scatter": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_void_p, c_u64]),
     "sd_op_attention_prepare": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_void_p, c_float, c_u64,

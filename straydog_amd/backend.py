@@ -153,6 +153,15 @@ class Backend:
     def rms_norm(self, x, weight, rows, width, eps, out):
         self.check(self.lib.sd_op_rms_norm(self.handle, x, weight, rows, width, eps, out))
 
+    def norm_rope(self, x, weight, rows, width, eps, rope_dims, positions, frequencies, out_rows, out, out_count):
+        self.check(self.lib.sd_op_norm_rope(self.handle, x, weight, rows, width, eps, rope_dims, positions, frequencies, out_rows, out, out_count))
+
+    def attention_turns_reserve(self, rows, rope_dims):
+        self.check(self.lib.sd_attention_turns_reserve(self.handle, rows, rope_dims))
+
+    def attention_turns_arm(self, rows):
+        self.check(self.lib.sd_attention_turns_arm(self.handle, rows))
+
     def rope_halves(self, x, rows, vectors, width, rope_dims, positions, frequencies):
         self.check(self.lib.sd_op_rope_halves(self.handle, x, rows, vectors, width, rope_dims, positions, frequencies))
 

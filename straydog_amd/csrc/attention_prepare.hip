@@ -4,6 +4,9 @@
 //   sd_op_rope_halves       pairs (i, i + pairs) turned, angles in double   gpu/token_mixing.hpp:254-274, :639-650
 //   sd_op_scatter           rows to the rows an index list names            gpu/ops.hpp:1171-1175, gpu/kernels.cpp:5244-5252
 //   sd_op_attention_prepare all of it for one step in one launch            gpu/token_mixing.hpp:276-338, :601-626
+//   sd_op_norm_rope         rms norm, then the last values turned in adjacent pairs, rows scattered; fills the attention rope
+//                           table when one is armed                          gpu/ops.hpp:60-106, gpu/kernels.cpp:4915-4940
+//   sd_attention_turns_reserve / _arm   that table                          gpu/kernels.cpp:558-616, :5288-5303
 // The fused entry gives the bits of the separate ones (the reference's own test of it, tests/fused_gpu.rs:225-268): the sum of
 // squares is formed per thread over the columns c = t, t + 256, ... by fused multiply-adds and then over the 256 threads in
 // halving-tree order, the scale is rsqrt of the mean plus eps, a value is (x * scale) * weight, and a pair is turned by
@@ -109,6 +112,41 @@ __global__ void __launch_bounds__(THREADS) prepare_kernel(const float* q_full, f
     }
 }
 
+// rms norm of row blockIdx.x, its last 2 * pairs values turned in adjacent pairs, stored at row rows[blockIdx.x] of the output
+// (the row itself without `rows`).  With a table the turns go there too: forward, and the inverse from the angle times -1.
+__global__ void __launch_bounds__(THREADS) norm_rope_kernel(const float* input, const float* weight, size_t width, float eps, size_t pairs,
+                                                            const int32_t* positions, const float* frequencies, const int32_t* rows, float* output,
+                                                            size_t out_count, double2* forward, double2* inverse) {
+    __shared__ float sums[THREADS];
+    const size_t index = blockIdx.x;
+    const float* row = input + index * width;
+    const int64_t target = rows ? int64_t(rows[index]) : int64_t(index);
+    const bool stored = target >= 0 && size_t(target) < out_count;      // a row outside the output is not stored (its table entry is)
+    float* out = output + (stored ? size_t(target) : 0) * width;
+    float sum = 0.0f;
+    for (size_t col = threadIdx.x; col < width; col += THREADS) sum = fmaf(row[col], row[col], sum);
+    const float scale = rsqrtf(tree_sum(sum, sums, THREADS) / float(width) + eps);
+    const size_t plain = width - 2 * pairs;
+    if (stored)
+        for (size_t col = threadIdx.x; col < plain; col += THREADS) out[col] = row[col] * scale * weight[col];
+    for (size_t pair = threadIdx.x; pair < pairs; pair += THREADS) {
+        const size_t col = plain + 2 * pair;
+        const double angle = double(positions[index]) * double(frequencies[pair]);
+        double s, c;
+        sincos(angle, &s, &c);
+        const double a = row[col] * scale * weight[col], b = row[col + 1] * scale * weight[col + 1];
+        if (stored) {
+            out[col] = float(a * c - b * s);
+            out[col + 1] = float(a * s + b * c);
+        }
+        if (forward) {
+            forward[index * pairs + pair] = make_double2(c, s);
+            sincos(angle * -1.0, &s, &c);
+            inverse[index * pairs + pair] = make_double2(c, s);
+        }
+    }
+}
+
 unsigned launch_dim(uint64_t count, uint64_t most) {
     if (!count || count > most) throw std::runtime_error("Straydog op: a launch is out of range");
     return unsigned(count);
@@ -136,6 +174,55 @@ int sd_op_rms_norm(void* handle, const float* input, const float* weight, uint64
     op_span(value, weight, checked_floats({width}), "a norm weight");
     op_span(value, output, checked_floats({rows, width}), "a norm output");
     rms_norm_kernel<<<launch_dim(rows, 0x7fffffffu), THREADS, 0, value.stream>>>(input, weight, size_t(width), eps, output);
+    SD_OP_END
+}
+
+int sd_op_norm_rope(void* handle, const float* input, const float* weight, uint64_t rows, uint64_t width, float eps, uint64_t rope_dims,
+                    const int32_t* positions, const float* frequencies, const int32_t* out_rows, float* out, uint64_t out_count) {
+    SD_OP_BEGIN
+    if (!rows || !width || rope_dims % 2 || rope_dims > width || (!out_rows && out_count < rows)) throw std::runtime_error("invalid Straydog norm shape");
+    op_span(value, input, checked_floats({rows, width}), "a norm input");
+    op_span(value, weight, checked_floats({width}), "a norm weight");
+    if (rope_dims) {
+        op_span(value, positions, checked_floats({rows}), "rope positions");
+        op_span(value, frequencies, checked_floats({rope_dims / 2}), "rope frequencies");
+    }
+    op_span(value, out, checked_floats({out_count, width}), "a norm output");
+    if (out_rows) {
+        op_span(value, out_rows, checked_floats({rows}), "output rows");
+        if (out == input) throw std::runtime_error("a scattered norm cannot run in place");
+    }
+    // an armed table of exactly these rows and pairs is filled by this launch (the arm is spent either way)
+    const size_t pairs = size_t(rope_dims / 2), armed = value.turns_armed;
+    value.turns_armed = 0;
+    const bool publish = armed && armed == rows && pairs && pairs == value.turns_pairs && value.turns && value.turns_rows >= rows;
+    norm_rope_kernel<<<launch_dim(rows, 0x7fffffffu), THREADS, 0, value.stream>>>(input, weight, size_t(width), eps, pairs, positions, frequencies,
+                                                                                 out_rows, out, size_t(out_count), publish ? value.turns : nullptr,
+                                                                                 publish ? value.turns + value.turns_rows * value.turns_pairs : nullptr);
+    if (publish) { value.turns_ready = true; value.turns_ready_rows = size_t(rows); value.turns_ready_pairs = pairs; }
+    SD_OP_END
+}
+
+int sd_attention_turns_reserve(void* handle, uint64_t rows, uint64_t rope_dims) {
+    SD_OP_BEGIN
+    if (rope_dims > 128 || rope_dims % 2) throw std::runtime_error("invalid Straydog attention rope");
+    const size_t pairs = size_t(rope_dims / 2);
+    if (rows && pairs && !(value.turns && value.turns_pairs == pairs && value.turns_rows >= rows)) {
+        if (value.turns) {
+            SD_CHECK(hipStreamSynchronize(value.stream));
+            release(value, value.turns);
+            value.turns = nullptr;
+        }
+        value.turns = static_cast<double2*>(allocate(value, checked_product({rows, uint64_t(pairs), sizeof(double2), 2}), false));
+        value.turns_rows = size_t(rows); value.turns_pairs = pairs; value.turns_armed = 0; value.turns_ready = false;
+    }
+    SD_OP_END
+}
+
+int sd_attention_turns_arm(void* handle, uint64_t rows) {
+    SD_OP_BEGIN
+    value.turns_armed = size_t(rows);
+    value.turns_ready = false;
     SD_OP_END
 }
 

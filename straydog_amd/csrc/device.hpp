@@ -51,6 +51,12 @@ struct Device {
     void* sequence_input = nullptr; size_t sequence_input_bytes = 0;
     void* sequence_output = nullptr; size_t sequence_output_bytes = 0;
     void* workspace = nullptr; size_t workspace_bytes = 0;
+    // The attention rope table of a pass (sd_attention_turns_reserve / _arm): forward[row][pair] = (cosine, sine), then the
+    // inverse turns at the same stride.  Armed for `turns_armed` rows, the next sd_op_norm_rope of that many rows fills it;
+    // ready, the next sd_op_sparse_attention of those rows reads it instead of forming the angles again.
+    double2* turns = nullptr;
+    size_t turns_rows = 0, turns_pairs = 0, turns_armed = 0, turns_ready_rows = 0, turns_ready_pairs = 0;
+    bool turns_ready = false;
     std::vector<hipEvent_t> events;
     // Optional kernel timing for harnesses (sdx_profile): event pairs around the launches of the op's main kernel.
     bool profile = false;

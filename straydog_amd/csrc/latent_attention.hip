@@ -34,6 +34,7 @@ struct LatentArgs {
     size_t heads, kdim, vdim;
     float scale;
     size_t pairs; const float* frequencies;
+    const double2* forward; const double2* inverse;   // the pass's rope table (cosine, sine per row and pair), or null: angles formed here
     float* out;
 };
 
@@ -65,7 +66,8 @@ __global__ void __launch_bounds__(THREADS) latent_attention_kernel(LatentArgs a)
         if (c >= rotated) {
             const size_t pair = (c - rotated) / 2;
             double s, co;
-            sincos(double(p) * double(a.frequencies[pair]), &s, &co);
+            if (a.forward) { const double2 turn = a.forward[row * a.pairs + pair]; co = turn.x; s = turn.y; }
+            else sincos(double(p) * double(a.frequencies[pair]), &s, &co);
             const double x = load(rotated + 2 * pair), y = load(rotated + 2 * pair + 1);
             value = (c - rotated) & 1 ? float(x * s + y * co) : float(x * co - y * s);
         }
@@ -150,7 +152,8 @@ __global__ void __launch_bounds__(THREADS) latent_attention_kernel(LatentArgs a)
         if (c >= back) {
             const size_t pair = (c - back) / 2;
             double s, co;
-            sincos(double(p) * double(a.frequencies[pair]) * -1.0, &s, &co);
+            if (a.inverse) { const double2 turn = a.inverse[row * a.pairs + pair]; co = turn.x; s = turn.y; }
+            else sincos(double(p) * double(a.frequencies[pair]) * -1.0, &s, &co);
             const double x = rows_out[h * a.vdim + back + 2 * pair], y = rows_out[h * a.vdim + back + 2 * pair + 1];
             value = (c - back) & 1 ? float(x * s + y * co) : float(x * co - y * s);
         }
@@ -199,6 +202,12 @@ int sd_op_sparse_attention(void* handle, const float* q, const float* raw, uint6
     args.compressed = state_base(compressed); args.selected = selected; args.selections = size_t(selections); args.sinks = sinks;
     args.heads = size_t(heads); args.kdim = args.vdim = size_t(dim); args.scale = scale; args.pairs = size_t(rope_dims / 2);
     args.frequencies = frequencies; args.out = out;
+    // a table that sd_op_norm_rope filled for exactly these rows stands in for the angles (gpu/kernels.cpp:5349-5361); it serves once
+    if (args.pairs && value.turns_ready && value.turns_ready_rows == size_t(rows) && value.turns_ready_pairs == args.pairs) {
+        args.forward = value.turns;
+        args.inverse = value.turns + value.turns_rows * value.turns_pairs;
+    }
+    value.turns_ready = false;
     launch(value, args, size_t(rows), size_t(window + selections), state_bf16(compressed));
     SD_OP_END
 }

@@ -92,3 +92,79 @@ def test_shapes_that_overflow_are_refused(gpu):
     with pytest.raises(StraydogError, match="outside"):
         gpu.rms_norm(b, f, 1, 257, 1e-6, b)                      # the weight holds 256 values
     gpu.release(buffer); gpu.release(floats)
+
+
+def test_norm_rope_matches_its_ops_and_scatters(gpu):
+    # sd_op_norm_rope == sd_op_rms_norm then sd_op_rope (the last rope_dims values, adjacent pairs), rows stored where out_rows says
+    rng = np.random.default_rng(31)
+    rows, width, rope_dims, out_count = 6, 576, 64, 9
+    x = (rng.standard_normal((rows, width)) * 3).astype(np.float32)
+    weight = (rng.standard_normal(width) * 2).astype(np.float32)
+    positions = np.array([70001, 3, 0, 123456, 9, 77], dtype=np.int32)
+    frequencies = (1.6e5 ** (-(2.0 * np.arange(rope_dims // 2)) / rope_dims)).astype(np.float32)
+    out_rows = np.array([4, 0, 8, 2, 11, -1], dtype=np.int32)            # the last two lie outside the output: not stored
+    xb, wb, pb, fb, rb = (gpu.upload(a) for a in (x, weight, positions, frequencies, out_rows))
+    apart = gpu.buffer(rows * width * 4)
+    gpu.rms_norm(xb.base(), wb.base(), rows, width, 1e-6, apart.base())
+    gpu.rope(apart.base(), rows, 1, width, rope_dims, pb.base(), fb.base())
+    want = _read(gpu, apart, rows * width).reshape(rows, width)
+    fused = gpu.buffer(rows * width * 4)
+    gpu.norm_rope(xb.base(), wb.base(), rows, width, 1e-6, rope_dims, pb.base(), fb.base(), None, fused.base(), rows)
+    assert np.array_equal(_read(gpu, fused, rows * width).view(np.uint32), want.reshape(-1).view(np.uint32))
+    canary = np.full((out_count, width), -3.25, dtype=np.float32)
+    spread = gpu.upload(canary)
+    gpu.norm_rope(xb.base(), wb.base(), rows, width, 1e-6, rope_dims, pb.base(), fb.base(), rb.base(), spread.base(), out_count)
+    got = _read(gpu, spread, out_count * width).reshape(out_count, width)
+    for r in range(rows):
+        if 0 <= out_rows[r] < out_count:
+            assert np.array_equal(got[out_rows[r]], want[r])
+            canary[out_rows[r]] = want[r]
+    assert np.array_equal(got, canary), "rows that no index names are left alone"
+    from straydog_amd.backend import StraydogError
+    with pytest.raises(StraydogError, match="in place"):
+        gpu.norm_rope(xb.base(), wb.base(), rows, width, 1e-6, rope_dims, pb.base(), fb.base(), rb.base(), xb.base(), rows)
+    for b in (xb, wb, pb, fb, rb, apart, fused, spread):
+        gpu.release(b)
+
+
+def test_attention_rope_table_serves_the_next_attention_once(gpu):
+    # sd_attention_turns_reserve / _arm: the norm of the pass's rows writes the table, the next sd_op_sparse_attention of those rows
+    # reads it (the same bits as forming the angles), and only that one
+    rng = np.random.default_rng(32)
+    rows, heads, dim, window, n, selections, rope_dims = 3, 8, 128, 8, 40, 12, 64
+    q = rng.standard_normal((rows, heads, dim)).astype(np.float32)
+    raw = rng.standard_normal((window, dim)).astype(np.float32)
+    compressed = rng.standard_normal((n, dim)).astype(np.float32)
+    positions = np.array([70001, 5, 131], dtype=np.int32)
+    elsewhere = np.array([11, 70001, 5], dtype=np.int32)
+    selected = np.stack([rng.permutation(n)[:selections] for _ in range(rows)]).astype(np.int32)
+    sinks = rng.standard_normal(heads).astype(np.float32)
+    frequencies = (1.6e5 ** (-(2.0 * np.arange(rope_dims // 2)) / rope_dims)).astype(np.float32)
+    side = rng.standard_normal((rows, dim)).astype(np.float32)           # the rows whose norm fills the table
+    qb, rb, cb, pb, eb, sb, kb, fb, nb = (gpu.upload(a) for a in (q, raw, compressed, positions, elsewhere, selected, sinks, frequencies, side))
+    weight = gpu.upload(np.ones(dim, dtype=np.float32))
+    out, normed = gpu.buffer(q.size * 4), gpu.buffer(side.size * 4)
+
+    def attend():
+        gpu.sparse_attention(qb.base(), rb.base(), window, pb.base(), window, cb.base(), n, sb.base(), selections, kb.base(), rows, heads, dim,
+                             float(1.0 / np.sqrt(dim)), rope_dims, fb.base(), None, out.base())
+        return _read(gpu, out, q.size).copy()
+    plain = attend()
+    gpu.attention_turns_reserve(rows, rope_dims)
+    gpu.attention_turns_arm(rows)
+    gpu.norm_rope(nb.base(), weight.base(), rows, dim, 1e-6, rope_dims, pb.base(), fb.base(), None, normed.base(), rows)
+    assert np.array_equal(attend().view(np.uint32), plain.view(np.uint32)), "the table's turns are the angles' own"
+    # a table filled for other positions shows that it is what the next attention reads, and that the one after does not
+    gpu.attention_turns_arm(rows)
+    gpu.norm_rope(nb.base(), weight.base(), rows, dim, 1e-6, rope_dims, eb.base(), fb.base(), None, normed.base(), rows)
+    assert not np.array_equal(attend(), plain)
+    assert np.array_equal(attend().view(np.uint32), plain.view(np.uint32))
+    # an arm for another number of rows is spent without a table
+    gpu.attention_turns_arm(rows + 1)
+    gpu.norm_rope(nb.base(), weight.base(), rows, dim, 1e-6, rope_dims, eb.base(), fb.base(), None, normed.base(), rows)
+    assert np.array_equal(attend().view(np.uint32), plain.view(np.uint32))
+    from straydog_amd.backend import StraydogError
+    with pytest.raises(StraydogError, match="rope"):
+        gpu.attention_turns_reserve(rows, 130)
+    for b in (qb, rb, cb, pb, eb, sb, kb, fb, nb, weight, out, normed):
+        gpu.release(b)
