@@ -85,6 +85,12 @@ int sd_op_sparse_attention(void* handle, const float* q, const float* raw, uint6
                            const float* compressed, uint64_t compressed_rows, const int32_t* selected, uint64_t selections,
                            const float* sinks, uint64_t rows, uint64_t heads, uint64_t dim, float scale, uint64_t rope_dims,
                            const float* frequencies, float* scratch, uint64_t scratch_bytes, float* out);
+/* reference straydog_gpu.h:399-406 (gpu/dspark_attention.hpp:1-101): DSpark's noncausal block attention.  q/out [slots][heads][512]
+ * (1..64 heads, 1..5 slots), K = V ring [128][512], block keys [slots][512], sinks [heads]; rope already applied.  Every query sees
+ * the history positions [anchor - history, anchor) (row p % 128 of the ring) and all the block's keys; scale 1/sqrt(512); the sink
+ * enters the maximum and the denominator only.  anchor_at, when not null, is a device-resident anchor that replaces `anchor`. */
+int sd_op_dspark_attention(void* handle, const float* q, const float* ring, const float* block, const float* sinks, uint64_t heads, uint64_t slots,
+                           uint32_t anchor, const int32_t* anchor_at, uint64_t history, float* out);
 /* reference straydog_gpu.h:271 (gpu/kernels.cpp:4942-4956, kernel gpu/ops.hpp:107-120): the last rope_dims values of each of
  * a row's `vectors` vectors of `width` rotated in adjacent pairs by positions[row] * frequencies[pair] (sine and cosine in
  * double); inverse: by the angle times -1. */

@@ -73,6 +73,7 @@ _latent = _sig("sdo_latent_attention", None, _vp, _vp, _sz, _vp, _sz, _vp, ctype
                ctypes.c_float, _sz, _vp, _vp, _vp, ctypes.c_int)
 _compress = _sig("sdo_compress", None, _vp, _vp, _sz, _sz, _sz, _vp)
 _qsa_select = _sig("sdo_qsa_select", _sz, _vp, _sz, _sz, _vp)
+_dspark = _sig("sdo_dspark_attention", None, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp)
 _rms_norm = _sig("sdo_rms_norm", None, _vp, _vp, _sz, _sz, ctypes.c_float, _vp)
 _rope_halves = _sig("sdo_rope_halves", None, _vp, _sz, _sz, _sz, _sz, _vp, _vp)
 _attention_prepare = _sig("sdo_attention_prepare", None, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp, ctypes.c_float, _sz, _vp, _vp, _vp, _vp,
@@ -286,6 +287,13 @@ def qsa_select(scores, position, keep_blocks=512):
     out = np.zeros(keep_blocks * 4 + 4 + max(0, position + 1), dtype=np.float32)
     count = _qsa_select(_ptr(scores), position, keep_blocks, _ptr(out))
     return out[:count].copy()
+
+
+def dspark_attention(q, ring, block, sinks, heads, slots, anchor, history):
+    q, ring, block, sinks = _f32(q), _f32(ring), _f32(block), _f32(sinks)
+    out = np.zeros(slots * heads * 512, dtype=np.float64)
+    _dspark(_ptr(q), _ptr(ring), _ptr(block), _ptr(sinks), heads, slots, anchor, history, _ptr(out))
+    return out
 
 
 def rms_norm(x, weight, eps):

@@ -799,6 +799,39 @@ void sdo_attention_prepare(const float* q_full, float* k, const float* v, size_t
     }
 }
 
+/* ------------------------------------------------------------------ DSpark block attention */
+
+/* dspark_attention.hpp:1-101, in double as the reference's own test states it (crates/straydog-engine/tests/dspark_attention_gpu.rs:
+ * 26-40): the keys are the ring rows of positions [anchor - history, anchor) (row p % 128) and all the block's keys; the head's sink
+ * enters the maximum and the denominator only. */
+void sdo_dspark_attention(const float* q, const float* ring, const float* block, const float* sinks, size_t heads, size_t slots,
+                          size_t anchor, size_t history, double* out) {
+    const size_t dim = 512, total = history + slots;
+    double scores[128 + 5];
+    for (size_t row = 0; row < slots * heads; ++row) {
+        const float* query = q + row * dim;
+        const double sink = sinks[row % heads];
+        double top = sink;
+        for (size_t i = 0; i < total; ++i) {
+            const float* key = i < history ? ring + ((anchor - history + i) % 128) * dim : block + (i - history) * dim;
+            double dot = 0.0;
+            for (size_t d = 0; d < dim; ++d) dot += (double)query[d] * (double)key[d];
+            scores[i] = dot / sqrt((double)dim);
+            if (scores[i] > top) top = scores[i];
+        }
+        double denominator = exp(sink - top);
+        for (size_t i = 0; i < total; ++i) { scores[i] = exp(scores[i] - top); denominator += scores[i]; }
+        for (size_t d = 0; d < dim; ++d) {
+            double sum = 0.0;
+            for (size_t i = 0; i < total; ++i) {
+                const float* key = i < history ? ring + ((anchor - history + i) % 128) * dim : block + (i - history) * dim;
+                sum += scores[i] * (double)key[d];
+            }
+            out[row * dim + d] = sum / denominator;
+        }
+    }
+}
+
 /* ------------------------------------------------------------------ seeded inputs */
 
 static inline uint64_t xorshift64(uint64_t* s) { *s ^= *s << 13; *s ^= *s >> 7; *s ^= *s << 17; return *s; }

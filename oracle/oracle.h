@@ -20,7 +20,8 @@
  * sdo_qsa_block_scores (exact rational arithmetic rounded once per fused step, in pure Python, + float64 closed form),
  * sdo_qsa_normalize / sdo_qsa_pool (float64 closed form; rotation invariants: pair norms kept, position 0 and columns
  * from 64 on unturned; the ring's contents), sdo_rms_norm / sdo_rope_halves / sdo_attention_prepare (float64 closed forms; a
- * rotation keeps pair norms; the fused step equals its parts).
+ * rotation keeps pair norms; the fused step equals its parts), sdo_dspark_attention (the known answers of the reference's test,
+ * dspark_attention_gpu.rs:101-124, + float64 numpy).
  * PARITY UNPINNED: none of the above; bit-level agreement with the reference's device summation
  * order inside its flash kernels is not claimed anywhere (tolerance-based, see the tests).
  */
@@ -145,6 +146,11 @@ void sdo_rope_halves(float* x, size_t rows, size_t vectors, size_t width, size_t
 void sdo_attention_prepare(const float* q_full, float* k, const float* v, size_t rows, size_t heads, size_t kv_heads, size_t dim,
                            const float* q_weight, const float* k_weight, float eps, size_t rope_dims, const int32_t* positions,
                            const float* frequencies, float* q, float* gate, float* keys, float* values, size_t context);
+
+/* ---- DSpark's noncausal block attention in double: gpu/dspark_attention.hpp:1-101; the statement of
+ * crates/straydog-engine/tests/dspark_attention_gpu.rs:26-40.  q/out [slots][heads][512], ring [128][512], block [slots][512]. */
+void sdo_dspark_attention(const float* q, const float* ring, const float* block, const float* sinks, size_t heads, size_t slots,
+                          size_t anchor, size_t history, double* out);
 
 /* ---- Seeded inputs: xorshift64 (crates/straydog-engine/tests/fused_gpu.rs:39-53) -> Box-Muller
  *      (gpu/tests/qsa_interval_test.cpp:12-18). */

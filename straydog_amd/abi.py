@@ -56,6 +56,7 @@ SIGNATURES = {
                                    c_void_p, c_void_p, c_void_p, c_u64, c_void_p, c_void_p, c_u64, c_u64]),
     "sd_op_to_bf16": (c_int, [c_void_p, c_void_p, c_u64, c_void_p]),
     # straydog_gpu_ext.h
+    "sd_op_dspark_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, ctypes.c_uint32, c_void_p, c_u64, c_void_p]),
     "sd_op_split": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_void_p, c_void_p]),
     "sd_op_rms_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_float, c_void_p]),
     "sd_op_norm_rope": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_float, c_u64, c_void_p, c_void_p, c_void_p, c_void_p, c_u64]),

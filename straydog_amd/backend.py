@@ -120,6 +120,9 @@ class Backend:
                                                    selected, selections, sinks, rows, heads, dim, scale, rope_dims, frequencies,
                                                    scratch.pointer if scratch else None, scratch.size if scratch else 0, out))
 
+    def dspark_attention(self, q, ring, block, sinks, heads, slots, anchor, anchor_at, history, out):
+        self.check(self.lib.sd_op_dspark_attention(self.handle, q, ring, block, sinks, heads, slots, anchor, anchor_at, history, out))
+
     def rope(self, x, rows, vectors, width, rope_dims, positions, frequencies, inverse=False):
         self.check(self.lib.sd_op_rope(self.handle, x, rows, vectors, width, rope_dims, positions, frequencies, int(inverse)))
 

@@ -177,7 +177,84 @@ void launch(Device& d, const LatentArgs& args, size_t rows, size_t total_keys, b
 
 }  // namespace
 
+namespace {
+
+// DSpark's noncausal block attention (reference gpu/dspark_attention.hpp:1-101): every query of the block sees the history
+// positions [anchor - history, anchor) of the K = V ring of 128 rows and all the block's keys, 512 columns, scale 1/sqrt(512),
+// the head's sink in the maximum and the denominator only.  A workgroup per (query, head): at most 133 keys, so a wave takes
+// every fourth key with its lanes across the columns (two 16-byte loads a lane, a wave-wide sum), the weights are formed a
+// thread per key, and the output two columns a thread over the keys in order.
+constexpr size_t DSPARK_DIM = 512, DSPARK_RING = 128, DSPARK_MOST = DSPARK_RING + 5;
+__global__ void __launch_bounds__(256) dspark_attention_kernel(const float* q, const float* ring, const float* block, const float* sinks, size_t heads,
+                                                               size_t slots, uint32_t anchor, const int32_t* anchor_at, size_t window, float scale,
+                                                               float* out) {
+    __shared__ __align__(16) float qs[DSPARK_DIM];
+    __shared__ float scores[DSPARK_MOST];
+    const size_t row = blockIdx.x / heads, head = blockIdx.x % heads;
+    const unsigned t = threadIdx.x, lane = t % 64, wave = t / 64;
+    const int64_t p = int64_t(anchor_at ? anchor_at[0] : int32_t(anchor)) - 1;
+    const int64_t first = p - int64_t(window) + 1 < 0 ? 0 : p - int64_t(window) + 1;
+    const size_t raw_count = size_t(p - first + 1), total = raw_count + slots;
+    const float* query = q + (row * heads + head) * DSPARK_DIM;
+    for (size_t i = t; i < DSPARK_DIM; i += 256) qs[i] = query[i];
+    __syncthreads();
+    const auto key = [&](size_t index) {
+        return index < raw_count ? ring + size_t(first + int64_t(index)) % DSPARK_RING * DSPARK_DIM : block + (index - raw_count) * DSPARK_DIM;
+    };
+    for (size_t index = wave; index < total; index += 4) {
+        const float* k = key(index) + 8 * lane;
+        const float4 k0 = *reinterpret_cast<const float4*>(k), k1 = *reinterpret_cast<const float4*>(k + 4);
+        const float4 q0 = *reinterpret_cast<const float4*>(qs + 8 * lane), q1 = *reinterpret_cast<const float4*>(qs + 8 * lane + 4);
+        float dot = q0.x * k0.x;
+        dot = fmaf(q0.y, k0.y, dot); dot = fmaf(q0.z, k0.z, dot); dot = fmaf(q0.w, k0.w, dot);
+        dot = fmaf(q1.x, k1.x, dot); dot = fmaf(q1.y, k1.y, dot); dot = fmaf(q1.z, k1.z, dot); dot = fmaf(q1.w, k1.w, dot);
+        #pragma unroll
+        for (int offset = 32; offset; offset /= 2) dot += __shfl_xor(dot, offset);
+        if (lane == 0) scores[index] = dot * scale;
+    }
+    __syncthreads();
+    float top = sinks[head];
+    for (size_t index = 0; index < total; ++index) top = fmaxf(top, scores[index]);
+    __syncthreads();
+    if (t < total) scores[t] = scores[t] == -INFINITY ? 0.0f : expf(scores[t] - top);
+    __syncthreads();
+    float denominator = 0.0f;
+    for (size_t index = 0; index < total; ++index) denominator += scores[index];
+    denominator += expf(sinks[head] - top);
+    const size_t dim = 2 * size_t(t);
+    float a0 = 0.0f, a1 = 0.0f;
+    #pragma unroll 8
+    for (size_t index = 0; index < total; ++index) {
+        const float w = scores[index];
+        const float2 v = *reinterpret_cast<const float2*>(key(index) + dim);
+        a0 = w == 0.0f ? a0 : fmaf(w, v.x, a0);
+        a1 = w == 0.0f ? a1 : fmaf(w, v.y, a1);
+    }
+    float* o = out + (row * heads + head) * DSPARK_DIM;
+    o[dim] = a0 / denominator;
+    o[dim + 1] = a1 / denominator;
+}
+
+}  // namespace
+
 extern "C" {
+
+int sd_op_dspark_attention(void* handle, const float* q, const float* ring, const float* block, const float* sinks, uint64_t heads, uint64_t slots,
+                           uint32_t anchor, const int32_t* anchor_at, uint64_t history, float* out) {
+    SD_OP_BEGIN
+    if (!heads || heads > 64 || !slots || slots > 5 || history > DSPARK_RING || anchor > uint32_t(INT32_MAX) || history > anchor)
+        throw std::runtime_error("invalid DSpark attention block or history range");
+    op_span(value, q, checked_floats({slots, heads, uint64_t(DSPARK_DIM)}), "DSpark rotated queries");
+    op_span(value, ring, DSPARK_RING * DSPARK_DIM * 4, "DSpark history K ring");
+    op_span(value, block, checked_floats({slots, uint64_t(DSPARK_DIM)}), "DSpark rotated block keys");
+    op_span(value, sinks, checked_floats({heads}), "DSpark attention sinks");
+    op_span(value, out, checked_floats({slots, heads, uint64_t(DSPARK_DIM)}), "DSpark attention output");
+    if (anchor_at) op_span(value, anchor_at, 4, "DSpark anchor position");
+    // p = anchor - 1 and a window of `history` give exactly [anchor - history, anchor); anchor = history = 0 gives no ring keys
+    dspark_attention_kernel<<<unsigned(slots * heads), 256, 0, value.stream>>>(q, ring, block, sinks, size_t(heads), size_t(slots), anchor, anchor_at,
+                                                                              size_t(history), 1.0f / sqrtf(float(DSPARK_DIM)), out);
+    SD_OP_END
+}
 
 int sd_op_sparse_attention(void* handle, const float* q, const float* raw, uint64_t raw_rows, const int32_t* positions, uint64_t window,
                            const float* compressed, uint64_t compressed_rows, const int32_t* selected, uint64_t selections,

@@ -372,3 +372,57 @@ def test_batched_sparse_path_small(gpu, oracle):
         assert np.abs(got[b] - want[0]).max() < 5e-5
     for b in (qb, kb, wb, vb, scores, indices, ab, lb, out):
         gpu.release(b)
+
+
+def _dspark_check(label, actual, expected):
+    # the reference's own bar (dspark_attention_gpu.rs:41-50): |a - b| / (1 + |b|) <= 2e-5
+    error = np.abs(actual.astype(np.float64) - expected) / (1.0 + np.abs(expected))
+    assert error.max() <= 2e-5, f"{label}: {error.max():.3e}"
+
+
+def test_dspark_block_attention(gpu, oracle):
+    # crates/straydog-engine/tests/dspark_attention_gpu.rs:52-124: 1..5 slots x histories 0, 37, 128 against the F64 statement, half the
+    # heads, an anchor that moves on the device, the refusals, and the observable key set and sink mass
+    from test_oracle_attention import _dspark_inputs
+    from straydog_amd.backend import StraydogError
+    q, ring, block, sinks = _dspark_inputs()
+    qb, rb, bb, sb = (gpu.upload(a) for a in (q, ring, block, sinks))
+    out = gpu.buffer(q.size * 4)
+    for slots in range(1, 6):
+        for history, anchor in ((0, 0), (37, 149), (128, 389)):
+            gpu.dspark_attention(qb.base(), rb.base(), bb.base(), sb.base(), 64, slots, anchor, None, history, out.base())
+            want = oracle.dspark_attention(q, ring, block, sinks, 64, slots, anchor, history)
+            _dspark_check(f"B={slots} H={history} anchor={anchor}", _read(gpu, out, np.float32, want.size), want)
+    for slots in (1, 4):
+        gpu.dspark_attention(qb.base(), rb.base(), bb.base(), sb.base(), 32, slots, 149, None, 37, out.base())
+        want = oracle.dspark_attention(q, ring, block, sinks, 32, slots, 149, 37)
+        _dspark_check(f"B={slots} 32 heads", _read(gpu, out, np.float32, want.size), want)
+    anchor = gpu.upload(np.array([389], dtype=np.int32))
+    for at in (389, 200, 128):
+        gpu.write_buffer(anchor, 0, np.array([at], dtype=np.int32))
+        gpu.dspark_attention(qb.base(), rb.base(), bb.base(), sb.base(), 64, 3, 389, anchor.base(), 128, out.base())
+        want = oracle.dspark_attention(q, ring, block, sinks, 64, 3, at, 128)
+        _dspark_check(f"B=3 anchor on the device at {at}", _read(gpu, out, np.float32, want.size), want)
+    for heads, slots, where, history in ((64, 0, 0, 0), (64, 6, 0, 0), (64, 1, 129, 129), (64, 1, 36, 37), (64, 1, 0xffffffff, 0), (0, 1, 0, 0),
+                                         (65, 1, 0, 0)):
+        with pytest.raises(StraydogError):
+            gpu.dspark_attention(qb.base(), rb.base(), bb.base(), sb.base(), heads, slots, where, None, history, out.base())
+    # zero queries, a ring that must never be attended, block keys of constant 1..5
+    gpu.write_buffer(qb, 0, np.zeros(q.size, np.float32))
+    gpu.write_buffer(rb, 0, np.full(ring.size, 23.0, np.float32))
+    keys = np.repeat(np.arange(1, 6, dtype=np.float32), 512)
+    gpu.write_buffer(bb, 0, keys)
+    gpu.write_buffer(sb, 0, np.zeros(64, np.float32))
+
+    def constant():
+        gpu.dspark_attention(qb.base(), rb.base(), bb.base(), sb.base(), 64, 5, 0, None, 0, out.base())
+        return _read(gpu, out, np.float32, q.size)
+    _dspark_check("five keys and one sink", constant(), np.full(q.size, 2.5))
+    keys[4 * 512:] = 11.0
+    gpu.write_buffer(bb, 0, keys)
+    _dspark_check("the last key changed", constant(), np.full(q.size, 3.5))
+    for sink, expected in ((1000.0, 0.0), (-1000.0, 4.2)):
+        gpu.write_buffer(sb, 0, np.full(64, sink, np.float32))
+        _dspark_check(f"sink={sink}", constant(), np.full(q.size, expected))
+    for b in (qb, rb, bb, sb, out, anchor):
+        gpu.release(b)

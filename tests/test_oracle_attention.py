@@ -278,3 +278,45 @@ def test_compress_matches_f64(oracle):
     want = (w * kv.reshape(groups, ratio, dim)).sum(axis=1)
     assert np.abs(got - want).max() < 1e-6
     assert np.array_equal(oracle.compress(kv[:groups], None, 1), kv[:groups])
+
+
+def _dspark_inputs(seed=0x9e3779b97f4a7c15):
+    # the generator and magnitudes of crates/straydog-engine/tests/dspark_attention_gpu.rs:9-16, 55-60
+    state = [seed]
+
+    def floats(n, scale):
+        out = np.empty(n, dtype=np.float32)
+        s = state[0]
+        for i in range(n):
+            s ^= (s << 13) & 0xffffffffffffffff
+            s ^= s >> 7
+            s ^= (s << 17) & 0xffffffffffffffff
+            out[i] = np.float32((np.float32(s >> 40) / np.float32(1 << 24) - np.float32(0.5)) * np.float32(2.0) * np.float32(scale))
+        state[0] = s
+        return out
+    q, ring, block, sinks = floats(5 * 64 * 512, 0.3), floats(128 * 512, 0.4), floats(5 * 512, 0.6), floats(64, 2.0)
+    sinks[0::16] = 30.0
+    sinks[1::16] = -30.0
+    return q, ring, block, sinks
+
+
+def test_dspark_known_answers_and_float64(oracle):
+    # the reference's own known answers (dspark_attention_gpu.rs:101-124): zero queries, block keys of constant 1..5, a sink of 0:
+    # every query sees five keys and one sink, (1+2+3+4+5)/6; a changed last key; a huge sink takes everything, a tiny one nothing
+    q, ring = np.zeros(5 * 64 * 512, np.float32), np.full(128 * 512, 23.0, np.float32)
+    block = np.repeat(np.arange(1, 6, dtype=np.float32), 512)
+    assert np.allclose(oracle.dspark_attention(q, ring, block, np.zeros(64, np.float32), 64, 5, 0, 0), 2.5, rtol=0, atol=1e-12)
+    block[4 * 512:] = 11.0
+    assert np.allclose(oracle.dspark_attention(q, ring, block, np.zeros(64, np.float32), 64, 5, 0, 0), 3.5, rtol=0, atol=1e-12)
+    assert np.allclose(oracle.dspark_attention(q, ring, block, np.full(64, 1000.0, np.float32), 64, 5, 0, 0), 0.0, atol=1e-12)
+    assert np.allclose(oracle.dspark_attention(q, ring, block, np.full(64, -1000.0, np.float32), 64, 5, 0, 0), 4.2, rtol=0, atol=1e-12)
+    # random inputs against numpy in float64, a ring that wraps
+    q, ring, block, sinks = _dspark_inputs()
+    heads, slots, anchor, history = 64, 3, 389, 128
+    got = oracle.dspark_attention(q, ring, block, sinks, heads, slots, anchor, history).reshape(slots, heads, 512)
+    keys = np.concatenate([ring.reshape(128, 512)[np.arange(anchor - history, anchor) % 128], block.reshape(5, 512)[:slots]]).astype(np.float64)
+    scores = q.reshape(5, 64, 512)[:slots].astype(np.float64) @ keys.T / np.sqrt(512.0)
+    top = np.maximum(scores.max(axis=-1), sinks.astype(np.float64)[None, :])
+    weights = np.exp(scores - top[..., None])
+    want = weights @ keys / (weights.sum(axis=-1) + np.exp(sinks.astype(np.float64)[None, :] - top))[..., None]
+    assert np.allclose(got, want, rtol=1e-12, atol=1e-14)
