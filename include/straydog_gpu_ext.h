@@ -39,6 +39,27 @@ typedef struct sdx_kv_pool {
 int sdx_kv_write(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
                  const void* keys, const void* values, int input_f16, uint64_t seqs, uint64_t span);
 
+/* A paged K/V cache kept by the library: the pool and the sequences' page tables, both in device memory, in the layout the
+ * entry points above and below take.  It stands where the reference has its K/V residency code (gpu/kv_stage.hpp:1-184: the mirror
+ * ring, the prefix stage, kv_layout / kv_prefetch) and sd_kv_grow (gpu/straydog_gpu.h:105-109): with the rows resident in HBM
+ * what is left of that is which pages a sequence owns.  Table changes are uploaded in stream order; no call waits for the device.
+ *   create    a pool of `pages` pages and a table for `sequences` sequences of up to max_context tokens (null on failure)
+ *   view      the pool struct, the device table and its stride, for sdx_kv_write / sdx_paged_attention / sdx_selected_attention
+ *   reserve   the sequence holds pages for `tokens` positions afterwards (growth without copies; "out of pages" changes nothing)
+ *   truncate  pages past `tokens` positions are given back (a rejected speculation, a rewind; 0 releases the sequence)
+ *   fork      sequence `to` (empty) starts as the first `tokens` positions of `from`: whole pages are shared by reference count,
+ *             the last, partial page is copied, so either sequence may append from position `tokens` on
+ *   usage     pages the sequence holds, pages free
+ * Destroy a cache before its device. */
+void* sdx_kv_cache_create(void* handle, uint64_t pages, uint32_t page_tokens, uint32_t kv_heads, uint32_t dim, uint32_t row_bytes,
+                          uint64_t sequences, uint64_t max_context);
+int sdx_kv_cache_destroy(void* handle, void* cache);
+int sdx_kv_cache_view(void* handle, void* cache, sdx_kv_pool* pool, const int32_t** page_table, uint64_t* table_stride);
+int sdx_kv_cache_reserve(void* handle, void* cache, uint64_t sequence, uint64_t tokens);
+int sdx_kv_cache_truncate(void* handle, void* cache, uint64_t sequence, uint64_t tokens);
+int sdx_kv_cache_fork(void* handle, void* cache, uint64_t from, uint64_t to, uint64_t tokens);
+int sdx_kv_cache_usage(void* handle, void* cache, uint64_t sequence, uint64_t* pages_held, uint64_t* pages_free);
+
 /* Causal grouped-query attention over the paged cache: the attention step of a decode (span 1), a speculative
  * verify (span <= 8) or a prefill chunk (any span), i.e. qsa_decode_parts/qsa_decode_merge, qsa_flash and
  * qsa_prompt_attention of the reference (gpu/sparse_attention_compute.hpp:41-170, :176-279,

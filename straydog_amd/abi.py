@@ -66,6 +66,13 @@ SIGNATURES = {
     "sd_op_scatter": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_void_p, c_u64]),
     "sd_op_attention_prepare": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_void_p, c_float, c_u64,
                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64]),
+    "sdx_kv_cache_create": (c_void_p, [c_void_p, c_u64, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, c_u64, c_u64]),
+    "sdx_kv_cache_destroy": (c_int, [c_void_p, c_void_p]),
+    "sdx_kv_cache_view": (c_int, [c_void_p, c_void_p, _P(KvPool), _P(c_void_p), _P(c_u64)]),
+    "sdx_kv_cache_reserve": (c_int, [c_void_p, c_void_p, c_u64, c_u64]),
+    "sdx_kv_cache_truncate": (c_int, [c_void_p, c_void_p, c_u64, c_u64]),
+    "sdx_kv_cache_fork": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64]),
+    "sdx_kv_cache_usage": (c_int, [c_void_p, c_void_p, c_u64, _P(c_u64), _P(c_u64)]),
     "sdx_kv_write": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_void_p, c_void_p, c_int, c_u64, c_u64]),
     "sdx_paged_attention_scratch": (c_u64, [c_u64, c_u64, c_u64, c_u64, c_u64]),
     "sdx_paged_attention": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_u64, c_void_p, c_int, c_u64, c_u64, c_u64,

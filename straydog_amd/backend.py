@@ -181,6 +181,33 @@ class Backend:
         buffer = self.buffer(size)
         return abi.KvPool(buffer.pointer, pages, page_tokens, kv_heads, dim, row_bytes), buffer
 
+    # ---- the paged K/V cache the library keeps ----
+    def kv_cache(self, pages, page_tokens, kv_heads, dim, row_bytes, sequences, max_context):
+        """(cache, pool struct, device page table, table stride)."""
+        cache = self.lib.sdx_kv_cache_create(self.handle, pages, page_tokens, kv_heads, dim, row_bytes, sequences, max_context)
+        if not cache:
+            raise StraydogError(self.error())
+        pool, table, stride = abi.KvPool(), ctypes.c_void_p(), abi.c_u64()
+        self.check(self.lib.sdx_kv_cache_view(self.handle, cache, ctypes.byref(pool), ctypes.byref(table), ctypes.byref(stride)))
+        return cache, pool, table.value, stride.value
+
+    def kv_cache_destroy(self, cache):
+        self.check(self.lib.sdx_kv_cache_destroy(self.handle, cache))
+
+    def kv_cache_reserve(self, cache, sequence, tokens):
+        self.check(self.lib.sdx_kv_cache_reserve(self.handle, cache, sequence, tokens))
+
+    def kv_cache_truncate(self, cache, sequence, tokens):
+        self.check(self.lib.sdx_kv_cache_truncate(self.handle, cache, sequence, tokens))
+
+    def kv_cache_fork(self, cache, source, target, tokens):
+        self.check(self.lib.sdx_kv_cache_fork(self.handle, cache, source, target, tokens))
+
+    def kv_cache_usage(self, cache, sequence=0):
+        held, free = abi.c_u64(), abi.c_u64()
+        self.check(self.lib.sdx_kv_cache_usage(self.handle, cache, sequence, ctypes.byref(held), ctypes.byref(free)))
+        return held.value, free.value
+
     def kv_write(self, pool, page_table, table_stride, positions, keys, values, input_f16, seqs, span):
         self.check(self.lib.sdx_kv_write(self.handle, ctypes.byref(pool), page_table, table_stride, positions, keys, values,
                                          int(input_f16), seqs, span))

@@ -228,3 +228,80 @@ def test_refusals(gpu):
     bad = type(pool)(buffer.pointer, 2, 33, 1, 128, 136)
     with pytest.raises(StraydogError, match="invalid Straydog K/V pool"):
         gpu.kv_write(bad, small.base(), 1, small.base(), small.base(), small.base(), False, 1, 1)
+
+
+def test_the_library_kept_cache_pages_grow_fork_and_truncate(gpu, oracle):
+    # sdx_kv_cache_*: sequences grow without copies, a fork shares whole pages and copies the partial one, a truncation gives pages
+    # back.  What the sequences hold is checked through attention against the oracle on each sequence's own logical rows.
+    from straydog_amd.backend import StraydogError
+    rng = np.random.default_rng(44)
+    page_tokens, kv_heads, dim, row_bytes, heads = 64, 2, 128, 136, 8
+    cache, pool, table, stride = gpu.kv_cache(12, page_tokens, kv_heads, dim, row_bytes, 3, 1024)
+    assert stride == 16 and gpu.kv_cache_usage(cache) == (0, 12)
+    logical = {s: (np.zeros((0, kv_heads, dim), np.float32), np.zeros((0, kv_heads, dim), np.float32)) for s in range(3)}
+
+    def append(sequence, count):
+        k = rng.standard_normal((count, kv_heads, dim)).astype(np.float32)
+        v = rng.standard_normal((count, kv_heads, dim)).astype(np.float32)
+        start = logical[sequence][0].shape[0]
+        gpu.kv_cache_reserve(cache, sequence, start + count)
+        kb, vb, pb = gpu.upload(k), gpu.upload(v), gpu.upload(np.array([start], dtype=np.int32))
+        gpu.kv_write(pool, table + sequence * stride * 4, stride, pb.base(), kb.base(), vb.base(), False, 1, count)
+        for b in (kb, vb, pb):
+            gpu.release(b)
+        logical[sequence] = (np.concatenate([logical[sequence][0], k]), np.concatenate([logical[sequence][1], v]))
+
+    def check(sequence):
+        k, v = logical[sequence]
+        length = k.shape[0]
+        q = rng.standard_normal((1, 1, heads, dim)).astype(np.float32)
+        qb, pb = gpu.upload(q), gpu.upload(np.array([length - 1], dtype=np.int32))
+        out = gpu.buffer(q.size * 4)
+        scratch = gpu.buffer(gpu.paged_attention_scratch(1, 1, heads, dim, 1024))
+        gpu.paged_attention(pool, table + sequence * stride * 4, stride, pb.base(), 1024, qb.base(), False, 1, 1, heads, 0.09, out.base(), False, scratch)
+        got = gpu.read_buffer(out, 0, np.float32, q.size).reshape(q.shape)
+        # the oracle on the sequence's rows laid out in pages of its own
+        pages = (length + page_tokens - 1) // page_tokens
+        host = np.zeros(oracle.pool_bytes(pages, kv_heads, page_tokens, row_bytes), dtype=np.uint8)
+        own = np.arange(pages, dtype=np.int32)[None, :]
+        oracle.kv_write(host, row_bytes, page_tokens, kv_heads, dim, own, np.zeros(1, np.int32), k[None], v[None])
+        want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, own, np.array([length - 1], np.int32), q, 0.09)
+        close_enough(got, want, f"sequence {sequence} of {length} tokens")
+        for b in (qb, pb, out, scratch):
+            gpu.release(b)
+
+    append(0, 200)                                   # 4 pages
+    append(0, 1)
+    check(0)
+    assert gpu.kv_cache_usage(cache, 0) == (4, 8)
+    gpu.kv_cache_fork(cache, 0, 1, 150)              # 2 whole pages shared, the third copied up to row 22
+    logical[1] = (logical[0][0][:150].copy(), logical[0][1][:150].copy())
+    assert gpu.kv_cache_usage(cache, 1) == (3, 7)
+    append(1, 70)                                    # the fork writes on from position 150; the source's rows 150.. are untouched
+    append(0, 100)
+    check(0); check(1)
+    assert gpu.kv_cache_usage(cache, 0) == (5, 5) and gpu.kv_cache_usage(cache, 1) == (4, 5)
+    gpu.kv_cache_truncate(cache, 1, 130)             # a rewind: the fork's fourth page goes back, its copy of the third stays
+    logical[1] = (logical[1][0][:130], logical[1][1][:130])
+    assert gpu.kv_cache_usage(cache, 1) == (3, 6)
+    append(1, 5)                                     # rows 130..134 land in the fork's own copy of page 3
+    check(1); check(0)
+    gpu.kv_cache_truncate(cache, 0, 0)               # the source goes: the shared pages stay with the fork
+    assert gpu.kv_cache_usage(cache, 0) == (0, 9)
+    check(1)
+    append(2, 9 * page_tokens)                       # exactly what is free
+    check(2)
+    with pytest.raises(StraydogError, match="out of pages"):
+        gpu.kv_cache_reserve(cache, 0, 1)
+    assert gpu.kv_cache_usage(cache, 0) == (0, 0)
+    with pytest.raises(StraydogError, match="max_context"):
+        gpu.kv_cache_reserve(cache, 0, 1025)
+    with pytest.raises(StraydogError, match="no such sequence"):
+        gpu.kv_cache_reserve(cache, 3, 1)
+    with pytest.raises(StraydogError, match="fork"):
+        gpu.kv_cache_fork(cache, 1, 2, 10)
+    gpu.kv_cache_destroy(cache)
+    used, _ = gpu.memory()
+    with pytest.raises(StraydogError):
+        gpu.kv_cache(0, 64, 2, 128, 136, 1, 64)
+    assert gpu.memory()[0] == used, "a refused cache leaves no allocation behind"
