@@ -187,6 +187,11 @@ def main():
                 out[name].update({"selected_attention_us": ms * 1e3, "selected_attention_kernel_us": None if kernel_ms is None else kernel_ms * 1e3,
                                   "selected_attention_gbps": work.attention_bytes() / ms / 1e6})
             work.release()
+            if rows <= 8:
+                stage = workloads.QwenStageWorkload(gpu, rows)
+                ms, _ = timed(gpu, stage.step, max(args.steps // 5, 3), 2)
+                out[name]["whole_stage_us"] = ms * 1e3        # norm + rope + K/V append + pooling, index, attention over the selection, gate
+                stage.release()
         return out
 
     if args.workload == "config4":

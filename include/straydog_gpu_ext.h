@@ -97,6 +97,33 @@ int sdx_qsa_pool(void* handle, const float* incoming, float* history, const floa
 int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, const float* blocks, uint64_t pool, uint64_t base,
                   const uint32_t* dynamic_base, uint64_t steps, uint64_t selected, float* scores, float* indices, float* counts);
 
+/* The attention stage of a Qwen decode or verification pass in one call: the reference's qsa_decode_attend / qsa_decode_attend_rows
+ * (gpu/qsa_decode.hpp:28-44, 113-129; kernel qsa_normalize_rows :86-111).  For rows r < steps (1..8) at the consecutive positions
+ * positions[r] with rope positions ropes[r], both device-resident (a recorded pass replays at the next position):
+ *   projections + r * stride holds the row's [heads x (query 256 | gate 256) | kv_heads x key 256 | kv_heads x value 256 |
+ *   4 x index query 128 | index key 128];
+ *   1. one launch: queries, keys and index queries RMS-normalised and turned (sdx_qsa_normalize's arithmetic; index queries in
+ *      place), the keys and values appended to the K/V rows at the positions (sdx_kv_write's bytes), the index keys pooled into
+ *      blocks / history row by row (sdx_qsa_pool's arithmetic);
+ *   2. sdx_qsa_index on the normalised index queries;  3. sdx_selected_attention over each row's selection with the gate.
+ * attended: [steps][heads][256] FP32.  scratch: sdx_qsa_decode_attend_scratch bytes (normalised queries, scores, selections,
+ * attention partials). */
+typedef struct sdx_qsa_state {
+    const sdx_kv_pool* kv;          /* rows of 256 columns, Q8_0 or FP16 */
+    const int32_t* page_table;      /* the sequence's pages, or null when one page holds the context (the reference's state layout) */
+    uint64_t context;
+    float* blocks;                  /* [128][context / 4 + 1] pooled index keys */
+    float* history;                 /* [16][128] the index keys' ring */
+    const float* q_norm;            /* 256 */
+    const float* k_norm;            /* 256 */
+    const float* index_q_norm;      /* 128 */
+    const float* index_k_norm;      /* 128 */
+    uint64_t heads;                 /* query heads, a multiple of the K/V heads, at most 16 each */
+} sdx_qsa_state;
+uint64_t sdx_qsa_decode_attend_scratch(uint64_t steps, uint64_t heads, uint64_t kv_heads, uint64_t context);
+int sdx_qsa_decode_attend(void* handle, const sdx_qsa_state* state, float* projections, uint64_t stride, uint64_t steps, const uint32_t* positions,
+                          const uint32_t* ropes, void* scratch, uint64_t scratch_bytes, float* attended);
+
 /* Selection-list attention over K/V rows of 256 columns (Q8_0 or FP16): the reference's qsa_attention / qsa_attention_rows
  * (gpu/sparse_attention_compute.hpp:609-647: qsa_decode_parts :41-135 + qsa_decode_merge :139-170) followed by qsa_gate
  * (gpu/sparse_attention.hpp:439-442).  Row r, at position base + r (or *dynamic_base + r, a device-resident position),
@@ -104,12 +131,12 @@ int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, con
  * reference's packed buffer hold them; an entry counts iff 0 <= raw <= position and raw < context (gpu/kernels.cpp:100-165).
  * The rows come from `pool` through page_table ([ceil(context / page_tokens)] pages of the one sequence) or, with a null
  * page_table, from a pool whose single page holds the context (which is the reference's state layout, planes x context).
- * q and out are [rows][heads][256], FP32 or FP16 each; gate (optional) is read at gate[(r * heads + h) * gate_stride + c] and
- * out *= sigmoid(gate).  heads / kv_heads <= 16.  scratch: sdx_selected_attention_scratch(rows, kv_heads, selected) bytes. */
+ * q and out are [rows][heads][256], FP32 or FP16 each; gate (optional) is read at gate[r * gate_row_stride + h * gate_stride + c]
+ * (gate_row_stride 0: heads * gate_stride) and out *= sigmoid(gate).  heads / kv_heads <= 16.  scratch: sdx_selected_attention_scratch(rows, kv_heads, selected) bytes. */
 uint64_t sdx_selected_attention_scratch(uint64_t rows, uint64_t kv_heads, uint64_t selected);
 int sdx_selected_attention(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t context, uint64_t base,
                            const uint32_t* dynamic_base, const float* indices, uint64_t selected, const float* counts, const void* q, int q_f16,
-                           uint64_t rows, uint64_t heads, float scale, const float* gate, uint64_t gate_stride, void* out, int out_f16,
+                           uint64_t rows, uint64_t heads, float scale, const float* gate, uint64_t gate_stride, uint64_t gate_row_stride, void* out, int out_f16,
                            void* scratch, uint64_t scratch_bytes);
 
 /* Top-k indexed sparse attention over BF16 latent K/V for a batch of sequences (one decode row each):

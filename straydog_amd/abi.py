@@ -22,6 +22,12 @@ class KvPool(ctypes.Structure):
 
 _P = ctypes.POINTER
 
+
+class QsaState(ctypes.Structure):
+    """sdx_qsa_state"""
+    _fields_ = [("kv", _P(KvPool)), ("page_table", c_void_p), ("context", c_u64), ("blocks", c_void_p), ("history", c_void_p), ("q_norm", c_void_p),
+                ("k_norm", c_void_p), ("index_q_norm", c_void_p), ("index_k_norm", c_void_p), ("heads", c_u64)]
+
 # name -> (restype, argtypes); the order is that of the headers
 SIGNATURES = {
     # straydog_gpu.h
@@ -82,7 +88,9 @@ SIGNATURES = {
     "sdx_qsa_index": (c_int, [c_void_p, c_void_p, c_u64, c_void_p, c_u64, c_u64, c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_void_p]),
     "sdx_selected_attention_scratch": (c_u64, [c_u64, c_u64, c_u64]),
     "sdx_selected_attention": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_u64, c_void_p, c_void_p, c_int,
-                                       c_u64, c_u64, c_float, c_void_p, c_u64, c_void_p, c_int, c_void_p, c_u64]),
+                                       c_u64, c_u64, c_float, c_void_p, c_u64, c_u64, c_void_p, c_int, c_void_p, c_u64]),
+    "sdx_qsa_decode_attend_scratch": (c_u64, [c_u64, c_u64, c_u64, c_u64]),
+    "sdx_qsa_decode_attend": (c_int, [c_void_p, _P(QsaState), c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_void_p, c_u64, c_void_p]),
     "sdx_index_score_bounds": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float, c_void_p, c_void_p]),
     "sdx_index_top_k": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float, c_void_p,
                                 c_u64, c_void_p]),

@@ -225,10 +225,23 @@ class Backend:
         return int(self.lib.sdx_selected_attention_scratch(rows, kv_heads, selected))
 
     def selected_attention(self, pool, page_table, context, base, indices, selected, counts, q, q_f16, rows, heads, scale, out, out_f16,
-                           scratch, gate=None, gate_stride=0, dynamic_base=None):
+                           scratch, gate=None, gate_stride=0, gate_row_stride=0, dynamic_base=None):
         self.check(self.lib.sdx_selected_attention(self.handle, ctypes.byref(pool), page_table, context, base, dynamic_base, indices, selected,
-                                                   counts, q, int(q_f16), rows, heads, scale, gate, gate_stride, out, int(out_f16),
+                                                   counts, q, int(q_f16), rows, heads, scale, gate, gate_stride, gate_row_stride, out, int(out_f16),
                                                    scratch.pointer, scratch.size))
+
+    def qsa_state(self, pool, page_table, context, blocks, history, q_norm, k_norm, index_q_norm, index_k_norm, heads):
+        """An sdx_qsa_state over device pointers (the pool struct is kept alive by the returned object)."""
+        state = abi.QsaState(ctypes.pointer(pool), page_table, context, blocks, history, q_norm, k_norm, index_q_norm, index_k_norm, heads)
+        state._pool = pool
+        return state
+
+    def qsa_decode_attend_scratch(self, steps, heads, kv_heads, context):
+        return int(self.lib.sdx_qsa_decode_attend_scratch(steps, heads, kv_heads, context))
+
+    def qsa_decode_attend(self, state, projections, stride, steps, positions, ropes, scratch, attended):
+        self.check(self.lib.sdx_qsa_decode_attend(self.handle, ctypes.byref(state), projections, stride, steps, positions, ropes, scratch.pointer,
+                                                  scratch.size, attended))
 
     def index_top_k(self, q_index, keys, weights, visible, batch, groups, heads, dim, scale, scores, k, indices):
         self.check(self.lib.sdx_index_top_k(self.handle, q_index, keys, weights, visible, batch, groups, heads, dim, scale, scores,

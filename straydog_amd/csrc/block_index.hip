@@ -17,6 +17,7 @@
 // beyond 32768 blocks), four 8-bit radix passes over per-wave LDS histograms (the first, where nearly all values share a digit, counted by ballots), and
 // one ordered pass whose slots come from 64-wide ballots and a scan over (run, wave) counts.
 #include "device.hpp"
+#include "kv_codec.hpp"
 #include "tree_sum.hpp"
 #include "../../include/straydog_gpu_ext.h"
 
@@ -32,38 +33,46 @@ __device__ __forceinline__ float turn(float own, float partner, unsigned column,
     return own * cosf(angle) + (column < 32 ? -partner : partner) * sinf(angle);
 }
 
+// A vector of `width` values (128 or 256), one per thread c < width: x * norm / sqrt(mean(x^2) + 1e-6), the first 64 columns turned
+// for `position`.  Every thread of the workgroup calls it (the sum has barriers); values and sums are 256 floats of LDS each.
+__device__ __forceinline__ float normalized(float x, const float* norm, unsigned width, size_t position, float* values, float* sums) {
+    const unsigned c = threadIdx.x;
+    if (c < width) values[c] = x * norm[c];
+    const float denominator = sqrtf(tree_sum(c < width ? x * x : 0.0f, sums, width) / float(width) + 1e-6f);
+    const float own = c < width ? values[c] / denominator : 0.0f;
+    const float partner = c < 64 ? values[(c + 32) % 64] / denominator : 0.0f;
+    const float value = turn(own, partner, c, position);
+    __syncthreads();        // (values may be written again at once)
+    return value;
+}
+
 // One workgroup of `width` threads per (row, head).
 __global__ void __launch_bounds__(256) normalize_kernel(const float* source, const float* norm, unsigned heads, unsigned width, size_t stride,
                                                         size_t position, float* target) {
     __shared__ float values[256], sums[256];
     const size_t head = blockIdx.x, token = head / heads;
     const unsigned c = threadIdx.x;
-    const float x = source[head * stride + c];
-    values[c] = x * norm[c];
-    const float denominator = sqrtf(tree_sum(x * x, sums, width) / float(width) + 1e-6f);
-    const float own = values[c] / denominator;
-    const float partner = c < 64 ? values[(c + 32) % 64] / denominator : 0.0f;
-    target[head * width + c] = turn(own, partner, c, position + token);
+    target[head * width + c] = normalized(source[head * stride + c], norm, width, position + token, values, sums);
+}
+
+// The mean of a block's four index-key inputs as a thread's column: taps in position order, earlier ones from the ring.
+__device__ __forceinline__ float pooled_mean(const float* incoming, size_t incoming_stride, const float* history, size_t begin, size_t base, unsigned c) {
+    float x = 0.0f;
+    #pragma unroll
+    for (size_t tap = 0; tap < 4; ++tap) {
+        const size_t pos = begin + tap;
+        x += pos < base ? history[(pos % RING) * COLUMNS + c] : incoming[(pos - base) * incoming_stride + c];
+    }
+    return x / 4.0f;
 }
 
 // One workgroup of 128 threads per block completed by the span.
 __global__ void __launch_bounds__(COLUMNS) pool_kernel(const float* incoming, const float* history, const float* norm, size_t pool, size_t base,
                                                        float* blocks) {
-    __shared__ float values[COLUMNS], sums[COLUMNS];
+    __shared__ float values[256], sums[256];
     const size_t block = base / 4 + blockIdx.x, begin = block * 4;
     const unsigned c = threadIdx.x;
-    float x = 0.0f;
-    #pragma unroll
-    for (size_t tap = 0; tap < 4; ++tap) {
-        const size_t pos = begin + tap;
-        x += pos < base ? history[(pos % RING) * COLUMNS + c] : incoming[(pos - base) * COLUMNS + c];
-    }
-    x /= 4.0f;
-    values[c] = x * norm[c];
-    const float denominator = sqrtf(tree_sum(x * x, sums, COLUMNS) / float(COLUMNS) + 1e-6f);
-    const float own = values[c] / denominator;
-    const float partner = c < 64 ? values[(c + 32) % 64] / denominator : 0.0f;
-    blocks[c * pool + block] = turn(own, partner, c, begin);
+    blocks[c * pool + block] = normalized(pooled_mean(incoming, COLUMNS, history, begin, base, c), norm, COLUMNS, begin, values, sums);
 }
 
 __global__ void __launch_bounds__(256) save_history_kernel(const float* incoming, size_t base, size_t steps, float* history) {
@@ -459,6 +468,69 @@ void launch_select(Device& d, const float* scores, size_t pool, size_t base, con
     select_kernel<REGS><<<rows, SELECT_THREADS, shared, d.stream>>>(scores, pool, base, dynamic, selected, held_runs, indices, counts);
 }
 
+// ---- a decode or verification pass's inputs in one launch --------------------------------------------------------------
+// The reference's qsa_normalize_rows (gpu/qsa_decode.hpp:86-111): blockIdx.y = row; blockIdx.x = a query head (normalised and turned
+// into `queries`), then a K/V head (the key normalised and turned, key and value rows encoded into the cache at the row's
+// position), then the four index-query heads (in place), then one workgroup that pools the index keys of all rows in turn
+// (a row completes a block from the ring the rows before it wrote).  Positions and rope positions are read on the device.
+struct StageArgs {
+    float* projections;            // row r at r * stride: heads x [query 256 | gate 256], kv x key 256, kv x value 256, 4 x index query 128, index key 128
+    size_t stride;
+    const float *q_norm, *k_norm, *index_q_norm, *index_k_norm;
+    unsigned heads, kv_heads, steps;
+    const uint32_t *positions, *ropes;
+    uint8_t* pages;
+    unsigned page_tokens, row_bytes;
+    const int32_t* page_table;
+    size_t context;
+    float* queries;                // [steps][heads][256]
+    float *blocks, *history;
+    size_t pool;
+};
+__global__ void __launch_bounds__(256) stage_prepare_kernel(StageArgs a) {
+    __shared__ float values[256], sums[256];
+    __shared__ __align__(16) float key[256];
+    const unsigned block = blockIdx.x, c = threadIdx.x;
+    const size_t row = blockIdx.y, pos = a.positions[row], rope = a.ropes[row];
+    float* own = a.projections + row * a.stride;
+    const size_t keys_at = size_t(a.heads) * 512, values_at = keys_at + size_t(a.kv_heads) * 256, index_at = keys_at + size_t(a.kv_heads) * 512;
+    if (block < a.heads) {
+        a.queries[(row * a.heads + block) * 256 + c] = normalized(own[size_t(block) * 512 + c], a.q_norm, 256, rope, values, sums);
+    } else if (block < a.heads + a.kv_heads) {
+        const unsigned head = block - a.heads;
+        key[c] = normalized(own[keys_at + head * 256 + c], a.k_norm, 256, rope, values, sums);
+        __syncthreads();
+        if (pos >= a.context || c >= 128) return;           // a position outside the cache writes no row; two waves encode
+        const size_t page = a.page_table ? size_t(a.page_table[pos / a.page_tokens]) : 0, in_page = a.page_table ? pos % a.page_tokens : pos;
+        const bool is_value = c >= 64;
+        const unsigned quad = c % 64;                       // four columns a thread: a wave holds the row, 8 lanes a 32-column block
+        uint8_t* target = a.pages + ((page * 2 * a.kv_heads + (is_value ? a.kv_heads : 0) + head) * a.page_tokens + in_page) * a.row_bytes;
+        const float* from = is_value ? own + values_at + head * 256 + 4 * quad : key + 4 * quad;
+        const float x[4] = {from[0], from[1], from[2], from[3]};
+        kv_store_quad(target, quad, 256, a.row_bytes != 512, x, true);
+    } else if (block < a.heads + a.kv_heads + HEADS) {
+        const unsigned head = block - a.heads - a.kv_heads;
+        float* vector = own + index_at + head * COLUMNS;
+        const float value = normalized(c < COLUMNS ? vector[c] : 0.0f, a.index_q_norm, COLUMNS, rope, values, sums);
+        if (c < COLUMNS) vector[c] = value;
+    } else if (row == 0) {
+        for (size_t r = 0; r < a.steps; ++r) {
+            const size_t at = a.positions[r];
+            if (c < COLUMNS) a.history[(at % RING) * COLUMNS + c] = a.projections[r * a.stride + index_at + HEADS * COLUMNS + c];
+            if ((at + 1) % 4 == 0 && at / 4 < a.pool) {
+                float x = 0.0f;
+                if (c < COLUMNS) {
+                    #pragma unroll
+                    for (size_t tap = 0; tap < 4; ++tap) x += a.history[((at - 3 + tap) % RING) * COLUMNS + c];
+                    x /= 4.0f;
+                }
+                const float value = normalized(x, a.index_k_norm, COLUMNS, size_t(a.ropes[r]) - 3, values, sums);
+                if (c < COLUMNS) a.blocks[c * a.pool + at / 4] = value;
+            }
+        }
+    }
+}
+
 template<int T>
 void launch_rows(Device& d, const float* queries, size_t stride, const float* blocks, size_t pool, size_t base, const uint32_t* dynamic, size_t steps,
                  size_t most, float* scores) {
@@ -529,6 +601,62 @@ int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, con
     if (most <= size_t(LDS_RUNS) * SELECT_THREADS) launch_select<0>(value, scores, pool, base, dynamic_base, selected, most, rows, indices, counts);
     else launch_select<33>(value, scores, pool, base, dynamic_base, selected, most, rows, indices, counts);
     SD_OP_END
+}
+
+uint64_t sdx_qsa_decode_attend_scratch(uint64_t steps, uint64_t heads, uint64_t kv_heads, uint64_t context) {
+    try {
+        const uint64_t pool = context / 4 + 1;
+        return checked_floats({steps, heads * 256 + pool + 2052 + 1}) + 256 + sdx_selected_attention_scratch(steps, kv_heads, 2052);
+    } catch (const std::exception&) { return 0; }
+}
+
+int sdx_qsa_decode_attend(void* handle, const sdx_qsa_state* state, float* projections, uint64_t stride, uint64_t steps, const uint32_t* positions,
+                          const uint32_t* ropes, void* scratch, uint64_t scratch_bytes, float* attended) {
+    {
+        SD_OP_BEGIN
+        if (!state || !state->kv) throw std::runtime_error("sdx_qsa_decode_attend: no state");
+        const sdx_kv_pool& kv = *state->kv;
+        const uint64_t heads = state->heads, context = state->context, pool = context / 4 + 1;
+        if (kv.dim != 256 || !heads || heads % kv.kv_heads || heads / kv.kv_heads > 16 || !steps || steps > 8 || !context || context > (uint64_t(1) << 24) ||
+            stride < heads * 512 + uint64_t(kv.kv_heads) * 512 + HEADS * COLUMNS + COLUMNS)
+            throw std::runtime_error("sdx_qsa_decode_attend: 1..8 rows of heads x 512 + K/V heads x 512 + 640 projections, K/V rows of 256 columns");
+        if (!state->page_table && kv.page_tokens < context) throw std::runtime_error("sdx_qsa_decode_attend: without a page table one page must hold the context");
+        if (state->page_table) op_span(value, state->page_table, checked_floats({(context + kv.page_tokens - 1) / kv.page_tokens}), "a page table");
+        op_span(value, kv.pages, checked_product({kv.page_count, 2, kv.kv_heads, kv.page_tokens, kv.row_bytes}), "a K/V pool");
+        op_span(value, state->blocks, checked_floats({pool, uint64_t(COLUMNS)}), "pooled index keys");
+        op_span(value, state->history, size_t(RING) * COLUMNS * 4, "the index history");
+        op_span(value, state->q_norm, 256 * 4, "a query norm weight");
+        op_span(value, state->k_norm, 256 * 4, "a key norm weight");
+        op_span(value, state->index_q_norm, COLUMNS * 4, "an index query norm weight");
+        op_span(value, state->index_k_norm, COLUMNS * 4, "an index key norm weight");
+        op_span(value, projections, checked_floats({steps - 1, stride}) + (heads * 512 + uint64_t(kv.kv_heads) * 512 + 640) * 4, "projections");
+        op_span(value, positions, checked_floats({steps}), "positions");
+        op_span(value, ropes, checked_floats({steps}), "rope positions");
+        op_span(value, attended, checked_floats({steps, heads, 256}), "an attention output");
+        const uint64_t need = sdx_qsa_decode_attend_scratch(steps, heads, kv.kv_heads, context);
+        if (!need || scratch_bytes < need) throw std::runtime_error("sdx_qsa_decode_attend: scratch too small (see sdx_qsa_decode_attend_scratch)");
+        op_span(value, scratch, need, "stage scratch");
+        StageArgs args{};
+        args.projections = projections; args.stride = stride;
+        args.q_norm = state->q_norm; args.k_norm = state->k_norm; args.index_q_norm = state->index_q_norm; args.index_k_norm = state->index_k_norm;
+        args.heads = unsigned(heads); args.kv_heads = kv.kv_heads; args.steps = unsigned(steps); args.positions = positions; args.ropes = ropes;
+        args.pages = static_cast<uint8_t*>(kv.pages); args.page_tokens = kv.page_tokens; args.row_bytes = kv.row_bytes; args.page_table = state->page_table;
+        args.context = context; args.queries = static_cast<float*>(scratch); args.blocks = state->blocks; args.history = state->history; args.pool = pool;
+        stage_prepare_kernel<<<dim3(unsigned(heads + kv.kv_heads + HEADS + 1), unsigned(steps)), 256, 0, value.stream>>>(args);
+        SD_CHECK(hipGetLastError());
+    } catch (const std::exception& e) { ::sd::last_error = e.what(); return -1; }
+    }
+    // the two stages behind it, on the position the device holds
+    const uint64_t heads = state->heads, pool = state->context / 4 + 1;
+    float* queries = static_cast<float*>(scratch);
+    float* scores = queries + steps * heads * 256;
+    float* indices = scores + steps * pool;
+    float* counts = indices + steps * 2052;
+    uint8_t* partial = reinterpret_cast<uint8_t*>((reinterpret_cast<uintptr_t>(counts + steps) + 255) & ~uintptr_t(255));
+    const size_t index_at = heads * 512 + size_t(state->kv->kv_heads) * 512;
+    if (sdx_qsa_index(handle, projections + index_at, stride, state->blocks, pool, 0, positions, steps, 2052, scores, indices, counts) < 0) return -1;
+    return sdx_selected_attention(handle, state->kv, state->page_table, state->context, 0, positions, indices, 2052, counts, queries, 0, steps, heads, 0.0625f,
+                                  projections + 256, 512, stride, attended, 0, partial, sdx_selected_attention_scratch(steps, state->kv->kv_heads, 2052));
 }
 
 }  // extern "C"

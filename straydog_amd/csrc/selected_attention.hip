@@ -167,7 +167,7 @@ __global__ void __launch_bounds__(WAVES * 64) selected_attention_kernel(Selected
 
 // A block per (row, head), a thread per column: the row's chunks merged, normalised, gated.
 template<bool F16_OUT>
-__global__ void __launch_bounds__(DIM) selected_merge_kernel(SelectedArgs a, const float* gate, size_t gate_stride, void* out) {
+__global__ void __launch_bounds__(DIM) selected_merge_kernel(SelectedArgs a, const float* gate, size_t gate_stride, size_t gate_row_stride, void* out) {
     constexpr int STRIDE = DIM + 2;
     const size_t row = blockIdx.x / a.heads;
     const unsigned head = blockIdx.x % a.heads, kvh = head / a.group, col = threadIdx.x;
@@ -184,7 +184,7 @@ __global__ void __launch_bounds__(DIM) selected_merge_kernel(SelectedArgs a, con
     }
     value = sum > 0.0f ? value / sum : 0.0f;
     if (gate) {
-        const float x = gate[(row * a.heads + head) * gate_stride + col], e = expf(-fabsf(x));
+        const float x = gate[row * gate_row_stride + head * gate_stride + col], e = expf(-fabsf(x));
         value *= x >= 0.0f ? 1.0f / (1.0f + e) : e / (1.0f + e);
     }
     const size_t at = (row * a.heads + head) * DIM + col;
@@ -219,7 +219,7 @@ uint64_t sdx_selected_attention_scratch(uint64_t rows, uint64_t kv_heads, uint64
 
 int sdx_selected_attention(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t context, uint64_t base,
                            const uint32_t* dynamic_base, const float* indices, uint64_t selected, const float* counts, const void* q, int q_f16,
-                           uint64_t rows, uint64_t heads, float scale, const float* gate, uint64_t gate_stride, void* out, int out_f16,
+                           uint64_t rows, uint64_t heads, float scale, const float* gate, uint64_t gate_stride, uint64_t gate_row_stride, void* out, int out_f16,
                            void* scratch, uint64_t scratch_bytes) {
     SD_OP_BEGIN
     validate_pool(value, pool);
@@ -237,8 +237,9 @@ int sdx_selected_attention(void* handle, const sdx_kv_pool* pool, const int32_t*
     op_span(value, q, checked_product({rows, heads, uint64_t(DIM), q_f16 ? 2u : 4u}), "attention queries");
     op_span(value, out, checked_product({rows, heads, uint64_t(DIM), out_f16 ? 2u : 4u}), "an attention output");
     if (gate) {
-        if (gate_stride < DIM) throw std::runtime_error("sdx_selected_attention: a gate stride below 256");
-        op_span(value, gate, checked_floats({rows * heads - 1, gate_stride}) + DIM * 4, "an attention gate");
+        if (!gate_row_stride) gate_row_stride = heads * gate_stride;
+        if (gate_stride < DIM || gate_row_stride < (heads - 1) * gate_stride + DIM) throw std::runtime_error("sdx_selected_attention: gate strides below a head's 256 values or a row's heads");
+        op_span(value, gate, checked_floats({rows - 1, gate_row_stride}) + ((heads - 1) * gate_stride + DIM) * 4, "an attention gate");
     }
     const size_t need = scratch_bytes_for(rows, pool->kv_heads, selected);
     if (scratch_bytes < need) throw std::runtime_error("sdx_selected_attention: scratch too small (see sdx_selected_attention_scratch)");
@@ -253,8 +254,8 @@ int sdx_selected_attention(void* handle, const sdx_kv_pool* pool, const int32_t*
     args.chunks = unsigned((selected + CHUNK - 1) / CHUNK);
     if (pool->row_bytes != 2 * pool->dim) launch<true>(value, args, rows); else launch<false>(value, args, rows);
     SD_CHECK(hipGetLastError());
-    if (out_f16) selected_merge_kernel<true><<<unsigned(rows * heads), DIM, 0, value.stream>>>(args, gate, gate_stride, out);
-    else selected_merge_kernel<false><<<unsigned(rows * heads), DIM, 0, value.stream>>>(args, gate, gate_stride, out);
+    if (out_f16) selected_merge_kernel<true><<<unsigned(rows * heads), DIM, 0, value.stream>>>(args, gate, gate_stride, gate_row_stride, out);
+    else selected_merge_kernel<false><<<unsigned(rows * heads), DIM, 0, value.stream>>>(args, gate, gate_stride, gate_row_stride, out);
     SD_OP_END
 }
 

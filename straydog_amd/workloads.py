@@ -255,6 +255,45 @@ class BlockIndexWorkload:
                 self.gpu.release(b)
 
 
+class QwenStageWorkload:
+    """The whole attention stage of a Qwen decode / verification pass in one call (sdx_qsa_decode_attend) at 242K tokens:
+    24 query / 2 K/V heads of 256 columns, Q8_0 rows in the reference's state layout, 4 x 128 index heads."""
+
+    def __init__(self, gpu, steps, base=242000, context=262144, heads=24, kv_heads=2, row_bytes=272, seed=8):
+        self.gpu, self.steps, self.heads = gpu, steps, heads
+        pool = context // 4 + 1
+        self.stride = heads * 512 + kv_heads * 512 + 640
+        self.kv, self.kv_buffer = gpu.kv_pool(1, context, kv_heads, 256, row_bytes)
+        k, table = gpu.buffer(8192 * kv_heads * 256 * 2), gpu.upload(np.zeros(1, dtype=np.int32))
+        gpu.fill_normal(k.base(), 8192 * kv_heads * 256, seed * 11 + 3, 1)
+        for first in range(0, context, 8192):
+            start = gpu.upload(np.array([first], dtype=np.int32))
+            gpu.kv_write(self.kv, table.base(), 1, start.base(), k.base(), k.base(), True, 1, 8192)
+            gpu.release(start)
+        self.projections = gpu.buffer(steps * self.stride * 4)
+        self.blocks, self.history = gpu.buffer(128 * pool * 4), gpu.buffer(16 * 128 * 4)
+        self.norms = [gpu.buffer(n * 4) for n in (256, 256, 128, 128)]
+        gpu.fill_normal(self.projections.base(), steps * self.stride, seed * 11 + 1, 0)
+        gpu.fill_normal(self.blocks.base(), 128 * pool, seed * 11 + 2, 0)
+        for i, n in enumerate((256, 256, 128, 128)):
+            gpu.fill_uniform(self.norms[i].base(), n, seed * 11 + 5 + i, 0.5, 1.5)
+        self.positions = gpu.upload(np.arange(base, base + steps, dtype=np.uint32))
+        self.state = gpu.qsa_state(self.kv, None, context, self.blocks.base(), self.history.base(), *[n.base() for n in self.norms], heads)
+        self.scratch = gpu.buffer(gpu.qsa_decode_attend_scratch(steps, heads, kv_heads, context))
+        self.attended = gpu.buffer(steps * heads * 256 * 4)
+        gpu.synchronize()
+        gpu.release(k); gpu.release(table)
+
+    def step(self):
+        # (the projections are normalised in place again on every call: values shrink towards the norm weights, the work is the same)
+        self.gpu.qsa_decode_attend(self.state, self.projections.base(), self.stride, self.steps, self.positions.base(), self.positions.base(),
+                                   self.scratch, self.attended.base())
+
+    def release(self):
+        for b in [self.kv_buffer, self.projections, self.blocks, self.history, self.positions, self.scratch, self.attended] + self.norms:
+            self.gpu.release(b)
+
+
 def config1_lengths(seed=0x9e3779b97f4a7c15 ^ 1, seqs=32, low=1024, high=32768):
     rng = np.random.default_rng(seed & 0xffffffff)
     return rng.integers(low, high + 1, size=seqs)

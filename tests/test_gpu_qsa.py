@@ -304,3 +304,79 @@ def test_index_then_attend_on_the_device(gpu, oracle):
     close_enough(got, want, "index then attend")
     for b in (qb, kb, qq, sb, ib, cb, out, scratch, buffer):
         gpu.release(b)
+
+
+@pytest.mark.parametrize("row_bytes,paged,steps,first", [(272, False, 1, 2047), (272, True, 5, 2047), (512, False, 8, 3001)])
+def test_decode_stage_in_one_call_equals_its_parts(gpu, oracle, row_bytes, paged, steps, first):
+    # sdx_qsa_decode_attend (qsa_decode_attend_rows, gpu/qsa_decode.hpp:113-129): "three launches in one, the same values" -- the
+    # prepared queries, K/V bytes, pooled blocks and ring equal those of sdx_qsa_normalize + sdx_kv_write + sdx_qsa_pool, and the
+    # attended rows equal sdx_qsa_index + sdx_selected_attention on them, bit for bit; the rows cross a block's end and the
+    # 512-block line, positions live on the device
+    rng = np.random.default_rng(steps * 10 + row_bytes)
+    heads, kv_heads, context = 24, 2, 4096
+    pool_blocks, stride = context // 4 + 1, 24 * 512 + 2 * 512 + 640 + 11
+    projections = (rng.standard_normal((steps, stride)) * 2).astype(np.float32)
+    norms = [(0.4 + 1.2 * rng.random(n)).astype(np.float32) for n in (256, 256, 128, 128)]
+    blocks = np.zeros((128, pool_blocks), dtype=np.float32)
+    blocks[:, :first // 4] = rng.standard_normal((128, first // 4)).astype(np.float32)
+    history = rng.standard_normal((16, 128)).astype(np.float32)
+    positions = np.arange(first, first + steps, dtype=np.uint32)
+    page_tokens = 256 if paged else context
+    pages = context // page_tokens
+    order = rng.permutation(pages).astype(np.int32)
+    if row_bytes == 272:
+        filled = rng.integers(0, 256, pages * 4 * page_tokens * row_bytes, dtype=np.uint8)
+    else:
+        filled = rng.standard_normal(pages * 4 * page_tokens * 256).astype(np.float16).view(np.uint8)
+    if row_bytes == 272:                                   # random bytes would make NaN scales: give every row sane FP16 scales
+        rows = filled.reshape(-1, 272)
+        rows[:, 256:] = np.tile(np.frombuffer(np.float16(0.01).tobytes(), np.uint8), 8)
+
+    def fresh():
+        kv, buffer = gpu.kv_pool(pages, page_tokens, kv_heads, 256, row_bytes)
+        gpu.write_buffer(buffer, 0, filled)
+        return dict(kv=kv, buffer=buffer, table=gpu.upload(order) if paged else None, projections=gpu.upload(projections), blocks=gpu.upload(blocks),
+                    history=gpu.upload(history), norms=[gpu.upload(n) for n in norms], positions=gpu.upload(positions),
+                    attended=gpu.buffer(steps * heads * 256 * 4))
+
+    def read_state(s):
+        return dict(kv=_read(gpu, s["buffer"], np.uint8, filled.size), blocks=_read(gpu, s["blocks"], np.float32, blocks.size),
+                    history=_read(gpu, s["history"], np.float32, history.size), projections=_read(gpu, s["projections"], np.float32, projections.size),
+                    attended=_read(gpu, s["attended"], np.float32, steps * heads * 256))
+    # one call
+    one = fresh()
+    state = gpu.qsa_state(one["kv"], one["table"].base() if paged else None, context, one["blocks"].base(), one["history"].base(),
+                          *[n.base() for n in one["norms"]], heads)
+    scratch = gpu.buffer(gpu.qsa_decode_attend_scratch(steps, heads, kv_heads, context))
+    gpu.qsa_decode_attend(state, one["projections"].base(), stride, steps, one["positions"].base(), one["positions"].base(), scratch, one["attended"].base())
+    got = read_state(one)
+    # the parts
+    two = fresh()
+    base = two["projections"].base()
+    queries = gpu.buffer(steps * heads * 256 * 4)
+    keys = gpu.buffer(steps * kv_heads * 256 * 4)
+    values = gpu.buffer(steps * kv_heads * 256 * 4)
+    index_keys = gpu.buffer(steps * 128 * 4)
+    for r in range(steps):
+        at = base + r * stride * 4
+        gpu.qsa_normalize(at, two["norms"][0].base(), 1, heads, 256, 512, first + r, queries.at(r * heads * 256 * 4))
+        gpu.qsa_normalize(at + heads * 512 * 4, two["norms"][1].base(), 1, kv_heads, 256, 256, first + r, keys.at(r * kv_heads * 256 * 4))
+        gpu.qsa_normalize(at + (heads * 512 + kv_heads * 512) * 4, two["norms"][2].base(), 1, 4, 128, 128, first + r, at + (heads * 512 + kv_heads * 512) * 4)
+        gpu.write_buffer(values, r * kv_heads * 256 * 4, projections[r, heads * 512 + kv_heads * 256:heads * 512 + kv_heads * 512])
+        gpu.write_buffer(index_keys, r * 128 * 4, projections[r, heads * 512 + kv_heads * 512 + 512:heads * 512 + kv_heads * 512 + 640])
+    start = gpu.upload(np.array([first], dtype=np.int32))
+    table = two["table"].base() if paged else gpu.upload(np.zeros(1, np.int32)).base()
+    gpu.kv_write(two["kv"], table, pages, start.base(), keys.base(), values.base(), False, 1, steps)
+    for r in range(steps):           # row by row, as a verification's rows are pooled: every row enters the ring
+        gpu.qsa_pool(index_keys.at(r * 128 * 4), two["history"].base(), two["norms"][3].base(), pool_blocks, first + r, 1, two["blocks"].base())
+    scores, indices, counts = gpu.buffer(steps * pool_blocks * 4), gpu.buffer(steps * 2052 * 4), gpu.buffer(steps * 4)
+    gpu.qsa_index(base + (heads * 512 + kv_heads * 512) * 4, stride, two["blocks"].base(), pool_blocks, first, steps, 2052, scores.base(), indices.base(),
+                  counts.base())
+    partial = gpu.buffer(gpu.selected_attention_scratch(steps, kv_heads, 2052))
+    gpu.selected_attention(two["kv"], two["table"].base() if paged else None, context, first, indices.base(), 2052, counts.base(), queries.base(), False,
+                           steps, heads, 0.0625, two["attended"].base(), False, partial, gate=base + 256 * 4, gate_stride=512, gate_row_stride=stride)
+    want = read_state(two)
+    for what in ("kv", "blocks", "history", "projections", "attended"):
+        a, b = got[what], want[what]
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), what
+    assert np.all(np.isfinite(got["attended"])) and np.abs(got["attended"]).max() > 0
