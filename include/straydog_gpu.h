@@ -56,6 +56,15 @@ void* sd_buffer(void* handle, uint64_t bytes);
 int sd_buffer_write(void* handle, void* buffer, uint64_t offset, const void* data, uint64_t bytes);
 int sd_buffer_read(void* handle, const void* buffer, uint64_t offset, void* output, uint64_t bytes);
 
+/* ---- Graphs of ops ---- */
+/* reference straydog_gpu.h:177-183 (gpu/kernels.cpp:4765-4813): between sd_graph_begin and sd_graph_end (keep: store it under key,
+ * replacing any; else drop it) the ops queued on the device's stream are recorded rather than run; only ops with no host data
+ * (no buffer writes) that allocate nothing may be recorded.  sd_graph_run queues a recorded graph: 0, or 1 when none is stored
+ * under key. */
+int sd_graph_begin(void* handle);
+int sd_graph_end(void* handle, uint64_t key, int keep);
+int sd_graph_run(void* handle, uint64_t key);
+
 /* ---- K/V format ---- */
 /* reference straydog_gpu.h:113 (gpu/kernels.cpp:4266-4274): the bytes of a K/V row of the Qwen state, 512 (FP16) or
  * 272 (Q8_0: 256 int8 then eight FP16 block scales, gpu/core.hpp:397-403).  Default 272. */

@@ -47,6 +47,9 @@ SIGNATURES = {
     "sd_buffer": (c_void_p, [c_void_p, c_u64]),
     "sd_buffer_write": (c_int, [c_void_p, c_void_p, c_u64, c_void_p, c_u64]),
     "sd_buffer_read": (c_int, [c_void_p, c_void_p, c_u64, c_void_p, c_u64]),
+    "sd_graph_begin": (c_int, [c_void_p]),
+    "sd_graph_end": (c_int, [c_void_p, c_u64, c_int]),
+    "sd_graph_run": (c_int, [c_void_p, c_u64]),
     "sd_kv_format": (c_int, [c_void_p, c_u32]),
     "sd_attention_sequence": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_u64, c_void_p, c_u64]),
     "sd_op_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float,

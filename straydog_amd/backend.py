@@ -264,6 +264,17 @@ class Backend:
     def latent_attention(self, q, latents, selected, batch, groups, k, heads, kdim, vdim, scale, out):
         self.check(self.lib.sdx_latent_attention(self.handle, q, latents, selected, batch, groups, k, heads, kdim, vdim, scale, out))
 
+    # ---- graphs of ops (gpu.rs graph_begin / graph_end / graph_run) ----
+    def graph_begin(self):
+        self.check(self.lib.sd_graph_begin(self.handle))
+
+    def graph_end(self, key, keep=True):
+        self.check(self.lib.sd_graph_end(self.handle, key, int(keep)))
+
+    def graph_run(self, key):
+        """True when a graph is stored under key and was queued."""
+        return self.check(self.lib.sd_graph_run(self.handle, key)) == 0
+
     # ---- harness helpers ----------------------------------------------------------------
     def event(self):
         return self.check(self.lib.sdx_event_record(self.handle))

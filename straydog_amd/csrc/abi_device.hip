@@ -176,6 +176,10 @@ void sd_destroy(void* handle) {
     Device* d = static_cast<Device*>(handle);
     (void)hipSetDevice(d->ordinal);
     if (d->stream) (void)hipStreamSynchronize(d->stream);
+    for (auto& entry : d->graphs) {
+        if (entry.second.executable) (void)hipGraphExecDestroy(entry.second.executable);
+        if (entry.second.graph) (void)hipGraphDestroy(entry.second.graph);
+    }
     for (const auto& entry : d->allocations) (void)hipFree(const_cast<uint8_t*>(entry.first));
     for (auto& event : d->events) if (event) (void)hipEventDestroy(event);
     for (auto& event : d->profile_events) (void)hipEventDestroy(event);
@@ -296,6 +300,54 @@ int sd_kv_format(void* handle, uint32_t row) {
         Device& d = device(handle);
         if (row != 512 && row != 272) throw std::runtime_error("invalid Straydog K/V format");
         d.kv_row = row;
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+// ---- graphs of ops (reference gpu/kernels.cpp:4765-4813) ----
+// Between begin and end the ops queued on the device's stream are recorded rather than run.  Only ops that take no host data and
+// allocate nothing may be recorded; the ops that keep a workspace (see the extension header) are called once before.
+
+int sd_graph_begin(void* handle) {
+    try {
+        Device& d = device(handle);
+        if (d.recording) throw std::runtime_error("a Straydog graph is already being recorded");
+        SD_CHECK(hipStreamBeginCapture(d.stream, hipStreamCaptureModeThreadLocal));
+        d.recording = true;
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sd_graph_end(void* handle, uint64_t key, int keep) {
+    try {
+        Device& d = device(handle);
+        if (!d.recording) throw std::runtime_error("no Straydog graph is being recorded");
+        d.recording = false;
+        Device::Recorded made;
+        SD_CHECK(hipStreamEndCapture(d.stream, &made.graph));
+        if (!keep) {
+            (void)hipGraphDestroy(made.graph);
+            return 0;
+        }
+        const hipError_t instantiated = hipGraphInstantiate(&made.executable, made.graph, nullptr, nullptr, 0);
+        if (instantiated != hipSuccess) {
+            (void)hipGraphDestroy(made.graph);
+            SD_CHECK(instantiated);
+        }
+        Device::Recorded& slot = d.graphs[key];
+        if (slot.executable) (void)hipGraphExecDestroy(slot.executable);
+        if (slot.graph) (void)hipGraphDestroy(slot.graph);
+        slot = made;
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sd_graph_run(void* handle, uint64_t key) {
+    try {
+        Device& d = device(handle);
+        const auto found = d.graphs.find(key);
+        if (found == d.graphs.end()) return 1;
+        SD_CHECK(hipGraphLaunch(found->second.executable, d.stream));
         return 0;
     } catch (const std::exception& e) { last_error = e.what(); return -1; }
 }

@@ -208,6 +208,8 @@ int sd_attention_turns_reserve(void* handle, uint64_t rows, uint64_t rope_dims) 
     if (rope_dims > 128 || rope_dims % 2) throw std::runtime_error("invalid Straydog attention rope");
     const size_t pairs = size_t(rope_dims / 2);
     if (rows && pairs && !(value.turns && value.turns_pairs == pairs && value.turns_rows >= rows)) {
+        if (value.recording) throw std::runtime_error("an attention rope table cannot be allocated while a graph is recorded");
+        if (value.turns && !value.graphs.empty()) throw std::runtime_error("an attention rope table cannot grow after a graph was recorded");
         if (value.turns) {
             SD_CHECK(hipStreamSynchronize(value.stream));
             release(value, value.turns);

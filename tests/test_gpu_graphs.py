@@ -1,0 +1,153 @@
+"""Recorded graphs of the attention ops (sd_graph_begin / sd_graph_end / sd_graph_run), after the reference's own uses of them:
+crates/straydog-engine/tests/dspark_attention_gpu.rs:81-124 (a recorded op follows a device-resident position as it moves; what a
+replay reads is what the buffers hold then) -- here for the DSpark block attention, a paged decode step (K/V append + attention) and
+the whole Qwen decode stage.  Every replay is checked against the same work run eagerly, with eager work and waits between replays."""
+import numpy as np
+import pytest
+
+from gpu_util import backend, close_enough, make_pool
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    with backend(4 << 30) as handle:
+        yield handle
+
+
+def _read(gpu, buffer, dtype, count):
+    return gpu.read_buffer(buffer, 0, dtype, count)
+
+
+def test_graph_bookkeeping(gpu):
+    from straydog_amd.backend import StraydogError
+    assert not gpu.graph_run(12345), "no graph is stored under that key"
+    with pytest.raises(StraydogError, match="no Straydog graph"):
+        gpu.graph_end(1)
+    gpu.graph_begin()
+    with pytest.raises(StraydogError, match="already"):
+        gpu.graph_begin()
+    gpu.graph_end(1, keep=False)
+    assert not gpu.graph_run(1), "a dropped graph is not stored"
+
+
+def test_dspark_attention_recorded(gpu, oracle):
+    from test_oracle_attention import _dspark_inputs
+    from test_gpu_ops import _dspark_check
+    q, ring, block, sinks = _dspark_inputs()
+    qb, rb, bb, sb = (gpu.upload(a) for a in (q, ring, block, sinks))
+    out = gpu.buffer(q.size * 4)
+    anchor = gpu.upload(np.array([389], dtype=np.int32))
+    gpu.graph_begin()
+    gpu.dspark_attention(qb.base(), rb.base(), bb.base(), sb.base(), 64, 3, 389, anchor.base(), 128, out.base())
+    gpu.graph_end(140)
+    for at in (389, 200, 128, 389):
+        gpu.write_buffer(anchor, 0, np.array([at], dtype=np.int32))
+        assert gpu.graph_run(140)
+        want = oracle.dspark_attention(q, ring, block, sinks, 64, 3, at, 128)
+        _dspark_check(f"replayed at {at}", _read(gpu, out, np.float32, want.size), want)
+    # the first capture, a key that changes later and the sink's mass are observable (dspark_attention_gpu.rs:101-124)
+    gpu.write_buffer(qb, 0, np.zeros(q.size, np.float32))
+    gpu.write_buffer(rb, 0, np.full(ring.size, 23.0, np.float32))
+    keys = np.repeat(np.arange(1, 6, dtype=np.float32), 512)
+    gpu.write_buffer(bb, 0, keys)
+    gpu.write_buffer(sb, 0, np.zeros(64, np.float32))
+    gpu.graph_begin()
+    gpu.dspark_attention(qb.base(), rb.base(), bb.base(), sb.base(), 64, 5, 0, None, 0, out.base())
+    gpu.graph_end(139)
+    assert gpu.graph_run(139)
+    _dspark_check("captured noncausal block", _read(gpu, out, np.float32, q.size), np.full(q.size, 2.5))
+    keys[4 * 512:] = 11.0
+    gpu.write_buffer(bb, 0, keys)
+    assert gpu.graph_run(139)
+    _dspark_check("future key changed", _read(gpu, out, np.float32, q.size), np.full(q.size, 3.5))
+    for sink, expected in ((1000.0, 0.0), (-1000.0, 4.2)):
+        gpu.write_buffer(sb, 0, np.full(64, sink, np.float32))
+        assert gpu.graph_run(139)
+        _dspark_check(f"sink={sink}", _read(gpu, out, np.float32, q.size), np.full(q.size, expected))
+    for b in (qb, rb, bb, sb, out, anchor):
+        gpu.release(b)
+
+
+def test_paged_decode_step_recorded(gpu, oracle):
+    # one decode step of a ragged batch -- append the new K/V rows, attend -- recorded once and replayed as the positions advance
+    rng = np.random.default_rng(5)
+    seqs, heads, kv_heads, dim, page_tokens, row_bytes = 3, 16, 2, 128, 64, 136
+    lengths = [700, 65, 1000]
+    capacity = [n + 8 for n in lengths]
+    pool, buffer, host, table, table_buffer = make_pool(gpu, oracle, rng, capacity, kv_heads, dim, page_tokens, row_bytes)
+    max_context = max(capacity)
+    positions = gpu.upload(np.array(lengths, dtype=np.int32))
+    kb, vb = gpu.buffer(seqs * kv_heads * dim * 4), gpu.buffer(seqs * kv_heads * dim * 4)
+    qb, out = gpu.buffer(seqs * heads * dim * 4), gpu.buffer(seqs * heads * dim * 4)
+    scratch = gpu.buffer(gpu.paged_attention_scratch(seqs, 1, heads, dim, max_context))
+
+    def step():
+        gpu.kv_write(pool, table_buffer.base(), table.shape[1], positions.base(), kb.base(), vb.base(), False, seqs, 1)
+        gpu.paged_attention(pool, table_buffer.base(), table.shape[1], positions.base(), max_context, qb.base(), False, seqs, 1, heads, 0.088, out.base(),
+                            False, scratch)
+    step()                                  # once eagerly: whatever a first call sets up is set up outside the recording
+    gpu.graph_begin()
+    step()
+    gpu.graph_end(7)
+    for turn in range(4):
+        at = np.array([n + turn for n in lengths], dtype=np.int32)
+        k = rng.standard_normal((seqs, 1, kv_heads, dim)).astype(np.float32)
+        v = rng.standard_normal((seqs, 1, kv_heads, dim)).astype(np.float32)
+        q = rng.standard_normal((seqs, 1, heads, dim)).astype(np.float32)
+        for b, a in ((positions, at), (kb, k), (vb, v), (qb, q)):
+            gpu.write_buffer(b, 0, a)
+        assert gpu.graph_run(7)
+        got = _read(gpu, out, np.float32, q.size).reshape(q.shape)
+        oracle.kv_write(host, row_bytes, page_tokens, kv_heads, dim, table, at, k, v)
+        want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, at, q, 0.088)
+        close_enough(got, want, f"replay {turn}")
+        assert np.array_equal(_read(gpu, buffer, np.uint8, host.size), host), "the appended rows"
+    for b in (buffer, table_buffer, positions, kb, vb, qb, out, scratch):
+        gpu.release(b)
+
+
+def test_qwen_decode_stage_recorded(gpu, oracle):
+    # sdx_qsa_decode_attend recorded once; replays at advancing device-resident positions give the bits of eager calls on a twin state
+    rng = np.random.default_rng(6)
+    heads, kv_heads, context, first, row_bytes = 24, 2, 4096, 2300, 272
+    pool_blocks, stride = context // 4 + 1, 24 * 512 + 2 * 512 + 640
+    blocks = np.zeros((128, pool_blocks), dtype=np.float32)
+    blocks[:, :first // 4] = rng.standard_normal((128, first // 4)).astype(np.float32)
+    history = rng.standard_normal((16, 128)).astype(np.float32)
+    norms = [(0.4 + 1.2 * rng.random(n)).astype(np.float32) for n in (256, 256, 128, 128)]
+    cached = np.zeros(context * 4 * row_bytes, dtype=np.uint8)
+    oracle.kv_write(cached, row_bytes, context, kv_heads, 256, np.zeros((1, 1), np.int32), np.zeros(1, np.int32),
+                    rng.standard_normal((1, first, kv_heads, 256)).astype(np.float32), rng.standard_normal((1, first, kv_heads, 256)).astype(np.float32))
+
+    def twin():
+        kv, buffer = gpu.kv_pool(1, context, kv_heads, 256, row_bytes)
+        gpu.write_buffer(buffer, 0, cached)
+        s = dict(kv=kv, buffer=buffer, projections=gpu.buffer(stride * 4), blocks=gpu.upload(blocks), history=gpu.upload(history),
+                 norms=[gpu.upload(n) for n in norms], position=gpu.upload(np.array([first], dtype=np.uint32)), attended=gpu.buffer(heads * 256 * 4),
+                 scratch=gpu.buffer(gpu.qsa_decode_attend_scratch(1, heads, kv_heads, context)))
+        s["state"] = gpu.qsa_state(kv, None, context, s["blocks"].base(), s["history"].base(), *[n.base() for n in s["norms"]], heads)
+        return s
+
+    def call(s):
+        gpu.qsa_decode_attend(s["state"], s["projections"].base(), stride, 1, s["position"].base(), s["position"].base(), s["scratch"], s["attended"].base())
+    recorded, eager = twin(), twin()
+    warm = twin()
+    call(warm)                               # a first call outside the recording
+    gpu.graph_begin()
+    call(recorded)
+    gpu.graph_end(9)
+    for turn in range(6):                    # positions 2300 .. 2305: a block is completed at 2303
+        row = (rng.standard_normal(stride) * 2).astype(np.float32)
+        at = np.array([first + turn], dtype=np.uint32)
+        for s in (recorded, eager):
+            gpu.write_buffer(s["projections"], 0, row)
+            gpu.write_buffer(s["position"], 0, at)
+        assert gpu.graph_run(9)
+        call(eager)
+        for what, count, dtype in (("attended", heads * 256, np.float32), ("blocks", blocks.size, np.float32), ("history", history.size, np.float32),
+                                   ("buffer", cached.size, np.uint8)):
+            a, b = _read(gpu, recorded[what], dtype, count), _read(gpu, eager[what], dtype, count)
+            assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), f"replay {turn}: {what}"
+        assert np.abs(_read(gpu, recorded["attended"], np.float32, heads * 256)).max() > 0
