@@ -597,6 +597,289 @@ void launch_pairs(Device& d, const PrefillArgs& args, unsigned seqs) {
     prefill_pairs_kernel<DIM, QT, Q8><<<dim3((runs + 1) / 2, args.kv_heads, seqs), TEAM * 64, shared, d.stream>>>(args);
 }
 
+// ---- the third form, for 128 columns: K/V unpacked once per call into FP16 tiles in a workspace -------------------------
+// A pass before the attention turns the cached rows of every (sequence, K/V head) into tiles of 64 keys, each a K block
+// [64 keys][128 columns] and a V^T block [128 columns][64 keys] of FP16, 32 KiB together, laid out in the order LDS wants them:
+// the 16-byte pieces of a K row sit at piece ^ (key % 16); a V^T row keeps the eight keys a lane multiplies at once (keys 4g.. and
+// 16 + 4g.. of a 32-key half) side by side as one 16-byte piece, at piece ^ (column / 2 % 8): the sixteen lanes of an operand
+// read then fall on sixteen different bank groups without any padding, and an operand is one 16-byte read.  The attention
+// kernel then copies a step's tile by plain 1 KiB global->LDS loads and has no conversion in its loop at all; the tiles are
+// read by every workgroup of the K/V head (from L2), the pass itself costs a few microseconds per call.
+constexpr int TILE_KEYS = 64;
+template<int DIM> constexpr int tile_bytes() { return 2 * TILE_KEYS * DIM * 2; }
+
+template<int DIM, bool Q8>
+__global__ void __launch_bounds__(256) unpack_tiles_kernel(PrefillArgs args, uint8_t* tiles_out, unsigned tiles_per_seq) {
+    constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, KT = TILE_KEYS * DIM * 2, PIECES = DIM / 8;
+    static_assert(DIM == 128, "a K row is 16 pieces, a V^T row 16 units");
+    const int tile = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z, t = threadIdx.x;
+    const int cached = min(args.positions[seq] + int(args.span), args.max_context), key0 = tile * TILE_KEYS;
+    if (key0 >= cached) return;
+    const int32_t* table = args.page_table + size_t(seq) * args.table_stride;
+    const size_t plane_bytes = size_t(args.page_tokens) * ROW;
+    uint8_t* out = tiles_out + ((size_t(seq) * args.kv_heads + kvh) * tiles_per_seq + tile) * tile_bytes<DIM>();
+    const auto row_of = [&](int key, bool value) {
+        const int token = min(key0 + key, cached - 1);
+        return args.pages + (size_t(table[token / int(args.page_tokens)]) * 2 * args.kv_heads + (value ? args.kv_heads : 0) + kvh) * plane_bytes +
+               size_t(token % int(args.page_tokens)) * ROW;
+    };
+    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+    // K: a thread takes pieces of 8 columns; rows past the sequence's end become zeros
+    #pragma unroll
+    for (int j = 0; j < TILE_KEYS * PIECES / 256; ++j) {
+        const int piece = t + 256 * j, key = piece / PIECES, c = piece % PIECES;
+        const uint8_t* row = row_of(key, false);
+        half8 values;
+        if (Q8) {
+            const uint2 bytes = *reinterpret_cast<const uint2*>(row + 8 * c);
+            const _Float16 scale = *reinterpret_cast<const _Float16*>(row + DIM + 2 * (c / 4));
+            #pragma unroll
+            for (int i = 0; i < 8; ++i) values[i] = (_Float16)float(int8_t((i < 4 ? bytes.x : bytes.y) >> (8 * (i & 3)))) * scale;
+        } else values = *reinterpret_cast<const half8*>(row + 16 * c);
+        if (key0 + key >= cached) values = half8{};
+        *reinterpret_cast<half8*>(out + key * (2 * DIM) + ((c ^ (key & 15)) * 16)) = values;
+    }
+    // V^T: a thread takes 4 keys x 4 columns
+    #pragma unroll
+    for (int j = 0; j < (TILE_KEYS / 4) * (DIM / 4) / 256; ++j) {
+        const int block = t + 256 * j, keys4 = block % (TILE_KEYS / 4), cols4 = block / (TILE_KEYS / 4);
+        _Float16 v[4][4];       // [key][column]
+        #pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint8_t* row = row_of(4 * keys4 + e, true);
+            const bool live = key0 + 4 * keys4 + e < cached;
+            if (Q8) {
+                const uint32_t bytes = *reinterpret_cast<const uint32_t*>(row + 4 * cols4);
+                const _Float16 scale = *reinterpret_cast<const _Float16*>(row + DIM + 2 * (cols4 / 8));
+                #pragma unroll
+                for (int c = 0; c < 4; ++c) v[e][c] = live ? (_Float16)float(int8_t(bytes >> (8 * c))) * scale : (_Float16)0.0f;
+            } else {
+                const half4 four = *reinterpret_cast<const half4*>(row + 8 * cols4);
+                #pragma unroll
+                for (int c = 0; c < 4; ++c) v[e][c] = live ? four[c] : (_Float16)0.0f;
+            }
+        }
+        #pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int column = 4 * cols4 + c;
+            // keys 32 part + 16 h + 4 g + (0..3) go to piece 4 part + g, its first (h = 0) or second 8 bytes
+            const int piece = 4 * (keys4 / 8) + keys4 % 4, second = (keys4 / 4) % 2;
+            *reinterpret_cast<half4*>(out + KT + column * (2 * TILE_KEYS) + ((piece ^ ((column >> 1) & 7)) * 16) + 8 * second) = half4{v[0][c], v[1][c], v[2][c], v[3][c]};
+        }
+    }
+}
+
+// Two runs of 4 x QT x 16 rows per workgroup (a late one and its mirror, as prefill_pairs_kernel), every wave 32 rows and both
+// halves of a 64-key step; a step's tile arrives by 32 global->LDS loads of 1 KiB, four a wave, into a ring of stages.
+template<int DIM, int QT>
+__global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) prefill_dense_kernel(PrefillArgs args, const uint8_t* tiles_in,
+                                                                                                       unsigned tiles_per_seq) {
+    constexpr int BLOCKS = DIM / 32, TILES = DIM / 16, KT = TILE_KEYS * DIM * 2, TILE = tile_bytes<DIM>();
+    constexpr int WAVE_ROWS = QT * 16, GROUP_ROWS = GROUPS * WAVE_ROWS, RING = 4, PER = TILE / 1024 / TEAM;
+    static_assert(WALK == TILE_KEYS && TILE % (1024 * TEAM) == 0 && RING * TILE <= 160 * 1024 - 1024, "a step is one tile, copied by the eight waves alike");
+    const int kvh = blockIdx.y, seq = blockIdx.z;
+    const int thread = threadIdx.x, lane = thread & 63, wave = __builtin_amdgcn_readfirstlane(thread >> 6), li = lane & 15, g = lane >> 4;
+    const int position = args.positions[seq];
+    const int cached = min(position + int(args.span), args.max_context);
+    const int quarter = wave % GROUPS, half = wave / GROUPS;       // half 0: the run from the end of the span, half 1: its mirror
+    const int runs = (int(args.rows) + GROUP_ROWS - 1) / GROUP_ROWS;
+    const int late = runs - 1 - int(blockIdx.x), early = int(blockIdx.x), run = half == 0 ? late : early;
+    const int row0 = run * GROUP_ROWS + quarter * WAVE_ROWS;
+    const int group_last = min(int(args.rows), (late + 1) * GROUP_ROWS) - 1;
+    const int keys = min(position + group_last / int(args.group) + 1, cached);     // the walk is the late run's
+    const bool idle = row0 >= int(args.rows) || (half == 1 && early == late);      // an odd number of runs: the middle one is alone
+    const int wave_first = position + row0 / int(args.group);
+    const int wave_last = position + (min(int(args.rows), row0 + WAVE_ROWS) - 1) / int(args.group);
+    extern __shared__ __attribute__((aligned(16))) uint8_t stages[];              // [RING][K block | V^T block]
+    const uint8_t* const source = tiles_in + (size_t(seq) * args.kv_heads + kvh) * tiles_per_seq * TILE + 1024 * PER * wave + 16 * lane;
+    const int last_tile = (keys - 1) / WALK;
+    const auto copy_in = [&](int step) {
+        const uint8_t* from = source + size_t(min(step, last_tile)) * TILE;
+        uint8_t* stage = stages + (step % RING) * TILE + 1024 * PER * wave;
+        #pragma unroll
+        for (int k = 0; k < PER; ++k) load_to_lds<false>(from + 1024 * k, stage + 1024 * k);
+    };
+
+    half8 qf[QT][BLOCKS];
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int row = row0 + qt * 16 + li;
+        const bool real = row < int(args.rows);
+        const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
+        const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
+        #pragma unroll
+        for (int b = 0; b < BLOCKS; ++b) {
+            half8 value = {};
+            if (real) {
+                if (args.q_f16) value = *reinterpret_cast<const half8*>(static_cast<const _Float16*>(args.q) + at + 32 * b + 8 * g);
+                else {
+                    const float* from = static_cast<const float*>(args.q) + at + 32 * b + 8 * g;
+                    #pragma unroll
+                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)from[i];
+                }
+            }
+            qf[qt][b] = value;
+        }
+    }
+    floatx4 acc[QT][TILES];
+    float m[QT], l[QT];
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        m[qt] = NEG_BIG; l[qt] = 0.0f;
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    // The weights of a step and the V^T operands they meet; the second wave of a SIMD keeps them over the barrier (below).
+    half8 pb[2][QT];
+    half8 va[2][TILES];
+    const auto weigh_in = [&] {
+        #pragma unroll
+        for (int part = 0; part < 2; ++part)
+            #pragma unroll
+            for (int jj = 0; jj < TILES; ++jj)
+                #pragma unroll
+                for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[part][jj], pb[part][qt], acc[qt][jj], 0, 0, 0);
+    };
+    // The two waves of a SIMD (a late run's and an early run's) meet at every step's barrier, so left alone both would multiply
+    // and then both would exponentiate.  The second one therefore carries its O^T += V^T . P^T over the barrier into the next
+    // step: while the first forms its weights (VALU), the second is at its products (MFMA), and the other way round.
+    const auto walk = [&](auto defer) {
+    constexpr bool DEFER = decltype(defer)::value;
+    bool pending = false;
+    for (int walk0 = 0, step = 0; walk0 < keys; walk0 += WALK, ++step) {
+        wait_loads<PER * (RING - 2)>();      // this step's pieces have landed when only the later steps' are outstanding
+        ring_barrier();                      // everybody's have, and everybody is done with the step before: its stage is free
+        copy_in(step + RING - 1);
+        const uint8_t* const kblock = stages + (step % RING) * TILE;
+        const uint8_t* const vblock = kblock + KT;
+        if (DEFER && pending) { weigh_in(); pending = false; }
+        if (idle || walk0 > wave_last) continue;         // (the barriers above are everybody's; the step's work is not)
+        // S^T for the step's four 16-key tiles: all of K's operands are asked for at once
+        constexpr int KEY_TILES = WALK / 16;
+        floatx4 s[QT][KEY_TILES];
+        {
+            half8 ka[KEY_TILES][BLOCKS];
+            #pragma unroll
+            for (int t = 0; t < KEY_TILES; ++t)
+                #pragma unroll
+                for (int b = 0; b < BLOCKS; ++b) ka[t][b] = *reinterpret_cast<const half8*>(kblock + (16 * t + li) * (2 * DIM) + (((4 * b + g) ^ li) * 16));
+            // eight independent chains, a column block at a time: no product waits for the one before it
+            #pragma unroll
+            for (int t = 0; t < KEY_TILES; ++t)
+                #pragma unroll
+                for (int qt = 0; qt < QT; ++qt) s[qt][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            #pragma unroll
+            for (int b = 0; b < BLOCKS; ++b)
+                #pragma unroll
+                for (int t = 0; t < KEY_TILES; ++t)
+                    #pragma unroll
+                    for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][b], qf[qt][b], s[qt][t], 0, 0, 0);
+        }
+        // V^T's operands travel while the scores are formed: a lane's keys of a 32-key half are {4g.., 16+4g..}
+        #pragma unroll
+        for (int part = 0; part < 2; ++part)
+            #pragma unroll
+            for (int jj = 0; jj < TILES; ++jj)
+                va[part][jj] = *reinterpret_cast<const half8*>(vblock + (16 * jj + li) * (2 * TILE_KEYS) + (((4 * part + g) ^ (li >> 1)) * 16));
+        if (walk0 + WALK - 1 > wave_first) {          // wave-uniform: some key of the step is past some row's position
+            asm volatile("; the step crosses the diagonal" ::: "memory");      // keeps the block a branch: it is rare
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt) {
+                const int row = row0 + qt * 16 + li;
+                const int limit = row < int(args.rows) ? position + row / int(args.group) : 0x7fffffff;   // a padding row masks nothing
+                #pragma unroll
+                for (int t = 0; t < KEY_TILES; ++t)
+                    #pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (walk0 + 16 * t + 4 * g + r > limit) s[qt][t][r] = -INFINITY;
+            }
+        }
+        float top[QT];
+        bool grown = false;
+        #pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            float most = s[qt][0][0];
+            #pragma unroll
+            for (int t = 0; t < KEY_TILES; ++t)
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) most = fmaxf(most, s[qt][t][r]);
+            top[qt] = row_max(most);
+            grown |= (top[qt] - m[qt]) * args.scale_log2 > SLACK;
+        }
+        if (__any(grown)) {
+            asm volatile("; new reference maxima" ::: "memory");          // keeps the block a branch: it is rare
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt) {
+                const float m_new = fmaxf(m[qt], top[qt]);
+                const float alpha = __builtin_amdgcn_exp2f((m[qt] - m_new) * args.scale_log2);
+                m[qt] = m_new;
+                l[qt] *= alpha;
+                #pragma unroll
+                for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] *= alpha;
+            }
+        }
+        #pragma unroll
+        for (int part = 0; part < 2; ++part)
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt) {
+                const float offset = -m[qt] * args.scale_log2;
+                float sum = 0.0f;
+                half8 p;
+                #pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    #pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float w = __builtin_amdgcn_exp2f(fmaf(s[qt][2 * part + t][r], args.scale_log2, offset));
+                        sum += w;
+                        p[4 * t + r] = (_Float16)w;
+                    }
+                pb[part][qt] = p;
+                l[qt] += sum;
+            }
+        if (DEFER) pending = true; else weigh_in();
+    }
+    if (DEFER && pending) weigh_in();
+    };
+    settle_loads();
+    #pragma unroll
+    for (int ahead = 0; ahead < RING - 1; ++ahead) copy_in(ahead);
+    if (half == 0) walk(std::false_type{}); else walk(std::true_type{});
+
+    if (idle) return;
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int row = row0 + qt * 16 + li;
+        const float inverse = 1.0f / row_sum(l[qt]);
+        if (row >= int(args.rows)) continue;
+        const int span_row = row / int(args.group), head = kvh * int(args.group) + row % int(args.group);
+        const size_t first = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM + 4 * g;
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj) {
+            const floatx4 value = acc[qt][jj] * inverse;
+            if (args.out_f16) {
+                typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+                *reinterpret_cast<half4*>(static_cast<_Float16*>(args.out) + first + 16 * jj) = half4{(_Float16)value[0], (_Float16)value[1], (_Float16)value[2], (_Float16)value[3]};
+            } else *reinterpret_cast<floatx4*>(static_cast<float*>(args.out) + first + 16 * jj) = value;
+        }
+    }
+}
+
+template<int DIM, int QT, bool Q8>
+void launch_dense(Device& d, const PrefillArgs& args, unsigned seqs) {
+    const unsigned tiles_per_seq = unsigned((args.max_context + TILE_KEYS - 1) / TILE_KEYS);
+    auto* tiles = static_cast<uint8_t*>(workspace(d, checked_product({seqs, args.kv_heads, tiles_per_seq, uint64_t(tile_bytes<DIM>())})));
+    constexpr int shared = 4 * tile_bytes<DIM>();
+    static bool raised = false;
+    if (!raised) {
+        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_dense_kernel<DIM, QT>), hipFuncAttributeMaxDynamicSharedMemorySize, shared));
+        raised = true;
+    }
+    unpack_tiles_kernel<DIM, Q8><<<dim3(tiles_per_seq, args.kv_heads, seqs), 256, 0, d.stream>>>(args, tiles, tiles_per_seq);
+    const unsigned runs = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
+    prefill_dense_kernel<DIM, QT><<<dim3((runs + 1) / 2, args.kv_heads, seqs), TEAM * 64, shared, d.stream>>>(args, tiles, tiles_per_seq);
+}
+
 template<int DIM, int QT, bool Q8, int OCC>
 void launch(Device& d, const PrefillArgs& args, unsigned seqs) {
     constexpr size_t merge = size_t(GROUPS) * QT * (DIM / 16 * 4 + 2) * 64 * 4;
@@ -631,7 +914,9 @@ void prefill_attention(Device& d, const sdx_kv_pool* pool, const int32_t* page_t
     args.out = out; args.out_f16 = out_f16;
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     KernelTimer timer(d);
-    if (pool->dim == 128) { if (q8) launch_pairs<128, 2, true>(d, args, unsigned(seqs)); else launch_pairs<128, 2, false>(d, args, unsigned(seqs)); }
+    static const bool dense = std::getenv("STRAYDOG_PREFILL_PAIRS") == nullptr;
+    if (pool->dim == 128 && dense) { if (q8) launch_dense<128, 2, true>(d, args, unsigned(seqs)); else launch_dense<128, 2, false>(d, args, unsigned(seqs)); }
+    else if (pool->dim == 128) { if (q8) launch_pairs<128, 2, true>(d, args, unsigned(seqs)); else launch_pairs<128, 2, false>(d, args, unsigned(seqs)); }
     else { if (q8) launch<256, 1, true, 2>(d, args, unsigned(seqs)); else launch<256, 1, false, 2>(d, args, unsigned(seqs)); }
 }
 
