@@ -7,21 +7,20 @@
 //
 // Shape of the work on gfx950 (wave64, v_mfma_f32_16x16x32_f16).  Query rows are ordered (span row, head in group), so a
 // run of consecutive rows is a run of consecutive tokens with all their grouped heads and every K/V row read serves all of
-// them.  A workgroup of 8 waves (two per SIMD) walks the keys 64 at a time; a step's K and V slabs (64 contiguous rows of a
-// page plane) arrive by coalesced 16-byte global->LDS loads, an eighth by each wave, into a ring of stages, so the copies
-// of the next steps are in flight while this one is computed; one barrier per step; steps that lie wholly after a wave's
-// rows are skipped.  Two kernels:
-//   * prefill_pairs_kernel (128 columns, the headline shape): the workgroup converts a step's raw rows once into FP16
-//     tiles in LDS which all eight waves read as MFMA operands; it owns two runs of 128 rows, one from the end of the span
-//     and its mirror image from the start, so every workgroup does about the same work, and writes its outputs normalised,
-//     with no merge (details at the kernel);
+// them.  A workgroup of 8 waves (two per SIMD) walks the keys 64 at a time, the next steps' operands travelling by 16-byte
+// global->LDS loads into a ring of stages while this one is computed; one barrier per step; steps that lie wholly after a
+// wave's rows are skipped.  Two kernels:
+//   * prefill_dense_kernel (128 columns, the headline shape): a pass before it unpacks the cached rows once per call into
+//     FP16 tiles in a workspace, laid out as LDS wants them, so the kernel's loop converts nothing: it copies a tile, reads
+//     operands without bank conflicts, multiplies and exponentiates.  A workgroup owns two runs of 128 rows, one from the
+//     end of the span and its mirror image from the start, so every workgroup does about the same work, and writes its
+//     outputs normalised, with no merge (details at the kernels);
 //   * prefill_attention_kernel (256 columns): 4 x QT x 16 rows per workgroup; every wave builds its own operands from the
-//     stage (paged_rows.hpp); a quarter of the rows belongs to a pair of waves, one taking the first 32 keys of every step
-//     and one the last 32, each with its own online softmax, merged through LDS at the end; the workgroups with the
-//     longest walks are dispatched first.
+//     raw rows in the stage (paged_rows.hpp); a quarter of the rows belongs to a pair of waves, one taking the first 32
+//     keys of every step and one the last 32, each with its own online softmax, merged through LDS at the end; the
+//     workgroups with the longest walks are dispatched first.
 #include "paged_rows.hpp"
 
-#include <cstdlib>
 #include <type_traits>
 
 using namespace sd;
@@ -31,8 +30,6 @@ namespace {
 
 constexpr float SLACK = 8.0f;     // how far (base-2 exponent) a row's true maximum may run ahead of its reference maximum
 // The ring of K/V stages: the copies of STAGES - 1 steps are in flight or landed; as many as fit beside nothing else, at most 4.
-// The same for the kernel that also keeps two pairs of FP16 tiles, at most 3.
-constexpr int tiles_ring(int stage_bytes, int tiles_bytes) { return (158 * 1024 - tiles_bytes) / stage_bytes < 3 ? (158 * 1024 - tiles_bytes) / stage_bytes : 3; }
 constexpr int stages_for(int stage_bytes) { return 150 * 1024 / stage_bytes < 4 ? 150 * 1024 / stage_bytes : 4; }
 constexpr int GROUPS = 4, HALVES = 2, TEAM = GROUPS * HALVES;   // row quarters x key halves = waves of a workgroup
 constexpr int WALK = HALVES * STEP;                            // keys per step of the workgroup
@@ -282,322 +279,7 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     }
 }
 
-// The second form of the kernel, for 128 columns.  The workgroup converts every step's rows once into FP16 tiles in LDS (K
-// as rows with a 16-byte pad, V transposed with an 8-byte pad: both read without bank conflicts as MFMA operands), so the
-// Q8_0 -> FP16 work is shared by the eight waves instead of being done by each; while a step is computed from one pair of
-// tiles the next step's raw rows (already landed) are converted into the other pair; one barrier per step.  Columns of an
-// output tile jj are 16 jj + (0..15), a lane holding 16 jj + 4 g + r.  The causal triangle is evened out inside every
-// workgroup: it owns two runs of 4 x QT x 16 query rows: one from the end of the span (its rows see the most keys)
-// on waves 0-3 and its mirror image from the start of the span on waves 4-7, so every workgroup walks about the same number
-// of (row, key) pairs and every SIMD hosts one wave of each run -- when the short run's waves are done the long run's have
-// the SIMD to themselves.  A wave takes both 32-key halves of a step in turn, so nothing is merged at the end.
-template<int DIM, int QT, bool Q8>
-__global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) prefill_pairs_kernel(PrefillArgs args) {
-    constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, BLOCKS = DIM / 32, TILES = DIM / 16;
-    constexpr int SLAB = WALK * ROW, UNITS = (SLAB + 1023) / 1024;
-    constexpr int WAVE_ROWS = QT * 16, GROUP_ROWS = GROUPS * WAVE_ROWS;
-    constexpr int KP = 2 * DIM + 16, VP = 2 * WALK + 8, KT = WALK * KP, VT = DIM * VP;     // pitches and sizes of the FP16 tiles
-    constexpr int RING = tiles_ring(2 * SLAB, 2 * (KT + VT));
-    static_assert(RING >= 2 && WALK == 64 && TEAM == 8, "512 threads convert a step of 64 rows, one piece each");
-    const int kvh = blockIdx.y, seq = blockIdx.z;
-    const int thread = threadIdx.x, lane = thread & 63, wave = __builtin_amdgcn_readfirstlane(thread >> 6), li = lane & 15, g = lane >> 4;
-    const int position = args.positions[seq];
-    const int cached = min(position + int(args.span), args.max_context);
-    const int quarter = wave % GROUPS, half = wave / GROUPS;       // half 0: the run from the end of the span, half 1: its mirror
-    const int runs = (int(args.rows) + GROUP_ROWS - 1) / GROUP_ROWS;
-    const int late = runs - 1 - int(blockIdx.x), early = int(blockIdx.x), tile = half == 0 ? late : early;
-    const int row0 = tile * GROUP_ROWS + quarter * WAVE_ROWS;
-    const int group_last = min(int(args.rows), (late + 1) * GROUP_ROWS) - 1;
-    const int keys = min(position + group_last / int(args.group) + 1, cached);     // the walk is the late run's
-    const bool idle = row0 >= int(args.rows) || (half == 1 && early == late);      // an odd number of runs: the middle one is alone
-    const int wave_first = position + row0 / int(args.group);
-    const int wave_last = position + (min(int(args.rows), row0 + WAVE_ROWS) - 1) / int(args.group);
-    const table_ptr table = (table_ptr)(args.page_table + size_t(seq) * args.table_stride);
-    const size_t plane_bytes = size_t(args.page_tokens) * ROW;
-    // Two objects, so that the compiler knows the tiles apart from the stages the global->LDS loads fill (it would otherwise
-    // guard every access to the tiles against those loads).
-    __shared__ __attribute__((aligned(16))) uint8_t stages[RING * 2 * SLAB];     // [RING][K slab | V slab] raw rows
-    extern __shared__ __attribute__((aligned(16))) uint8_t tiles[];              // [2][K tile | V tile]
-    constexpr int MOST = (2 * UNITS + TEAM - 1) / TEAM, LEAST = 2 * UNITS / TEAM;
-    const bool most = wave < 2 * UNITS - LEAST * TEAM;
-
-    const auto copy_in = [&](int buffer, int token0, int page) {
-        const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(token0 % int(args.page_tokens)) * ROW + 16 * lane;
-        uint8_t* stage = stages + buffer * (2 * SLAB);
-        #pragma unroll
-        for (int k = 0; k < MOST; ++k) {
-            const int unit = wave + TEAM * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS;
-            if (unit < 2 * UNITS && 16 * lane + 1024 * j < SLAB)
-                load_to_lds<false>(base + size_t(part ? args.kv_heads : 0) * plane_bytes + 1024 * j, stage + part * SLAB + 1024 * j);
-        }
-    };
-    // One step's raw rows into FP16 tiles; rows past the sequence's end become zeros (the page holds anything there).
-    const auto convert = [&](int buffer, int into, int walk0) {
-        int thread = threadIdx.x;
-        asm volatile("" : "+v"(thread));                       // the piece's addresses are formed here, not kept across the walk
-        const uint8_t* raw = stages + buffer * (2 * SLAB);
-        uint8_t* ktile = tiles + into * (KT + VT);
-        uint8_t* vtile = ktile + KT;
-        const int valid = cached - walk0;                      // rows of the step the cache holds
-        if (Q8) {
-            // K: 16 columns of one row; V: 4 rows x 4 columns, transposed.  All of the thread's raw reads are asked for at once.
-            const int key = thread >> 3, piece = thread & 7, rows4 = thread & 15, cols4 = thread >> 4;
-            const uint32_t from_k = lds_address(raw + key * ROW), from_v = lds_address(raw + SLAB + 4 * rows4 * ROW);
-            words2 a, b;
-            uint32_t scale_bits, words[4], scales[4];
-            asm volatile("ds_read_b64 %0, %11\n\tds_read_b64 %1, %11 offset:8\n\tds_read_u16 %2, %12\n\t"
-                         "ds_read_b32 %3, %13\n\tds_read_b32 %4, %13 offset:%c15\n\tds_read_b32 %5, %13 offset:%c16\n\tds_read_b32 %6, %13 offset:%c17\n\t"
-                         "ds_read_u16 %7, %14\n\tds_read_u16 %8, %14 offset:%c15\n\tds_read_u16 %9, %14 offset:%c16\n\tds_read_u16 %10, %14 offset:%c17\n\t"
-                         "s_waitcnt lgkmcnt(0)"
-                         : "=&v"(a), "=&v"(b), "=&v"(scale_bits), "=&v"(words[0]), "=&v"(words[1]), "=&v"(words[2]), "=&v"(words[3]),
-                           "=&v"(scales[0]), "=&v"(scales[1]), "=&v"(scales[2]), "=&v"(scales[3])
-                         : "v"(from_k + 16 * piece), "v"(from_k + DIM + 2 * (piece >> 1)), "v"(from_v + 4 * cols4), "v"(from_v + DIM + 2 * (cols4 >> 3)),
-                           "n"(ROW), "n"(2 * ROW), "n"(3 * ROW) : "memory");
-            {
-                if (key >= valid) scale_bits = 0;
-                const half2v scale = as_half2(scale_bits | (scale_bits << 16));
-                const uint32_t pieces[4] = {a.x, a.y, b.x, b.y};
-                half2v out[8];
-                #pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const uint32_t bits = pieces[w] ^ 0x80808080u;
-                    out[2 * w] = magic_to_half2(byte_perm(0x64646464u, bits, 0x04010400u), scale);
-                    out[2 * w + 1] = magic_to_half2(byte_perm(0x64646464u, bits, 0x04030402u), scale);
-                }
-                half8* to = reinterpret_cast<half8*>(ktile + key * KP + 32 * piece);
-                to[0] = half8{out[0].x, out[0].y, out[1].x, out[1].y, out[2].x, out[2].y, out[3].x, out[3].y};
-                to[1] = half8{out[4].x, out[4].y, out[5].x, out[5].y, out[6].x, out[6].y, out[7].x, out[7].y};
-            }
-            {
-                #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (4 * rows4 + e >= valid) scales[e] = 0u;
-                const half2v first = as_half2(scales[0] | (scales[1] << 16)), second = as_half2(scales[2] | (scales[3] << 16));
-                #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const uint32_t sel = 0x0c000c00u | uint32_t(c) | (uint32_t(4 + c) << 16);
-                    const half2v lo = magic_to_half2(byte_perm(words[1], words[0], sel) ^ 0x64806480u, first);
-                    const half2v hi = magic_to_half2(byte_perm(words[3], words[2], sel) ^ 0x64806480u, second);
-                    uint2 packed;
-                    packed.x = __builtin_bit_cast(uint32_t, lo); packed.y = __builtin_bit_cast(uint32_t, hi);
-                    *reinterpret_cast<uint2*>(vtile + (4 * cols4 + c) * VP + 8 * rows4) = packed;
-                }
-            }
-        } else {
-            // K: the slab is 16-byte pieces one after the other; piece c goes to its row's place in the padded tile
-            #pragma unroll
-            for (int k = 0; k < SLAB / 16 / (TEAM * 64); ++k) {
-                const int c = thread + TEAM * 64 * k, key = c / (ROW / 16), at = (c % (ROW / 16)) * 16;
-                words4 piece;
-                asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(piece) : "v"(lds_address(raw + 16 * c)) : "memory");
-                if (key >= valid) piece = words4{0u, 0u, 0u, 0u};
-                *reinterpret_cast<words4*>(ktile + key * KP + at) = piece;
-            }
-            // V: 4 rows x 4 columns, transposed
-            #pragma unroll
-            for (int k = 0; k < (WALK / 4) * (DIM / 4) / (TEAM * 64); ++k) {
-                const int block = thread + TEAM * 64 * k, rows4 = block & 15, cols4 = block >> 4;
-                const uint32_t from = lds_address(raw + SLAB + 4 * rows4 * ROW + 8 * cols4);
-                words2 words[4];
-                asm volatile("ds_read_b64 %0, %4\n\tds_read_b64 %1, %4 offset:%c5\n\tds_read_b64 %2, %4 offset:%c6\n\tds_read_b64 %3, %4 offset:%c7\n\ts_waitcnt lgkmcnt(0)"
-                             : "=&v"(words[0]), "=&v"(words[1]), "=&v"(words[2]), "=&v"(words[3]) : "v"(from), "n"(ROW), "n"(2 * ROW), "n"(3 * ROW) : "memory");
-                #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (4 * rows4 + e >= valid) words[e] = words2{0u, 0u};
-                #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
-                    uint2 packed;
-                    packed.x = byte_perm(c < 2 ? words[1].x : words[1].y, c < 2 ? words[0].x : words[0].y, sel);
-                    packed.y = byte_perm(c < 2 ? words[3].x : words[3].y, c < 2 ? words[2].x : words[2].y, sel);
-                    *reinterpret_cast<uint2*>(vtile + (4 * cols4 + c) * VP + 8 * rows4) = packed;
-                }
-            }
-        }
-    };
-
-
-    half8 qf[QT][BLOCKS];
-    #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-        const int row = row0 + qt * 16 + li;
-        const bool real = row < int(args.rows);
-        const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
-        const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
-        #pragma unroll
-        for (int b = 0; b < BLOCKS; ++b) {
-            half8 value = {};
-            if (real) {
-                if (args.q_f16) value = *reinterpret_cast<const half8*>(static_cast<const _Float16*>(args.q) + at + 32 * b + 8 * g);
-                else {
-                    const float* from = static_cast<const float*>(args.q) + at + 32 * b + 8 * g;
-                    #pragma unroll
-                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)from[i];
-                }
-            }
-            qf[qt][b] = value;
-        }
-    }
-    floatx4 acc[QT][TILES];
-    float m[QT], l[QT];
-    #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-        m[qt] = NEG_BIG; l[qt] = 0.0f;
-        #pragma unroll
-        for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-
-    settle_loads();
-    const int last_step = (keys - 1) / WALK * WALK;
-    #pragma unroll
-    for (int ahead = 0; ahead < RING; ++ahead) copy_in(ahead, min(ahead * WALK, last_step), table[min(ahead * WALK, last_step) / int(args.page_tokens)]);
-    int page_ahead = table[min(RING * WALK, last_step) / int(args.page_tokens)];      // of the step the walk's first copy brings in
-    // the first step's tiles
-    if (most) wait_loads<MOST * (RING - 1)>(); else wait_loads<LEAST * (RING - 1)>();
-    ring_barrier();
-    convert(0, 0, 0);
-
-    // The two waves of a SIMD walk in different orders: the first half's converts its piece of the next step and then computes,
-    // the second half's computes and then converts, so that one's MFMA phases meet the other's VALU phases.  (Two loops: the
-    // order is fixed at compile time in each.)
-    const auto walk = [&](auto convert_first) {
-    for (int walk0 = 0, step = 0; walk0 < keys; walk0 += WALK, ++step) {
-        // the next step's raw rows have landed when only the later steps' copies are outstanding
-        if (most) wait_loads<MOST * (RING - 2)>(); else wait_loads<LEAST * (RING - 2)>();
-        ring_barrier();       // everybody's pieces have; this step's tiles are written; the other tiles and the raw stage of this step are free
-        copy_in(step % RING, min(walk0 + RING * WALK, last_step), page_ahead);
-        page_ahead = table[min(walk0 + (RING + 1) * WALK, last_step) / int(args.page_tokens)];     // a scalar load, back long before the next step
-        if (decltype(convert_first)::value && walk0 + WALK < keys) convert((step + 1) % RING, (step + 1) & 1, walk0 + WALK);
-        #pragma unroll 1
-        for (int part = 0; part < WALK / STEP; ++part) {
-        const int token0 = walk0 + part * STEP;
-        if (!(idle || token0 > wave_last || token0 >= keys)) {
-        const uint8_t* ktile = tiles + (step & 1) * (KT + VT) + part * STEP * KP;
-        const uint8_t* vtile = tiles + (step & 1) * (KT + VT) + KT + part * STEP * 2;
-        // all of the step's operands are asked for at once: one LDS round trip for K, and V's is hidden behind the softmax
-        half8 ka[2][BLOCKS];
-        #pragma unroll
-        for (int t = 0; t < 2; ++t)
-            #pragma unroll
-            for (int b = 0; b < BLOCKS; ++b) ka[t][b] = *reinterpret_cast<const half8*>(ktile + (16 * t + li) * KP + 64 * b + 16 * g);
-        uint2 va[TILES][2];
-        #pragma unroll
-        for (int jj = 0; jj < TILES; ++jj) {
-            const uint8_t* from = vtile + (16 * jj + li) * VP + 8 * g;
-            va[jj][0] = *reinterpret_cast<const uint2*>(from); va[jj][1] = *reinterpret_cast<const uint2*>(from + 32);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        floatx4 s[QT][2];
-        #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            #pragma unroll
-            for (int qt = 0; qt < QT; ++qt) s[qt][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-            #pragma unroll
-            for (int b = 0; b < BLOCKS; ++b)
-                #pragma unroll
-                for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][b], qf[qt][b], s[qt][t], 0, 0, 0);
-        }
-        if (token0 + STEP - 1 > wave_first) {          // wave-uniform: some token of the step is past some row's position
-            asm volatile("; the step crosses the diagonal" ::: "memory");      // keeps the block a branch: it is rare
-            #pragma unroll
-            for (int qt = 0; qt < QT; ++qt) {
-                const int row = row0 + qt * 16 + li;
-                const int limit = row < int(args.rows) ? position + row / int(args.group) : 0x7fffffff;   // a padding row masks nothing
-                #pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    #pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (token0 + 16 * t + 4 * g + r > limit) s[qt][t][r] = -INFINITY;
-            }
-        }
-        // Every row's new maximum first; one rare block moves the reference maxima of the rows that need it; then the weights.
-        // Scores stay unscaled (the scale goes into the exponent's multiply-add); m is a row's reference maximum in unscaled
-        // units.  It follows the true maximum only when that has grown by more than SLACK (in base-2 exponent units): weights
-        // then stay below 2^SLACK, far inside FP16 and FP32 range, and the accumulators are rescaled a few times per row
-        // instead of at every new maximum.  The quotient acc/sum does not depend on the reference.
-        float top[QT];
-        bool grown = false;
-        #pragma unroll
-        for (int qt = 0; qt < QT; ++qt) {
-            top[qt] = row_max(fmaxf(fmaxf(fmaxf(s[qt][0][0], s[qt][0][1]), fmaxf(s[qt][0][2], s[qt][0][3])),
-                                    fmaxf(fmaxf(s[qt][1][0], s[qt][1][1]), fmaxf(s[qt][1][2], s[qt][1][3]))));
-            grown |= (top[qt] - m[qt]) * args.scale_log2 > SLACK;
-        }
-        if (__any(grown)) {
-            asm volatile("; new reference maxima" ::: "memory");          // keeps the block a branch: it is rare
-            #pragma unroll
-            for (int qt = 0; qt < QT; ++qt) {
-                const float m_new = fmaxf(m[qt], top[qt]);
-                const float alpha = __builtin_amdgcn_exp2f((m[qt] - m_new) * args.scale_log2);
-                m[qt] = m_new;
-                l[qt] *= alpha;
-                #pragma unroll
-                for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] *= alpha;
-            }
-        }
-        half8 pb[QT];
-        #pragma unroll
-        for (int qt = 0; qt < QT; ++qt) {
-            const float offset = -m[qt] * args.scale_log2;
-            float sum = 0.0f;
-            half8 p;
-            #pragma unroll
-            for (int t = 0; t < 2; ++t)
-                #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float w = __builtin_amdgcn_exp2f(fmaf(s[qt][t][r], args.scale_log2, offset));
-                    sum += w;
-                    p[4 * t + r] = (_Float16)w;
-                }
-            pb[qt] = p;
-            l[qt] += sum;
-        }
-        #pragma unroll
-        for (int jj = 0; jj < TILES; ++jj) {
-            const uint4 both = {va[jj][0].x, va[jj][0].y, va[jj][1].x, va[jj][1].y};
-            #pragma unroll
-            for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, both), pb[qt], acc[qt][jj], 0, 0, 0);
-        }
-        }
-        }
-        if (!decltype(convert_first)::value && walk0 + WALK < keys) convert((step + 1) % RING, (step + 1) & 1, walk0 + WALK);
-    }
-    };
-    if (half == 0) walk(std::true_type{}); else walk(std::false_type{});
-
-    if (idle) return;
-    #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-        const int row = row0 + qt * 16 + li;
-        const float inverse = 1.0f / row_sum(l[qt]);
-        if (row >= int(args.rows)) continue;
-        const int span_row = row / int(args.group), head = kvh * int(args.group) + row % int(args.group);
-        const size_t first = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM + 4 * g;
-        #pragma unroll
-        for (int jj = 0; jj < TILES; ++jj) {
-            const floatx4 value = acc[qt][jj] * inverse;
-            if (args.out_f16) {
-                typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-                *reinterpret_cast<half4*>(static_cast<_Float16*>(args.out) + first + 16 * jj) = half4{(_Float16)value[0], (_Float16)value[1], (_Float16)value[2], (_Float16)value[3]};
-            } else *reinterpret_cast<floatx4*>(static_cast<float*>(args.out) + first + 16 * jj) = value;
-        }
-    }
-}
-
-template<int DIM, int QT, bool Q8>
-void launch_pairs(Device& d, const PrefillArgs& args, unsigned seqs) {
-    constexpr size_t stage = size_t(2) * WALK * (Q8 ? DIM + DIM / 16 : 2 * DIM), shared = size_t(2) * (WALK * (2 * DIM + 16) + DIM * (2 * WALK + 8));
-    static_assert(tiles_ring(int(stage), int(shared)) * stage + shared <= 160 * 1024, "the stages and the tiles share the compute unit's LDS");
-    static bool raised = false;
-    if (!raised && shared > 64 * 1024) {
-        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_pairs_kernel<DIM, QT, Q8>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
-        raised = true;
-    }
-    const unsigned runs = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
-    prefill_pairs_kernel<DIM, QT, Q8><<<dim3((runs + 1) / 2, args.kv_heads, seqs), TEAM * 64, shared, d.stream>>>(args);
-}
-
-// ---- the third form, for 128 columns: K/V unpacked once per call into FP16 tiles in a workspace -------------------------
+// ---- the form for 128 columns: K/V unpacked once per call into FP16 tiles in a workspace -----------------------------------
 // A pass before the attention turns the cached rows of every (sequence, K/V head) into tiles of 64 keys, each a K block
 // [64 keys][128 columns] and a V^T block [128 columns][64 keys] of FP16, 32 KiB together, laid out in the order LDS wants them:
 // the 16-byte pieces of a K row sit at piece ^ (key % 16); a V^T row keeps the eight keys a lane multiplies at once (keys 4g.. and
@@ -669,8 +351,9 @@ __global__ void __launch_bounds__(256) unpack_tiles_kernel(PrefillArgs args, uin
     }
 }
 
-// Two runs of 4 x QT x 16 rows per workgroup (a late one and its mirror, as prefill_pairs_kernel), every wave 32 rows and both
-// halves of a 64-key step; a step's tile arrives by 32 global->LDS loads of 1 KiB, four a wave, into a ring of stages.
+// Two runs of 4 x QT x 16 rows per workgroup: one counted from the end of the span on waves 0-3 (its rows see the most keys) and
+// its mirror image from the start on waves 4-7, so every workgroup walks about the same number of (row, key) pairs and every
+// SIMD hosts one wave of each run.  Every wave holds 32 rows and takes a 64-key step whole; a step's tile arrives by 32 global->LDS loads of 1 KiB, four a wave, into a ring of stages.
 template<int DIM, int QT>
 __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) prefill_dense_kernel(PrefillArgs args, const uint8_t* tiles_in,
                                                                                                        unsigned tiles_per_seq) {
@@ -914,9 +597,7 @@ void prefill_attention(Device& d, const sdx_kv_pool* pool, const int32_t* page_t
     args.out = out; args.out_f16 = out_f16;
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     KernelTimer timer(d);
-    static const bool dense = std::getenv("STRAYDOG_PREFILL_PAIRS") == nullptr;
-    if (pool->dim == 128 && dense) { if (q8) launch_dense<128, 2, true>(d, args, unsigned(seqs)); else launch_dense<128, 2, false>(d, args, unsigned(seqs)); }
-    else if (pool->dim == 128) { if (q8) launch_pairs<128, 2, true>(d, args, unsigned(seqs)); else launch_pairs<128, 2, false>(d, args, unsigned(seqs)); }
+    if (pool->dim == 128) { if (q8) launch_dense<128, 2, true>(d, args, unsigned(seqs)); else launch_dense<128, 2, false>(d, args, unsigned(seqs)); }
     else { if (q8) launch<256, 1, true, 2>(d, args, unsigned(seqs)); else launch<256, 1, false, 2>(d, args, unsigned(seqs)); }
 }
 
