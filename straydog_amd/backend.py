@@ -305,6 +305,12 @@ class Backend:
     def fill_uniform(self, out, count, seed, lo=0.0, hi=1.0):
         self.check(self.lib.sdx_fill_uniform(self.handle, out, count, seed, lo, hi))
 
+    def mfma_probe(self, trips):
+        """Queues the matrix-core probe; returns the floating-point operations it performs."""
+        flops = ctypes.c_double()
+        self.check(self.lib.sdx_mfma_probe(self.handle, trips, ctypes.byref(flops)))
+        return flops.value
+
     def read_probe(self, source, size, blocks_per_cu=8, unroll=4):
         self.check(self.lib.sdx_read_probe(self.handle, source, size, blocks_per_cu, unroll))
 

@@ -93,6 +93,30 @@ __global__ void __launch_bounds__(256) read_probe_kernel(const probe_u4* __restr
     if (fold == 0x9e3779b9u && sink) *sink = fold;
 }
 
+// Matrix-core probe: every wave keeps eight independent chains of v_mfma_f32_16x16x32_f16 going on operands it holds in
+// registers, two waves a SIMD, nothing else in the loop.  The measured dense FP16 ceiling of the box at the clock it holds under
+// that load.
+typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
+typedef float probe_float4 __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(512) mfma_probe_kernel(unsigned trips, float* sink) {
+    probe_half8 a, b;
+    #pragma unroll
+    for (int i = 0; i < 8; ++i) { a[i] = (_Float16)(float(threadIdx.x % 7) * 0.125f); b[i] = (_Float16)(float(threadIdx.x % 5) * 0.25f); }
+    probe_float4 c[8];
+    #pragma unroll
+    for (int i = 0; i < 8; ++i) c[i] = probe_float4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (unsigned trip = 0; trip < trips; ++trip) {
+        #pragma unroll
+        for (int repeat = 0; repeat < 4; ++repeat)
+            #pragma unroll
+            for (int i = 0; i < 8; ++i) c[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c[i], 0, 0, 0);
+    }
+    float fold = 0.0f;
+    #pragma unroll
+    for (int i = 0; i < 8; ++i) fold += c[i][0] + c[i][1] + c[i][2] + c[i][3];
+    if (fold == -1.0f && sink) *sink = fold;       // never: the sums are not negative
+}
+
 }  // namespace
 
 namespace sd {
@@ -152,6 +176,16 @@ int sdx_read_probe(void* handle, const void* source, uint64_t bytes, uint32_t bl
     if (unroll >= 8) read_probe_kernel<8><<<grid, 256, 0, value.stream>>>(static_cast<const probe_u4*>(source), size_t(bytes / 16), sink);
     else if (unroll >= 4) read_probe_kernel<4><<<grid, 256, 0, value.stream>>>(static_cast<const probe_u4*>(source), size_t(bytes / 16), sink);
     else read_probe_kernel<2><<<grid, 256, 0, value.stream>>>(static_cast<const probe_u4*>(source), size_t(bytes / 16), sink);
+    SD_OP_END
+}
+
+int sdx_mfma_probe(void* handle, uint32_t trips, double* flops) {
+    SD_OP_BEGIN
+    if (!trips || trips > (1u << 24)) throw std::runtime_error("invalid Straydog matrix probe");
+    float* sink = static_cast<float*>(workspace(value, 256));
+    const unsigned groups = value.compute_units;        // one workgroup of eight waves per compute unit
+    mfma_probe_kernel<<<groups, 512, 0, value.stream>>>(trips, sink);
+    if (flops) *flops = double(groups) * 8 * double(trips) * 32 * (2.0 * 16 * 16 * 32);
     SD_OP_END
 }
 
