@@ -177,8 +177,10 @@ int sdx_copy(void* handle, void* target, const void* source, uint64_t bytes);
 /* Read-only streaming probe (16-byte loads, `unroll` per lane per trip, `blocks_per_cu` workgroups per compute unit). */
 int sdx_read_probe(void* handle, const void* source, uint64_t bytes, uint32_t blocks_per_cu, uint32_t unroll);
 /* Matrix-core probe: eight waves per compute unit, each `trips` x 32 independent v_mfma_f32_16x16x32_f16; *flops receives the
- * floating-point operations the launch performs (time it with the events above). */
-int sdx_mfma_probe(void* handle, uint32_t trips, double* flops);
+ * floating-point operations the launch performs (time it with the events above).  live = 0: tame constant operands, the
+ * rate at the clock the box holds for them; live = 1: pseudo-random operands that change from product to product, as real
+ * data does -- the matrix cores then draw more and the clock (and the rate) settles lower. */
+int sdx_mfma_probe(void* handle, uint32_t trips, int live, double* flops);
 
 #ifdef __cplusplus
 }

@@ -305,10 +305,11 @@ class Backend:
     def fill_uniform(self, out, count, seed, lo=0.0, hi=1.0):
         self.check(self.lib.sdx_fill_uniform(self.handle, out, count, seed, lo, hi))
 
-    def mfma_probe(self, trips):
-        """Queues the matrix-core probe; returns the floating-point operations it performs."""
+    def mfma_probe(self, trips, live=False):
+        """Queues the matrix-core probe (live: operands that change from product to product); returns the floating-point
+        operations it performs."""
         flops = ctypes.c_double()
-        self.check(self.lib.sdx_mfma_probe(self.handle, trips, ctypes.byref(flops)))
+        self.check(self.lib.sdx_mfma_probe(self.handle, trips, int(live), ctypes.byref(flops)))
         return flops.value
 
     def read_probe(self, source, size, blocks_per_cu=8, unroll=4):

@@ -94,27 +94,37 @@ __global__ void __launch_bounds__(256) read_probe_kernel(const probe_u4* __restr
 }
 
 // Matrix-core probe: every wave keeps eight independent chains of v_mfma_f32_16x16x32_f16 going on operands it holds in
-// registers, two waves a SIMD, nothing else in the loop.  The measured dense FP16 ceiling of the box at the clock it holds under
-// that load.
+// registers, two waves a SIMD, nothing else in the loop: the dense FP16 ceiling of the box at the clock it holds under
+// that load.  The clock depends on the operands: with LIVE ones (pseudo-random values, another pair of registers for every
+// product, as a kernel working on real data presents them) the matrix cores draw more and the shader clock settles well
+// below what it holds for the tame constants of the other variant.
 typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
 typedef float probe_float4 __attribute__((ext_vector_type(4)));
+__device__ unsigned probe_mix(unsigned x) { x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16; return x; }
+template<bool LIVE>
 __global__ void __launch_bounds__(512) mfma_probe_kernel(unsigned trips, float* sink) {
-    probe_half8 a, b;
+    probe_half8 a[4], b[4];
     #pragma unroll
-    for (int i = 0; i < 8; ++i) { a[i] = (_Float16)(float(threadIdx.x % 7) * 0.125f); b[i] = (_Float16)(float(threadIdx.x % 5) * 0.25f); }
+    for (int k = 0; k < 4; ++k)
+        #pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (LIVE) {
+                const unsigned h = probe_mix(threadIdx.x * 64 + k * 8 + i + blockIdx.x * 7919);
+                a[k][i] = (_Float16)((float(h & 0xffff) / 65536.0f - 0.5f) * 4.0f);
+                b[k][i] = (_Float16)((float(h >> 16) / 65536.0f - 0.5f) * 4.0f);
+            } else { a[k][i] = (_Float16)(float(threadIdx.x % 7) * 0.125f); b[k][i] = (_Float16)(float(threadIdx.x % 5) * 0.25f); }
+        }
     probe_float4 c[8];
     #pragma unroll
     for (int i = 0; i < 8; ++i) c[i] = probe_float4{0.0f, 0.0f, 0.0f, 0.0f};
     for (unsigned trip = 0; trip < trips; ++trip) {
         #pragma unroll
-        for (int repeat = 0; repeat < 4; ++repeat)
-            #pragma unroll
-            for (int i = 0; i < 8; ++i) c[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c[i], 0, 0, 0);
+        for (int i = 0; i < 32; ++i) c[i % 8] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i % 4], b[(i / 4) % 4], c[i % 8], 0, 0, 0);
     }
     float fold = 0.0f;
     #pragma unroll
     for (int i = 0; i < 8; ++i) fold += c[i][0] + c[i][1] + c[i][2] + c[i][3];
-    if (fold == -1.0f && sink) *sink = fold;       // never: the sums are not negative
+    if (fold == -1.0f && sink) *sink = fold;       // never in practice; keeps the products
 }
 
 }  // namespace
@@ -179,12 +189,13 @@ int sdx_read_probe(void* handle, const void* source, uint64_t bytes, uint32_t bl
     SD_OP_END
 }
 
-int sdx_mfma_probe(void* handle, uint32_t trips, double* flops) {
+int sdx_mfma_probe(void* handle, uint32_t trips, int live, double* flops) {
     SD_OP_BEGIN
     if (!trips || trips > (1u << 24)) throw std::runtime_error("invalid Straydog matrix probe");
     float* sink = static_cast<float*>(workspace(value, 256));
     const unsigned groups = value.compute_units;        // one workgroup of eight waves per compute unit
-    mfma_probe_kernel<<<groups, 512, 0, value.stream>>>(trips, sink);
+    if (live) mfma_probe_kernel<true><<<groups, 512, 0, value.stream>>>(trips, sink);
+    else mfma_probe_kernel<false><<<groups, 512, 0, value.stream>>>(trips, sink);
     if (flops) *flops = double(groups) * 8 * double(trips) * 32 * (2.0 * 16 * 16 * 32);
     SD_OP_END
 }

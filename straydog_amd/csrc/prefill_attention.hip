@@ -8,13 +8,13 @@
 // Shape of the work on gfx950 (wave64, v_mfma_f32_16x16x32_f16).  Query rows are ordered (span row, head in group), so a
 // run of consecutive rows is a run of consecutive tokens with all their grouped heads and every K/V row read serves all of
 // them.  A workgroup of 8 waves (two per SIMD) walks the keys 64 at a time, the next steps' operands travelling by 16-byte
-// global->LDS loads into a ring of stages while this one is computed; one barrier per step; steps that lie wholly after a
-// wave's rows are skipped.  Two kernels:
+// global->LDS loads into a ring of stages while this one is computed; one barrier per 64 keys; steps that lie wholly after
+// a wave's rows are skipped.  Two kernels:
 //   * prefill_dense_kernel (128 columns, the headline shape): a pass before it unpacks the cached rows once per call into
 //     FP16 tiles in a workspace, laid out as LDS wants them, so the kernel's loop converts nothing: it copies a tile, reads
-//     operands without bank conflicts, multiplies and exponentiates.  A workgroup owns two runs of 128 rows, one from the
-//     end of the span and its mirror image from the start, so every workgroup does about the same work, and writes its
-//     outputs normalised, with no merge (details at the kernels);
+//     operands without bank conflicts, multiplies and exponentiates, every wave's stream pipelined by hand.  A workgroup
+//     owns two runs of 128 rows, one from the end of the span and its mirror image from the start, so every workgroup does
+//     about the same work, and writes its outputs normalised, with no merge (details at the kernels);
 //   * prefill_attention_kernel (256 columns): 4 x QT x 16 rows per workgroup; every wave builds its own operands from the
 //     raw rows in the stage (paged_rows.hpp); a quarter of the rows belongs to a pair of waves, one taking the first 32
 //     keys of every step and one the last 32, each with its own online softmax, merged through LDS at the end; the
@@ -288,6 +288,7 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
 // kernel then copies a step's tile by plain 1 KiB global->LDS loads and has no conversion in its loop at all; the tiles are
 // read by every workgroup of the K/V head (from L2), the pass itself costs a few microseconds per call.
 constexpr int TILE_KEYS = 64;
+typedef float float2v __attribute__((ext_vector_type(2)));
 template<int DIM> constexpr int tile_bytes() { return 2 * TILE_KEYS * DIM * 2; }
 
 template<int DIM, bool Q8>
@@ -353,181 +354,227 @@ __global__ void __launch_bounds__(256) unpack_tiles_kernel(PrefillArgs args, uin
 
 // Two runs of 4 x QT x 16 rows per workgroup: one counted from the end of the span on waves 0-3 (its rows see the most keys) and
 // its mirror image from the start on waves 4-7, so every workgroup walks about the same number of (row, key) pairs and every
-// SIMD hosts one wave of each run.  Every wave holds 32 rows and takes a 64-key step whole; a step's tile arrives by 32 global->LDS loads of 1 KiB, four a wave, into a ring of stages.
+// SIMD hosts one wave of each run.  A tile of 64 keys arrives by 32 global->LDS loads of 1 KiB, four a wave, into a ring of
+// four stages; the workgroup meets once a tile.
+//
+// Every wave holds 32 rows and its own instruction stream is pipelined by hand: a step of the wave is 32 keys, and while the
+// weights of step u are formed (exponentials) the scores of step u + 1 are multiplied, the K operands of step u + 2 and the
+// V^T operands of step u are on their way from LDS, and the products O^T += V^T . P^T of step u follow -- one matrix
+// instruction, then the one or two vector instructions that fit beside it, in an order that is written out and fenced, since
+// a wave issues in order and the matrix core idles whenever the wave at its head has something else to do first.  Measured
+// on this hardware, a matrix instruction leaves room for about three plain vector instructions or one exponential; so
+// there are as few vector instructions as the arithmetic allows:
+//   * the queries carry the softmax scale (times log2 e), and the products S^T = K . Q^T start from minus the rows'
+//     reference maxima instead of zero: a score leaves the matrix core ready to be exponentiated;
+//   * the causal mask is -inf in those starting values (set up only for the one or two steps of a wave that cross its
+//     diagonal), so a masked score leaves the matrix core as -inf and costs the loop nothing;
+//   * whether some row has outgrown its reference maximum by more than the slack is one comparison per lane of the largest
+//     score a lane holds; only then (rarely) are row maxima reduced across lanes, the references moved, the sums so far
+//     scaled down, and the step's scores multiplied again from the new references -- the score registers are only ever
+//     written by the matrix cores.
 template<int DIM, int QT>
 __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) prefill_dense_kernel(PrefillArgs args, const uint8_t* tiles_in,
                                                                                                        unsigned tiles_per_seq) {
     constexpr int BLOCKS = DIM / 32, TILES = DIM / 16, KT = TILE_KEYS * DIM * 2, TILE = tile_bytes<DIM>();
-    constexpr int WAVE_ROWS = QT * 16, GROUP_ROWS = GROUPS * WAVE_ROWS, RING = 4, PER = TILE / 1024 / TEAM;
-    static_assert(WALK == TILE_KEYS && TILE % (1024 * TEAM) == 0 && RING * TILE <= 160 * 1024 - 1024, "a step is one tile, copied by the eight waves alike");
+    constexpr int WAVE_ROWS = QT * 16, GROUP_ROWS = GROUPS * WAVE_ROWS, RING = 4, PER = TILE / 1024 / TEAM, SUB = 32;
+    static_assert(TILE % (1024 * TEAM) == 0 && RING * TILE <= 160 * 1024 - 1024 && TILE_KEYS == 2 * SUB, "a tile is two steps of a wave");
     const int kvh = blockIdx.y, seq = blockIdx.z;
     const int thread = threadIdx.x, lane = thread & 63, wave = __builtin_amdgcn_readfirstlane(thread >> 6), li = lane & 15, g = lane >> 4;
     const int position = args.positions[seq];
     const int cached = min(position + int(args.span), args.max_context);
-    const int quarter = wave % GROUPS, half = wave / GROUPS;       // half 0: the run from the end of the span, half 1: its mirror
+    const int quarter = wave % GROUPS, half = wave / GROUPS;
     const int runs = (int(args.rows) + GROUP_ROWS - 1) / GROUP_ROWS;
     const int late = runs - 1 - int(blockIdx.x), early = int(blockIdx.x), run = half == 0 ? late : early;
     const int row0 = run * GROUP_ROWS + quarter * WAVE_ROWS;
     const int group_last = min(int(args.rows), (late + 1) * GROUP_ROWS) - 1;
-    const int keys = min(position + group_last / int(args.group) + 1, cached);     // the walk is the late run's
-    const bool idle = row0 >= int(args.rows) || (half == 1 && early == late);      // an odd number of runs: the middle one is alone
+    const int keys = min(position + group_last / int(args.group) + 1, cached);
+    const bool idle = row0 >= int(args.rows) || (half == 1 && early == late);
     const int wave_first = position + row0 / int(args.group);
-    const int wave_last = position + (min(int(args.rows), row0 + WAVE_ROWS) - 1) / int(args.group);
+    const int wave_last = min(position + (min(int(args.rows), row0 + WAVE_ROWS) - 1) / int(args.group), keys - 1);
+    const int steps = idle ? 0 : wave_last / SUB + 1;                              // the wave's own steps of 32 keys
     extern __shared__ __attribute__((aligned(16))) uint8_t stages[];              // [RING][K block | V^T block]
     const uint8_t* const source = tiles_in + (size_t(seq) * args.kv_heads + kvh) * tiles_per_seq * TILE + 1024 * PER * wave + 16 * lane;
-    const int last_tile = (keys - 1) / WALK;
-    const auto copy_in = [&](int step) {
-        const uint8_t* from = source + size_t(min(step, last_tile)) * TILE;
-        uint8_t* stage = stages + (step % RING) * TILE + 1024 * PER * wave;
+    const int last_tile = (keys - 1) / TILE_KEYS;
+    const auto copy_in = [&](int tile) {
+        const uint8_t* from = source + size_t(min(tile, last_tile)) * TILE;
+        uint8_t* stage = stages + (tile % RING) * TILE + 1024 * PER * wave;
         #pragma unroll
         for (int k = 0; k < PER; ++k) load_to_lds<false>(from + 1024 * k, stage + 1024 * k);
     };
 
-    half8 qf[QT][BLOCKS];
+    half8 qf[QT][BLOCKS];          // the queries times scale * log2 e: a score is a base-2 exponent
+    int limit[QT];
     #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
         const int row = row0 + qt * 16 + li;
         const bool real = row < int(args.rows);
         const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
+        limit[qt] = real ? position + span_row : 0x7fffffff;                      // a padding row masks nothing
         const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
         #pragma unroll
         for (int b = 0; b < BLOCKS; ++b) {
             half8 value = {};
             if (real) {
-                if (args.q_f16) value = *reinterpret_cast<const half8*>(static_cast<const _Float16*>(args.q) + at + 32 * b + 8 * g);
-                else {
+                if (args.q_f16) {
+                    const half8 raw = *reinterpret_cast<const half8*>(static_cast<const _Float16*>(args.q) + at + 32 * b + 8 * g);
+                    #pragma unroll
+                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)(float(raw[i]) * args.scale_log2);
+                } else {
                     const float* from = static_cast<const float*>(args.q) + at + 32 * b + 8 * g;
                     #pragma unroll
-                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)from[i];
+                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)(from[i] * args.scale_log2);
                 }
             }
             qf[qt][b] = value;
         }
     }
-    floatx4 acc[QT][TILES];
-    float m[QT], l[QT];
+    // start: where the score products of a step begin instead of zero: minus the row's reference maximum, or -inf for a key
+    // after the row's own position -- the causal mask costs the loop nothing, a masked score leaves the matrix core as -inf
+    floatx4 acc[QT][TILES], start[QT][2];
+    float l[QT], ref[QT];
     #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
-        m[qt] = NEG_BIG; l[qt] = 0.0f;
+        l[qt] = 0.0f; ref[qt] = 0.0f;
+        start[qt][0] = start[qt][1] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
         #pragma unroll
         for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
-
-    // The weights of a step and the V^T operands they meet; the second wave of a SIMD keeps them over the barrier (below).
-    half8 pb[2][QT];
-    half8 va[2][TILES];
-    const auto weigh_in = [&] {
+    const auto crosses = [&](int u) { return SUB * u + SUB - 1 > wave_first; };
+    // the starting values of a step that crosses the wave's diagonal (every later step of the wave does)
+    const auto veil = [&](int u) {
+        asm volatile("; the step crosses the diagonal" ::: "memory");
         #pragma unroll
-        for (int part = 0; part < 2; ++part)
+        for (int qt = 0; qt < QT; ++qt)
             #pragma unroll
-            for (int jj = 0; jj < TILES; ++jj)
+            for (int t = 0; t < 2; ++t)
                 #pragma unroll
-                for (int qt = 0; qt < QT; ++qt) acc[qt][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[part][jj], pb[part][qt], acc[qt][jj], 0, 0, 0);
+                for (int r = 0; r < 4; ++r) start[qt][t][r] = SUB * u + 16 * t + 4 * g + r > limit[qt] ? -INFINITY : ref[qt];
     };
-    // The two waves of a SIMD (a late run's and an early run's) meet at every step's barrier, so left alone both would multiply
-    // and then both would exponentiate.  The second one therefore carries its O^T += V^T . P^T over the barrier into the next
-    // step: while the first forms its weights (VALU), the second is at its products (MFMA), and the other way round.
-    const auto walk = [&](auto defer) {
-    constexpr bool DEFER = decltype(defer)::value;
-    bool pending = false;
-    for (int walk0 = 0, step = 0; walk0 < keys; walk0 += WALK, ++step) {
-        wait_loads<PER * (RING - 2)>();      // this step's pieces have landed when only the later steps' are outstanding
-        ring_barrier();                      // everybody's have, and everybody is done with the step before: its stage is free
-        copy_in(step + RING - 1);
-        const uint8_t* const kblock = stages + (step % RING) * TILE;
-        const uint8_t* const vblock = kblock + KT;
-        if (DEFER && pending) { weigh_in(); pending = false; }
-        if (idle || walk0 > wave_last) continue;         // (the barriers above are everybody's; the step's work is not)
-        // S^T for the step's four 16-key tiles: all of K's operands are asked for at once
-        constexpr int KEY_TILES = WALK / 16;
-        floatx4 s[QT][KEY_TILES];
-        {
-            half8 ka[KEY_TILES][BLOCKS];
-            #pragma unroll
-            for (int t = 0; t < KEY_TILES; ++t)
-                #pragma unroll
-                for (int b = 0; b < BLOCKS; ++b) ka[t][b] = *reinterpret_cast<const half8*>(kblock + (16 * t + li) * (2 * DIM) + (((4 * b + g) ^ li) * 16));
-            // eight independent chains, a column block at a time: no product waits for the one before it
-            #pragma unroll
-            for (int t = 0; t < KEY_TILES; ++t)
-                #pragma unroll
-                for (int qt = 0; qt < QT; ++qt) s[qt][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-            #pragma unroll
-            for (int b = 0; b < BLOCKS; ++b)
-                #pragma unroll
-                for (int t = 0; t < KEY_TILES; ++t)
-                    #pragma unroll
-                    for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][b], qf[qt][b], s[qt][t], 0, 0, 0);
-        }
-        // V^T's operands travel while the scores are formed: a lane's keys of a 32-key half are {4g.., 16+4g..}
+    // K operands of step u and the scores they give, relative to the references
+    const auto scores = [&](int u, floatx4 (&s)[QT][2]) {
+        const uint8_t* const kblock = stages + ((u >> 1) % RING) * TILE + (u & 1) * (SUB * 2 * DIM);
+        half8 ka[2][BLOCKS];
         #pragma unroll
-        for (int part = 0; part < 2; ++part)
+        for (int t = 0; t < 2; ++t)
             #pragma unroll
-            for (int jj = 0; jj < TILES; ++jj)
-                va[part][jj] = *reinterpret_cast<const half8*>(vblock + (16 * jj + li) * (2 * TILE_KEYS) + (((4 * part + g) ^ (li >> 1)) * 16));
-        if (walk0 + WALK - 1 > wave_first) {          // wave-uniform: some key of the step is past some row's position
-            asm volatile("; the step crosses the diagonal" ::: "memory");      // keeps the block a branch: it is rare
+            for (int b = 0; b < BLOCKS; ++b) ka[t][b] = *reinterpret_cast<const half8*>(kblock + (16 * t + li) * (2 * DIM) + (((4 * b + g) ^ li) * 16));
+        #pragma unroll
+        for (int b = 0; b < BLOCKS; ++b)
             #pragma unroll
-            for (int qt = 0; qt < QT; ++qt) {
-                const int row = row0 + qt * 16 + li;
-                const int limit = row < int(args.rows) ? position + row / int(args.group) : 0x7fffffff;   // a padding row masks nothing
+            for (int t = 0; t < 2; ++t)
                 #pragma unroll
-                for (int t = 0; t < KEY_TILES; ++t)
-                    #pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (walk0 + 16 * t + 4 * g + r > limit) s[qt][t][r] = -INFINITY;
-            }
-        }
-        float top[QT];
-        bool grown = false;
+                for (int qt = 0; qt < QT; ++qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][b], qf[qt][b], b == 0 ? start[qt][t] : s[qt][t], 0, 0, 0);
+    };
+    // The rows' maxima of step u's scores (of the keys a row may see) become (FIRST) or raise (otherwise) the references: what
+    // has been summed so far is scaled down, and the step's scores are multiplied again from the new references -- the
+    // score registers are only ever written by the matrix cores, which keeps them where they are.
+    const auto raise = [&](auto first, int u, floatx4 (&s)[QT][2]) {
+        asm volatile("; new reference maxima" ::: "memory");
         #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
             float most = s[qt][0][0];
             #pragma unroll
-            for (int t = 0; t < KEY_TILES; ++t)
+            for (int t = 0; t < 2; ++t)
                 #pragma unroll
                 for (int r = 0; r < 4; ++r) most = fmaxf(most, s[qt][t][r]);
-            top[qt] = row_max(most);
-            grown |= (top[qt] - m[qt]) * args.scale_log2 > SLACK;
-        }
-        if (__any(grown)) {
-            asm volatile("; new reference maxima" ::: "memory");          // keeps the block a branch: it is rare
-            #pragma unroll
-            for (int qt = 0; qt < QT; ++qt) {
-                const float m_new = fmaxf(m[qt], top[qt]);
-                const float alpha = __builtin_amdgcn_exp2f((m[qt] - m_new) * args.scale_log2);
-                m[qt] = m_new;
+            const float top = row_max(most);
+            const float delta = decltype(first)::value ? top : fmaxf(top, 0.0f);
+            ref[qt] -= delta;
+            start[qt][0] -= delta; start[qt][1] -= delta;
+            if (!decltype(first)::value) {
+                const float alpha = __builtin_amdgcn_exp2f(-delta);
                 l[qt] *= alpha;
                 #pragma unroll
                 for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] *= alpha;
             }
         }
-        #pragma unroll
-        for (int part = 0; part < 2; ++part)
-            #pragma unroll
-            for (int qt = 0; qt < QT; ++qt) {
-                const float offset = -m[qt] * args.scale_log2;
-                float sum = 0.0f;
-                half8 p;
-                #pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float w = __builtin_amdgcn_exp2f(fmaf(s[qt][2 * part + t][r], args.scale_log2, offset));
-                        sum += w;
-                        p[4 * t + r] = (_Float16)w;
-                    }
-                pb[part][qt] = p;
-                l[qt] += sum;
-            }
-        if (DEFER) pending = true; else weigh_in();
-    }
-    if (DEFER && pending) weigh_in();
+        scores(u, s);
     };
+    // One step: weights of step u from `now`, scores of step u + 1 into `next`, the products of step u, the maxima of step
+    // u + 1.  The order of issue is written out: between two fences the compiler finds one product and the few vector
+    // instructions that run beside it, nothing crosses a fence.
+    static_assert(QT == 2 && BLOCKS == 4 && TILES == 8, "the interleaving below is written for 32 rows x 32 keys x 128 columns");
+    half8 ka[2][BLOCKS];           // the K operands of the step after the one whose weights are being formed: read a step ahead
+    const auto read_k = [&](int u, int t, int b) {
+        const uint8_t* const kblock = stages + ((u >> 1) % RING) * TILE + (u & 1) * (SUB * 2 * DIM);
+        ka[t][b] = *reinterpret_cast<const half8*>(kblock + (16 * t + li) * (2 * DIM) + (((4 * b + g) ^ li) * 16));
+    };
+    // the workgroup's meeting once a tile: the next tile has landed (the wave's own pieces: only the tile after it is still
+    // outstanding; everybody's: the barrier), and everybody is done with the tile before this one, whose stage the tile
+    // three ahead now goes to
+    const auto meet = [&](int tile) {
+        wait_loads<PER * (RING - 3)>();
+        ring_barrier();
+        copy_in(tile + RING - 1);
+    };
+    const auto advance = [&](auto even, int u, floatx4 (&now)[QT][2], floatx4 (&next)[QT][2]) {
+        if (crosses(u + 1)) veil(u + 1);
+        const uint8_t* const vblock = stages + ((u >> 1) % RING) * TILE + KT;
+        const int part = u & 1;
+        half8 va[TILES];
+        __builtin_amdgcn_sched_barrier(0);
+        words4 pw[QT];
+        float w0[8], w1[8];
+        const auto weight = [&](float score) { return __builtin_amdgcn_exp2f(score); };
+        const auto packed = [&](float first, float second) { return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{first, second}, half2v)); };
+        #pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            // the product: column block b of key tile t for row tile qt (past the wave's last step: of whatever the stage holds, never used)
+            const int b = i / 4, t = (i / 2) % 2, qt = i % 2;
+            next[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[t][b], qf[qt][b], b == 0 ? start[qt][t] : next[qt][t], 0, 0, 0);
+            // beside it: a weight of this step's first row tile, or its sum and packing and a V^T operand
+            const int e = i / 2;
+            if (i % 2 == 0) w0[e] = weight(now[0][e / 4][e % 4]);
+            else {
+                l[0] += w0[e];
+                if (e % 2) pw[0][e / 2] = packed(w0[e - 1], w0[e]);
+            }
+            if (i < 8) {
+                va[i] = *reinterpret_cast<const half8*>(vblock + (16 * i + li) * (2 * TILE_KEYS) + (((4 * part + g) ^ (li >> 1)) * 16));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (decltype(even)::value) meet(u >> 1);        // the step after the next reads the next tile
+        __builtin_amdgcn_sched_barrier(0);
+        #pragma unroll
+        for (int j = 0; j < 8; ++j) {       // the first row tile's products, the second's weights, the K operands of the step after the next
+            acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[j], __builtin_bit_cast(half8, pw[0]), acc[0][j], 0, 0, 0);
+            w1[j] = weight(now[1][j / 4][j % 4]);
+            if (j % 2) pw[1][j / 2] = packed(w1[j - 1], w1[j]);
+            read_k(u + 2, j % 2, j / 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        float most = next[0][0][0];
+        #pragma unroll
+        for (int j = 0; j < 8; ++j) {       // the second row tile's products, its weights' sum, the next step's largest score
+            acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[j], __builtin_bit_cast(half8, pw[1]), acc[1][j], 0, 0, 0);
+            l[1] += w1[j];
+            most = fmaxf(fmaxf(most, next[j / 4][(j / 2) % 2][2 * (j % 2)]), next[j / 4][(j / 2) % 2][2 * (j % 2) + 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (__any(most > SLACK) && u + 1 < steps) raise(std::false_type{}, u + 1, next);
+    };
+
+
     settle_loads();
     #pragma unroll
     for (int ahead = 0; ahead < RING - 1; ++ahead) copy_in(ahead);
-    if (half == 0) walk(std::false_type{}); else walk(std::true_type{});
+    floatx4 even[QT][2], odd[QT][2];
+    wait_loads<PER * (RING - 2)>();
+    ring_barrier();
+    if (steps > 0) {
+        if (crosses(0)) veil(0);
+        scores(0, even);
+        raise(std::true_type{}, 0, even);
+        #pragma unroll
+        for (int b = 0; b < BLOCKS; ++b)
+            #pragma unroll
+            for (int t = 0; t < 2; ++t) read_k(1, t, b);
+    }
+    for (int tile = 0; tile <= last_tile; ++tile) {
+        if (2 * tile < steps) advance(std::true_type{}, 2 * tile, even, odd); else meet(tile);
+        if (2 * tile + 1 < steps) advance(std::false_type{}, 2 * tile + 1, odd, even);
+    }
 
     if (idle) return;
     #pragma unroll
