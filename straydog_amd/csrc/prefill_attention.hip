@@ -402,6 +402,10 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
         for (int k = 0; k < PER; ++k) load_to_lds<false>(from + 1024 * k, stage + 1024 * k);
     };
 
+    // the first tiles are on their way while the queries are fetched (the compiler's wait for the queries, which it places
+    // before their conversion right below, covers these loads too: they are older)
+    #pragma unroll
+    for (int ahead = 0; ahead < RING - 1; ++ahead) copy_in(ahead);
     half8 qf[QT][BLOCKS];          // the queries times scale * log2 e: a score is a base-2 exponent
     int limit[QT];
     #pragma unroll
@@ -556,9 +560,6 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     };
 
 
-    settle_loads();
-    #pragma unroll
-    for (int ahead = 0; ahead < RING - 1; ++ahead) copy_in(ahead);
     floatx4 even[QT][2], odd[QT][2];
     wait_loads<PER * (RING - 2)>();
     ring_barrier();
