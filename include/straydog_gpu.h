@@ -65,6 +65,24 @@ int sd_graph_begin(void* handle);
 int sd_graph_end(void* handle, uint64_t key, int keep);
 int sd_graph_run(void* handle, uint64_t key);
 
+/* ---- conversation checkpoints ---- */
+/* reference straydog_gpu.h:115 (gpu/kernels.cpp:3905-3915): page-locked host memory of `bytes` for copies of sequence state;
+ * it lives until the handle is destroyed (or sdx_checkpoint_release, straydog_gpu_ext.h). */
+void* sd_checkpoint_buffer(void* handle, uint64_t bytes);
+/* reference straydog_gpu.h:116 (gpu/kernels.cpp:3962-3990): `count` (1..4096) whole device allocations copied into (save != 0)
+ * or out of a checkpoint buffer, packed in the order given, the stream waited for once; refuses a buffer that is not a
+ * checkpoint buffer, a state that is not an allocation, and states that do not fit the buffer. */
+int sd_checkpoint_copy(void* handle, int save, void* const* states, uint64_t count, void* buffer);
+/* reference straydog_gpu.h:118 (gpu/kernels.cpp:3951-3961): checkpoint buffer `to` receives what `from` holds (equal sizes),
+ * after the stream -- and the copies into `from` it still had -- is done. */
+int sd_checkpoint_clone(void* handle, void* from, void* to);
+/* reference straydog_gpu.h:120-121 (gpu/kernels.cpp:3996-4041): part of a state to (save != 0) or from host memory: `height`
+ * runs of `width` floats, `pitch` floats apart, from float `offset` of the allocation (a K/V plane's positions are one run, a
+ * block indexer's pooled blocks one run per column); host rows are packed.  `first` is where the reference truncates the VRAM
+ * mirrors of a host-resident K/V; this library keeps K/V in HBM only and ignores it. */
+int sd_state_copy(void* handle, void* state, uint64_t offset, uint64_t pitch, uint64_t width, uint64_t height, float* host, uint64_t first,
+                  int save);
+
 /* ---- K/V format ---- */
 /* reference straydog_gpu.h:113 (gpu/kernels.cpp:4266-4274): the bytes of a K/V row of the Qwen state, 512 (FP16) or
  * 272 (Q8_0: 256 int8 then eight FP16 block scales, gpu/core.hpp:397-403).  Default 272. */

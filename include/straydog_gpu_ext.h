@@ -174,6 +174,8 @@ int sdx_profile_read(void* handle, double* milliseconds, uint64_t* launches);
 int sdx_fill_normal(void* handle, void* out, uint64_t count, uint64_t seed, int out_kind /* 0 f32, 1 f16, 2 bf16 */);
 int sdx_fill_uniform(void* handle, float* out, uint64_t count, uint64_t seed, float lo, float hi);
 int sdx_copy(void* handle, void* target, const void* source, uint64_t bytes);
+/* Frees a buffer of sd_checkpoint_buffer before the handle is destroyed (the reference keeps them for the handle's life). */
+int sdx_checkpoint_release(void* handle, void* buffer);
 /* Read-only streaming probe (16-byte loads, `unroll` per lane per trip, `blocks_per_cu` workgroups per compute unit). */
 int sdx_read_probe(void* handle, const void* source, uint64_t bytes, uint32_t blocks_per_cu, uint32_t unroll);
 /* Matrix-core probe: eight waves per compute unit, each `trips` x 32 independent v_mfma_f32_16x16x32_f16; *flops receives the

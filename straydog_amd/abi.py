@@ -50,6 +50,11 @@ SIGNATURES = {
     "sd_graph_begin": (c_int, [c_void_p]),
     "sd_graph_end": (c_int, [c_void_p, c_u64, c_int]),
     "sd_graph_run": (c_int, [c_void_p, c_u64]),
+    "sd_checkpoint_buffer": (c_void_p, [c_void_p, c_u64]),
+    "sd_checkpoint_copy": (c_int, [c_void_p, c_int, _P(c_void_p), c_u64, c_void_p]),
+    "sd_checkpoint_clone": (c_int, [c_void_p, c_void_p, c_void_p]),
+    "sd_state_copy": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_u64, c_int]),
+    "sdx_checkpoint_release": (c_int, [c_void_p, c_void_p]),
     "sd_kv_format": (c_int, [c_void_p, c_u32]),
     "sd_attention_sequence": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_u64, c_void_p, c_u64]),
     "sd_op_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float,

@@ -275,6 +275,31 @@ class Backend:
         """True when a graph is stored under key and was queued."""
         return self.check(self.lib.sd_graph_run(self.handle, key)) == 0
 
+    # ---- conversation checkpoints --------------------------------------------------------
+    def checkpoint_buffer(self, size):
+        """Page-locked host memory of `size` bytes; returns its address."""
+        pointer = self.lib.sd_checkpoint_buffer(self.handle, size)
+        if not pointer:
+            raise StraydogError(self.error())
+        return pointer
+
+    def checkpoint_release(self, pointer):
+        self.check(self.lib.sdx_checkpoint_release(self.handle, pointer))
+
+    def checkpoint_copy(self, save, states, buffer):
+        """Whole allocations (device pointers) into (save) or out of a checkpoint buffer, packed in order."""
+        array = (ctypes.c_void_p * len(states))(*states)
+        self.check(self.lib.sd_checkpoint_copy(self.handle, int(save), array, len(states), buffer))
+
+    def checkpoint_clone(self, source, target):
+        self.check(self.lib.sd_checkpoint_clone(self.handle, source, target))
+
+    def state_copy(self, state, offset, pitch, width, height, host, first, save):
+        """`height` runs of `width` floats, `pitch` apart, from float `offset` of the allocation, to (save) or from the
+        C-contiguous float32 array `host` of height x width."""
+        assert host.dtype == np.float32 and host.flags["C_CONTIGUOUS"] and host.size == width * height
+        self.check(self.lib.sd_state_copy(self.handle, state, offset, pitch, width, height, host.ctypes.data, first, int(save)))
+
     # ---- harness helpers ----------------------------------------------------------------
     def event(self):
         return self.check(self.lib.sdx_event_record(self.handle))

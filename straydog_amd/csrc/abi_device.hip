@@ -6,6 +6,7 @@
 #include "../../include/straydog_gpu_ext.h"
 
 #include <algorithm>
+#include <cstring>
 
 namespace sd {
 
@@ -183,6 +184,7 @@ void sd_destroy(void* handle) {
     for (const auto& entry : d->allocations) (void)hipFree(const_cast<uint8_t*>(entry.first));
     for (auto& event : d->events) if (event) (void)hipEventDestroy(event);
     for (auto& event : d->profile_events) (void)hipEventDestroy(event);
+    for (const auto& entry : d->checkpoints) (void)hipHostFree(entry.first);
     if (d->arena) (void)hipHostFree(d->arena);
     if (d->stream) (void)hipStreamDestroy(d->stream);
     delete d;
@@ -291,6 +293,103 @@ int sd_buffer_read(void* handle, const void* buffer, uint64_t offset, void* outp
         if (!output || offset > UINT64_MAX - bytes) throw std::runtime_error("invalid Straydog buffer read");
         op_span(d, static_cast<const uint8_t*>(buffer) + offset, size_t(bytes), "a read buffer");
         download(d, output, static_cast<const uint8_t*>(buffer) + offset, size_t(bytes));
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+// Conversation checkpoints (reference gpu/kernels.cpp:3905-3915 sd_checkpoint_buffer, :3962-3990 sd_checkpoint_copy, :3951-3961
+// sd_checkpoint_clone, :3996-4041 sd_state_copy): sequence state -- K/V pools, page tables, the block indexer's pooled blocks --
+// saved to and restored from page-locked host memory.  With the rows resident in HBM a checkpoint is the only time they cross
+// PCIe; whole allocations go as one copy each, a part of a state (a sequence's positions within a plane, one run per plane)
+// as one strided copy.
+void* sd_checkpoint_buffer(void* handle, uint64_t bytes) {
+    try {
+        Device& d = device(handle);
+        if (!bytes) throw std::runtime_error("invalid Straydog checkpoint buffer");
+        void* host = nullptr;
+        SD_CHECK(hipHostMalloc(&host, size_t(bytes), hipHostMallocDefault));
+        try {
+            std::lock_guard<std::mutex> lock(d.mutex);
+            d.checkpoints.emplace(host, size_t(bytes));
+        } catch (...) { (void)hipHostFree(host); throw; }
+        return host;
+    } catch (const std::exception& e) { last_error = e.what(); return nullptr; }
+}
+
+int sdx_checkpoint_release(void* handle, void* buffer) {
+    try {
+        Device& d = device(handle);
+        {
+            std::lock_guard<std::mutex> lock(d.mutex);
+            if (!d.checkpoints.erase(buffer)) throw std::runtime_error("Straydog: not a checkpoint buffer of this device");
+        }
+        SD_CHECK(hipStreamSynchronize(d.stream));
+        SD_CHECK(hipHostFree(buffer));
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sd_checkpoint_copy(void* handle, int save, void* const* states, uint64_t count, void* buffer) {
+    try {
+        Device& d = device(handle);
+        std::vector<size_t> sizes;
+        {
+            std::lock_guard<std::mutex> lock(d.mutex);
+            const auto found = d.checkpoints.find(buffer);
+            if (found == d.checkpoints.end() || !states || !count || count > 4096) throw std::runtime_error("invalid Straydog checkpoint copy");
+            size_t total = 0;
+            for (uint64_t i = 0; i < count; ++i) {
+                const auto state = d.allocations.find(static_cast<const uint8_t*>(states[i]));
+                if (state == d.allocations.end() || state->second > found->second - total) throw std::runtime_error("invalid Straydog checkpoint state");
+                sizes.push_back(state->second);
+                total += state->second;
+            }
+        }
+        auto* host = static_cast<uint8_t*>(buffer);
+        for (uint64_t i = 0; i < count; ++i) {
+            if (save) SD_CHECK(hipMemcpyAsync(host, states[i], sizes[i], hipMemcpyDeviceToHost, d.stream));
+            else SD_CHECK(hipMemcpyAsync(states[i], host, sizes[i], hipMemcpyHostToDevice, d.stream));
+            host += sizes[i];
+        }
+        SD_CHECK(hipStreamSynchronize(d.stream));
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sd_checkpoint_clone(void* handle, void* from, void* to) {
+    try {
+        Device& d = device(handle);
+        size_t bytes = 0;
+        {
+            std::lock_guard<std::mutex> lock(d.mutex);
+            const auto source = d.checkpoints.find(from), target = d.checkpoints.find(to);
+            if (source == d.checkpoints.end() || target == d.checkpoints.end() || source->second != target->second || from == to)
+                throw std::runtime_error("invalid Straydog checkpoint clone");
+            bytes = source->second;
+        }
+        SD_CHECK(hipStreamSynchronize(d.stream));       // the copies into `from` among what the stream still had
+        std::memcpy(to, from, bytes);
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sd_state_copy(void* handle, void* state, uint64_t offset, uint64_t pitch, uint64_t width, uint64_t height, float* host, uint64_t first, int save) {
+    try {
+        Device& d = device(handle);
+        (void)first;        // (the reference truncates its VRAM mirrors of a host-resident K/V there; here the state is the only copy)
+        size_t floats = 0;
+        {
+            std::lock_guard<std::mutex> lock(d.mutex);
+            const auto found = d.allocations.find(static_cast<const uint8_t*>(state));
+            if (found == d.allocations.end() || !host || !width || !height || pitch < width) throw std::runtime_error("invalid Straydog state copy");
+            floats = found->second / 4;
+        }
+        if (offset > floats || height - 1 > (floats - offset) / pitch || width > floats - offset - (height - 1) * pitch)
+            throw std::runtime_error("Straydog state copy outside its state");
+        float* base = static_cast<float*>(state) + offset;
+        if (save) SD_CHECK(hipMemcpy2DAsync(host, width * 4, base, pitch * 4, width * 4, height, hipMemcpyDeviceToHost, d.stream));
+        else SD_CHECK(hipMemcpy2DAsync(base, pitch * 4, host, width * 4, width * 4, height, hipMemcpyHostToDevice, d.stream));
+        SD_CHECK(hipStreamSynchronize(d.stream));
         return 0;
     } catch (const std::exception& e) { last_error = e.what(); return -1; }
 }

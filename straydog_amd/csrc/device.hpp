@@ -57,6 +57,8 @@ struct Device {
     double2* turns = nullptr;
     size_t turns_rows = 0, turns_pairs = 0, turns_armed = 0, turns_ready_rows = 0, turns_ready_pairs = 0;
     bool turns_ready = false;
+    // Page-locked host copies of sequence state (conversation checkpoints): pointer -> bytes.
+    std::map<void*, size_t> checkpoints;
     // Recorded graphs of ops (sd_graph_begin / _end / _run), by the caller's key.
     struct Recorded { hipGraph_t graph = nullptr; hipGraphExec_t executable = nullptr; };
     std::map<uint64_t, Recorded> graphs;
