@@ -305,8 +305,9 @@ __global__ void __launch_bounds__(256) block_tops_kernel(const float* scores, co
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int RADIX_BINS = 2048, RADIX_LEVELS = 3, INTERVAL_KEYS = 1024;   // digits of 11, 11 and 10 bits; groups per workgroup
-constexpr int SCORE_WAVES = 4, SCORE_BATCH = 4;                             // the rescoring kernel: waves per workgroup, groups a wave takes at a time
+constexpr int RADIX_BINS = 2048, RADIX_LEVELS = 2, INTERVAL_KEYS = 1024;   // digits of 11 and 11 bits (the cut is the k-th highest lower bound's leading 22 bits: the
+                                                                           // last 10 would spare a candidate in a thousand and cost a pass over the bounds); groups per workgroup
+constexpr int SCORE_WAVES = 4, SCORE_BATCH = 8;                             // the rescoring kernel: waves per workgroup, groups a wave takes at a time
 constexpr int BRACKET_WAVES = 8, BRACKET_KEYS = 2048, BRACKET_RING = 4;     // the bracket kernel: waves, groups per workgroup, stages per wave
 __device__ __forceinline__ uint32_t radix_digit(uint32_t key, int level) { return level == 0 ? key >> 21 : level == 1 ? (key >> 10) & 2047u : key & 1023u; }
 
@@ -329,11 +330,18 @@ __device__ __forceinline__ void load_to_lds(const void* from, const void* to) {
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt\n\ts_mov_b32 m0, %0" : "=&s"(keep) : "v"(from), "s"(base) : "memory");
 }
 
-// W of the margin for every row: sum_h |w_h| |q_h| * |scale| * 2^-14, rounded up a little.
-__global__ void __launch_bounds__(256) index_margin_kernel(const uint16_t* q, const float* weights, size_t heads, size_t dim, float scale, float* margin) {
-    // four lanes per head, 8 values a load
+// Before the bounds, a few workgroups per row: the row's histograms zeroed, its queries widened to FP32 for the canonical
+// rescoring, and (the first of them) W of the margin: sum_h |w_h| |q_h| * |scale| * 2^-14, rounded up a little.
+__global__ void __launch_bounds__(256) index_prepare_kernel(const uint16_t* q, const float* weights, size_t heads, size_t dim, float scale, size_t rows,
+                                                            float* margin, float* wide_q, uint32_t* histogram) {
     const size_t row = blockIdx.x;
-    const unsigned t = threadIdx.x, h = t / 4, part = t % 4;
+    const unsigned t = threadIdx.x, h = t / 4, part = t % 4, slice = blockIdx.y, slices = gridDim.y;
+    for (int level = 0; level < RADIX_LEVELS; ++level)
+        for (unsigned i = slice * 256 + t; i < unsigned(RADIX_BINS); i += slices * 256) histogram[(size_t(level) * rows + row) * RADIX_BINS + i] = 0u;
+    // (transposed, [column][head]: a lane per head then reads neighbouring words)
+    for (size_t i = slice * 256 + t; i < heads * dim; i += slices * 256) wide_q[row * heads * dim + (i % dim) * heads + i / dim] = bf16_value(q[row * heads * dim + i]);
+    if (slice) return;
+    // four lanes per head, 8 values a load
     float square = 0.0f;
     if (h < heads)
         for (size_t d = 8 * part; d < dim; d += 32) {
@@ -556,10 +564,11 @@ __global__ void __launch_bounds__(256) candidate_list_kernel(const float* upper,
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 255) totals[row] = at;
 }
 
-// The canonical score of every listed group: a wave takes a few groups at a time, a lane per head (the key rows in scalar
-// registers), and then adds each group's 64 terms in head order -- lane c the terms of group c, read from LDS, so the
-// ordered sums run side by side.  The workgroup's waves share one copy of the row's queries in LDS, transposed so
-// that the lanes of a wave read neighbouring words; few registers, so many waves hide the loads' latency.
+// The canonical score of every listed group: a wave takes a few groups at a time, a lane per head with the head's 128 query
+// values in its registers; a key row is 64 words, lane i fetches word i (one coalesced load, the next group's row on its
+// way while this one is used) and the words go round by v_readlane, so a group costs a wave 64 broadcasts and 128
+// multiply-adds in the canonical column order.  Then each group's 64 terms are added in head order -- lane c the terms of
+// group c, read from LDS, so the ordered sums run side by side.
 template<int HEADS>
 __global__ void __launch_bounds__(SCORE_WAVES * 64) candidate_score_kernel(const float* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
                                                               size_t groups, float scale, const int32_t* __restrict__ list, const uint32_t* __restrict__ totals,
@@ -570,28 +579,24 @@ __global__ void __launch_bounds__(SCORE_WAVES * 64) candidate_score_kernel(const
     const int head = min(lane, HEADS - 1);
     const uint32_t total = totals[row];
     if (blockIdx.x * SCORE_WAVES * BATCH >= total) return;
-    __shared__ float shared_q[DIM][HEADS + 1];
     __shared__ float terms[SCORE_WAVES][BATCH][HEADS + 1];
-    for (int i = threadIdx.x; i < HEADS * DIM; i += SCORE_WAVES * 64) shared_q[i % DIM][i / DIM] = q[row * HEADS * DIM + i];
-    __syncthreads();
+    float mine[DIM];
+    #pragma unroll
+    for (int d = 0; d < DIM; ++d) mine[d] = q[(row * DIM + d) * HEADS + head];          // [column][head]
     const float weight = weights[row * HEADS + head];
     const uint32_t* row_keys = reinterpret_cast<const uint32_t*>(keys + row * groups * DIM);
     for (uint32_t first = (blockIdx.x * SCORE_WAVES + wave) * BATCH; first < total; first += gridDim.x * SCORE_WAVES * BATCH) {
         const int count = int(min(uint32_t(BATCH), total - first));
-        // A key row is 64 words: lane i fetches word i (one coalesced load), the words then go round by v_readlane.  The next
-        // group's row is on its way while this one is used.
         uint32_t words = row_keys[size_t(list[row * groups + first]) * (DIM / 2) + lane];
         for (int c = 0; c < count; ++c) {
             const uint32_t current = words;
             if (c + 1 < count) words = row_keys[size_t(list[row * groups + first + c + 1]) * (DIM / 2) + lane];
-            const float* mine = &shared_q[0][head];
-            asm volatile("" : "+v"(mine));               // read anew for every group: the values are not kept in registers
             float dot = 0.0f;
             #pragma unroll
             for (int d = 0; d < DIM; d += 2) {
                 const uint32_t pair = __builtin_amdgcn_readlane(current, d / 2);
-                dot = __builtin_fmaf(mine[d * (HEADS + 1)], __uint_as_float(pair << 16), dot);
-                dot = __builtin_fmaf(mine[(d + 1) * (HEADS + 1)], __uint_as_float(pair & 0xffff0000u), dot);
+                dot = __builtin_fmaf(mine[d], __uint_as_float(pair << 16), dot);
+                dot = __builtin_fmaf(mine[d + 1], __uint_as_float(pair & 0xffff0000u), dot);
             }
             if (lane < HEADS) terms[wave][c][lane] = rounded_product(fmaxf(dot, 0.0f), weight);
         }
@@ -610,7 +615,16 @@ __global__ void __launch_bounds__(TOPK_THREADS) top_k_listed_kernel(const float*
                                                                     int32_t* out) {
     const float* s = scores + size_t(blockIdx.x) * groups;
     const int32_t* c = list + size_t(blockIdx.x) * groups;
-    top_k_row([=](size_t v) { return s[v]; }, [=](size_t v) { return c[v]; }, totals[blockIdx.x], k, out + size_t(blockIdx.x) * k);
+    const uint32_t total = totals[blockIdx.x];
+    // the select passes over the scores five times: a list this short (k and a few) is read from memory once
+    constexpr uint32_t HELD = 6144;
+    __shared__ float held_scores[HELD];
+    __shared__ int32_t held_list[HELD];
+    if (total <= HELD) {
+        for (uint32_t v = threadIdx.x; v < total; v += TOPK_THREADS) { held_scores[v] = s[v]; held_list[v] = c[v]; }
+        __syncthreads();
+        top_k_row([&](size_t v) { return held_scores[v]; }, [&](size_t v) { return held_list[v]; }, total, k, out + size_t(blockIdx.x) * k);
+    } else top_k_row([=](size_t v) { return s[v]; }, [=](size_t v) { return c[v]; }, total, k, out + size_t(blockIdx.x) * k);
 }
 
 __global__ void fill_words_kernel(uint32_t* to, size_t count) {
@@ -664,8 +678,7 @@ FastIndexSpace fast_index_space(void* base, size_t batch, size_t groups, size_t 
 template<int HEADS>
 void fast_index_bounds(Device& d, const FastIndexSpace& s, const void* q_index, const void* keys, const float* weights, const int32_t* visible, size_t batch,
                        size_t groups, float scale) {
-    fill_words_kernel<<<unsigned(std::min<size_t>(checked_blocks(RADIX_LEVELS * batch * RADIX_BINS), 1024)), 256, 0, d.stream>>>(s.histogram, RADIX_LEVELS * batch * RADIX_BINS);
-    index_margin_kernel<<<unsigned(batch), 256, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), weights, HEADS, 128, scale, s.margin);
+    index_prepare_kernel<<<dim3(unsigned(batch), 8), 256, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), weights, HEADS, 128, scale, batch, s.margin, s.wide_q, s.histogram);
     index_interval_kernel<HEADS><<<dim3(unsigned((groups + BRACKET_KEYS - 1) / BRACKET_KEYS), unsigned(batch)), BRACKET_WAVES * 64, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys),
                                                                                                    weights, visible, s.margin, groups, scale, s.lower, s.upper, s.histogram);
     SD_CHECK(hipGetLastError());
@@ -675,14 +688,12 @@ template<int HEADS>
 void fast_index_top_k(Device& d, const FastIndexSpace& s, const void* q_index, const void* keys, const float* weights, const int32_t* visible, size_t batch,
                       size_t groups, float scale, size_t k, int32_t* indices) {
     const dim3 grid(unsigned(s.blocks), unsigned(batch));
-    widen_bf16(d, q_index, s.wide_q, batch * HEADS * 128);
     {
         KernelTimer timer(d);
         fast_index_bounds<HEADS>(d, s, q_index, keys, weights, visible, batch, groups, scale);
     }
     const uint32_t rank = uint32_t(std::min<size_t>(k, 0xffffffffu));
     radix_histogram_kernel<<<grid, 256, 0, d.stream>>>(s.lower, groups, batch, 1, rank, s.histogram);
-    radix_histogram_kernel<<<grid, 256, 0, d.stream>>>(s.lower, groups, batch, 2, rank, s.histogram);
     candidate_count_kernel<<<grid, 256, 0, d.stream>>>(s.upper, groups, batch, rank, s.histogram, s.counts);
     candidate_list_kernel<<<grid, 256, 0, d.stream>>>(s.upper, groups, batch, rank, s.histogram, s.counts, s.list, s.totals);
     candidate_score_kernel<HEADS><<<dim3(unsigned((k + k / 8 + 64 + SCORE_WAVES * SCORE_BATCH - 1) / (SCORE_WAVES * SCORE_BATCH)), unsigned(batch)), SCORE_WAVES * 64, 0, d.stream>>>(s.wide_q, static_cast<const uint16_t*>(keys), weights, groups, scale, s.list, s.totals,

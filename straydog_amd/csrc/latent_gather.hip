@@ -62,17 +62,37 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
     float m = NEG_BIG, l = 0.0f;
 
     const int first = chunk * CHUNK, last = min(int(a.k), first + CHUNK);
+    // gather: a row is PIECES pieces of 16 bytes, a thread takes every 256th piece of a step; a missing row is read from row 0
+    // and masked.  The pieces of the step after this one are fetched into registers before this one is multiplied.
+    constexpr int MINE = (STEP * PIECES + 255) / 256;
+    uint4 fetched[MINE];
+    uint32_t present = 0;                                     // bit j: the row of the thread's j-th piece exists
+    const auto fetch = [&](int key0) {
+        present = 0;
+        #pragma unroll
+        for (int j = 0; j < MINE; ++j) {
+            const int piece = thread + 256 * j, row = piece / PIECES, part = piece % PIECES;
+            fetched[j] = uint4{0u, 0u, 0u, 0u};
+            if (piece < STEP * PIECES) {
+                const int index = key0 + row < last ? a.selected[size_t(batch) * a.k + key0 + row] : -1;
+                const bool exists = index >= 0 && index < int(a.groups);
+                fetched[j] = *reinterpret_cast<const uint4*>(a.latents + (size_t(batch) * a.groups + (exists ? index : 0)) * KDIM + 8 * part);
+                present |= exists ? 1u << j : 0u;
+            }
+        }
+    };
+    if (first < last) fetch(first);
     for (int key0 = first; key0 < last; key0 += STEP) {
         __syncthreads();                                      // the tiles of the step before are done with
-        // gather: a row is PIECES pieces of 16 bytes; a missing row is read from row 0 and masked
-        for (int piece = thread; piece < STEP * PIECES; piece += 256) {
-            const int row = piece / PIECES, part = piece % PIECES;
-            const int index = key0 + row < last ? a.selected[size_t(batch) * a.k + key0 + row] : -1;
-            const bool exists = index >= 0 && index < int(a.groups);
-            const uint4 bits = *reinterpret_cast<const uint4*>(a.latents + (size_t(batch) * a.groups + (exists ? index : 0)) * KDIM + 8 * part);
-            *reinterpret_cast<uint4*>(ktile + row * KP + 16 * part) = bits;
-            if (part == 0) seen[row] = exists ? 1u : 0u;
+        #pragma unroll
+        for (int j = 0; j < MINE; ++j) {
+            const int piece = thread + 256 * j, row = piece / PIECES, part = piece % PIECES;
+            if (piece < STEP * PIECES) {
+                *reinterpret_cast<uint4*>(ktile + row * KP + 16 * part) = fetched[j];
+                if (part == 0) seen[row] = (present >> j) & 1u;
+            }
         }
+        if (key0 + STEP < last) fetch(key0 + STEP);
         __syncthreads();
         // V tile: 4 rows x 4 columns at a time, transposed
         for (int block = thread; block < (STEP / 4) * (VDIM / 4); block += 256) {
