@@ -308,7 +308,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 constexpr int RADIX_BINS = 2048, RADIX_LEVELS = 2, INTERVAL_KEYS = 1024;   // digits of 11 and 11 bits (the cut is the k-th highest lower bound's leading 22 bits: the
                                                                            // last 10 would spare a candidate in a thousand and cost a pass over the bounds); groups per workgroup
 constexpr int SCORE_WAVES = 4, SCORE_BATCH = 8;                             // the rescoring kernel: waves per workgroup, groups a wave takes at a time
-constexpr int BRACKET_WAVES = 8, BRACKET_KEYS = 2048, BRACKET_RING = 4;     // the bracket kernel: waves, groups per workgroup, stages per wave
+constexpr int BRACKET_WAVES = 8, BRACKET_KEYS = 4096, BRACKET_RING = 4;     // the bracket kernel: waves, groups per workgroup, stages per wave
 __device__ __forceinline__ uint32_t radix_digit(uint32_t key, int level) { return level == 0 ? key >> 21 : level == 1 ? (key >> 10) & 2047u : key & 1023u; }
 
 // The sum over the four lanes li, li + 16, li + 32, li + 48 in all of them (see paged_rows.hpp for the instructions).

@@ -19,7 +19,7 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-constexpr int CHUNK = 128;          // selected rows per workgroup
+constexpr int CHUNK = 64;           // selected rows per workgroup
 
 struct GatherArgs {
     const uint16_t* q;              // [batch][heads][kdim] BF16
@@ -131,7 +131,11 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
             }
         }
         top = row_max(top);
-        if (__any(top > m)) {
+        // The reference maximum moves only when some head's maximum has outgrown it by more than 2^8 (weights stay below 2^8,
+        // and 128 accumulator registers are not multiplied through at every step); the first step sets it, nothing is summed yet.
+        if (key0 == first) m = top;
+        else if (__any((top - m) * a.scale_log2 > 8.0f)) {
+            asm volatile("; new reference maxima" ::: "memory");
             const float m_new = fmaxf(m, top), alpha = __builtin_amdgcn_exp2f((m - m_new) * a.scale_log2);
             m = m_new;
             l *= alpha;
@@ -174,20 +178,39 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
 }
 
 // One block per (sequence, head): the chunks merged under their common maximum and normalised; a head none of whose
-// rows exists gives zeros.
+// rows exists gives zeros.  The chunks' pieces are asked for eight at a time, so that eight loads are in flight and not one.
 template<int VDIM>
 __global__ void __launch_bounds__(VDIM / 4) latent_merge_kernel(GatherArgs a) {
     const size_t item = blockIdx.x, batch = item / a.heads, head = item % a.heads;
     const float* base = a.partial + (batch * a.chunks * a.heads + head) * (VDIM + 2);
     const size_t step = size_t(a.heads) * (VDIM + 2);
+    constexpr unsigned AT_ONCE = 8;
     float top = NEG_BIG;
-    for (unsigned c = 0; c < a.chunks; ++c) top = fmaxf(top, base[c * step + VDIM]);
+    for (unsigned c0 = 0; c0 < a.chunks; c0 += AT_ONCE) {
+        float tops[AT_ONCE];
+        #pragma unroll
+        for (unsigned i = 0; i < AT_ONCE; ++i) tops[i] = base[min(c0 + i, a.chunks - 1) * step + VDIM];
+        #pragma unroll
+        for (unsigned i = 0; i < AT_ONCE; ++i) top = fmaxf(top, tops[i]);
+    }
     floatx4 value = {0.0f, 0.0f, 0.0f, 0.0f};
     float sum = 0.0f;
-    for (unsigned c = 0; c < a.chunks; ++c) {
-        const float weight = __builtin_amdgcn_exp2f((base[c * step + VDIM] - top) * a.scale_log2);
-        sum += base[c * step + VDIM + 1] * weight;
-        value += *reinterpret_cast<const floatx4*>(base + c * step + 4 * threadIdx.x) * weight;
+    for (unsigned c0 = 0; c0 < a.chunks; c0 += AT_ONCE) {
+        floatx4 values[AT_ONCE];
+        float tops[AT_ONCE], sums[AT_ONCE];
+        #pragma unroll
+        for (unsigned i = 0; i < AT_ONCE; ++i) {
+            const size_t at = min(c0 + i, a.chunks - 1) * step;
+            values[i] = *reinterpret_cast<const floatx4*>(base + at + 4 * threadIdx.x);
+            tops[i] = base[at + VDIM];
+            sums[i] = base[at + VDIM + 1];
+        }
+        #pragma unroll
+        for (unsigned i = 0; i < AT_ONCE; ++i) {
+            const float weight = c0 + i < a.chunks ? __builtin_amdgcn_exp2f((tops[i] - top) * a.scale_log2) : 0.0f;
+            sum += sums[i] * weight;
+            value += values[i] * weight;
+        }
     }
     if (sum > 0.0f) value *= 1.0f / sum; else value = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     *reinterpret_cast<floatx4*>(a.out + item * VDIM + 4 * threadIdx.x) = value;
