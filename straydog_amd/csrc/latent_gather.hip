@@ -48,6 +48,10 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
     uint8_t* ktile = lds;                                     // [32 rows][KP]
     uint8_t* vtile = ktile + STEP * KP;                       // [VDIM columns][VP]
     uint32_t* seen = reinterpret_cast<uint32_t*>(vtile + VDIM * VP);   // [32]: 1 where the step's row exists
+    int32_t* chosen = reinterpret_cast<int32_t*>(seen + STEP);         // [CHUNK]: the workgroup's selected rows, -1 where there is none
+    const int first = chunk * CHUNK, last = min(int(a.k), first + CHUNK);
+    // the selection is read once, ahead of everything else: a step's rows then wait for one load, not for two in a row
+    if (thread < CHUNK) chosen[thread] = first + thread < last ? a.selected[size_t(batch) * a.k + first + thread] : -1;
 
     bf16x8 qf[KSTEPS];
     #pragma unroll
@@ -61,7 +65,7 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
     for (int jj = 0; jj < TILES; ++jj) acc[jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     float m = NEG_BIG, l = 0.0f;
 
-    const int first = chunk * CHUNK, last = min(int(a.k), first + CHUNK);
+    __syncthreads();
     // gather: a row is PIECES pieces of 16 bytes, a thread takes every 256th piece of a step; a missing row is read from row 0
     // and masked.  The pieces of the step after this one are fetched into registers before this one is multiplied.
     constexpr int MINE = (STEP * PIECES + 255) / 256;
@@ -74,7 +78,8 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
             const int piece = thread + 256 * j, row = piece / PIECES, part = piece % PIECES;
             fetched[j] = uint4{0u, 0u, 0u, 0u};
             if (piece < STEP * PIECES) {
-                const int index = key0 + row < last ? a.selected[size_t(batch) * a.k + key0 + row] : -1;
+ 
+                const int index = chosen[key0 - first + row];
                 const bool exists = index >= 0 && index < int(a.groups);
                 fetched[j] = *reinterpret_cast<const uint4*>(a.latents + (size_t(batch) * a.groups + (exists ? index : 0)) * KDIM + 8 * part);
                 present |= exists ? 1u << j : 0u;
@@ -234,7 +239,7 @@ void latent_gather(Device& d, const void* q, const void* latents, const int32_t*
     args.q = static_cast<const uint16_t*>(q); args.latents = static_cast<const uint16_t*>(latents); args.selected = selected;
     args.groups = unsigned(groups); args.k = unsigned(k); args.heads = unsigned(heads); args.chunks = unsigned((k + CHUNK - 1) / CHUNK);
     args.scale_log2 = scale * 1.44269504088896341f; args.partial = partial; args.out = out;
-    constexpr size_t shared = size_t(STEP) * (2 * KDIM + 16) + size_t(VDIM) * (2 * STEP + 8) + STEP * 4;
+    constexpr size_t shared = size_t(STEP) * (2 * KDIM + 16) + size_t(VDIM) * (2 * STEP + 8) + STEP * 4 + CHUNK * 4;
     static bool raised = false;
     if (!raised) {
         SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_gather_kernel<KDIM, VDIM>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
