@@ -30,19 +30,24 @@ MEASURED_TRAFFIC = {"config1": 630.7e6, "config1_32k": 1147.4e6}
 
 
 def timed(gpu, step, steps, warmup):
-    """(ms per step over the whole stream, ms per launch of the dominant kernel) for `steps` steps after `warmup`."""
+    """(ms per step over the whole stream, ms per launch of the dominant kernel) for `steps` steps after `warmup`.  Two passes of
+    the same `steps` steps: the first is bracketed by two events and nothing else (the step time), the second also brackets
+    every launch of the dominant kernel (the kernel time) -- the extra events stall the queue for a few microseconds per
+    launch, which the step time should not carry."""
     for _ in range(warmup):
         step()
     gpu.synchronize()
-    gpu.profile(True)
     begin = gpu.event()
     for _ in range(steps):
         step()
     end = gpu.event()
     total = gpu.elapsed_ms(begin, end)
+    gpu.events_clear()
+    gpu.profile(True)
+    for _ in range(steps):
+        step()
     kernel_ms, launches = gpu.profile_read()
     gpu.profile(False)
-    gpu.events_clear()
     return total / steps, (kernel_ms / launches if launches else None)
 
 
