@@ -343,9 +343,17 @@ __global__ void __launch_bounds__(256) paged_merge_kernel(PagedArgs args, void* 
         sum = sum * keep + (reduce[1][0] + reduce[1][1]) + (reduce[1][2] + reduce[1][3]);
         value.x *= keep; value.y *= keep;
         top = top_new;
-        for (unsigned k = group; k < count; k += GROUPS) {
-            const float2 v = *reinterpret_cast<const float2*>(base + (first + k) * step + col);
-            value.x += v.x * weights[k]; value.y += v.y * weights[k];
+        // eight of a group's chunks at a time: eight loads in flight, not one after the other
+        constexpr unsigned AT_ONCE = 8;
+        for (unsigned k0 = group; k0 < count; k0 += AT_ONCE * GROUPS) {
+            float2 v[AT_ONCE];
+            #pragma unroll
+            for (unsigned i = 0; i < AT_ONCE; ++i) v[i] = *reinterpret_cast<const float2*>(base + (first + min(k0 + i * GROUPS, count - 1)) * step + col);
+            #pragma unroll
+            for (unsigned i = 0; i < AT_ONCE; ++i) {
+                const float w_k = k0 + i * GROUPS < count ? weights[k0 + i * GROUPS] : 0.0f;
+                value.x += v[i].x * w_k; value.y += v[i].y * w_k;
+            }
         }
         __syncthreads();      // weights and reduce are rewritten by the next pass
     }
