@@ -173,14 +173,30 @@ __global__ void __launch_bounds__(DIM) selected_merge_kernel(SelectedArgs a, con
     const unsigned head = blockIdx.x % a.heads, kvh = head / a.group, col = threadIdx.x;
     const unsigned used = (list_length(a, row) + CHUNK - 1) / CHUNK;
     const float* base = a.partial + ((row * a.kv_heads + kvh) * a.chunks) * 16 * STRIDE + size_t(head % a.group) * STRIDE;
+    // the chunks' pieces are asked for eight at a time: eight loads in flight, not one after the other
+    constexpr unsigned AT_ONCE = 8;
     float top = NEG_BIG;
-    for (unsigned c = 0; c < used; ++c) top = fmaxf(top, base[size_t(c) * 16 * STRIDE + DIM]);
+    for (unsigned c0 = 0; c0 < used; c0 += AT_ONCE) {
+        float tops[AT_ONCE];
+        #pragma unroll
+        for (unsigned i = 0; i < AT_ONCE; ++i) tops[i] = base[size_t(min(c0 + i, used - 1)) * 16 * STRIDE + DIM];
+        #pragma unroll
+        for (unsigned i = 0; i < AT_ONCE; ++i) top = fmaxf(top, tops[i]);
+    }
     float sum = 0.0f, value = 0.0f;
-    for (unsigned c = 0; c < used; ++c) {
-        const float* part = base + size_t(c) * 16 * STRIDE;
-        const float weight = __builtin_amdgcn_exp2f(part[DIM] - top);
-        sum += part[DIM + 1] * weight;
-        value += part[col] * weight;
+    for (unsigned c0 = 0; c0 < used; c0 += AT_ONCE) {
+        float tops[AT_ONCE], sums[AT_ONCE], values[AT_ONCE];
+        #pragma unroll
+        for (unsigned i = 0; i < AT_ONCE; ++i) {
+            const float* part = base + size_t(min(c0 + i, used - 1)) * 16 * STRIDE;
+            tops[i] = part[DIM]; sums[i] = part[DIM + 1]; values[i] = part[col];
+        }
+        #pragma unroll
+        for (unsigned i = 0; i < AT_ONCE; ++i) {
+            const float weight = c0 + i < used ? __builtin_amdgcn_exp2f(tops[i] - top) : 0.0f;
+            sum += sums[i] * weight;
+            value += values[i] * weight;
+        }
     }
     value = sum > 0.0f ? value / sum : 0.0f;
     if (gate) {
