@@ -166,6 +166,42 @@ def test_prefill_span_rows(gpu, oracle, dim, fmt, span, heads, kv_heads):
     gpu.release(buffer); gpu.release(tb)
 
 
+@pytest.mark.parametrize("fmt", ["q8", "f16"])
+def test_prefill_with_scores_that_keep_growing(gpu, oracle, fmt):
+    # Keys whose scores rise along the sequence (k_t = t/8 * u + noise, queries along u) make every row's maximum outgrow its
+    # reference again and again: the path that moves the references, scales what was summed and multiplies the step's scores
+    # anew runs many times per row; rows of small and large magnitude sit side by side, one head has zero queries.
+    rng = np.random.default_rng(91)
+    dim, page_tokens, heads, kv_heads, span, context = 128, 64, 16, 2, 160, 300
+    row_bytes = (dim + dim // 16) if fmt == "q8" else 2 * dim
+    total = span + context
+    pages = (total + page_tokens - 1) // page_tokens
+    table = rng.permutation(pages + 1)[:pages].astype(np.int32).reshape(1, pages)
+    host = np.zeros(oracle.pool_bytes(pages + 1, kv_heads, page_tokens, row_bytes), dtype=np.uint8)
+    u = rng.standard_normal(dim).astype(np.float32)
+    u /= np.linalg.norm(u)
+    rise = (np.arange(total, dtype=np.float32) / 8.0)[None, :, None, None] * u[None, None, None, :]
+    k = (rise + 0.3 * rng.standard_normal((1, total, kv_heads, dim))).astype(np.float16).astype(np.float32)
+    v = rng.standard_normal((1, total, kv_heads, dim)).astype(np.float16).astype(np.float32)
+    oracle.kv_write(host, row_bytes, page_tokens, kv_heads, dim, table, np.zeros(1, np.int32), k, v)
+    pool, buffer = gpu.kv_pool(pages + 1, page_tokens, kv_heads, dim, row_bytes)
+    gpu.write_buffer(buffer, 0, host)
+    tb = gpu.upload(table)
+    # (with Q8_0 rows the operands' FP16 rounding of values around 50 limits how sharp a softmax the 2e-3 bound can be asked
+    # of: the decode kernel shows the same errors; FP16 rows carry no such rounding)
+    strength = rng.choice([0.5, 4.0, 30.0] if fmt == "f16" else [0.5, 2.0, 4.0], size=(1, span, heads, 1)).astype(np.float32)
+    q = (strength * u[None, None, None, :] + 0.2 * rng.standard_normal((1, span, heads, dim))).astype(np.float16).astype(np.float32)
+    q[:, :, 3] = 0.0
+    scale = 1.0 / np.sqrt(dim)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array([context], np.int32), q, scale)
+    got = _run(gpu, pool, table, tb, [context], q, span, heads, scale, True, False)
+    close_enough(got, want, f"growing scores {fmt}")
+    for r in (0, 77, span - 1):                 # the decode kernel at the same rows: another route to the same numbers
+        single = _run(gpu, pool, table, tb, [context + r], q[:, r:r + 1], 1, heads, scale, True, False, max_context=total)
+        assert np.abs(single[:, 0] - got[:, r]).max() < 1e-3
+    gpu.release(buffer); gpu.release(tb)
+
+
 def test_prefill_in_chunks_equals_prefill_at_once(gpu, oracle):
     # a prompt prefilled in 4 chunks (each chunk attends the cache so far) gives the rows of one whole-prompt pass
     rng = np.random.default_rng(5)
