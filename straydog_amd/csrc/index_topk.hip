@@ -627,10 +627,6 @@ __global__ void __launch_bounds__(TOPK_THREADS) top_k_listed_kernel(const float*
     } else top_k_row([=](size_t v) { return s[v]; }, [=](size_t v) { return c[v]; }, total, k, out + size_t(blockIdx.x) * k);
 }
 
-__global__ void fill_words_kernel(uint32_t* to, size_t count) {
-    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) to[i] = 0u;
-}
-
 __global__ void widen_bf16_kernel(const uint16_t* from, float* to, size_t count) {
     for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) to[i] = bf16_value(from[i]);
 }
