@@ -316,6 +316,81 @@ __device__ __forceinline__ void choose_blocks(SelectShared& sh, Each each_run, B
     });
 }
 
+// A short span's rows (a decode step, a verification span) would leave all but a few compute units idle while one workgroup a
+// row sweeps 60K values.  For those the thinning is spread out: THIN_SEGMENTS workgroups a row each find the same guess from the
+// same sample of the row (the R-th highest of 4096 values spread evenly over it, to 24 bits) and list, in block order, the values
+// of their own stretch of the row that reach it; the row's workgroup then only gathers the lists.  A stretch whose list does
+// not fit says so and the row's workgroup does all the work itself, as it does for rows too short to be worth it.
+constexpr int THIN_SEGMENTS = 32, THIN_THREADS = 256, THIN_CAP = 256, THIN_ROWS = 8, THIN_SAMPLE = 4096;
+constexpr uint32_t THIN_NONE = 0xffffffffu;
+__global__ void __launch_bounds__(THIN_THREADS) thin_kernel(const float* __restrict__ scores, size_t pool, size_t base, const uint32_t* dynamic,
+                                                            uint2* __restrict__ listed, uint32_t* __restrict__ listed_counts) {
+    __shared__ uint32_t bins[THIN_SAMPLE];
+    __shared__ uint32_t wave_sums[THIN_THREADS / 64], found[2];
+    if (dynamic) base = *dynamic;
+    const size_t token = blockIdx.y, position = base + token, complete = (position + 1) / 4;
+    const unsigned t = threadIdx.x, lane = t % 64, wave = t / 64, segment = blockIdx.x;
+    uint32_t* const count_out = listed_counts + token * THIN_SEGMENTS + segment;
+    if (position + 1 > 4 * pool || complete < size_t(8) * SELECT_THREADS) {          // (the row's workgroup decides the same way)
+        if (t == 0) *count_out = THIN_NONE;
+        return;
+    }
+    const uint32_t* row = reinterpret_cast<const uint32_t*>(scores + token * pool);   // scores are sums of max(., 0): their bits order as they do
+    constexpr unsigned MINE = THIN_SAMPLE / THIN_THREADS;
+    uint32_t sample[MINE];
+    #pragma unroll
+    for (unsigned k = 0; k < MINE; ++k) sample[k] = row[size_t(t + THIN_THREADS * k) * complete / THIN_SAMPLE];
+    uint32_t guess = 0, rank = uint32_t(3 * size_t(KEEP) * THIN_SAMPLE / (2 * complete)) + 16;
+    #pragma unroll 1
+    for (int shift = 20; shift >= 8; shift -= 12) {          // the sample's rank-th highest value to 24 bits: 12 bits a level
+        for (unsigned i = t; i < unsigned(THIN_SAMPLE); i += THIN_THREADS) bins[i] = 0;
+        __syncthreads();
+        #pragma unroll
+        for (unsigned k = 0; k < MINE; ++k)
+            if (shift == 20 || (sample[k] >> 20) == (guess >> 20)) atomicAdd(bins + ((sample[k] >> shift) & 4095u), 1u);
+        __syncthreads();
+        // thread t holds the 16 bins below 4096 - 16 t, highest first: a scan in thread order counts the values in higher bins
+        uint32_t mine[MINE], sum = 0;
+        #pragma unroll
+        for (unsigned j = 0; j < MINE; ++j) { mine[j] = bins[4095 - MINE * t - j]; sum += mine[j]; }
+        uint32_t inclusive = sum;
+        #pragma unroll
+        for (unsigned offset = 1; offset < 64; offset *= 2) { const uint32_t other = __shfl_up(inclusive, offset); if (lane >= offset) inclusive += other; }
+        if (lane == 63) wave_sums[wave] = inclusive;
+        __syncthreads();
+        uint32_t above = inclusive - sum;
+        for (unsigned w = 0; w < wave; ++w) above += wave_sums[w];
+        #pragma unroll
+        for (unsigned j = 0; j < MINE; ++j) {
+            if (above < rank && above + mine[j] >= rank) { found[0] = guess | ((4095 - MINE * t - j) << shift); found[1] = rank - above; }
+            above += mine[j];
+        }
+        __syncthreads();
+        guess = found[0]; rank = found[1];
+    }
+    // the stretch's values that reach the guess, in block order
+    const size_t stretch = (complete + THIN_SEGMENTS - 1) / THIN_SEGMENTS, first = segment * stretch, last = min(first + stretch, complete);
+    uint2* const out = listed + (token * THIN_SEGMENTS + segment) * THIN_CAP;
+    uint32_t written = 0;
+    const uint64_t below = (uint64_t(1) << lane) - 1;
+    for (size_t at = first; at < last; at += THIN_THREADS) {
+        const size_t block = at + t;
+        const uint32_t bits = block < last ? row[block] : 0u;
+        const bool reaches = block < last && bits >= guess;
+        const uint64_t reaching = __ballot(reaches);
+        __syncthreads();                                     // the counts of the round before are read
+        if (lane == 0) wave_sums[wave] = uint32_t(__popcll(reaching));
+        __syncthreads();
+        uint32_t before = written, round = 0;
+        #pragma unroll
+        for (unsigned w = 0; w < THIN_THREADS / 64; ++w) { before += w < wave ? wave_sums[w] : 0u; round += wave_sums[w]; }
+        const uint32_t slot = before + uint32_t(__popcll(reaching & below));
+        if (reaches && slot < uint32_t(THIN_CAP)) out[slot] = make_uint2(bits, uint32_t(block));
+        written += round;
+    }
+    if (t == 0) *count_out = written <= uint32_t(THIN_CAP) ? written : THIN_NONE;
+}
+
 // One workgroup per row; block i * 1024 + t is thread t's value i.  The row is read once and stays on the chip: its first
 // LDS_RUNS runs of 1024 values in LDS (as many as the row has: the launch sizes the array), the runs beyond, for the longest
 // rows, in REGS registers a thread.
@@ -328,7 +403,8 @@ constexpr int LDS_RUNS = 31, LIST_RUNS = 2, LIST = LIST_RUNS * SELECT_THREADS;
 template<int REGS>
 __global__ void __launch_bounds__(SELECT_THREADS) select_kernel(const float* __restrict__ scores, size_t pool, size_t base, const uint32_t* dynamic,
                                                                 size_t selected, unsigned held_runs, float* __restrict__ indices,
-                                                                float* __restrict__ counts) {
+                                                                float* __restrict__ counts, const uint2* __restrict__ thinned,
+                                                                const uint32_t* __restrict__ thinned_counts) {
     extern __shared__ uint32_t held[];                       // [run][1024]
     __shared__ SelectShared sh;
     __shared__ uint2 list[LIST];                             // (score bits, block) of the values that reach the guess
@@ -348,6 +424,27 @@ __global__ void __launch_bounds__(SELECT_THREADS) select_kernel(const float* __r
     const float* row = scores + token * pool;
     const unsigned runs = unsigned((complete + SELECT_THREADS - 1) / SELECT_THREADS), lds_runs = min(runs, held_runs);
     uint32_t values[REGS ? REGS : 1];
+    uint32_t guess = 0;
+    bool listed = false;
+    uint32_t list_count = 0;
+    // The row thinned by thin_kernel: its stretches' lists, one after the other, are the row's list -- when every stretch's
+    // fitted and they hold at least 512 values and no more than the list does; the row itself is then not read at all.
+    if (thinned && runs >= 8) {
+        const uint32_t mine = t < unsigned(THIN_SEGMENTS) ? thinned_counts[token * THIN_SEGMENTS + t] : 0u;
+        const bool none = __syncthreads_or(mine == THIN_NONE);
+        const uint32_t before = group_scan(none ? 0u : mine, sh.wave_sums, list_count);
+        listed = !none && list_count >= KEEP && list_count <= LIST;
+        if (listed) {
+            if (t < unsigned(THIN_SEGMENTS)) { sh.bins[2 * t] = before; sh.bins[2 * t + 1] = mine; }
+            __syncthreads();
+            for (unsigned slot = t; slot < unsigned(THIN_SEGMENTS * THIN_CAP); slot += SELECT_THREADS) {
+                const unsigned segment = slot / THIN_CAP, entry = slot % THIN_CAP;
+                if (entry < sh.bins[2 * segment + 1]) list[sh.bins[2 * segment] + entry] = thinned[(token * THIN_SEGMENTS + segment) * THIN_CAP + entry];
+            }
+            __syncthreads();
+        }
+    }
+    if (!listed) {
     #pragma unroll 8
     for (unsigned i = 0; i < lds_runs; ++i) {
         const size_t block = size_t(i) * SELECT_THREADS + t;
@@ -359,6 +456,7 @@ __global__ void __launch_bounds__(SELECT_THREADS) select_kernel(const float* __r
             const size_t block = size_t(LDS_RUNS + j) * SELECT_THREADS + t;
             values[j] = block < complete ? __float_as_uint(row[block]) : 0u;
         }
+    }
     }
     // body(run, bits, valid) for every run of the row, in run order (every thread reads back only what it wrote)
     const auto each_run = [&](auto body) {
@@ -377,10 +475,7 @@ __global__ void __launch_bounds__(SELECT_THREADS) select_kernel(const float* __r
                 if (unsigned(LDS_RUNS + j) < runs) body(unsigned(LDS_RUNS + j), values[j], size_t(LDS_RUNS + j) * SELECT_THREADS + t < complete);
         }
     };
-    uint32_t guess = 0;
-    bool listed = false;
-    uint32_t list_count = 0;
-    if (runs >= 8) {
+    if (!listed && runs >= 8) {
         constexpr unsigned SAMPLES = 4;                      // values a thread gives to the sample
         uint32_t sample[SAMPLES];
         bool sampled[SAMPLES];
@@ -457,7 +552,7 @@ __global__ void __launch_bounds__(SELECT_THREADS) select_kernel(const float* __r
 
 template<int REGS>
 void launch_select(Device& d, const float* scores, size_t pool, size_t base, const uint32_t* dynamic, size_t selected, size_t most, unsigned rows,
-                   float* indices, float* counts) {
+                   float* indices, float* counts, const uint2* thinned, const uint32_t* thinned_counts) {
     const unsigned held_runs = unsigned(std::min<size_t>((most + SELECT_THREADS - 1) / SELECT_THREADS, LDS_RUNS));
     const size_t shared = size_t(std::max(held_runs, 1u)) * SELECT_THREADS * 4;
     static bool raised[2] = {false, false};
@@ -465,7 +560,7 @@ void launch_select(Device& d, const float* scores, size_t pool, size_t base, con
         SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&select_kernel<REGS>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_RUNS * SELECT_THREADS * 4));
         raised[REGS ? 1 : 0] = true;
     }
-    select_kernel<REGS><<<rows, SELECT_THREADS, shared, d.stream>>>(scores, pool, base, dynamic, selected, held_runs, indices, counts);
+    select_kernel<REGS><<<rows, SELECT_THREADS, shared, d.stream>>>(scores, pool, base, dynamic, selected, held_runs, indices, counts, thinned, thinned_counts);
 }
 
 // ---- a decode or verification pass's inputs in one launch --------------------------------------------------------------
@@ -598,8 +693,26 @@ int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, con
         }
     }
     const unsigned rows = checked_blocks(steps, 1);
-    if (most <= size_t(LDS_RUNS) * SELECT_THREADS) launch_select<0>(value, scores, pool, base, dynamic_base, selected, most, rows, indices, counts);
-    else launch_select<33>(value, scores, pool, base, dynamic_base, selected, most, rows, indices, counts);
+    // a few long rows: the thinning goes to many workgroups first (their lists live in a small buffer the handle keeps; were
+    // the first such call recorded into a graph, it does without)
+    const uint2* thinned = nullptr;
+    const uint32_t* thinned_counts = nullptr;
+    if (rows <= unsigned(THIN_ROWS) && most >= size_t(8) * SELECT_THREADS) {
+        constexpr size_t lists = size_t(THIN_ROWS) * THIN_SEGMENTS * THIN_CAP * sizeof(uint2);
+        if (!value.select_thin) {
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            SD_CHECK(hipStreamIsCapturing(value.stream, &capturing));
+            if (capturing == hipStreamCaptureStatusNone) value.select_thin = allocate(value, lists + size_t(THIN_ROWS) * THIN_SEGMENTS * 4, true);
+        }
+        if (value.select_thin) {
+            uint2* listed = static_cast<uint2*>(value.select_thin);
+            uint32_t* listed_counts = reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(value.select_thin) + lists);
+            thin_kernel<<<dim3(THIN_SEGMENTS, rows), THIN_THREADS, 0, value.stream>>>(scores, pool, base, dynamic_base, listed, listed_counts);
+            thinned = listed; thinned_counts = listed_counts;
+        }
+    }
+    if (most <= size_t(LDS_RUNS) * SELECT_THREADS) launch_select<0>(value, scores, pool, base, dynamic_base, selected, most, rows, indices, counts, thinned, thinned_counts);
+    else launch_select<33>(value, scores, pool, base, dynamic_base, selected, most, rows, indices, counts, thinned, thinned_counts);
     SD_OP_END
 }
 

@@ -57,6 +57,8 @@ struct Device {
     double2* turns = nullptr;
     size_t turns_rows = 0, turns_pairs = 0, turns_armed = 0, turns_ready_rows = 0, turns_ready_pairs = 0;
     bool turns_ready = false;
+    // The lists of a short span's thinned index rows (block_index.hip), allocated at the first such call and kept.
+    void* select_thin = nullptr;
     // Page-locked host copies of sequence state (conversation checkpoints): pointer -> bytes.
     std::map<void*, size_t> checkpoints;
     // Recorded graphs of ops (sd_graph_begin / _end / _run), by the caller's key.

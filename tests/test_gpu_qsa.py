@@ -104,6 +104,9 @@ def _check(oracle, queries, blocks, base, selected, got):
     ("g", 262100, 3, 262144, 512),      # the longest context: rows re-read per pass
     ("g", 70000, 2, 131072, 512),       # 16 values a thread
     ("g", 100, 20, 1024, 512),          # a short context: every row keeps every causal position
+    ("d", 60000, 4, 65536, 512),        # a few long rows are thinned by many workgroups first: exact ties where the cut falls,
+    ("t", 100000, 8, 131072, 512),      # ... clustered scores,
+    ("z", 40000, 2, 65536, 512),        # ... and zero queries, whose lists do not fit: the row's workgroup does it all
 ])
 def test_block_scores_and_selection(gpu, oracle, mode, base, steps, context, stride):
     pool = context // 4 + 1
