@@ -89,44 +89,43 @@ __device__ __forceinline__ float positive_sum(const float (&dot)[HEADS]) {
     return total;
 }
 
-// ---- scores of a short span: a lane per block, T rows per lane ------------------------------------------------------------
-// The queries sit in LDS as [row][column][head], so the four heads of a column come by one wave-uniform 16-byte read.
+// ---- scores of a short span: a lane per block, a wave per head, T rows per lane ----------------------------------------------
+// The chains of a block's four heads run in four waves of the workgroup (the same 64 blocks, the keys read by each: the second
+// to fourth find them in the cache), so a compute unit holds four times the waves to hide the loads behind; the four sums meet
+// in LDS and are added in head order.  The queries sit in LDS as [row][head][column]: a wave-uniform read a column.
 template<int T>
-__global__ void __launch_bounds__(64) scores_rows_kernel(const float* __restrict__ queries, size_t query_stride, const float* __restrict__ blocks,
-                                                         size_t pool, size_t base, const uint32_t* dynamic, unsigned steps, float* __restrict__ scores) {
-    __shared__ __align__(16) float q[T][COLUMNS][HEADS];
+__global__ void __launch_bounds__(64 * HEADS) scores_rows_kernel(const float* __restrict__ queries, size_t query_stride, const float* __restrict__ blocks,
+                                                                size_t pool, size_t base, const uint32_t* dynamic, unsigned steps, float* __restrict__ scores) {
+    __shared__ float q[T][HEADS][COLUMNS];
+    __shared__ float sums[HEADS][T][64];
     if (dynamic) base = *dynamic;
     const size_t most = min((base + steps) / 4, pool), first = size_t(blockIdx.x) * 64;   // the last row's complete blocks
-    const unsigned lane = threadIdx.x;
+    const unsigned lane = threadIdx.x % 64, head = threadIdx.x / 64;
     if (most <= KEEP || first >= most) return;
-    for (unsigned i = lane; i < T * HEADS * COLUMNS; i += 64) {
-        const unsigned row = i / (HEADS * COLUMNS), h = i / COLUMNS % HEADS, c = i % COLUMNS;
-        q[row][c][h] = row < steps ? queries[row * query_stride + h * COLUMNS + c] : 0.0f;
+    for (unsigned i = threadIdx.x; i < T * HEADS * COLUMNS; i += 64 * HEADS) {
+        const unsigned row = i / (HEADS * COLUMNS);
+        q[row][i / COLUMNS % HEADS][i % COLUMNS] = row < steps ? queries[row * query_stride + i % (HEADS * COLUMNS)] : 0.0f;
     }
     __syncthreads();
     const float* column = blocks + min(first + lane, pool - 1);
-    float dot[T][HEADS] = {};
+    float dot[T] = {};
     #pragma unroll 1
     for (unsigned c0 = 0; c0 < COLUMNS; c0 += 16) {
         float key[16];
         #pragma unroll
         for (unsigned j = 0; j < 16; ++j) key[j] = column[size_t(c0 + j) * pool];
         #pragma unroll
-        for (unsigned j = 0; j < 16; ++j) {
+        for (unsigned j = 0; j < 16; ++j)
             #pragma unroll
-            for (int row = 0; row < T; ++row) {
-                const float4 heads = *reinterpret_cast<const float4*>(q[row][c0 + j]);
-                dot[row][0] = fmaf(key[j], heads.x, dot[row][0]);
-                dot[row][1] = fmaf(key[j], heads.y, dot[row][1]);
-                dot[row][2] = fmaf(key[j], heads.z, dot[row][2]);
-                dot[row][3] = fmaf(key[j], heads.w, dot[row][3]);
-            }
-        }
+            for (int row = 0; row < T; ++row) dot[row] = fmaf(key[j], q[row][head][c0 + j], dot[row]);
     }
     #pragma unroll
-    for (int row = 0; row < T; ++row) {
+    for (int row = 0; row < T; ++row) sums[head][row][lane] = dot[row];
+    __syncthreads();
+    for (unsigned row = head; row < unsigned(T); row += HEADS) {
         const size_t complete = (base + row + 1) / 4;
-        if (unsigned(row) < steps && complete > KEEP && first + lane < min(complete, pool)) scores[row * pool + first + lane] = positive_sum(dot[row]);
+        const float four[HEADS] = {sums[0][row][lane], sums[1][row][lane], sums[2][row][lane], sums[3][row][lane]};
+        if (row < steps && complete > KEEP && first + lane < min(complete, pool)) scores[row * pool + first + lane] = positive_sum(four);
     }
 }
 
@@ -629,7 +628,7 @@ __global__ void __launch_bounds__(256) stage_prepare_kernel(StageArgs a) {
 template<int T>
 void launch_rows(Device& d, const float* queries, size_t stride, const float* blocks, size_t pool, size_t base, const uint32_t* dynamic, size_t steps,
                  size_t most, float* scores) {
-    scores_rows_kernel<T><<<checked_blocks(most, 64), 64, 0, d.stream>>>(queries, stride, blocks, pool, base, dynamic, unsigned(steps), scores);
+    scores_rows_kernel<T><<<checked_blocks(most, 64), 64 * HEADS, 0, d.stream>>>(queries, stride, blocks, pool, base, dynamic, unsigned(steps), scores);
 }
 
 }  // namespace
