@@ -5,10 +5,11 @@
 // block scale, FP32 sums: gpu/qsa_prompt_attention.hpp:15-33, :144-150).
 //
 // Shape of the work on gfx950 (wave64, v_mfma_f32_16x16x32_f16):
-//   * a workgroup (4 waves) owns one (sequence, K/V head, chunk of the context); the chunk size is chosen on the device
-//     from the batch, and the chunks that hold tokens are numbered densely so that the grid's first workgroups all work;
-//   * the waves take alternate 32-token steps, each with its own online softmax, and merge through LDS at the end; a
-//     second kernel merges the chunks of a sequence;
+//   * the batch's cached tokens, all K/V heads, are cut on the device into equal shares, one per workgroup (4 waves) and as
+//     many workgroups as are resident at once: all start together and end together, whatever the mix of lengths.  A share
+//     that crosses from one (sequence, K/V head) into the next is worked in segments, one partial result each;
+//   * the waves take alternate 32-token steps, each with its own online softmax, and merge through LDS at the end of a
+//     segment; a second kernel merges the segments of a sequence;
 //   * a step's K and V slabs (32 contiguous rows of a page plane) are copied by coalesced, non-temporal 16-byte
 //     global->LDS loads into the wave's own LDS stage, operands are read from there in MFMA layout, and the next step's
 //     copy is in flight while this step is computed;
@@ -28,51 +29,69 @@ using namespace sd::paged;
 
 namespace {
 
-// Tokens per chunk, the same for every workgroup of a launch and for the merge after it: the batch's cached tokens (all K/V
-// heads) cut into `rounds` workgroups per resident slot, in whole 128-token rounds of the four waves.  Workgroups are
-// dispatched in order as earlier ones finish: sequences of one length fill the device evenly in a single round, which has
-// the least start-up work; unequal ones even out over two rounds of smaller chunks.
-__device__ __forceinline__ unsigned chunk_tokens(const PagedArgs& args, int lane) {
-    if (args.chunk_min == args.chunk_max) return args.chunk_min;
-    float tokens = 0.0f;
-    int longest = 0;
-    for (unsigned s = lane; s < args.seqs; s += 64) {
-        const int total = min(args.positions[s] + int(args.span), args.max_context);
-        tokens += float(total);
-        longest = max(longest, total);
-    }
+// The batch's work is counted in units of 128 tokens (one step of each of the four waves): a sequence of n tokens has
+// ceil(n / 128) units per K/V head, laid out sequence by sequence and, within one, K/V head by K/V head.  Workgroup w of G
+// takes the units floor(w U / G) up to floor((w + 1) U / G): G is as many workgroups as are resident at once (fewer when
+// that would leave a workgroup less than share_min units).  Every wave finds the same numbers from the positions alone.
+constexpr unsigned UNIT = STEP * WAVES;
+struct Share { unsigned units, groups; };
+__device__ __forceinline__ Share batch_share(const PagedArgs& args, int lane) {
+    unsigned units = 0;
+    for (unsigned s = lane; s < args.seqs; s += 64) units += unsigned(min(args.positions[s] + int(args.span), args.max_context) + int(UNIT) - 1) / UNIT;
     #pragma unroll
-    for (int d = 32; d; d >>= 1) { tokens += __shfl_xor(tokens, d); longest = max(longest, __shfl_xor(longest, d)); }
-    const float rounds = tokens > 0.9f * float(args.seqs) * float(longest) ? args.rounds_even : args.rounds;
-    const float cut = tokens * float(args.kv_heads) / (args.slots * rounds);
-    const unsigned chunk = (unsigned(fminf(cut, 1.0e6f)) + 127u) / 128u * 128u;
-    return __builtin_amdgcn_readfirstlane(min(max(chunk, args.chunk_min), args.chunk_max));
+    for (int d = 32; d; d >>= 1) units += __shfl_xor(units, d);
+    units = __builtin_amdgcn_readfirstlane(units * args.kv_heads);
+    return Share{units, min(args.groups_max, max(1u, units / args.share_min))};
 }
+__device__ __forceinline__ unsigned share_begin(const Share& share, unsigned w) { return unsigned(uint64_t(w) * share.units / share.groups); }
+// the workgroup that takes unit u: the w with floor(w U / G) <= u < floor((w + 1) U / G)
+__device__ __forceinline__ unsigned share_owner(const Share& share, unsigned u) { return unsigned((uint64_t(u + 1) * share.groups - 1) / share.units); }
 
-// The work of workgroup `id`: the chunks that hold tokens are numbered sequence by sequence, then K/V head by K/V head, so
-// the workgroups with work are the first of the grid and the rest leave at once.  Every wave finds the same answer from
-// the positions alone (a running count over 64 sequences at a time).
-struct WorkItem { int seq, chunk, kvh, per_chunk, position, total; };
-__device__ __forceinline__ bool find_work(const PagedArgs& args, unsigned id, int lane, WorkItem& item) {
-    item.per_chunk = int(chunk_tokens(args, lane));
+// Where unit u lies: its sequence and K/V head, how many units into them, and how many they have (a running count over 64
+// sequences at a time; `before` = the units of the sequences before).
+// (The lane number is taken afresh, by an instruction the compiler may not move: what is derived from it here would
+// otherwise be kept in registers all through the caller's loop over the tokens.)
+__device__ __forceinline__ int fresh_lane() {
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    return lane;
+}
+// (Likewise the kernel's arguments, read afresh for each segment through a pointer the compiler cannot see through: fields
+// that only a segment's start or end needs do not then occupy scalar registers through the loop over the tokens.)
+typedef __attribute__((address_space(4))) const PagedArgs* args_ptr;
+__device__ __forceinline__ PagedArgs fresh_args() {
+    args_ptr at = (args_ptr)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(at));
+    PagedArgs args;
+    args.pages = at->pages; args.page_tokens = at->page_tokens; args.kv_heads = at->kv_heads; args.heads = at->heads; args.group = at->group;
+    args.span = at->span; args.page_table = at->page_table; args.table_stride = at->table_stride; args.positions = at->positions; args.q = at->q;
+    args.q_f16 = at->q_f16; args.scale_log2 = at->scale_log2; args.partial = at->partial; args.rows = at->rows; args.seqs = at->seqs;
+    args.groups_max = at->groups_max; args.share_min = at->share_min; args.max_context = at->max_context;
+    return args;
+}
+struct Segment { int seq, kvh, position, total; unsigned unit, units, before; };
+__device__ __forceinline__ bool locate(const PagedArgs& args, unsigned u, Segment& seg) {
+    const int lane = fresh_lane();
     unsigned before = 0;
     for (unsigned first = 0; first < args.seqs; first += 64) {
         const unsigned s = first + lane;
         const int position = s < args.seqs ? args.positions[s] : 0;
         const int total = s < args.seqs ? min(position + int(args.span), args.max_context) : 0;
-        const unsigned used = unsigned(total + item.per_chunk - 1) / unsigned(item.per_chunk);
-        unsigned upto = used * args.kv_heads;      // workgroups of this and the earlier sequences of the 64
+        const unsigned units = unsigned(total + int(UNIT) - 1) / UNIT;
+        unsigned upto = units * args.kv_heads;      // units of this and the earlier sequences of the 64
         #pragma unroll
         for (int d = 1; d < 64; d <<= 1) { const unsigned other = __shfl_up(upto, d); if (lane >= d) upto += other; }
         const unsigned all = __shfl(upto, 63);
-        if (id < before + all) {
-            const int owner = __popcll(__ballot(before + upto <= id));
-            const unsigned chunks = __shfl(used, owner), within = id - before - __shfl(upto - used * args.kv_heads, owner);
-            item.seq = int(first) + owner;
-            item.total = __shfl(total, owner);
-            item.position = __shfl(position, owner);
-            item.kvh = int(within / chunks);
-            item.chunk = int(within % chunks);
+        if (u < before + all) {
+            const int owner = __popcll(__ballot(before + upto <= u));
+            seg.units = __shfl(units, owner);
+            seg.before = before + __shfl(upto - units * args.kv_heads, owner);
+            const unsigned within = u - seg.before;
+            seg.seq = int(first) + owner;
+            seg.total = __shfl(total, owner);
+            seg.position = __shfl(position, owner);
+            seg.kvh = int(within / seg.units);
+            seg.unit = within % seg.units;
             return true;
         }
         before += all;
@@ -89,15 +108,25 @@ template<int N> __device__ __forceinline__ void wait_loads() { __builtin_amdgcn_
 // own LDS stage; operands are then read from LDS in MFMA layout while the next step's copy is in flight.  OCC = the waves per
 // SIMD the variant is compiled for (its register budget).
 template<int DIM, int QT, bool Q8, int OCC>
-__global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) paged_attention_kernel(PagedArgs args) {
+__global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) paged_attention_kernel(PagedArgs given) {
     constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, BLOCKS = DIM / 32, W = DIM / 16, TILES = DIM / 16;
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, g = lane >> 4;
-    WorkItem item;
-    if (!find_work(args, blockIdx.x, lane, item)) return;
-    const int seq = __builtin_amdgcn_readfirstlane(item.seq), chunk = __builtin_amdgcn_readfirstlane(item.chunk);
-    const int kvh = __builtin_amdgcn_readfirstlane(item.kvh), total = __builtin_amdgcn_readfirstlane(item.total);
-    const int position = __builtin_amdgcn_readfirstlane(item.position);
-    const int chunk_begin = chunk * item.per_chunk, chunk_end = min(total, chunk_begin + item.per_chunk);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const Share share = batch_share(given, threadIdx.x & 63);
+    if (blockIdx.x >= share.groups) return;
+    extern __shared__ float lds[];
+    const unsigned share_end = share_begin(share, blockIdx.x + 1);
+    for (unsigned unit = share_begin(share, blockIdx.x); unit < share_end;) {
+    // (a fresh lane number per segment: what a segment's start and end derive from it is then worked out there, not kept in
+    // registers through every other segment's loop over the tokens)
+    const int lane = fresh_lane(), li = lane & 15, g = lane >> 4;
+    const PagedArgs args = fresh_args();                    // (the kernel's only argument: it lies at the segment's start)
+    Segment found;
+    if (!locate(args, unit, found)) return;            // (cannot happen: the units were counted from the same positions)
+    const int seq = __builtin_amdgcn_readfirstlane(found.seq), kvh = __builtin_amdgcn_readfirstlane(found.kvh);
+    const int total = __builtin_amdgcn_readfirstlane(found.total), position = __builtin_amdgcn_readfirstlane(found.position);
+    const unsigned first_unit = __builtin_amdgcn_readfirstlane(found.unit);
+    const unsigned take = min(share_end - unit, unsigned(__builtin_amdgcn_readfirstlane(found.units)) - first_unit);
+    const int chunk_begin = int(first_unit * UNIT), chunk_end = min(total, int((first_unit + take) * UNIT));
     const table_ptr table = (table_ptr)(args.page_table + size_t(seq) * args.table_stride);
     const size_t plane_bytes = size_t(args.page_tokens) * ROW;
 
@@ -136,7 +165,6 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    extern __shared__ float lds[];
     constexpr int SLAB = STEP * ROW;                       // one step's rows of one plane: contiguous in the page
     // Stages per wave: with few waves per SIMD one step in flight per wave does not cover the memory latency, so a wave then
     // keeps two (where the workgroups resident at once still fit the 160 KiB of LDS).
@@ -271,19 +299,22 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
     // Merge the waves through LDS: per wave and query row the maximum, the sum and the unnormalised output.
     __syncthreads();    // the merge area overlays the stages
     constexpr int STRIDE = DIM + 2, QROWS = QT * 16;
+    const int lane_after = fresh_lane(), li_after = lane_after & 15, g_after = lane_after >> 4;   // (again: nothing of this is worked out before the loop)
+    const unsigned thread = unsigned(wave * 64 + lane_after);
     #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
         const float sum = row_sum(l[qt]);
-        float* row = lds + (size_t(wave) * QROWS + qt * 16 + li) * STRIDE;
-        if (g == 0) { row[DIM] = m[qt] * args.scale_log2; row[DIM + 1] = sum; }      // maxima leave in exponent units
+        float* row = lds + (size_t(wave) * QROWS + qt * 16 + li_after) * STRIDE;
+        if (g_after == 0) { row[DIM] = m[qt] * args.scale_log2; row[DIM + 1] = sum; }      // maxima leave in exponent units
         #pragma unroll
         for (int jj = 0; jj < TILES; ++jj)
             #pragma unroll
-            for (int r = 0; r < 4; ++r) row[W * (4 * g + r) + jj] = acc[qt][jj][r];
+            for (int r = 0; r < 4; ++r) row[W * (4 * g_after + r) + jj] = acc[qt][jj][r];
     }
     __syncthreads();
-    float* out = args.partial + ((size_t(seq) * args.kv_heads + kvh) * args.chunks + chunk) * args.rows * STRIDE;
-    for (unsigned i = threadIdx.x; i < args.rows * STRIDE; i += WAVES * 64) {
+    // a partial result per (workgroup, sequence and K/V head) met: both only grow along the units, so their sum numbers them
+    float* out = args.partial + (size_t(blockIdx.x) + size_t(seq) * args.kv_heads + kvh) * args.rows * STRIDE;
+    for (unsigned i = thread; i < args.rows * STRIDE; i += WAVES * 64) {
         const unsigned row = i / STRIDE, col = i % STRIDE;
         float top = NEG_BIG;
         #pragma unroll
@@ -300,9 +331,12 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         }
         out[i] = value;
     }
+    unit += take;
+    if (unit < share_end) __syncthreads();                  // the next segment's stages overlay the merge area
+    }
 }
 
-// One block per (sequence, span row, head): the chunks' partial results merged and normalised (the algebra of the
+// One block per (sequence, span row, head): the segments' partial results merged and normalised (the algebra of the
 // reference's qsa_decode_merge, gpu/sparse_attention_compute.hpp:139-170).  The block's 256 threads are GROUPS groups of
 // DIM/2 threads; a group takes every GROUPS-th chunk and a thread two columns, so all loads of a pass are in flight at
 // once; chunks are taken 256 at a time with a running maximum.
@@ -312,10 +346,17 @@ __global__ void __launch_bounds__(256) paged_merge_kernel(PagedArgs args, void* 
     const unsigned item = blockIdx.x, head = item % args.heads, span_row = item / args.heads % args.span, seq = item / args.heads / args.span;
     const unsigned kvh = head / args.group, row = span_row * args.group + head % args.group;
     const unsigned tid = threadIdx.x, group = tid / LANES, col = 2 * (tid % LANES), wave = tid >> 6;
-    const int total = min(args.positions[seq] + int(args.span), args.max_context);
-    const int per_chunk = int(chunk_tokens(args, int(tid & 63)));
-    const unsigned used = unsigned((total + per_chunk - 1) / per_chunk);
-    const float* base = args.partial + ((size_t(seq) * args.kv_heads + kvh) * args.chunks) * args.rows * STRIDE + size_t(row) * STRIDE;
+    // the workgroups whose shares met this sequence and K/V head
+    const int lane = int(tid & 63);
+    const Share share = batch_share(args, lane);
+    unsigned before = 0;
+    for (unsigned s = lane; s < seq; s += 64) before += unsigned(min(args.positions[s] + int(args.span), args.max_context) + int(UNIT) - 1) / UNIT;
+    #pragma unroll
+    for (int d = 32; d; d >>= 1) before += __shfl_xor(before, d);
+    const unsigned units = unsigned(min(args.positions[seq] + int(args.span), args.max_context) + int(UNIT) - 1) / UNIT;
+    const unsigned begin = (before * args.kv_heads + kvh * units), owner = share_owner(share, begin);
+    const unsigned used = share_owner(share, begin + units - 1) - owner + 1;
+    const float* base = args.partial + (size_t(owner) + size_t(seq) * args.kv_heads + kvh) * args.rows * STRIDE + size_t(row) * STRIDE;
     const size_t step = size_t(args.rows) * STRIDE;
     __shared__ float weights[256];
     __shared__ float reduce[2][4];
@@ -369,42 +410,22 @@ __global__ void __launch_bounds__(256) paged_merge_kernel(PagedArgs args, void* 
     }
 }
 
-// Tuning switches read once from the environment, as the reference reads its hot-path switches (STRAYDOG_QSA_MMA,
-// gpu/sparse_attention_compute.hpp:594): STRAYDOG_DECODE_CHUNK = tokens per workgroup (0: chosen on the device from the
-// batch), STRAYDOG_DECODE_ROUNDS = workgroups per resident slot the batch is cut into (0: chosen from the batch too).
-struct Tuning { unsigned chunk = 0; float rounds = 0.0f; };
-const Tuning& tuning() {
-    static const Tuning value = [] {
-        Tuning t;
-        if (const char* text = std::getenv("STRAYDOG_DECODE_CHUNK")) t.chunk = unsigned(std::strtoul(text, nullptr, 10));
-        if (const char* text = std::getenv("STRAYDOG_DECODE_ROUNDS")) t.rounds = std::max(0.0f, std::strtof(text, nullptr));
-        return t;
+// Tuning switch read once from the environment, as the reference reads its hot-path switches (STRAYDOG_QSA_MMA,
+// gpu/sparse_attention_compute.hpp:594): STRAYDOG_DECODE_GROUPS = the most workgroups a batch is shared among (0: as many as
+// are resident at once).
+unsigned tuned_groups() {
+    static const unsigned value = [] {
+        const char* text = std::getenv("STRAYDOG_DECODE_GROUPS");
+        return text ? unsigned(std::strtoul(text, nullptr, 10)) : 0u;
     }();
     return value;
 }
 
-constexpr unsigned smallest_chunk = 256, largest_chunk = 16384;
-
-// The host knows only max_context: it bounds the device's choice above by the chunk of a batch with every sequence full,
-// and sizes the grid for an eighth of that (the workgroups past the batch's last chunk leave at once).
-void plan_chunks(PagedArgs& args, uint64_t seqs, uint64_t kv_heads, uint64_t max_context, unsigned slots) {
-    args.slots = float(slots);
-    // One query tile (decode, 4 workgroups per compute unit): one round for even batches, two for uneven ones; the heavier
-    // variants (1-2 workgroups per compute unit) even out better over three, and their idle trailing workgroups cost more, so
-    // their grid allows less room below the largest chunk.
-    const bool decode = args.rows <= 16;
-    args.rounds = tuning().rounds > 0.0f ? tuning().rounds : decode ? 2.0f : 3.0f;
-    args.rounds_even = tuning().rounds > 0.0f ? tuning().rounds : decode ? 1.0f : 3.0f;
-    if (tuning().chunk) {
-        const unsigned chunk = std::min(std::max((tuning().chunk + 127u) / 128u * 128u, smallest_chunk), 1u << 20);
-        args.chunk_min = args.chunk_max = chunk;
-    } else {
-        const double full = double(max_context) * double(seqs) * double(kv_heads) / double(args.slots * args.rounds_even);
-        const unsigned chunk = unsigned(std::min(full, 1.0e6) + 127.0) / 128u * 128u;
-        args.chunk_max = std::min(std::max(chunk, smallest_chunk), largest_chunk);
-        args.chunk_min = std::max(smallest_chunk, args.chunk_max / (decode ? 4 : 2) / 128u * 128u);
-    }
-    args.chunks = unsigned((max_context + args.chunk_min - 1) / args.chunk_min);
+// A share is at least 256 tokens; the host knows only max_context, which bounds the units a batch can have and so the
+// workgroups worth launching.
+constexpr unsigned smallest_share = 2;
+uint64_t most_groups(uint64_t seqs, uint64_t kv_heads, uint64_t max_context) {
+    return seqs * kv_heads * ((max_context + smallest_share * UNIT - 1) / (smallest_share * UNIT));
 }
 
 template<int DIM, int QT, bool Q8, int OCC>
@@ -449,9 +470,9 @@ unsigned resident_slots(const Device& d, unsigned dim, bool q8, unsigned query_t
 extern "C" {
 
 uint64_t sdx_paged_attention_scratch(uint64_t seqs, uint64_t span, uint64_t heads, uint64_t dim, uint64_t max_context) {
-    // the smallest chunk a launch may use
-    const uint64_t chunks = (max_context + smallest_chunk - 1) / smallest_chunk;
-    return seqs * span * heads * chunks * (dim + 2) * 4;
+    // a partial result per workgroup and one more per (sequence, K/V head); at most a workgroup per 256 tokens of a sequence
+    const uint64_t shares = (max_context + smallest_share * UNIT - 1) / (smallest_share * UNIT);
+    return seqs * span * heads * (shares + 1) * (dim + 2) * 4;
 }
 
 int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride,
@@ -481,14 +502,16 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
     args.q = q; args.q_f16 = q_f16; args.scale_log2 = scale * 1.44269504088896341f;
     args.rows = unsigned(rows); args.seqs = unsigned(seqs);
     args.max_context = int(max_context);
-    plan_chunks(args, seqs, pool->kv_heads, max_context, resident_slots(value, pool->dim, pool->row_bytes != 2 * pool->dim, query_tiles));
-    if (args.chunks > 65535) throw std::runtime_error("invalid Straydog paged attention shape");
-    const size_t need = checked_floats({seqs, pool->kv_heads, args.chunks, rows, uint64_t(pool->dim) + 2});
+    const uint64_t items = checked_product({seqs, pool->kv_heads});
+    if (checked_product({items, (max_context + UNIT - 1) / UNIT}) > 0x7fffffffu) throw std::runtime_error("invalid Straydog paged attention shape");
+    const unsigned slots = resident_slots(value, pool->dim, pool->row_bytes != 2 * pool->dim, query_tiles);
+    args.groups_max = unsigned(std::min<uint64_t>(tuned_groups() ? tuned_groups() : slots, most_groups(seqs, pool->kv_heads, max_context)));
+    args.share_min = smallest_share;
+    const size_t need = checked_floats({uint64_t(args.groups_max) + items, rows, uint64_t(pool->dim) + 2});
     if (!scratch || scratch_bytes < need) throw std::runtime_error("Straydog paged attention scratch too small");
     op_span(value, scratch, need, "attention scratch");
     args.partial = static_cast<float*>(scratch);
-    if (checked_product({seqs, args.chunks, pool->kv_heads}) > 0x7fffffffu) throw std::runtime_error("invalid Straydog paged attention shape");
-    const dim3 grid(unsigned(seqs * args.chunks * pool->kv_heads));
+    const dim3 grid(args.groups_max);
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     {
         KernelTimer timer(value);
@@ -496,13 +519,13 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
         else { if (q8) launch_tiles<256, true>(value, args, query_tiles, grid); else launch_tiles<256, false>(value, args, query_tiles, grid); }
     }
     SD_CHECK(hipGetLastError());
-    const unsigned items = unsigned(checked_product({seqs, span, heads}));
+    const unsigned outputs = unsigned(checked_product({seqs, span, heads}));
     if (pool->dim == 128) {
-        if (out_f16) paged_merge_kernel<128, true><<<items, 256, 0, value.stream>>>(args, out);
-        else paged_merge_kernel<128, false><<<items, 256, 0, value.stream>>>(args, out);
+        if (out_f16) paged_merge_kernel<128, true><<<outputs, 256, 0, value.stream>>>(args, out);
+        else paged_merge_kernel<128, false><<<outputs, 256, 0, value.stream>>>(args, out);
     } else {
-        if (out_f16) paged_merge_kernel<256, true><<<items, 256, 0, value.stream>>>(args, out);
-        else paged_merge_kernel<256, false><<<items, 256, 0, value.stream>>>(args, out);
+        if (out_f16) paged_merge_kernel<256, true><<<outputs, 256, 0, value.stream>>>(args, out);
+        else paged_merge_kernel<256, false><<<outputs, 256, 0, value.stream>>>(args, out);
     }
     SD_OP_END
 }

@@ -32,10 +32,9 @@ struct PagedArgs {
     const void* q;
     int q_f16;
     float scale_log2;      // softmax scale * log2(e): scores live in the base-2 domain
-    float* partial;        // [seq][kv head][chunk][row][dim + 2]
-    unsigned chunks, rows;  // chunks = the most chunks a sequence can have; rows = span * group (query rows per K/V head)
-    unsigned chunk_min, chunk_max, seqs;   // tokens per chunk are chosen on the device between these (see chunk_tokens)
-    float slots, rounds, rounds_even;   // workgroups resident at once; workgroups per slot to cut an uneven / an even batch into
+    float* partial;        // [workgroup + sequence * kv_heads + kv head][row][dim + 2]: one per segment of a workgroup's share
+    unsigned rows, seqs;   // rows = span * group (query rows per K/V head)
+    unsigned groups_max, share_min;   // the most workgroups that share the batch's tokens; the fewest 128-token units a share may have
     int max_context;       // positions[s] + span is clipped to this (the launch and the page table are sized for it)
 };
 
