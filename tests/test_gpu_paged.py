@@ -237,6 +237,27 @@ def test_many_short_sequences(gpu, oracle):
     gpu.release(buffer); gpu.release(tb)
 
 
+@pytest.mark.parametrize("span", [1, 3])
+def test_shares_that_cross_sequences_and_heads(gpu, oracle, span):
+    # the batch's tokens are cut into equal shares: one long sequence is spread over hundreds of workgroups, the short ones
+    # around it are met several to a share, and a share ends anywhere (inside a sequence, at its end, between K/V heads);
+    # max_context far above the longest sequence, as a server that sizes for the worst case would pass it
+    rng = np.random.default_rng(808 + span)
+    dim, row_bytes, page_tokens, heads, kv_heads = 128, 136, 64, 16, 4
+    lengths = [int(n) for n in rng.integers(span, 600, size=20)] + [20000] + [int(n) for n in rng.integers(span, 600, size=20)]
+    lengths[0], lengths[5], lengths[30] = span, 128, 129
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, lengths, kv_heads, dim, page_tokens, row_bytes)
+    seqs = len(lengths)
+    q = rng.standard_normal((seqs, span, heads, dim)).astype(np.float16).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    positions = [n - span for n in lengths]
+    got = _run(gpu, pool, table, tb, positions, q, span, heads, scale, True, False, max_context=table.shape[1] * page_tokens)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array(positions, np.int32), q, scale)
+    for s in range(seqs):
+        close_enough(got[s], want[s], f"sequence {s} of {lengths[s]} tokens")
+    gpu.release(buffer); gpu.release(tb)
+
+
 def test_zero_queries_give_the_mean_of_the_values(gpu, oracle):
     rng = np.random.default_rng(5)
     heads, kv_heads, dim, row_bytes, page_tokens = 8, 2, 128, 136, 32
