@@ -5,6 +5,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdint>
 #include <cstring>
@@ -84,6 +85,21 @@ struct KernelTimer {
         d.profile_events.push_back(event);
     }
 };
+
+// Launches one kernel on the device's stream.  With the device's profiling on it goes through the extended launch, whose
+// two events take the kernel's own start and end times (what a tracer reads), not the times of event packets around it.
+template<typename... Params, typename... Args>
+void timed_launch(Device& d, void (*kernel)(Params...), dim3 grid, dim3 block, size_t shared, Args... args) {
+    hipEvent_t start = nullptr, stop = nullptr;
+    if (d.profile && (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess)) {
+        if (start) (void)hipEventDestroy(start);
+        start = stop = nullptr;
+    }
+    if (!start) { kernel<<<grid, block, shared, d.stream>>>(Params(args)...); return; }
+    hipExtLaunchKernelGGL(kernel, grid, block, uint32_t(shared), d.stream, start, stop, 0, Params(args)...);
+    d.profile_events.push_back(start);
+    d.profile_events.push_back(stop);
+}
 
 Device& device(void* handle);                         // sets the HIP device of the handle; throws on null
 void* allocate(Device& d, size_t bytes, bool zero);   // budget-checked hipMalloc (+ tail)

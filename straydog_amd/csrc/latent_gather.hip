@@ -245,10 +245,7 @@ void latent_gather(Device& d, const void* q, const void* latents, const int32_t*
         SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_gather_kernel<KDIM, VDIM>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
         raised = true;
     }
-    {
-        KernelTimer timer(d);
-        latent_gather_kernel<KDIM, VDIM><<<dim3(args.chunks, unsigned((heads + 63) / 64), unsigned(batch)), 256, shared, d.stream>>>(args);
-    }
+    timed_launch(d, &latent_gather_kernel<KDIM, VDIM>, dim3(args.chunks, unsigned((heads + 63) / 64), unsigned(batch)), dim3(256), shared, args);
     SD_CHECK(hipGetLastError());
     latent_merge_kernel<VDIM><<<unsigned(batch * heads), VDIM / 4, 0, d.stream>>>(args);
 }

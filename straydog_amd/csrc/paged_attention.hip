@@ -438,7 +438,7 @@ void launch(Device& d, const PagedArgs& args, dim3 grid) {
         SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_kernel<DIM, QT, Q8, OCC>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
         raised = true;
     }
-    paged_attention_kernel<DIM, QT, Q8, OCC><<<grid, WAVES * 64, shared, d.stream>>>(args);
+    timed_launch(d, &paged_attention_kernel<DIM, QT, Q8, OCC>, grid, dim3(WAVES * 64), shared, args);
 }
 
 // The variants that exist: (columns, query tiles, format) -> waves per SIMD the kernel is compiled for.  One query tile is
@@ -513,11 +513,8 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
     args.partial = static_cast<float*>(scratch);
     const dim3 grid(args.groups_max);
     const bool q8 = pool->row_bytes != 2 * pool->dim;
-    {
-        KernelTimer timer(value);
-        if (pool->dim == 128) { if (q8) launch_tiles<128, true>(value, args, query_tiles, grid); else launch_tiles<128, false>(value, args, query_tiles, grid); }
-        else { if (q8) launch_tiles<256, true>(value, args, query_tiles, grid); else launch_tiles<256, false>(value, args, query_tiles, grid); }
-    }
+    if (pool->dim == 128) { if (q8) launch_tiles<128, true>(value, args, query_tiles, grid); else launch_tiles<128, false>(value, args, query_tiles, grid); }
+    else { if (q8) launch_tiles<256, true>(value, args, query_tiles, grid); else launch_tiles<256, false>(value, args, query_tiles, grid); }
     SD_CHECK(hipGetLastError());
     const unsigned outputs = unsigned(checked_product({seqs, span, heads}));
     if (pool->dim == 128) {

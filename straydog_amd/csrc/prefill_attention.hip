@@ -608,7 +608,7 @@ void launch_dense(Device& d, const PrefillArgs& args, unsigned seqs) {
     }
     unpack_tiles_kernel<DIM, Q8><<<dim3(tiles_per_seq, args.kv_heads, seqs), 256, 0, d.stream>>>(args, tiles, tiles_per_seq);
     const unsigned runs = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
-    prefill_dense_kernel<DIM, QT><<<dim3((runs + 1) / 2, args.kv_heads, seqs), TEAM * 64, shared, d.stream>>>(args, tiles, tiles_per_seq);
+    timed_launch(d, &prefill_dense_kernel<DIM, QT>, dim3((runs + 1) / 2, args.kv_heads, seqs), dim3(TEAM * 64), shared, args, tiles, tiles_per_seq);
 }
 
 template<int DIM, int QT, bool Q8, int OCC>
@@ -623,7 +623,7 @@ void launch(Device& d, const PrefillArgs& args, unsigned seqs) {
         raised = true;
     }
     const unsigned tiles = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
-    prefill_attention_kernel<DIM, QT, Q8, OCC><<<dim3(tiles, args.kv_heads, seqs), TEAM * 64, shared, d.stream>>>(args);
+    timed_launch(d, &prefill_attention_kernel<DIM, QT, Q8, OCC>, dim3(tiles, args.kv_heads, seqs), dim3(TEAM * 64), shared, args);
 }
 
 }  // namespace
@@ -644,7 +644,6 @@ void prefill_attention(Device& d, const sdx_kv_pool* pool, const int32_t* page_t
     args.rows = unsigned(span * args.group); args.max_context = int(max_context);
     args.out = out; args.out_f16 = out_f16;
     const bool q8 = pool->row_bytes != 2 * pool->dim;
-    KernelTimer timer(d);
     if (pool->dim == 128) { if (q8) launch_dense<128, 2, true>(d, args, unsigned(seqs)); else launch_dense<128, 2, false>(d, args, unsigned(seqs)); }
     else { if (q8) launch<256, 1, true, 2>(d, args, unsigned(seqs)); else launch<256, 1, false, 2>(d, args, unsigned(seqs)); }
 }

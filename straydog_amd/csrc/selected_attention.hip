@@ -221,8 +221,7 @@ void launch(Device& d, const SelectedArgs& args, size_t rows) {
         SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&selected_attention_kernel<Q8>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
         raised = true;
     }
-    KernelTimer timer(d);
-    selected_attention_kernel<Q8><<<dim3(args.chunks, args.kv_heads, unsigned(rows)), WAVES * 64, shared, d.stream>>>(args);
+    timed_launch(d, &selected_attention_kernel<Q8>, dim3(args.chunks, args.kv_heads, unsigned(rows)), dim3(WAVES * 64), shared, args);
 }
 
 }  // namespace
