@@ -296,43 +296,67 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         }
     }
 
-    // Merge the waves through LDS: per wave and query row the maximum, the sum and the unnormalised output.
-    __syncthreads();    // the merge area overlays the stages
-    constexpr int STRIDE = DIM + 2, QROWS = QT * 16;
+    // Merge the waves, two by two, through LDS: waves 2 and 3 hand their maxima, sums and unnormalised outputs to waves 0 and
+    // 1, then wave 1 hands its own to wave 0.  Corresponding lanes hold corresponding elements, so a value goes from lane to
+    // lane ([register][lane] in LDS, no bank conflicts), and the area is two waves' registers: it fits the stages it overlays.
+    __syncthreads();    // the stages are free
+    constexpr int STRIDE = DIM + 2, HELD = QT * (TILES * 4 + 2);
     const int lane_after = fresh_lane(), li_after = lane_after & 15, g_after = lane_after >> 4;   // (again: nothing of this is worked out before the loop)
-    const unsigned thread = unsigned(wave * 64 + lane_after);
-    #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-        const float sum = row_sum(l[qt]);
-        float* row = lds + (size_t(wave) * QROWS + qt * 16 + li_after) * STRIDE;
-        if (g_after == 0) { row[DIM] = m[qt] * args.scale_log2; row[DIM + 1] = sum; }      // maxima leave in exponent units
+    const auto hand_over = [&](int slot) {
+        float* to = lds + size_t(slot) * HELD * 64 + lane_after;
         #pragma unroll
-        for (int jj = 0; jj < TILES; ++jj)
+        for (int qt = 0; qt < QT; ++qt) {
+            float* mine = to + qt * (TILES * 4 + 2) * 64;
+            mine[0] = m[qt]; mine[64] = l[qt];
             #pragma unroll
-            for (int r = 0; r < 4; ++r) row[W * (4 * g_after + r) + jj] = acc[qt][jj][r];
-    }
+            for (int jj = 0; jj < TILES; ++jj)
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) mine[(2 + 4 * jj + r) * 64] = acc[qt][jj][r];
+        }
+    };
+    const auto take_in = [&](int slot) {
+        const float* from = lds + size_t(slot) * HELD * 64 + lane_after;
+        #pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            const float* theirs = from + qt * (TILES * 4 + 2) * 64;
+            const float m_other = theirs[0], m_new = fmaxf(m[qt], m_other);
+            const float keep = __builtin_amdgcn_exp2f((m[qt] - m_new) * args.scale_log2), add = __builtin_amdgcn_exp2f((m_other - m_new) * args.scale_log2);
+            m[qt] = m_new;
+            l[qt] = l[qt] * keep + theirs[64] * add;
+            #pragma unroll
+            for (int jj = 0; jj < TILES; ++jj)
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) acc[qt][jj][r] = acc[qt][jj][r] * keep + theirs[(2 + 4 * jj + r) * 64] * add;
+        }
+    };
+    if (wave >= 2) hand_over(wave - 2);
     __syncthreads();
-    // a partial result per (workgroup, sequence and K/V head) met: both only grow along the units, so their sum numbers them
-    float* out = args.partial + (size_t(blockIdx.x) + size_t(seq) * args.kv_heads + kvh) * args.rows * STRIDE;
-    for (unsigned i = thread; i < args.rows * STRIDE; i += WAVES * 64) {
-        const unsigned row = i / STRIDE, col = i % STRIDE;
-        float top = NEG_BIG;
+    if (wave < 2) take_in(wave);
+    __syncthreads();
+    if (wave == 1) hand_over(0);
+    __syncthreads();
+    if (wave == 0) {
+        take_in(0);
+        // a partial result per (workgroup, sequence and K/V head) met: both only grow along the units, so their sum numbers
+        // them.  Row layout: DIM outputs, the maximum in exponent units, the sum; a lane holds 4 runs of 8 columns of its row.
+        float* out = args.partial + (size_t(blockIdx.x) + size_t(seq) * args.kv_heads + kvh) * args.rows * STRIDE;
         #pragma unroll
-        for (int w = 0; w < WAVES; ++w) top = fmaxf(top, lds[(size_t(w) * QROWS + row) * STRIDE + DIM]);
-        float value;
-        if (col == DIM) value = top;
-        else {
-            value = 0.0f;
-            #pragma unroll
-            for (int w = 0; w < WAVES; ++w) {
-                const float* other = lds + (size_t(w) * QROWS + row) * STRIDE;
-                value += other[col] * __builtin_amdgcn_exp2f(other[DIM] - top);
+        for (int qt = 0; qt < QT; ++qt) {
+            const float sum = row_sum(l[qt]);
+            const int row = qt * 16 + li_after;
+            if (row < int(args.rows)) {
+                float* to = out + size_t(row) * STRIDE;
+                if (g_after == 0) *reinterpret_cast<float2*>(to + DIM) = make_float2(m[qt] * args.scale_log2, sum);
+                #pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    #pragma unroll
+                    for (int jj = 0; jj < TILES; jj += 2)
+                        *reinterpret_cast<float2*>(to + W * (4 * g_after + r) + jj) = make_float2(acc[qt][jj][r], acc[qt][jj + 1][r]);
             }
         }
-        out[i] = value;
     }
     unit += take;
-    if (unit < share_end) __syncthreads();                  // the next segment's stages overlay the merge area
+    if (unit < share_end) __syncthreads();                  // the next segment's stages overlay what wave 0 has just read
     }
 }
 
@@ -431,7 +455,7 @@ uint64_t most_groups(uint64_t seqs, uint64_t kv_heads, uint64_t max_context) {
 template<int DIM, int QT, bool Q8, int OCC>
 void launch(Device& d, const PagedArgs& args, dim3 grid) {
     constexpr int slab = STEP * (Q8 ? DIM + DIM / 16 : 2 * DIM);
-    const size_t shared = std::max(size_t(WAVES) * QT * 16 * (DIM + 2) * 4, size_t(WAVES) * stages_per_wave(slab, OCC) * 2 * slab);
+    const size_t shared = std::max(size_t(2) * QT * (DIM / 16 * 4 + 2) * 64 * 4, size_t(WAVES) * stages_per_wave(slab, OCC) * 2 * slab);
     if (shared > 160 * 1024) throw std::runtime_error("Straydog paged attention: too many query rows per K/V head for the decode kernel");
     static bool raised = false;
     if (!raised && shared > 64 * 1024) {
@@ -461,7 +485,7 @@ void launch_tiles(Device& d, const PagedArgs& args, unsigned query_tiles, dim3 g
 // Workgroups resident at once: as many per compute unit as the variant's waves per SIMD and its LDS allow.
 unsigned resident_slots(const Device& d, unsigned dim, bool q8, unsigned query_tiles) {
     const int occupancy = variant_occupancy(int(dim), q8, query_tiles), slab = STEP * int(q8 ? dim + dim / 16 : 2 * dim);
-    const size_t shared = std::max(size_t(WAVES) * query_tiles * 16 * (dim + 2) * 4, size_t(WAVES) * stages_per_wave(slab, occupancy) * 2 * slab);
+    const size_t shared = std::max(size_t(2) * query_tiles * (dim / 16 * 4 + 2) * 64 * 4, size_t(WAVES) * stages_per_wave(slab, occupancy) * 2 * slab);
     return d.compute_units * unsigned(std::max<size_t>(1, std::min<size_t>(size_t(occupancy), (160 * 1024) / shared)));
 }
 
