@@ -389,6 +389,13 @@ __global__ void __launch_bounds__(256) paged_merge_kernel(PagedArgs args, void* 
     float2 value = {0.0f, 0.0f};
     for (unsigned first = 0; first < used; first += 256) {
         const unsigned c = first + tid, count = min(used - first, 256u);
+        // eight of a group's partial results at a time: eight loads in flight, not one after the other; the first eight are
+        // asked for together with the maxima and sums their weights come from
+        constexpr unsigned AT_ONCE = 8;
+        float2 v[AT_ONCE];
+        if (group < count)
+            #pragma unroll
+            for (unsigned i = 0; i < AT_ONCE; ++i) v[i] = *reinterpret_cast<const float2*>(base + (first + min(group + i * GROUPS, count - 1)) * step + col);
         float m = NEG_BIG, l = 0.0f;
         if (c < used) { const float2 pair = *reinterpret_cast<const float2*>(base + c * step + DIM); m = pair.x; l = pair.y; }
         float tile_top = m;
@@ -408,12 +415,10 @@ __global__ void __launch_bounds__(256) paged_merge_kernel(PagedArgs args, void* 
         sum = sum * keep + (reduce[1][0] + reduce[1][1]) + (reduce[1][2] + reduce[1][3]);
         value.x *= keep; value.y *= keep;
         top = top_new;
-        // eight of a group's chunks at a time: eight loads in flight, not one after the other
-        constexpr unsigned AT_ONCE = 8;
         for (unsigned k0 = group; k0 < count; k0 += AT_ONCE * GROUPS) {
-            float2 v[AT_ONCE];
-            #pragma unroll
-            for (unsigned i = 0; i < AT_ONCE; ++i) v[i] = *reinterpret_cast<const float2*>(base + (first + min(k0 + i * GROUPS, count - 1)) * step + col);
+            if (k0 != group)
+                #pragma unroll
+                for (unsigned i = 0; i < AT_ONCE; ++i) v[i] = *reinterpret_cast<const float2*>(base + (first + min(k0 + i * GROUPS, count - 1)) * step + col);
             #pragma unroll
             for (unsigned i = 0; i < AT_ONCE; ++i) {
                 const float w_k = k0 + i * GROUPS < count ? weights[k0 + i * GROUPS] : 0.0f;
