@@ -675,8 +675,8 @@ template<int HEADS>
 void fast_index_bounds(Device& d, const FastIndexSpace& s, const void* q_index, const void* keys, const float* weights, const int32_t* visible, size_t batch,
                        size_t groups, float scale) {
     index_prepare_kernel<<<dim3(unsigned(batch), 8), 256, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), weights, HEADS, 128, scale, batch, s.margin, s.wide_q, s.histogram);
-    index_interval_kernel<HEADS><<<dim3(unsigned((groups + BRACKET_KEYS - 1) / BRACKET_KEYS), unsigned(batch)), BRACKET_WAVES * 64, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys),
-                                                                                                   weights, visible, s.margin, groups, scale, s.lower, s.upper, s.histogram);
+    timed_launch(d, &index_interval_kernel<HEADS>, dim3(unsigned((groups + BRACKET_KEYS - 1) / BRACKET_KEYS), unsigned(batch)), dim3(BRACKET_WAVES * 64), 0,
+                 static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys), weights, visible, s.margin, groups, scale, s.lower, s.upper, s.histogram);
     SD_CHECK(hipGetLastError());
 }
 
@@ -684,10 +684,7 @@ template<int HEADS>
 void fast_index_top_k(Device& d, const FastIndexSpace& s, const void* q_index, const void* keys, const float* weights, const int32_t* visible, size_t batch,
                       size_t groups, float scale, size_t k, int32_t* indices) {
     const dim3 grid(unsigned(s.blocks), unsigned(batch));
-    {
-        KernelTimer timer(d);
-        fast_index_bounds<HEADS>(d, s, q_index, keys, weights, visible, batch, groups, scale);
-    }
+    fast_index_bounds<HEADS>(d, s, q_index, keys, weights, visible, batch, groups, scale);
     const uint32_t rank = uint32_t(std::min<size_t>(k, 0xffffffffu));
     radix_histogram_kernel<<<grid, 256, 0, d.stream>>>(s.lower, groups, batch, 1, rank, s.histogram);
     candidate_count_kernel<<<grid, 256, 0, d.stream>>>(s.upper, groups, batch, rank, s.histogram, s.counts);
