@@ -32,9 +32,9 @@ MEASURED_TRAFFIC = {"config1": 626.8e6, "config1_32k": 1147.4e6}
 def timed(gpu, step, steps, warmup):
     """(ms per step over the whole stream, ms per launch of the dominant kernel) for `steps` steps after `warmup`.  Two passes of
     the same `steps` steps: the first is bracketed by two events and nothing else (the step time), in the second the library
-    also times every launch of the dominant kernel: through the extended launch, whose events take the kernel's own start and
-    end (the duration a tracer reports), or, where the timed stage is two kernels, by events around them -- either way the
-    queue stalls for a few microseconds per launch, which the step time should not carry."""
+    also times every launch of the dominant kernel through the extended launch, whose events take the kernel's own start and
+    end (the duration a tracer reports) -- the queue stalls for a few microseconds per such launch, which the step time
+    should not carry."""
     for _ in range(warmup):
         step()
     gpu.synchronize()

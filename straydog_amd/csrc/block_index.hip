@@ -628,7 +628,7 @@ __global__ void __launch_bounds__(256) stage_prepare_kernel(StageArgs a) {
 template<int T>
 void launch_rows(Device& d, const float* queries, size_t stride, const float* blocks, size_t pool, size_t base, const uint32_t* dynamic, size_t steps,
                  size_t most, float* scores) {
-    scores_rows_kernel<T><<<checked_blocks(most, 64), 64 * HEADS, 0, d.stream>>>(queries, stride, blocks, pool, base, dynamic, unsigned(steps), scores);
+    timed_launch(d, &scores_rows_kernel<T>, dim3(checked_blocks(most, 64)), dim3(64 * HEADS), 0, queries, stride, blocks, pool, base, dynamic, unsigned(steps), scores);
 }
 
 }  // namespace
@@ -678,7 +678,6 @@ int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, con
     if (dynamic_base) op_span(value, dynamic_base, 4, "sdx_qsa_index position");
     const size_t most = dynamic_base ? size_t(pool) : size_t((base + steps) / 4);       // complete blocks of the last row, at most
     {
-        KernelTimer timer(value);
         if (most > KEEP) {
             if (steps <= 1) launch_rows<1>(value, queries, query_stride, blocks, pool, base, dynamic_base, steps, most, scores);
             else if (steps <= 2) launch_rows<2>(value, queries, query_stride, blocks, pool, base, dynamic_base, steps, most, scores);
@@ -686,8 +685,8 @@ int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, con
             else if (steps <= 8) launch_rows<8>(value, queries, query_stride, blocks, pool, base, dynamic_base, steps, most, scores);
             else {
                 if (dynamic_base) throw std::runtime_error("sdx_qsa_index: a device-resident position serves spans of up to 8 rows");
-                scores_tiled_kernel<<<dim3(checked_blocks(most, TILE_BLOCKS), checked_blocks(steps, TILE_ROWS)), TILE_THREADS, 0, value.stream>>>(
-                    queries, query_stride, blocks, pool, base, steps, scores);
+                timed_launch(value, &scores_tiled_kernel, dim3(checked_blocks(most, TILE_BLOCKS), checked_blocks(steps, TILE_ROWS)), dim3(TILE_THREADS), 0,
+                             queries, query_stride, blocks, pool, base, steps, scores);
             }
         }
     }

@@ -67,23 +67,9 @@ struct Device {
     std::map<uint64_t, Recorded> graphs;
     bool recording = false;
     std::vector<hipEvent_t> events;
-    // Optional kernel timing for harnesses (sdx_profile): event pairs around the launches of the op's main kernel.
+    // Optional kernel timing for harnesses (sdx_profile): an event pair per launch of the op's main kernel (timed_launch).
     bool profile = false;
     std::vector<hipEvent_t> profile_events;
-};
-
-// Brackets one kernel launch with events when the device's profiling is on.
-struct KernelTimer {
-    Device& d;
-    explicit KernelTimer(Device& device) : d(device) { mark(); }
-    ~KernelTimer() { mark(); }
-    void mark() {
-        if (!d.profile) return;
-        hipEvent_t event;
-        if (hipEventCreate(&event) != hipSuccess) return;
-        (void)hipEventRecord(event, d.stream);
-        d.profile_events.push_back(event);
-    }
 };
 
 // Launches one kernel on the device's stream.  With the device's profiling on it goes through the extended launch, whose
