@@ -37,7 +37,7 @@ constexpr unsigned UNIT = STEP * WAVES;
 struct Share { unsigned units, groups; };
 __device__ __forceinline__ Share batch_share(const PagedArgs& args, int lane) {
     unsigned units = 0;
-    for (unsigned s = lane; s < args.seqs; s += 64) units += unsigned(min(args.positions[s] + int(args.span), args.max_context) + int(UNIT) - 1) / UNIT;
+    for (unsigned s = lane; s < args.seqs; s += 64) units += unsigned(min(first_position(args.positions, s, args.max_context) + int(args.span), args.max_context) + int(UNIT) - 1) / UNIT;
     #pragma unroll
     for (int d = 32; d; d >>= 1) units += __shfl_xor(units, d);
     units = __builtin_amdgcn_readfirstlane(units * args.kv_heads);
@@ -75,7 +75,7 @@ __device__ __forceinline__ bool locate(const PagedArgs& args, unsigned u, Segmen
     unsigned before = 0;
     for (unsigned first = 0; first < args.seqs; first += 64) {
         const unsigned s = first + lane;
-        const int position = s < args.seqs ? args.positions[s] : 0;
+        const int position = s < args.seqs ? first_position(args.positions, s, args.max_context) : 0;
         const int total = s < args.seqs ? min(position + int(args.span), args.max_context) : 0;
         const unsigned units = unsigned(total + int(UNIT) - 1) / UNIT;
         unsigned upto = units * args.kv_heads;      // units of this and the earlier sequences of the 64
@@ -374,10 +374,10 @@ __global__ void __launch_bounds__(256) paged_merge_kernel(PagedArgs args, void* 
     const int lane = int(tid & 63);
     const Share share = batch_share(args, lane);
     unsigned before = 0;
-    for (unsigned s = lane; s < seq; s += 64) before += unsigned(min(args.positions[s] + int(args.span), args.max_context) + int(UNIT) - 1) / UNIT;
+    for (unsigned s = lane; s < seq; s += 64) before += unsigned(min(first_position(args.positions, s, args.max_context) + int(args.span), args.max_context) + int(UNIT) - 1) / UNIT;
     #pragma unroll
     for (int d = 32; d; d >>= 1) before += __shfl_xor(before, d);
-    const unsigned units = unsigned(min(args.positions[seq] + int(args.span), args.max_context) + int(UNIT) - 1) / UNIT;
+    const unsigned units = unsigned(min(first_position(args.positions, seq, args.max_context) + int(args.span), args.max_context) + int(UNIT) - 1) / UNIT;
     const unsigned begin = (before * args.kv_heads + kvh * units), owner = share_owner(share, begin);
     const unsigned used = share_owner(share, begin + units - 1) - owner + 1;
     const float* base = args.partial + (size_t(owner) + size_t(seq) * args.kv_heads + kvh) * args.rows * STRIDE + size_t(row) * STRIDE;

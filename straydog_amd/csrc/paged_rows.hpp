@@ -38,6 +38,10 @@ struct PagedArgs {
     int max_context;       // positions[s] + span is clipped to this (the launch and the page table are sized for it)
 };
 
+// A sequence's first query position as the kernels use it: the positions live on the device, where the host cannot check
+// them, so one outside [0, max_context] is taken as the nearest end (and addresses nothing outside the page table).
+__device__ __forceinline__ int first_position(const int32_t* positions, unsigned seq, int max_context) { return min(max(positions[seq], 0), max_context); }
+
 // The maximum / the sum over the four lanes li, li + 16, li + 32, li + 48 (one query row's four lane groups), in all four.
 // v_permlane16_swap exchanges the odd 16-lane rows of its first register with the even rows of its second, v_permlane32_swap
 // the upper half of the first with the lower half of the second: with both registers holding the same values, each lane

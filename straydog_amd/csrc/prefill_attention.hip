@@ -60,7 +60,7 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     static_assert(STAGES >= 2, "a step is copied while the one before is computed");
     const int tile = int(gridDim.x) - 1 - int(blockIdx.x), kvh = blockIdx.y, seq = blockIdx.z;   // later rows walk further: first
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, g = lane >> 4;
-    const int position = args.positions[seq];
+    const int position = first_position(args.positions, unsigned(seq), args.max_context);
     const int cached = min(position + int(args.span), args.max_context);          // rows of the sequence the cache holds
     const int quarter = wave % GROUPS, half = wave / GROUPS;                      // waves w and w + 4 share a SIMD and the rows
     const int row0 = tile * GROUP_ROWS + quarter * WAVE_ROWS;                     // the wave's first query row
@@ -296,7 +296,7 @@ __global__ void __launch_bounds__(256) unpack_tiles_kernel(PrefillArgs args, uin
     constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, KT = TILE_KEYS * DIM * 2, PIECES = DIM / 8;
     static_assert(DIM == 128, "a K row is 16 pieces, a V^T row 16 units");
     const int tile = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z, t = threadIdx.x;
-    const int cached = min(args.positions[seq] + int(args.span), args.max_context), key0 = tile * TILE_KEYS;
+    const int cached = min(first_position(args.positions, unsigned(seq), args.max_context) + int(args.span), args.max_context), key0 = tile * TILE_KEYS;
     if (key0 >= cached) return;
     const int32_t* table = args.page_table + size_t(seq) * args.table_stride;
     const size_t plane_bytes = size_t(args.page_tokens) * ROW;
@@ -380,7 +380,7 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     static_assert(TILE % (1024 * TEAM) == 0 && RING * TILE <= 160 * 1024 - 1024 && TILE_KEYS == 2 * SUB, "a tile is two steps of a wave");
     const int kvh = blockIdx.y, seq = blockIdx.z;
     const int thread = threadIdx.x, lane = thread & 63, wave = __builtin_amdgcn_readfirstlane(thread >> 6), li = lane & 15, g = lane >> 4;
-    const int position = args.positions[seq];
+    const int position = first_position(args.positions, unsigned(seq), args.max_context);
     const int cached = min(position + int(args.span), args.max_context);
     const int quarter = wave % GROUPS, half = wave / GROUPS;
     const int runs = (int(args.rows) + GROUP_ROWS - 1) / GROUP_ROWS;

@@ -258,6 +258,25 @@ def test_shares_that_cross_sequences_and_heads(gpu, oracle, span):
     gpu.release(buffer); gpu.release(tb)
 
 
+def test_positions_outside_the_context_are_taken_as_its_nearest_end(gpu, oracle):
+    # the positions live on the device, where the host cannot check them: a negative one counts as 0, one past max_context as
+    # max_context, and the sequences beside them are not disturbed
+    rng = np.random.default_rng(515)
+    dim, row_bytes, page_tokens, heads, kv_heads = 128, 136, 64, 8, 2
+    lengths = [300, 300, 300, 300]
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, lengths, kv_heads, dim, page_tokens, row_bytes)
+    q = rng.standard_normal((4, 1, heads, dim)).astype(np.float16).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    max_context = 300
+    given = [-7, 120, 2_000_000_000, 299]
+    meant = [0, 120, 299, 299]          # (a position of max_context with a span of 1 sees all max_context tokens, as 299 does)
+    got = _run(gpu, pool, table, tb, given, q, 1, heads, scale, True, False, max_context=max_context)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array(meant, np.int32), q, scale)
+    for s in range(4):
+        close_enough(got[s], want[s], f"position {given[s]}")
+    gpu.release(buffer); gpu.release(tb)
+
+
 def test_zero_queries_give_the_mean_of_the_values(gpu, oracle):
     rng = np.random.default_rng(5)
     heads, kv_heads, dim, row_bytes, page_tokens = 8, 2, 128, 136, 32
