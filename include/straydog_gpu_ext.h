@@ -166,9 +166,10 @@ int64_t sdx_event_record(void* handle);
 int sdx_event_elapsed(void* handle, int64_t begin, int64_t end, float* milliseconds);
 int sdx_events_clear(void* handle);
 int sdx_device_compute_units(void* handle);
-/* Kernel timing for benchmarks: while enabled, each op brackets the launch of its dominant kernel with events on the
- * handle's stream; sdx_profile_read waits for the stream and returns the summed kernel time and the launch count.
- * sdx_profile(handle, 0|1) clears what was recorded. */
+/* Kernel timing for benchmarks: while enabled, each op launches its dominant kernel through the extended launch, whose two
+ * events take the kernel's own start and end on the handle's stream; sdx_profile_read waits for the stream and returns the
+ * summed kernel time and the launch count.  sdx_profile(handle, 0|1) clears what was recorded.  Launches recorded into a graph
+ * (sd_graph_begin .. sd_graph_end) are not timed. */
 int sdx_profile(void* handle, int enable);
 int sdx_profile_read(void* handle, double* milliseconds, uint64_t* launches);
 int sdx_fill_normal(void* handle, void* out, uint64_t count, uint64_t seed, int out_kind /* 0 f32, 1 f16, 2 bf16 */);

@@ -77,7 +77,9 @@ struct Device {
 template<typename... Params, typename... Args>
 void timed_launch(Device& d, void (*kernel)(Params...), dim3 grid, dim3 block, size_t shared, Args... args) {
     hipEvent_t start = nullptr, stop = nullptr;
-    if (d.profile && (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess)) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    const bool timed = d.profile && hipStreamIsCapturing(d.stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone;
+    if (timed && (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess)) {
         if (start) (void)hipEventDestroy(start);
         start = stop = nullptr;
     }
