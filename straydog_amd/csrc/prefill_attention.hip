@@ -301,11 +301,28 @@ __global__ void __launch_bounds__(256) unpack_tiles_kernel(PrefillArgs args, uin
     const int32_t* table = args.page_table + size_t(seq) * args.table_stride;
     const size_t plane_bytes = size_t(args.page_tokens) * ROW;
     uint8_t* out = tiles_out + ((size_t(seq) * args.kv_heads + kvh) * tiles_per_seq + tile) * tile_bytes<DIM>();
-    const auto row_of = [&](int key, bool value) {
+    // The tile's raw rows come into LDS first, by 8-byte words that follow one another through a row and from row to row of
+    // a page (the small pieces the layouts below are made of would each be a memory access of their own otherwise).
+    __shared__ __attribute__((aligned(16))) uint8_t raw[2][TILE_KEYS][ROW];
+    constexpr int WORDS = ROW / 8;
+    constexpr int ALL = 2 * TILE_KEYS * WORDS, MINE = (ALL + 255) / 256;
+    uint2 held[MINE];
+    #pragma unroll
+    for (int j = 0; j < MINE; ++j) {                        // all of a thread's words are asked for before the first is stored
+        const int word = min(t + 256 * j, ALL - 1);
+        const int value = word / (TILE_KEYS * WORDS), key = word / WORDS % TILE_KEYS, at = word % WORDS;
         const int token = min(key0 + key, cached - 1);
-        return args.pages + (size_t(table[token / int(args.page_tokens)]) * 2 * args.kv_heads + (value ? args.kv_heads : 0) + kvh) * plane_bytes +
-               size_t(token % int(args.page_tokens)) * ROW;
-    };
+        const uint8_t* row = args.pages + (size_t(table[token / int(args.page_tokens)]) * 2 * args.kv_heads + (value ? args.kv_heads : 0) + kvh) * plane_bytes +
+                             size_t(token % int(args.page_tokens)) * ROW;
+        held[j] = *reinterpret_cast<const uint2*>(row + 8 * at);
+    }
+    #pragma unroll
+    for (int j = 0; j < MINE; ++j) {
+        const int word = t + 256 * j;
+        if (word < ALL) *reinterpret_cast<uint2*>(&raw[0][0][0] + 8 * word) = held[j];
+    }
+    __syncthreads();
+    const auto row_of = [&](int key, bool value) -> const uint8_t* { return raw[value ? 1 : 0][key]; };
     typedef _Float16 half4 __attribute__((ext_vector_type(4)));
     // K: a thread takes pieces of 8 columns; rows past the sequence's end become zeros
     #pragma unroll
