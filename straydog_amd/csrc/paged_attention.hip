@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
     const int total = __builtin_amdgcn_readfirstlane(found.total), position = __builtin_amdgcn_readfirstlane(found.position);
     const unsigned first_unit = __builtin_amdgcn_readfirstlane(found.unit);
     const unsigned take = min(share_end - unit, unsigned(__builtin_amdgcn_readfirstlane(found.units)) - first_unit);
-    const int chunk_begin = int(first_unit * UNIT), chunk_end = min(total, int((first_unit + take) * UNIT));
+    const int segment_begin = int(first_unit * UNIT), segment_end = min(total, int((first_unit + take) * UNIT));
     const table_ptr table = (table_ptr)(args.page_table + size_t(seq) * args.table_stride);
     const size_t plane_bytes = size_t(args.page_tokens) * ROW;
 
@@ -195,7 +195,7 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
 
     // Where the step to copy next lies: page_index-th page of the sequence, in_page rows into it.  Its page number is fetched
     // (a scalar load) a step before its copy is issued.
-    int token0 = chunk_begin + STEP * wave;
+    int token0 = segment_begin + STEP * wave;
     const int last_page = (total - 1) / int(args.page_tokens);
     int page_index = token0 / int(args.page_tokens), in_page = token0 % int(args.page_tokens);
     const auto advance = [&] {
@@ -205,19 +205,19 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
     settle_loads();
     #pragma unroll
     for (int ahead = 0; ahead < DEPTH; ++ahead) {
-        if (token0 + ahead * STEP * WAVES < chunk_end) copy_in(stages + ahead * (2 * SLAB), table[min(page_index, last_page)], in_page);
+        if (token0 + ahead * STEP * WAVES < segment_end) copy_in(stages + ahead * (2 * SLAB), table[min(page_index, last_page)], in_page);
         advance();
     }
     int page_ahead = table[min(page_index, last_page)];
-    for (int buffer = 0; token0 < chunk_end; token0 += STEP * WAVES, buffer = DEPTH == 2 ? buffer ^ 1 : 0) {
+    for (int buffer = 0; token0 < segment_end; token0 += STEP * WAVES, buffer = DEPTH == 2 ? buffer ^ 1 : 0) {
         uint8_t* const stage = stages + buffer * (2 * SLAB);
-        const bool more = token0 + DEPTH * STEP * WAVES < chunk_end;      // a step to copy into this stage once it is read
+        const bool more = token0 + DEPTH * STEP * WAVES < segment_end;      // a step to copy into this stage once it is read
         const int page_now = page_ahead, in_page_now = in_page;
         advance();
         page_ahead = table[min(page_index, last_page)];
         RowLoad<DIM, Q8> current;
         // the stage holds this step when only the step after it is still on its way
-        if (DEPTH == 2 && token0 + STEP * WAVES < chunk_end) wait_loads<LOADS>(); else wait_loads<0>();
+        if (DEPTH == 2 && token0 + STEP * WAVES < segment_end) wait_loads<LOADS>(); else wait_loads<0>();
         request(current, stage, token0);
         __builtin_amdgcn_s_waitcnt(0xc07f);          // lgkmcnt(0): operands are in registers, the stage is free again
         __builtin_amdgcn_sched_barrier(0);
@@ -362,8 +362,8 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
 
 // One block per (sequence, span row, head): the segments' partial results merged and normalised (the algebra of the
 // reference's qsa_decode_merge, gpu/sparse_attention_compute.hpp:139-170).  The block's 256 threads are GROUPS groups of
-// DIM/2 threads; a group takes every GROUPS-th chunk and a thread two columns, so all loads of a pass are in flight at
-// once; chunks are taken 256 at a time with a running maximum.
+// DIM/2 threads; a group takes every GROUPS-th segment and a thread two columns, so all loads of a pass are in flight at
+// once; segments are taken 256 at a time with a running maximum.
 template<int DIM, bool F16_OUT>
 __global__ void __launch_bounds__(256) paged_merge_kernel(PagedArgs args, void* out) {
     constexpr int STRIDE = DIM + 2, LANES = DIM / 2, GROUPS = 256 / LANES;
