@@ -76,10 +76,27 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     const bool most = wave < 2 * UNITS - LEAST * TEAM;
 
     // The step's two slabs into a stage: 2 * UNITS pieces of 1 KiB, every fourth one by this wave.
+    // (Pages of fewer tokens than a step: the step's rows lie in two pages, and every lane looks up the page of its own
+    // 16 bytes; rows past the cached ones are the last cached row again, and never read.)
+    const bool split_pages = args.page_tokens % WALK != 0;
     const auto copy_in = [&](int buffer, int token0) {
+        uint8_t* stage = stages + buffer * (2 * SLAB);
+        if (split_pages) {
+            #pragma unroll
+            for (int k = 0; k < MOST; ++k) {
+                const int unit = wave + TEAM * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS, at = 16 * lane + 1024 * j;
+                if (unit < 2 * UNITS && at < SLAB) {
+                    const int token = min(token0 + at / ROW, cached - 1);
+                    const int page = args.page_table[size_t(seq) * args.table_stride + token / int(args.page_tokens)];
+                    const uint8_t* from = args.pages + (size_t(page) * 2 * args.kv_heads + (part ? args.kv_heads : 0) + kvh) * plane_bytes +
+                                          size_t(token % int(args.page_tokens)) * ROW + at % ROW;
+                    __builtin_amdgcn_global_load_lds((global_ptr)from, (lds_ptr)(stage + part * SLAB + 1024 * j), 16, 0, 0);
+                }
+            }
+            return;
+        }
         const int page = table[token0 / int(args.page_tokens)];
         const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(token0 % int(args.page_tokens)) * ROW + 16 * lane;
-        uint8_t* stage = stages + buffer * (2 * SLAB);
         #pragma unroll
         for (int k = 0; k < MOST; ++k) {
             const int unit = wave + TEAM * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS;

@@ -138,12 +138,13 @@ def test_verify_span_rows(gpu, oracle, span, heads, kv_heads):
 
 @pytest.mark.parametrize("dim,fmt,span,heads,kv_heads", [(128, "q8", 40, 32, 4), (128, "q8", 100, 8, 1), (128, "f16", 33, 16, 2),
                                                          (256, "q8", 24, 24, 2), (256, "f16", 9, 24, 2), (128, "q8", 9, 4, 4)])
-def test_prefill_span_rows(gpu, oracle, dim, fmt, span, heads, kv_heads):
+@pytest.mark.parametrize("page_tokens", [64, 32])
+def test_prefill_span_rows(gpu, oracle, dim, fmt, span, heads, kv_heads, page_tokens):
     # BASELINE config 2 in small: a chunk of new tokens attends the cache (which holds the chunk's own rows) causally.
     # Rows per K/V head = span * group exceed what the decode kernel's workgroup takes, so this is the many-rows kernel.
     rng = np.random.default_rng(77 + span + dim)
+    # Pages of 32 tokens are shorter than the 64 keys a workgroup of the 256-column kernel takes at a time.
     row_bytes = (dim + dim // 16) if fmt == "q8" else 2 * dim
-    page_tokens = 64
     contexts = [0, 31, 200, 517]
     lengths = [c + span for c in contexts]
     pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, lengths, kv_heads, dim, page_tokens, row_bytes,
