@@ -11,6 +11,19 @@
 namespace sd {
 
 thread_local std::string last_error;
+void select_thin_reserve(Device& d);     // block_index.hip
+
+// Recorded graphs hold the addresses their ops were given.  When a buffer the library owns moves (the workspace grows), the
+// graphs recorded so far would replay on freed memory: they are dropped, sd_graph_run then answers 1 ("none stored under
+// this key") and the caller records again -- what the reference does when its K/V views change (kv_clear_graphs,
+// gpu/kv_stage.hpp:96-104).
+static void drop_graphs(Device& d) {
+    for (auto& entry : d.graphs) {
+        if (entry.second.executable) (void)hipGraphExecDestroy(entry.second.executable);
+        if (entry.second.graph) (void)hipGraphDestroy(entry.second.graph);
+    }
+    d.graphs.clear();
+}
 
 Device& device(void* handle) {
     if (!handle) throw std::runtime_error("Straydog device handle is null");
@@ -92,7 +105,10 @@ void* workspace(Device& d, size_t bytes) {
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     SD_CHECK(hipStreamIsCapturing(d.stream, &capturing));
     if (capturing != hipStreamCaptureStatusNone) throw std::runtime_error("Straydog attention workspace cannot grow while a graph is recorded");
-    if (d.workspace) release(d, d.workspace);
+    if (d.workspace) {
+        drop_graphs(d);
+        release(d, d.workspace);
+    }
     d.workspace = nullptr; d.workspace_bytes = 0;
     const size_t rounded = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
     d.workspace = allocate(d, rounded, true);
@@ -411,6 +427,8 @@ int sd_graph_begin(void* handle) {
     try {
         Device& d = device(handle);
         if (d.recording) throw std::runtime_error("a Straydog graph is already being recorded");
+        // (made here, not by the op that uses it: a capture takes no allocation; reference gpu/kernels.cpp:4769-4773)
+        try { select_thin_reserve(d); } catch (const std::exception&) {}
         SD_CHECK(hipStreamBeginCapture(d.stream, hipStreamCaptureModeThreadLocal));
         d.recording = true;
         return 0;

@@ -554,11 +554,7 @@ void launch_select(Device& d, const float* scores, size_t pool, size_t base, con
                    float* indices, float* counts, const uint2* thinned, const uint32_t* thinned_counts) {
     const unsigned held_runs = unsigned(std::min<size_t>((most + SELECT_THREADS - 1) / SELECT_THREADS, LDS_RUNS));
     const size_t shared = size_t(std::max(held_runs, 1u)) * SELECT_THREADS * 4;
-    static bool raised[2] = {false, false};
-    if (shared > 48 * 1024 && !raised[REGS ? 1 : 0]) {
-        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&select_kernel<REGS>), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_RUNS * SELECT_THREADS * 4));
-        raised[REGS ? 1 : 0] = true;
-    }
+    if (shared > 48 * 1024) raise_shared_limit(d, reinterpret_cast<const void*>(&select_kernel<REGS>), LDS_RUNS * SELECT_THREADS * 4);
     select_kernel<REGS><<<rows, SELECT_THREADS, shared, d.stream>>>(scores, pool, base, dynamic, selected, held_runs, indices, counts, thinned, thinned_counts);
 }
 
@@ -576,6 +572,7 @@ struct StageArgs {
     uint8_t* pages;
     unsigned page_tokens, row_bytes;
     const int32_t* page_table;
+    size_t page_count;
     size_t context;
     float* queries;                // [steps][heads][256]
     float *blocks, *history;
@@ -595,7 +592,9 @@ __global__ void __launch_bounds__(256) stage_prepare_kernel(StageArgs a) {
         key[c] = normalized(own[keys_at + head * 256 + c], a.k_norm, 256, rope, values, sums);
         __syncthreads();
         if (pos >= a.context || c >= 128) return;           // a position outside the cache writes no row; two waves encode
-        const size_t page = a.page_table ? size_t(a.page_table[pos / a.page_tokens]) : 0, in_page = a.page_table ? pos % a.page_tokens : pos;
+        const long long entry = a.page_table ? a.page_table[pos / a.page_tokens] : 0;
+        if (entry < 0 || size_t(entry) >= a.page_count) return;   // nor does a table entry that names no page of the pool
+        const size_t page = size_t(entry), in_page = a.page_table ? pos % a.page_tokens : pos;
         const bool is_value = c >= 64;
         const unsigned quad = c % 64;                       // four columns a thread: a wave holds the row, 8 lanes a 32-column block
         uint8_t* target = a.pages + ((page * 2 * a.kv_heads + (is_value ? a.kv_heads : 0) + head) * a.page_tokens + in_page) * a.row_bytes;
@@ -632,6 +631,18 @@ void launch_rows(Device& d, const float* queries, size_t stride, const float* bl
 }
 
 }  // namespace
+
+namespace sd {
+// The lists of a short span's thinned rows: allocated once per handle, never while a graph is being recorded (sd_graph_begin
+// calls this first, so that a recorded pass takes the same path as an eager one).
+constexpr size_t thin_list_bytes = size_t(THIN_ROWS) * THIN_SEGMENTS * THIN_CAP * sizeof(uint2);
+void select_thin_reserve(Device& d) {
+    if (d.select_thin) return;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    SD_CHECK(hipStreamIsCapturing(d.stream, &capturing));
+    if (capturing == hipStreamCaptureStatusNone) d.select_thin = allocate(d, thin_list_bytes + size_t(THIN_ROWS) * THIN_SEGMENTS * 4, true);
+}
+}  // namespace sd
 
 extern "C" {
 
@@ -691,17 +702,13 @@ int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, con
         }
     }
     const unsigned rows = checked_blocks(steps, 1);
-    // a few long rows: the thinning goes to many workgroups first (their lists live in a small buffer the handle keeps; were
-    // the first such call recorded into a graph, it does without)
+    // a few long rows: the thinning goes to many workgroups first (their lists live in a small buffer the handle keeps from
+    // the first such call, or from the first sd_graph_begin, on: a call recorded into a graph finds it there)
     const uint2* thinned = nullptr;
     const uint32_t* thinned_counts = nullptr;
     if (rows <= unsigned(THIN_ROWS) && most >= size_t(8) * SELECT_THREADS) {
-        constexpr size_t lists = size_t(THIN_ROWS) * THIN_SEGMENTS * THIN_CAP * sizeof(uint2);
-        if (!value.select_thin) {
-            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-            SD_CHECK(hipStreamIsCapturing(value.stream, &capturing));
-            if (capturing == hipStreamCaptureStatusNone) value.select_thin = allocate(value, lists + size_t(THIN_ROWS) * THIN_SEGMENTS * 4, true);
-        }
+        constexpr size_t lists = thin_list_bytes;
+        select_thin_reserve(value);
         if (value.select_thin) {
             uint2* listed = static_cast<uint2*>(value.select_thin);
             uint32_t* listed_counts = reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(value.select_thin) + lists);
@@ -751,7 +758,7 @@ int sdx_qsa_decode_attend(void* handle, const sdx_qsa_state* state, float* proje
         args.projections = projections; args.stride = stride;
         args.q_norm = state->q_norm; args.k_norm = state->k_norm; args.index_q_norm = state->index_q_norm; args.index_k_norm = state->index_k_norm;
         args.heads = unsigned(heads); args.kv_heads = kv.kv_heads; args.steps = unsigned(steps); args.positions = positions; args.ropes = ropes;
-        args.pages = static_cast<uint8_t*>(kv.pages); args.page_tokens = kv.page_tokens; args.row_bytes = kv.row_bytes; args.page_table = state->page_table;
+        args.pages = static_cast<uint8_t*>(kv.pages); args.page_tokens = kv.page_tokens; args.row_bytes = kv.row_bytes; args.page_table = state->page_table; args.page_count = size_t(kv.page_count);
         args.context = context; args.queries = static_cast<float*>(scratch); args.blocks = state->blocks; args.history = state->history; args.pool = pool;
         stage_prepare_kernel<<<dim3(unsigned(heads + kv.kv_heads + HEADS + 1), unsigned(steps)), 256, 0, value.stream>>>(args);
         SD_CHECK(hipGetLastError());

@@ -193,8 +193,7 @@ template<class Source>
 void launch(Device& d, const Source& source, const float* q, size_t rows, size_t heads, size_t kv_heads, size_t dim, float scale,
             size_t splits, float* partial, const float* gate, float* out) {
     const size_t shared = attention_lds(heads / kv_heads, dim);
-    static bool raised = false;
-    if (!raised) { SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&fp32_attention_kernel<Source>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64)); raised = true; }
+    raise_shared_limit(d, reinterpret_cast<const void*>(&fp32_attention_kernel<Source>), 160 * 1024 - 64);
     fp32_attention_kernel<Source><<<dim3(unsigned(rows * kv_heads), unsigned(splits)), THREADS, shared, d.stream>>>(source, q, heads, kv_heads, dim, scale, partial);
     SD_CHECK(hipGetLastError());
     fp32_attention_merge_kernel<<<unsigned(rows * heads), THREADS, 0, d.stream>>>(partial, splits, dim, gate, out);

@@ -58,6 +58,9 @@ struct Device {
     double2* turns = nullptr;
     size_t turns_rows = 0, turns_pairs = 0, turns_armed = 0, turns_ready_rows = 0, turns_ready_pairs = 0;
     bool turns_ready = false;
+    // Dynamic LDS limits raised so far, by kernel: the attribute belongs to this device's copy of the kernel, so each
+    // handle raises it for itself (raise_shared_limit).
+    std::map<const void*, size_t> shared_limits;
     // The lists of a short span's thinned index rows (block_index.hip), allocated at the first such call and kept.
     void* select_thin = nullptr;
     // Page-locked host copies of sequence state (conversation checkpoints): pointer -> bytes.
@@ -87,6 +90,16 @@ void timed_launch(Device& d, void (*kernel)(Params...), dim3 grid, dim3 block, s
     hipExtLaunchKernelGGL(kernel, grid, block, uint32_t(shared), d.stream, start, stop, 0, Params(args)...);
     d.profile_events.push_back(start);
     d.profile_events.push_back(stop);
+}
+
+// A kernel that asks for more dynamic LDS than the default limit has the limit raised first, once per handle and size.
+inline void raise_shared_limit(Device& d, const void* kernel, size_t bytes) {
+    size_t& have = d.shared_limits[kernel];
+    if (bytes <= have) return;
+    if (bytes > 160 * 1024) throw std::runtime_error("Straydog op: a kernel asks for more LDS than a compute unit has");
+    const hipError_t error = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes));
+    if (error != hipSuccess) throw std::runtime_error(std::string("Straydog op: ") + gpu_error_text(error));
+    have = bytes;
 }
 
 Device& device(void* handle);                         // sets the HIP device of the handle; throws on null

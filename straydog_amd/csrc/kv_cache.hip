@@ -61,6 +61,15 @@ void upload_entries(KvCache& c, size_t sequence, size_t first, size_t count) {
     if (count) upload(*c.device, c.table + sequence * c.stride + first, c.pages_of.data() + sequence * c.stride + first, count * sizeof(int32_t));
 }
 
+// The first `rows` rows of every plane of page `source` into page `copy`, in stream order.
+void copy_rows(KvCache& c, Device& d, int32_t source, int32_t copy, size_t rows) {
+    const size_t plane = size_t(c.pool.page_tokens) * c.pool.row_bytes, planes = 2 * size_t(c.pool.kv_heads);
+    auto* base = static_cast<uint8_t*>(c.pool.pages);
+    for (size_t p = 0; p < planes; ++p)
+        SD_CHECK(hipMemcpyAsync(base + (size_t(copy) * planes + p) * plane, base + (size_t(source) * planes + p) * plane, rows * c.pool.row_bytes,
+                                hipMemcpyDeviceToDevice, d.stream));
+}
+
 }  // namespace
 
 extern "C" {
@@ -131,9 +140,21 @@ int sdx_kv_cache_truncate(void* handle, void* cache, uint64_t sequence, uint64_t
     SD_OP_BEGIN
     KvCache& c = cache_of(value, cache);
     check_sequence(c, sequence);
-    const size_t keep = pages_for(c, tokens);
+    const size_t keep = pages_for(c, tokens), rest = size_t(tokens % c.pool.page_tokens);
+    // Rows appended after a rewind land in the last kept page from row `rest` on.  If another sequence shares that page (a fork's
+    // whole pages are shared by reference count), those rows are still the sibling's: this sequence continues on a copy of the
+    // rows it keeps.  Without a free page for the copy nothing is changed.
+    const bool shared_tail = rest && keep <= c.held[sequence] && keep && c.references[size_t(c.pages_of[sequence * c.stride + keep - 1])] > 1;
+    if (shared_tail && c.free_pages.empty()) throw std::runtime_error("Straydog K/V cache: out of pages");
     for (size_t i = c.held[sequence]; i > keep; --i) drop_page(c, c.pages_of[sequence * c.stride + i - 1]);
     c.held[sequence] = uint32_t(std::min<size_t>(c.held[sequence], keep));
+    if (shared_tail) {
+        const int32_t source = c.pages_of[sequence * c.stride + keep - 1], copy = take_page(c);
+        copy_rows(c, value, source, copy, rest);
+        drop_page(c, source);
+        c.pages_of[sequence * c.stride + keep - 1] = copy;
+        upload_entries(c, sequence, keep - 1, 1);
+    }
     SD_OP_END
 }
 
@@ -154,11 +175,7 @@ int sdx_kv_cache_fork(void* handle, void* cache, uint64_t from, uint64_t to, uin
         // the prefix's last page is written on by both sequences from here on: the target gets its own copy of the rows so far
         const int32_t source = c.pages_of[from * c.stride + whole], copy = take_page(c);
         c.pages_of[to * c.stride + whole] = copy;
-        const size_t plane = size_t(c.pool.page_tokens) * c.pool.row_bytes, planes = 2 * size_t(c.pool.kv_heads);
-        auto* base = static_cast<uint8_t*>(c.pool.pages);
-        for (size_t p = 0; p < planes; ++p)
-            SD_CHECK(hipMemcpyAsync(base + (size_t(copy) * planes + p) * plane, base + (size_t(source) * planes + p) * plane, rest * c.pool.row_bytes,
-                                    hipMemcpyDeviceToDevice, value.stream));
+        copy_rows(c, value, source, copy, rest);
     }
     c.held[to] = uint32_t(need);
     upload_entries(c, to, 0, need);

@@ -14,7 +14,7 @@ namespace {
 // A thread holds 4 consecutive values of a row; the 8 threads of a 32-value block are adjacent lanes, so the
 // block's largest magnitude is three xor-shuffles away.  One 4-byte store per thread; lane 0 of a block stores the scale.
 template<bool F16_IN>
-__global__ void __launch_bounds__(256) kv_write_kernel(uint8_t* pages, unsigned page_tokens, unsigned kv_heads, unsigned dim, unsigned row_bytes,
+__global__ void __launch_bounds__(256) kv_write_kernel(uint8_t* pages, size_t page_count, unsigned page_tokens, unsigned kv_heads, unsigned dim, unsigned row_bytes,
                                                        const int32_t* page_table, size_t table_stride, const int32_t* positions,
                                                        const void* keys, const void* values, size_t span, size_t total) {
     const size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x;   // one per 4 values of [K|V][seq][row][head][dim/4]
@@ -34,11 +34,16 @@ __global__ void __launch_bounds__(256) kv_write_kernel(uint8_t* pages, unsigned 
         const float4 raw = *reinterpret_cast<const float4*>(static_cast<const float*>(source) + first);
         x[0] = raw.x; x[1] = raw.y; x[2] = raw.z; x[3] = raw.w;
     }
-    const size_t position = size_t(positions[seq]) + row;
-    const size_t page = size_t(page_table[seq * table_stride + position / page_tokens]);
+    // The positions are device-resident (a replayed graph advances them there), so the host cannot check them: a row whose
+    // position is negative or past the sequence's table row, or whose table entry names no page of the pool, is not stored.
+    const long long first_position = positions[seq];
+    const size_t position = size_t(first_position < 0 ? 0 : first_position) + row;
+    bool stored = live && first_position >= 0 && position < table_stride * page_tokens;
+    const long long page = stored ? page_table[seq * table_stride + position / page_tokens] : 0;
+    stored = stored && page >= 0 && size_t(page) < page_count;
     const size_t plane = is_value ? kv_heads + head : head;
-    uint8_t* out = pages + ((page * 2 * kv_heads + plane) * page_tokens + position % page_tokens) * row_bytes;
-    kv_store_quad(out, unsigned(quad), dim, row_bytes != 2 * dim, x, live);
+    uint8_t* out = pages + ((size_t(stored ? page : 0) * 2 * kv_heads + plane) * page_tokens + position % page_tokens) * row_bytes;
+    kv_store_quad(out, unsigned(quad), dim, row_bytes != 2 * dim, x, stored);
 }
 
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {   // splitmix64 finaliser
@@ -153,10 +158,10 @@ int sdx_kv_write(void* handle, const sdx_kv_pool* pool, const int32_t* page_tabl
     const size_t total = checked_product({2, seqs, span, pool->kv_heads, pool->dim / 4});
     auto* pages = static_cast<uint8_t*>(pool->pages);
     if (input_f16)
-        kv_write_kernel<true><<<checked_blocks(total), 256, 0, value.stream>>>(pages, pool->page_tokens, pool->kv_heads, pool->dim, pool->row_bytes,
+        kv_write_kernel<true><<<checked_blocks(total), 256, 0, value.stream>>>(pages, size_t(pool->page_count), pool->page_tokens, pool->kv_heads, pool->dim, pool->row_bytes,
             page_table, size_t(table_stride), positions, keys, values, size_t(span), total);
     else
-        kv_write_kernel<false><<<checked_blocks(total), 256, 0, value.stream>>>(pages, pool->page_tokens, pool->kv_heads, pool->dim, pool->row_bytes,
+        kv_write_kernel<false><<<checked_blocks(total), 256, 0, value.stream>>>(pages, size_t(pool->page_count), pool->page_tokens, pool->kv_heads, pool->dim, pool->row_bytes,
             page_table, size_t(table_stride), positions, keys, values, size_t(span), total);
     SD_OP_END
 }

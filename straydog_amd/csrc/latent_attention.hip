@@ -164,12 +164,8 @@ __global__ void __launch_bounds__(THREADS) latent_attention_kernel(LatentArgs a)
 void launch(Device& d, const LatentArgs& args, size_t rows, size_t total_keys, bool bf16) {
     const size_t shared = (HB * (args.kdim + PAD) + HB * total_keys + HB) * 4;
     if (shared > 160 * 1024 - 256) throw std::runtime_error("invalid Straydog attention shape");
-    static bool raised = false;
-    if (!raised) {
-        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attention_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
-        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attention_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256));
-        raised = true;
-    }
+    raise_shared_limit(d, reinterpret_cast<const void*>(&latent_attention_kernel<true>), 160 * 1024 - 256);
+    raise_shared_limit(d, reinterpret_cast<const void*>(&latent_attention_kernel<false>), 160 * 1024 - 256);
     const dim3 grid(unsigned((args.heads + HB - 1) / HB), unsigned(rows));
     if (bf16) latent_attention_kernel<true><<<grid, THREADS, shared, d.stream>>>(args);
     else latent_attention_kernel<false><<<grid, THREADS, shared, d.stream>>>(args);

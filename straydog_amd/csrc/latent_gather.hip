@@ -240,11 +240,7 @@ void latent_gather(Device& d, const void* q, const void* latents, const int32_t*
     args.groups = unsigned(groups); args.k = unsigned(k); args.heads = unsigned(heads); args.chunks = unsigned((k + CHUNK - 1) / CHUNK);
     args.scale_log2 = scale * 1.44269504088896341f; args.partial = partial; args.out = out;
     constexpr size_t shared = size_t(STEP) * (2 * KDIM + 16) + size_t(VDIM) * (2 * STEP + 8) + STEP * 4 + CHUNK * 4;
-    static bool raised = false;
-    if (!raised) {
-        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_gather_kernel<KDIM, VDIM>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
-        raised = true;
-    }
+    raise_shared_limit(d, reinterpret_cast<const void*>(&latent_gather_kernel<KDIM, VDIM>), shared);
     timed_launch(d, &latent_gather_kernel<KDIM, VDIM>, dim3(args.chunks, unsigned((heads + 63) / 64), unsigned(batch)), dim3(256), shared, args);
     SD_CHECK(hipGetLastError());
     latent_merge_kernel<VDIM><<<unsigned(batch * heads), VDIM / 4, 0, d.stream>>>(args);

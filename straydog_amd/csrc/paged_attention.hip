@@ -66,7 +66,7 @@ __device__ __forceinline__ PagedArgs fresh_args() {
     args.pages = at->pages; args.page_tokens = at->page_tokens; args.kv_heads = at->kv_heads; args.heads = at->heads; args.group = at->group;
     args.span = at->span; args.page_table = at->page_table; args.table_stride = at->table_stride; args.positions = at->positions; args.q = at->q;
     args.q_f16 = at->q_f16; args.scale_log2 = at->scale_log2; args.partial = at->partial; args.rows = at->rows; args.seqs = at->seqs;
-    args.groups_max = at->groups_max; args.share_min = at->share_min; args.max_context = at->max_context;
+    args.groups_max = at->groups_max; args.share_min = at->share_min; args.max_context = at->max_context; args.page_last = at->page_last;
     return args;
 }
 struct Segment { int seq, kvh, position, total; unsigned unit, units, before; };
@@ -182,7 +182,7 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
     };
     // The step's two slabs copied into the stage, 1 KiB per instruction, lanes past a slab's end switched off.
     const auto copy_in = [&](uint8_t* stage, int page, int in_page) {
-        const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(in_page) * ROW + 16 * lane;
+        const uint8_t* base = args.pages + (size_t(pool_page(page, args.page_last)) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(in_page) * ROW + 16 * lane;
         #pragma unroll
         for (int part = 0; part < 2; ++part) {
             const uint8_t* from = base + size_t(part ? args.kv_heads : 0) * plane_bytes;
@@ -462,11 +462,7 @@ void launch(Device& d, const PagedArgs& args, dim3 grid) {
     constexpr int slab = STEP * (Q8 ? DIM + DIM / 16 : 2 * DIM);
     const size_t shared = std::max(size_t(2) * QT * (DIM / 16 * 4 + 2) * 64 * 4, size_t(WAVES) * stages_per_wave(slab, OCC) * 2 * slab);
     if (shared > 160 * 1024) throw std::runtime_error("Straydog paged attention: too many query rows per K/V head for the decode kernel");
-    static bool raised = false;
-    if (!raised && shared > 64 * 1024) {
-        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&paged_attention_kernel<DIM, QT, Q8, OCC>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
-        raised = true;
-    }
+    if (shared > 64 * 1024) raise_shared_limit(d, reinterpret_cast<const void*>(&paged_attention_kernel<DIM, QT, Q8, OCC>), shared);
     timed_launch(d, &paged_attention_kernel<DIM, QT, Q8, OCC>, grid, dim3(WAVES * 64), shared, args);
 }
 
@@ -531,6 +527,7 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
     args.q = q; args.q_f16 = q_f16; args.scale_log2 = scale * 1.44269504088896341f;
     args.rows = unsigned(rows); args.seqs = unsigned(seqs);
     args.max_context = int(max_context);
+    args.page_last = unsigned(std::min<uint64_t>(pool->page_count - 1, 0x7fffffffu));
     const uint64_t items = checked_product({seqs, pool->kv_heads});
     if (checked_product({items, (max_context + UNIT - 1) / UNIT}) > 0x7fffffffu) throw std::runtime_error("invalid Straydog paged attention shape");
     const unsigned slots = resident_slots(value, pool->dim, pool->row_bytes != 2 * pool->dim, query_tiles);

@@ -36,11 +36,16 @@ struct PagedArgs {
     unsigned rows, seqs;   // rows = span * group (query rows per K/V head)
     unsigned groups_max, share_min;   // the most workgroups that share the batch's tokens; the fewest 128-token units a share may have
     int max_context;       // positions[s] + span is clipped to this (the launch and the page table are sized for it)
+    unsigned page_last;    // the pool's last page: a table entry outside the pool is taken as the nearest page of it
 };
 
 // A sequence's first query position as the kernels use it: the positions live on the device, where the host cannot check
 // them, so one outside [0, max_context] is taken as the nearest end (and addresses nothing outside the page table).
 __device__ __forceinline__ int first_position(const int32_t* positions, unsigned seq, int max_context) { return min(max(positions[seq], 0), max_context); }
+
+// A page-table entry as the kernels use it: the table is device memory the host does not read, so an entry that names no page
+// of the pool (negative, or past the last page) addresses the pool's last page instead of memory outside it.
+__device__ __forceinline__ int pool_page(int entry, unsigned page_last) { return int(min(unsigned(entry), page_last)); }
 
 // The maximum / the sum over the four lanes li, li + 16, li + 32, li + 48 (one query row's four lane groups), in all four.
 // v_permlane16_swap exchanges the odd 16-lane rows of its first register with the even rows of its second, v_permlane32_swap

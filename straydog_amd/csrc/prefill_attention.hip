@@ -48,6 +48,7 @@ struct PrefillArgs {
     float scale_log2;      // softmax scale * log2(e): scores live in the base-2 domain
     unsigned rows;         // span * group: query rows per K/V head
     int max_context;       // positions[s] + span is clipped to this
+    unsigned page_last;    // the pool's last page (table entries outside the pool are taken as the nearest page of it)
     void* out;
     int out_f16;
 };
@@ -87,7 +88,7 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
                 const int unit = wave + TEAM * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS, at = 16 * lane + 1024 * j;
                 if (unit < 2 * UNITS && at < SLAB) {
                     const int token = min(token0 + at / ROW, cached - 1);
-                    const int page = args.page_table[size_t(seq) * args.table_stride + token / int(args.page_tokens)];
+                    const int page = pool_page(args.page_table[size_t(seq) * args.table_stride + token / int(args.page_tokens)], args.page_last);
                     const uint8_t* from = args.pages + (size_t(page) * 2 * args.kv_heads + (part ? args.kv_heads : 0) + kvh) * plane_bytes +
                                           size_t(token % int(args.page_tokens)) * ROW + at % ROW;
                     __builtin_amdgcn_global_load_lds((global_ptr)from, (lds_ptr)(stage + part * SLAB + 1024 * j), 16, 0, 0);
@@ -95,7 +96,7 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
             }
             return;
         }
-        const int page = table[token0 / int(args.page_tokens)];
+        const int page = pool_page(table[token0 / int(args.page_tokens)], args.page_last);
         const uint8_t* base = args.pages + (size_t(page) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(token0 % int(args.page_tokens)) * ROW + 16 * lane;
         #pragma unroll
         for (int k = 0; k < MOST; ++k) {
@@ -329,7 +330,7 @@ __global__ void __launch_bounds__(256) unpack_tiles_kernel(PrefillArgs args, uin
         const int word = min(t + 256 * j, ALL - 1);
         const int value = word / (TILE_KEYS * WORDS), key = word / WORDS % TILE_KEYS, at = word % WORDS;
         const int token = min(key0 + key, cached - 1);
-        const uint8_t* row = args.pages + (size_t(table[token / int(args.page_tokens)]) * 2 * args.kv_heads + (value ? args.kv_heads : 0) + kvh) * plane_bytes +
+        const uint8_t* row = args.pages + (size_t(pool_page(table[token / int(args.page_tokens)], args.page_last)) * 2 * args.kv_heads + (value ? args.kv_heads : 0) + kvh) * plane_bytes +
                              size_t(token % int(args.page_tokens)) * ROW;
         held[j] = *reinterpret_cast<const uint2*>(row + 8 * at);
     }
@@ -635,11 +636,7 @@ void launch_dense(Device& d, const PrefillArgs& args, unsigned seqs) {
     const unsigned tiles_per_seq = unsigned((args.max_context + TILE_KEYS - 1) / TILE_KEYS);
     auto* tiles = static_cast<uint8_t*>(workspace(d, checked_product({seqs, args.kv_heads, tiles_per_seq, uint64_t(tile_bytes<DIM>())})));
     constexpr int shared = 4 * tile_bytes<DIM>();
-    static bool raised = false;
-    if (!raised) {
-        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_dense_kernel<DIM, QT>), hipFuncAttributeMaxDynamicSharedMemorySize, shared));
-        raised = true;
-    }
+    raise_shared_limit(d, reinterpret_cast<const void*>(&prefill_dense_kernel<DIM, QT>), shared);
     unpack_tiles_kernel<DIM, Q8><<<dim3(tiles_per_seq, args.kv_heads, seqs), 256, 0, d.stream>>>(args, tiles, tiles_per_seq);
     const unsigned runs = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
     timed_launch(d, &prefill_dense_kernel<DIM, QT>, dim3((runs + 1) / 2, args.kv_heads, seqs), dim3(TEAM * 64), shared, args, tiles, tiles_per_seq);
@@ -651,11 +648,7 @@ void launch(Device& d, const PrefillArgs& args, unsigned seqs) {
     constexpr size_t stage = size_t(2) * WALK * (Q8 ? DIM + DIM / 16 : 2 * DIM), ring = stages_for(int(stage)) * stage;
     constexpr size_t shared = ring > merge ? ring : merge;
     static_assert(shared <= 160 * 1024, "the stages and the merge area share the compute unit's LDS");
-    static bool raised = false;
-    if (!raised && shared > 64 * 1024) {
-        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&prefill_attention_kernel<DIM, QT, Q8, OCC>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
-        raised = true;
-    }
+    if (shared > 64 * 1024) raise_shared_limit(d, reinterpret_cast<const void*>(&prefill_attention_kernel<DIM, QT, Q8, OCC>), shared);
     const unsigned tiles = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
     timed_launch(d, &prefill_attention_kernel<DIM, QT, Q8, OCC>, dim3(tiles, args.kv_heads, seqs), dim3(TEAM * 64), shared, args);
 }
@@ -676,6 +669,7 @@ void prefill_attention(Device& d, const sdx_kv_pool* pool, const int32_t* page_t
     args.page_table = page_table; args.table_stride = size_t(table_stride); args.positions = positions;
     args.q = q; args.q_f16 = q_f16; args.scale_log2 = scale * 1.44269504088896341f;
     args.rows = unsigned(span * args.group); args.max_context = int(max_context);
+    args.page_last = unsigned(std::min<uint64_t>(pool->page_count - 1, 0x7fffffffu));
     args.out = out; args.out_f16 = out_f16;
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     if (pool->dim == 128) { if (q8) launch_dense<128, 2, true>(d, args, unsigned(seqs)); else launch_dense<128, 2, false>(d, args, unsigned(seqs)); }

@@ -28,6 +28,7 @@ struct SelectedArgs {
     const uint8_t* pages;
     unsigned page_tokens, kv_heads, heads, group;
     const int32_t* page_table;     // null: one page holds the context
+    unsigned page_last;            // the pool's last page (table entries outside the pool are taken as the nearest page of it)
     size_t context, base;
     const uint32_t* dynamic_base;
     const float* indices;
@@ -87,7 +88,7 @@ __global__ void __launch_bounds__(WAVES * 64) selected_attention_kernel(Selected
         const bool counts_in = raw >= 0.0f && raw <= float(position) && raw < float(a.context);
         const uint64_t usable = __ballot(counts_in);
         const size_t token = counts_in ? size_t(raw) : min(position, a.context - 1);
-        const size_t page = a.page_table ? size_t(a.page_table[token / a.page_tokens]) : 0, in_page = a.page_table ? token % a.page_tokens : token;
+        const size_t page = a.page_table ? size_t(pool_page(a.page_table[token / a.page_tokens], a.page_last)) : 0, in_page = a.page_table ? token % a.page_tokens : token;
         const size_t plane_bytes = size_t(a.page_tokens) * ROW;
         const uint8_t* const krow = a.pages + (page * 2 * a.kv_heads + kvh) * plane_bytes + in_page * ROW;
         settle_loads();
@@ -216,11 +217,7 @@ template<bool Q8>
 void launch(Device& d, const SelectedArgs& args, size_t rows) {
     constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM;
     const size_t shared = std::max<size_t>(size_t(WAVES) * 2 * STEP * ROW, size_t(WAVES) * 16 * (DIM + 2) * 4);
-    static bool raised = false;
-    if (!raised) {
-        SD_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&selected_attention_kernel<Q8>), hipFuncAttributeMaxDynamicSharedMemorySize, int(shared)));
-        raised = true;
-    }
+    raise_shared_limit(d, reinterpret_cast<const void*>(&selected_attention_kernel<Q8>), shared);
     timed_launch(d, &selected_attention_kernel<Q8>, dim3(args.chunks, args.kv_heads, unsigned(rows)), dim3(WAVES * 64), shared, args);
 }
 
@@ -262,7 +259,7 @@ int sdx_selected_attention(void* handle, const sdx_kv_pool* pool, const int32_t*
     SelectedArgs args{};
     args.pages = static_cast<const uint8_t*>(pool->pages);
     args.page_tokens = pool->page_tokens; args.kv_heads = pool->kv_heads; args.heads = unsigned(heads); args.group = unsigned(heads / pool->kv_heads);
-    args.page_table = page_table; args.context = context; args.base = base; args.dynamic_base = dynamic_base;
+    args.page_table = page_table; args.page_last = unsigned(std::min<uint64_t>(pool->page_count - 1, 0x7fffffffu)); args.context = context; args.base = base; args.dynamic_base = dynamic_base;
     args.indices = indices; args.selected = selected; args.counts = counts; args.q = q; args.q_f16 = q_f16;
     args.scale_log2 = scale * 1.4426950408889634f;
     args.partial = static_cast<float*>(scratch);

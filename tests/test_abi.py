@@ -45,8 +45,57 @@ def test_failures_are_codes_with_text(library):
     library.sd_destroy(None)   # a no-op
 
 
-def test_static_archive_is_built():
-    assert os.path.exists(os.path.join(ROOT, "straydog_amd", "libstraydog_gpu.a"))
+def _golden_symbols():
+    """name -> (kind of result, 'real' | 'stub') for every function the reference's gpu/straydog_gpu.h declares."""
+    table = {}
+    for line in open(os.path.join(ROOT, "tests", "golden", "abi_symbols.txt")):
+        if line.strip() and not line.startswith("#"):
+            name, kind, state = line.split()
+            table[name] = (kind, state)
+    return table
+
+
+def _defined(path):
+    import subprocess
+    listing = subprocess.run(["nm", "--defined-only", "-g", path], check=True, capture_output=True, text=True).stdout
+    return {parts[-1] for parts in (line.split() for line in listing.splitlines()) if len(parts) >= 3 and parts[-2] == "T" and parts[-1].startswith("sd_")}
+
+
+@pytest.mark.parametrize("artifact", ["libstraydog_gpu.a", "libstraydog_gpu.so"])
+def test_library_defines_the_whole_reference_abi(library, artifact):
+    # the reference's host links the static archive and binds every declared function (crates/straydog-gpu/build.rs:52):
+    # the archive must define each of the 321, no more and no fewer
+    golden = _golden_symbols()
+    assert len(golden) == 321
+    assert _defined(os.path.join(ROOT, "straydog_amd", artifact)) == set(golden)
+    assert {name for name, (_, state) in golden.items() if state == "real"} == set(_declared("straydog_gpu.h"))
+
+
+def test_symbol_list_matches_the_reference_header():
+    header = "/root/reference/gpu/straydog_gpu.h"
+    if not os.path.exists(header):
+        pytest.skip("no reference checkout on this machine; tests/golden/abi_symbols.txt was generated from it")
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("gen_stubs", os.path.join(ROOT, "straydog_amd", "csrc", "gen_stubs.py"))
+    module = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(module)
+    golden = _golden_symbols()
+    assert [(name, kind) for name, kind in module.declarations(header)] == [(name, kind) for name, (kind, _) in golden.items()]
+
+
+def test_stubs_fail_cleanly(library):
+    golden = _golden_symbols()
+    results = {"INT": (ctypes.c_int, -1), "PTR": (ctypes.c_void_p, None), "U64": (ctypes.c_uint64, 0), "I64": (ctypes.c_int64, -1),
+               "U32": (ctypes.c_uint32, 0), "VOID": (None, None)}
+    stubs = [(name, kind) for name, (kind, state) in golden.items() if state == "stub"]
+    assert len(stubs) > 250
+    for name, kind in stubs:
+        function = getattr(library, name)
+        function.restype, expected = results[kind]
+        function.argtypes = None
+        # arguments are ignored (the caller owns them in the C calling convention): pass a few, as a bound caller would
+        assert function(None, None, ctypes.c_uint64(3), None) == expected, name
+        assert library.sd_error().decode() == f"{name} is not implemented in the attention library"
 
 
 def test_backend_refuses_a_missing_library(tmp_path):

@@ -151,3 +151,48 @@ def test_qwen_decode_stage_recorded(gpu, oracle):
             a, b = _read(gpu, recorded[what], dtype, count), _read(gpu, eager[what], dtype, count)
             assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), f"replay {turn}: {what}"
         assert np.abs(_read(gpu, recorded["attended"], np.float32, heads * 256)).max() > 0
+
+
+def test_graphs_are_dropped_when_the_workspace_moves(gpu, oracle):
+    # ops that use the handle's workspace bake its address into a recorded graph; when a later, larger call makes the workspace
+    # grow (and move), the kept graphs are dropped: sd_graph_run answers "none stored" and the caller records again, instead of
+    # replaying on freed memory.  Growth while recording is refused.
+    from straydog_amd.backend import StraydogError
+    rng = np.random.default_rng(8)
+
+    def latent_case(batch, groups, k, heads=64):
+        q = rng.standard_normal((batch, heads, 576)).astype(np.float32)
+        latents = rng.standard_normal((batch, groups, 576)).astype(np.float32)
+        selected = np.stack([np.sort(rng.choice(groups, size=k, replace=False)) for _ in range(batch)]).astype(np.int32)
+        bf = lambda a: (a.view(np.uint32) >> 16).astype(np.uint16)     # truncation is fine here: both sides see the same bits
+        qb, lb, sb = gpu.upload(bf(q)), gpu.upload(bf(latents)), gpu.upload(selected)
+        out = gpu.buffer(batch * heads * 512 * 4)
+        def run():
+            gpu.latent_attention(qb.base(), lb.base(), sb.base(), batch, groups, k, heads, 576, 512, 1.0 / 24.0, out.base())
+        return run, out, (qb, lb, sb, out)
+
+    small, small_out, small_buffers = latent_case(1, 512, 128)
+    small()                                              # sizes the workspace for this shape
+    eager = _read(gpu, small_out, np.float32, 64 * 512).copy()
+    gpu.graph_begin()
+    small()
+    gpu.graph_end(21)
+    gpu.write_buffer(small_out, 0, np.zeros(64 * 512, np.float32))
+    assert gpu.graph_run(21)
+    assert np.array_equal(_read(gpu, small_out, np.float32, 64 * 512), eager)
+    large, large_out, large_buffers = latent_case(4, 4096, 2048)
+    gpu.graph_begin()
+    with pytest.raises(StraydogError, match="cannot grow while a graph is recorded"):
+        large()
+    gpu.graph_end(22, keep=False)
+    assert gpu.graph_run(21), "a refused growth leaves the kept graphs alone"
+    large()                                              # eager: the workspace grows and moves
+    assert not gpu.graph_run(21), "the graph that held the old workspace address is gone"
+    gpu.graph_begin()
+    small()
+    gpu.graph_end(21)
+    gpu.write_buffer(small_out, 0, np.zeros(64 * 512, np.float32))
+    assert gpu.graph_run(21)
+    assert np.array_equal(_read(gpu, small_out, np.float32, 64 * 512), eager)
+    for b in small_buffers + large_buffers:
+        gpu.release(b)

@@ -382,3 +382,127 @@ def test_the_library_kept_cache_pages_grow_fork_and_truncate(gpu, oracle):
     with pytest.raises(StraydogError):
         gpu.kv_cache(0, 64, 2, 128, 136, 1, 64)
     assert gpu.memory()[0] == used, "a refused cache leaves no allocation behind"
+
+
+def test_a_rewind_into_a_shared_page_continues_on_a_copy(gpu, oracle):
+    # a fork at a page boundary shares whole pages; when either sequence rewinds to a position inside a shared page and
+    # appends, its new rows must not overwrite the rows the sibling still attends to
+    from straydog_amd.backend import StraydogError
+    rng = np.random.default_rng(45)
+    page_tokens, kv_heads, dim, row_bytes, heads = 64, 2, 128, 136, 8
+    cache, pool, table, stride = gpu.kv_cache(12, page_tokens, kv_heads, dim, row_bytes, 2, 512)
+    logical = {}
+
+    def append(sequence, count):
+        k = rng.standard_normal((count, kv_heads, dim)).astype(np.float32)
+        v = rng.standard_normal((count, kv_heads, dim)).astype(np.float32)
+        have = logical.get(sequence, (np.zeros((0, kv_heads, dim), np.float32),) * 2)
+        start = have[0].shape[0]
+        gpu.kv_cache_reserve(cache, sequence, start + count)
+        kb, vb, pb = gpu.upload(k), gpu.upload(v), gpu.upload(np.array([start], dtype=np.int32))
+        gpu.kv_write(pool, table + sequence * stride * 4, stride, pb.base(), kb.base(), vb.base(), False, 1, count)
+        for b in (kb, vb, pb):
+            gpu.release(b)
+        logical[sequence] = (np.concatenate([have[0], k]), np.concatenate([have[1], v]))
+
+    def check(sequence):
+        k, v = logical[sequence]
+        length = k.shape[0]
+        q = rng.standard_normal((1, 1, heads, dim)).astype(np.float32)
+        qb, pb = gpu.upload(q), gpu.upload(np.array([length - 1], dtype=np.int32))
+        out = gpu.buffer(q.size * 4)
+        scratch = gpu.buffer(gpu.paged_attention_scratch(1, 1, heads, dim, 512))
+        gpu.paged_attention(pool, table + sequence * stride * 4, stride, pb.base(), 512, qb.base(), False, 1, 1, heads, 0.09, out.base(), False, scratch)
+        got = gpu.read_buffer(out, 0, np.float32, q.size).reshape(q.shape)
+        pages = (length + page_tokens - 1) // page_tokens
+        host = np.zeros(oracle.pool_bytes(pages, kv_heads, page_tokens, row_bytes), dtype=np.uint8)
+        own = np.arange(pages, dtype=np.int32)[None, :]
+        oracle.kv_write(host, row_bytes, page_tokens, kv_heads, dim, own, np.zeros(1, np.int32), k[None], v[None])
+        want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, own, np.array([length - 1], np.int32), q, 0.09)
+        close_enough(got, want, f"sequence {sequence} of {length} tokens")
+        for b in (qb, pb, out, scratch):
+            gpu.release(b)
+
+    append(0, 128)                                   # two whole pages
+    gpu.kv_cache_fork(cache, 0, 1, 128)              # both shared, nothing copied
+    logical[1] = (logical[0][0].copy(), logical[0][1].copy())
+    assert gpu.kv_cache_usage(cache, 1) == (2, 10)
+    gpu.kv_cache_truncate(cache, 1, 100)             # into the shared second page: the fork takes a copy of its rows 64..99
+    logical[1] = (logical[1][0][:100], logical[1][1][:100])
+    assert gpu.kv_cache_usage(cache, 1) == (2, 9)
+    append(1, 20)                                    # rows 100..119 of the fork
+    check(1); check(0)                               # the source still reads its own rows 100..127
+    gpu.kv_cache_truncate(cache, 0, 70)              # the source rewinds below the fork point: its second page is its own by now
+    logical[0] = (logical[0][0][:70], logical[0][1][:70])
+    append(0, 10)
+    check(0); check(1)
+    gpu.kv_cache_truncate(cache, 0, 30)              # into the first page, which the fork still shares
+    logical[0] = (logical[0][0][:30], logical[0][1][:30])
+    append(0, 3)
+    check(0); check(1)
+    # with no page free for the copy the rewind is refused and changes nothing
+    append(1, 512 - 120)
+    assert gpu.kv_cache_usage(cache, 1) == (8, 3)
+    gpu.kv_cache_truncate(cache, 0, 0)
+    assert gpu.kv_cache_usage(cache, 0) == (0, 4)
+    gpu.kv_cache_fork(cache, 1, 0, 64)               # the first page shared again
+    gpu.kv_cache_reserve(cache, 0, 320)              # takes the four free pages
+    with pytest.raises(StraydogError, match="out of pages"):
+        gpu.kv_cache_truncate(cache, 1, 10)          # page 0 is shared with sequence 0 and no page is left for a copy
+    assert gpu.kv_cache_usage(cache, 1)[0] == 8
+    check(1)
+    gpu.kv_cache_destroy(cache)
+
+
+def test_rows_at_positions_outside_the_table_are_not_written(gpu, oracle):
+    # K/V positions are read on the device: a negative one, one past the sequence's table row, or a table entry that names no
+    # page of the pool stores nothing, and the rows of the sequences beside it keep their bytes
+    rng = np.random.default_rng(616)
+    dim, row_bytes, page_tokens, kv_heads, seqs, span = 128, 136, 32, 2, 5, 3
+    stride, pages = 2, 12
+    table = np.arange(seqs * stride, dtype=np.int32).reshape(seqs, stride)
+    table[4, 1] = 4000                               # names no page
+    pool, buffer = gpu.kv_pool(pages, page_tokens, kv_heads, dim, row_bytes)
+    before = rng.integers(0, 255, size=buffer.size, dtype=np.uint8)
+    gpu.write_buffer(buffer, 0, before)
+    positions = np.array([-2, 62, 10, 2_000_000_000, 31], dtype=np.int32)
+    keys = rng.standard_normal((seqs, span, kv_heads, dim)).astype(np.float32)
+    values = rng.standard_normal((seqs, span, kv_heads, dim)).astype(np.float32)
+    tb, pb, kb, vb = gpu.upload(table), gpu.upload(positions), gpu.upload(keys), gpu.upload(values)
+    gpu.kv_write(pool, tb.base(), stride, pb.base(), kb.base(), vb.base(), False, seqs, span)
+    got = gpu.read_buffer(buffer, 0, np.uint8, buffer.size)
+    want = before.copy()
+    # what should have been stored: sequence 1 rows at 62, 63 (64 is past its table row), sequence 2 rows at 10..12, sequence 4
+    # row at 31 (32 and 33 fall into the page that does not exist); sequences 0 and 3 nothing
+    for s, rows in ((1, [0, 1]), (2, [0, 1, 2]), (4, [0])):
+        for r in rows:
+            one = np.array([[int(positions[s]) + r]], dtype=np.int32).reshape(1)
+            oracle.kv_write(want, row_bytes, page_tokens, kv_heads, dim, table[s:s + 1], one, keys[s:s + 1, r:r + 1], values[s:s + 1, r:r + 1])
+    assert np.array_equal(got, want)
+    for b in (tb, pb, kb, vb, buffer):
+        gpu.release(b)
+
+
+def test_table_entries_outside_the_pool_read_inside_it(gpu, oracle):
+    # a page-table entry that names no page of the pool is read as the pool's last page (never memory outside the pool); the
+    # sequences beside it are not disturbed
+    rng = np.random.default_rng(717)
+    dim, row_bytes, page_tokens, heads, kv_heads = 128, 136, 64, 8, 2
+    lengths = [200, 200, 200]
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, lengths, kv_heads, dim, page_tokens, row_bytes, spare_pages=0)
+    last = int(pool.page_count) - 1
+    bad = table.copy()
+    bad[1, 2] = -5
+    bad[1, 3] = 1 << 30
+    meant = table.copy()
+    meant[1, 2] = last
+    meant[1, 3] = last
+    bb = gpu.upload(bad)
+    q = rng.standard_normal((3, 1, heads, dim)).astype(np.float16).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    got = _run(gpu, pool, bad, bb, [199, 199, 199], q, 1, heads, scale, True, False)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, meant, np.array([199, 199, 199], np.int32), q, scale)
+    for s in range(3):
+        close_enough(got[s], want[s], f"sequence {s}")
+    for b in (buffer, tb, bb):
+        gpu.release(b)
