@@ -73,6 +73,19 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
                         const int32_t* positions, uint64_t max_context, const void* q, int q_f16, uint64_t seqs, uint64_t span,
                         uint64_t heads, float scale, void* out, int out_f16, void* scratch, uint64_t scratch_bytes);
 
+/* The same attention for callers that cannot allocate device memory or pass a scratch buffer: code under graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The split partial results live in
+ * an area of sdx_paged_attention_static_bytes() bytes (16 MiB) that the library itself holds on every GPU it runs on until the
+ * process ends; a batch that would need more (sdx_paged_attention_scratch says how much a shape can need at most; the call
+ * computes the exact figure) and spans with more query rows per K/V head than the decode kernel takes (64 at 128 columns, 32 at
+ * 256) are refused with an error.  The call allocates nothing.  All calls on one GPU share that area: calls that overlap in
+ * time on one GPU (two handles, two streams) race; calls queued on one handle's stream do not.  Same results, bit for bit, as
+ * sdx_paged_attention. */
+uint64_t sdx_paged_attention_static_bytes(void);
+int sdx_paged_attention_static(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride,
+                               const int32_t* positions, uint64_t max_context, const void* q, int q_f16, uint64_t seqs, uint64_t span,
+                               uint64_t heads, float scale, void* out, int out_f16);
+
 /* Qwen's block indexer (the reference runs it inside sd_qsa_sequence / sd_decode_span / sd_prefill_span; here its stages are
  * callable on their own).  All buffers are device memory of the handle.
  *

@@ -91,6 +91,9 @@ SIGNATURES = {
     "sdx_paged_attention_scratch": (c_u64, [c_u64, c_u64, c_u64, c_u64, c_u64]),
     "sdx_paged_attention": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_u64, c_void_p, c_int, c_u64, c_u64, c_u64,
                                     c_float, c_void_p, c_int, c_void_p, c_u64]),
+    "sdx_paged_attention_static_bytes": (c_u64, []),
+    "sdx_paged_attention_static": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_u64, c_void_p, c_int, c_u64, c_u64, c_u64,
+                                           c_float, c_void_p, c_int]),
     "sdx_qsa_normalize": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_u64, c_void_p]),
     "sdx_qsa_pool": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_void_p]),
     "sdx_qsa_index": (c_int, [c_void_p, c_void_p, c_u64, c_void_p, c_u64, c_u64, c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_void_p]),

@@ -221,6 +221,12 @@ class Backend:
                                                 q, int(q_f16), seqs, span, heads, scale, out, int(out_f16), scratch.pointer,
                                                 scratch.size))
 
+    def paged_attention_static(self, pool, page_table, table_stride, positions, max_context, q, q_f16, seqs, span, heads, scale, out,
+                               out_f16):
+        """sdx_paged_attention with the partial results in the library's own area: the call allocates nothing."""
+        self.check(self.lib.sdx_paged_attention_static(self.handle, ctypes.byref(pool), page_table, table_stride, positions, max_context,
+                                                       q, int(q_f16), seqs, span, heads, scale, out, int(out_f16)))
+
     def selected_attention_scratch(self, rows, kv_heads, selected):
         return int(self.lib.sdx_selected_attention_scratch(rows, kv_heads, selected))
 

@@ -11,6 +11,7 @@
 namespace sd {
 
 thread_local std::string last_error;
+void paged_attention_setup(Device& d);   // paged_attention.hip
 void select_thin_reserve(Device& d);     // block_index.hip
 
 // Recorded graphs hold the addresses their ops were given.  When a buffer the library owns moves (the workspace grows), the
@@ -180,6 +181,7 @@ void* sd_create(int ordinal, uint64_t budget) {
         SD_CHECK(hipHostMalloc(reinterpret_cast<void**>(&d->arena), io_arena_bytes, hipHostMallocDefault));
         d->events.resize(2);
         for (auto& event : d->events) { SD_CHECK(hipEventCreateWithFlags(&event, hipEventDisableTiming)); SD_CHECK(hipEventRecord(event, d->stream)); }
+        paged_attention_setup(*d);
         return d;
     } catch (const std::exception& e) {
         last_error = e.what();

@@ -61,6 +61,8 @@ struct Device {
     // Dynamic LDS limits raised so far, by kernel: the attribute belongs to this device's copy of the kernel, so each
     // handle raises it for itself (raise_shared_limit).
     std::map<const void*, size_t> shared_limits;
+    // This device's address of the partial-result area the library itself holds for sdx_paged_attention_static.
+    float* paged_static = nullptr;
     // The lists of a short span's thinned index rows (block_index.hip), allocated at the first such call and kept.
     void* select_thin = nullptr;
     // Page-locked host copies of sequence state (conversation checkpoints): pointer -> bytes.

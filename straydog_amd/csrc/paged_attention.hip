@@ -490,20 +490,17 @@ unsigned resident_slots(const Device& d, unsigned dim, bool q8, unsigned query_t
     return d.compute_units * unsigned(std::max<size_t>(1, std::min<size_t>(size_t(occupancy), (160 * 1024) / shared)));
 }
 
-}  // namespace
 
-extern "C" {
+// The partial results of the entry point that allocates nothing: device memory of the library itself, one copy per GPU,
+// held until the process ends.
+constexpr size_t static_scratch_bytes = size_t(16) << 20;
+static __device__ __align__(256) float scratch[static_scratch_bytes / 4];
 
-uint64_t sdx_paged_attention_scratch(uint64_t seqs, uint64_t span, uint64_t heads, uint64_t dim, uint64_t max_context) {
-    // a partial result per workgroup and one more per (sequence, K/V head); at most a workgroup per 256 tokens of a sequence
-    const uint64_t shares = (max_context + smallest_share * UNIT - 1) / (smallest_share * UNIT);
-    return seqs * span * heads * (shares + 1) * (dim + 2) * 4;
-}
-
-int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride,
-                        const int32_t* positions, uint64_t max_context, const void* q, int q_f16, uint64_t seqs, uint64_t span,
-                        uint64_t heads, float scale, void* out, int out_f16, void* scratch, uint64_t scratch_bytes) {
-    SD_OP_BEGIN
+// What both entry points do once their partial-result area is known.  `timed`: the main kernel may go through the extended
+// launch when the handle is being profiled (that creates events, which the entry point that allocates nothing must not).
+void paged_attention(Device& value, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
+                     uint64_t max_context, const void* q, int q_f16, uint64_t seqs, uint64_t span, uint64_t heads, float scale, void* out,
+                     int out_f16, float* partial, uint64_t partial_bytes, bool own_partial) {
     validate_pool(value, pool);
     if (!(scale > 0.0f) || !seqs || seqs > 65535 || !span || !heads || heads % pool->kv_heads || !max_context || max_context > (uint64_t(1) << 30) ||
         !table_stride || max_context > table_stride * pool->page_tokens)
@@ -515,10 +512,11 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
     op_span(value, q, checked_product({seqs, span, heads, pool->dim, q_f16 ? 2u : 4u}), "attention queries");
     op_span(value, out, checked_product({seqs, span, heads, pool->dim, out_f16 ? 2u : 4u}), "an attention output");
     if (query_tiles > (pool->dim == 128 ? 4u : 2u)) {
+        if (own_partial) throw std::runtime_error("Straydog paged attention: too many query rows per K/V head for the entry point that allocates nothing");
         // many rows per K/V head (a prefill chunk): every workgroup walks the keys once for a run of rows, nothing to merge
         prefill_attention(value, pool, page_table, table_stride, positions, max_context, q, q_f16, seqs, span, heads, scale, out, out_f16);
         SD_CHECK(hipGetLastError());
-        return 0;
+        return;
     }
     PagedArgs args{};
     args.pages = static_cast<const uint8_t*>(pool->pages);
@@ -534,9 +532,18 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
     args.groups_max = unsigned(std::min<uint64_t>(tuned_groups() ? tuned_groups() : slots, most_groups(seqs, pool->kv_heads, max_context)));
     args.share_min = smallest_share;
     const size_t need = checked_floats({uint64_t(args.groups_max) + items, rows, uint64_t(pool->dim) + 2});
-    if (!scratch || scratch_bytes < need) throw std::runtime_error("Straydog paged attention scratch too small");
-    op_span(value, scratch, need, "attention scratch");
-    args.partial = static_cast<float*>(scratch);
+    if (own_partial) {
+        if (need > partial_bytes)
+            throw std::runtime_error("Straydog paged attention: this batch needs " + std::to_string(need) + " bytes of partial results, the entry point that allocates nothing holds " +
+                                     std::to_string(partial_bytes));
+    } else {
+        if (!partial || partial_bytes < need) throw std::runtime_error("Straydog paged attention scratch too small");
+        op_span(value, partial, need, "attention scratch");
+    }
+    args.partial = partial;
+    const bool profiled = value.profile;
+    if (own_partial) value.profile = false;
+    struct Restore { Device& d; bool profile; ~Restore() { d.profile = profile; } } restore{value, profiled};
     const dim3 grid(args.groups_max);
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     if (pool->dim == 128) { if (q8) launch_tiles<128, true>(value, args, query_tiles, grid); else launch_tiles<128, false>(value, args, query_tiles, grid); }
@@ -550,6 +557,47 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
         if (out_f16) paged_merge_kernel<256, true><<<outputs, 256, 0, value.stream>>>(args, out);
         else paged_merge_kernel<256, false><<<outputs, 256, 0, value.stream>>>(args, out);
     }
+}
+
+
+}  // namespace
+
+namespace sd {
+// Called by sd_create with the handle's device current: the address this device holds the library's partial-result area at
+// (each GPU has its own copy of the array at its own address; the array's name is not a device address in host code).
+void paged_attention_setup(Device& d) {
+    float* address = nullptr;
+    SD_CHECK(hipGetSymbolAddress(reinterpret_cast<void**>(&address), HIP_SYMBOL(scratch)));
+    d.paged_static = address;
+}
+}  // namespace sd
+
+extern "C" {
+
+uint64_t sdx_paged_attention_scratch(uint64_t seqs, uint64_t span, uint64_t heads, uint64_t dim, uint64_t max_context) {
+    // a partial result per workgroup and one more per (sequence, K/V head); at most a workgroup per 256 tokens of a sequence
+    const uint64_t shares = (max_context + smallest_share * UNIT - 1) / (smallest_share * UNIT);
+    return seqs * span * heads * (shares + 1) * (dim + 2) * 4;
+}
+
+int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride,
+                        const int32_t* positions, uint64_t max_context, const void* q, int q_f16, uint64_t seqs, uint64_t span,
+                        uint64_t heads, float scale, void* out, int out_f16, void* scratch, uint64_t scratch_bytes) {
+    SD_OP_BEGIN
+    paged_attention(value, pool, page_table, table_stride, positions, max_context, q, q_f16, seqs, span, heads, scale, out, out_f16,
+                    static_cast<float*>(scratch), scratch_bytes, false);
+    SD_OP_END
+}
+
+uint64_t sdx_paged_attention_static_bytes(void) { return static_scratch_bytes; }
+
+int sdx_paged_attention_static(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride,
+                               const int32_t* positions, uint64_t max_context, const void* q, int q_f16, uint64_t seqs, uint64_t span,
+                               uint64_t heads, float scale, void* out, int out_f16) {
+    SD_OP_BEGIN
+    if (!value.paged_static) throw std::runtime_error("Straydog paged attention: the library's own partial-result area was not found on this device");
+    paged_attention(value, pool, page_table, table_stride, positions, max_context, q, q_f16, seqs, span, heads, scale, out, out_f16,
+                    value.paged_static, static_scratch_bytes, true);
     SD_OP_END
 }
 
