@@ -142,6 +142,14 @@ int sd_op_index_select(void* handle, const float* q, const float* keys, const fl
                        uint64_t groups, uint64_t heads, uint64_t dim, float scale, uint64_t rope_dims, const int32_t* positions,
                        const float* frequencies, float* scores, uint64_t k, int32_t* out, const int32_t* candidates, uint64_t blocks,
                        uint64_t block);
+/* reference straydog_gpu.h:422 (gpu/kernels.cpp:5620-5667, gpu/ops.hpp:2267-2300): sd_op_index_select of one decode row with the
+ * projection of x into the heads' weights ahead of it: weights[h] = row h of the heads x proj_cols matrix proj_weights . x, the
+ * rows BF16 (proj_kind 30) or ggml Q8_0 blocks (proj_kind 8); other kinds are refused.  `weights` receives them.  The same
+ * weights, scores and indices, bit for bit, as sdx_index_projection (straydog_gpu_ext.h) followed by sd_op_index_select. */
+int sd_op_index_select_proj(void* handle, const void* proj_weights, int proj_kind, uint64_t proj_cols, const float* x, const float* q,
+                            const float* keys, float* weights, const int32_t* visible, uint64_t groups, uint64_t heads, uint64_t dim, float scale,
+                            uint64_t rope_dims, const int32_t* positions, const float* frequencies, float* scores, uint64_t k, int32_t* out,
+                            const int32_t* candidates, uint64_t blocks, uint64_t block);
 /* ---- The inputs of a dense attention step (its neighbours in a span) ---- */
 /* reference straydog_gpu.h:446 (gpu/token_mixing.hpp:246-252, :628-637): rows of [first | second], `width` each, apart. */
 int sd_op_split(void* handle, const float* x, uint64_t rows, uint64_t width, float* first, float* second);

@@ -159,6 +159,13 @@ int sdx_selected_attention(void* handle, const sdx_kv_pool* pool, const int32_t*
  * ties to the lowest index, -1 padding: bit-exact. */
 int sdx_index_top_k(void* handle, const void* q_index, const void* keys, const float* weights, const int32_t* visible, uint64_t batch,
                     uint64_t groups, uint64_t heads, uint64_t dim, float scale, float* scores, uint64_t k, int32_t* indices);
+/* The projection inside sd_op_index_select_proj on its own (the reference forms it with sd_op_linear, its GEMV stack, whose
+ * summation order follows a per-device lane count: gpu/gemv_common.hpp:785-812): weights[h] = row h of proj_weights . x for
+ * heads <= 64 rows of proj_cols <= 8192 columns, BF16 (kind 30, 16-byte aligned rows, cols a multiple of 8) or ggml Q8_0 (kind 8,
+ * cols a multiple of 32).  The order of the sums is fixed: a unit (8 BF16 columns or a Q8_0 block) is one chain of fused
+ * multiply-adds over its columns from zero (Q8_0: over float(q) * x, then times the block's scale); unit u belongs to lane
+ * u % 64, which adds its units in order; the 64 lane sums are added pairwise at distances 32, 16, 8, 4, 2, 1. */
+int sdx_index_projection(void* handle, const void* proj_weights, int proj_kind, uint64_t proj_cols, const float* x, uint64_t heads, float* weights);
 /* The bracket the matrix cores put around every canonical score of stage 1 (dim 128, heads a multiple of 16 up to 64):
  * lower[b][g] <= score <= upper[b][g], -inf for groups that are not visible.  sdx_index_top_k without a scores buffer
  * scores canonically only the groups whose upper bound reaches the k-th highest lower bound (the approach of the

@@ -66,6 +66,7 @@ _op_att = _sig("sdo_op_attention", None, _vp, _vp, _vp, _sz, _vp, _sz, _sz, _sz,
 _op_att64 = _sig("sdo_op_attention_f64", None, _vp, _vp, _vp, _sz, _vp, _sz, _sz, _sz, _sz, ctypes.c_float, _vp, _vp, _vp)
 _idx = _sig("sdo_index_scores", None, _vp, _vp, ctypes.c_int, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_float, _vp, ctypes.c_int)
 _idx64 = _sig("sdo_index_scores_f64", None, _vp, _vp, ctypes.c_int, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_float, _vp)
+_idx_proj = _sig("sdo_index_projection", None, _vp, ctypes.c_int, _sz, _vp, _sz, _vp)
 _topk_key = _sig("sdo_top_k_key", ctypes.c_uint32, ctypes.c_float)
 _topk = _sig("sdo_top_k", None, _vp, _sz, _sz, _sz, _vp)
 _cand = _sig("sdo_index_candidates", None, _vp, _vp, _sz, _sz, _sz, _sz, _vp)
@@ -231,6 +232,14 @@ def index_scores_f64(q, keys, weights, visible, scale):
     groups = keys.shape[0]
     out = np.zeros((rows, groups), dtype=np.float64)
     _idx64(_ptr(q), _ptr(keys), bf16, _ptr(weights), _ptr(visible), rows, groups, heads, dim, ctypes.c_float(scale), _ptr(out))
+    return out
+
+
+def index_projection(matrix, kind, cols, x, heads):
+    """matrix: uint8 bytes of heads rows, BF16 (kind 30) or ggml Q8_0 blocks (kind 8); x [cols] fp32."""
+    matrix, x = np.ascontiguousarray(matrix, dtype=np.uint8), _f32(x)
+    out = np.zeros(heads, dtype=np.float32)
+    _idx_proj(_ptr(matrix), kind, cols, _ptr(x), heads, _ptr(out))
     return out
 
 

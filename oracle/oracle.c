@@ -425,6 +425,36 @@ void sdo_index_scores(const float* q, const void* keys, int keys_bf16, const flo
     }
 }
 
+/* The indexer's projection in the library's stated order for 64 lanes (see oracle.h). */
+void sdo_index_projection(const uint8_t* matrix, int kind, size_t cols, const float* x, size_t heads, float* weights) {
+    const size_t unit = kind == 30 ? 8 : 32, units = cols / unit, row_bytes = kind == 30 ? cols * 2 : cols / 32 * 34;
+    for (size_t head = 0; head < heads; ++head) {
+        const uint8_t* row = matrix + head * row_bytes;
+        float lanes[64];
+        for (size_t lane = 0; lane < 64; ++lane) {
+            float sum = 0.0f;
+            for (size_t u = lane; u < units; u += 64) {
+                float chain = 0.0f;
+                if (kind == 30) {
+                    for (size_t i = 0; i < 8; ++i) {
+                        const uint8_t* at = row + (u * 8 + i) * 2;
+                        chain = fmaf(sdo_bf16_to_f32((uint16_t)(at[0] | (at[1] << 8))), x[u * 8 + i], chain);
+                    }
+                } else {
+                    const uint8_t* block = row + u * 34;
+                    for (size_t i = 0; i < 32; ++i) chain = fmaf((float)(int8_t)block[2 + i], x[u * 32 + i], chain);
+                    chain *= sdo_f16_to_f32((uint16_t)(block[0] | (block[1] << 8)));
+                }
+                sum = sum + chain;
+            }
+            lanes[lane] = sum;
+        }
+        for (size_t offset = 32; offset; offset /= 2)
+            for (size_t lane = 0; lane < offset; ++lane) lanes[lane] = lanes[lane] + lanes[lane + offset];
+        weights[head] = lanes[0];
+    }
+}
+
 void sdo_index_scores_f64(const float* q, const void* keys, int keys_bf16, const float* weights, const int32_t* visible,
                           size_t rows, size_t groups, size_t heads, size_t dim, float scale, double* scores) {
     for (size_t row = 0; row < rows; ++row) {

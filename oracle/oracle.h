@@ -100,6 +100,13 @@ void sdo_index_scores(const float* q, const void* keys, int keys_bf16, const flo
 void sdo_index_scores_f64(const float* q, const void* keys, int keys_bf16, const float* weights, const int32_t* visible,
                           size_t rows, size_t groups, size_t heads, size_t dim, float scale, double* scores);
 
+/* ---- The indexer's projection (sd_op_index_select_proj, gpu/kernels.cpp:5620-5667): weights[h] = matrix row h . x, rows BF16
+ *      (kind 30) or ggml Q8_0 blocks (kind 8: FP16 scale then 32 int8, crates/straydog-engine/src/formats.rs:104-116, 232-236).
+ *      The reference's GEMV fixes no summation order across devices (gpu/gemv_common.hpp:785-812: `lanes` is tuned per device);
+ *      this is the library's stated order for 64 lanes: unit chains from zero, lane u % 64 adds its units in order, lane sums
+ *      added pairwise at distances 32 .. 1.  Pinned by a float64 dot product and by the order's own definition on small cases. */
+void sdo_index_projection(const uint8_t* matrix, int kind, size_t cols, const float* x, size_t heads, float* weights);
+
 /* ---- Top-k: gpu/ops.hpp:1766-1874 (top_k_key, top_k_row); rule crates/straydog-engine/tests/fused_gpu.rs:326-358. */
 uint32_t sdo_top_k_key(float value);
 void sdo_top_k(const float* scores, size_t rows, size_t groups, size_t k, int32_t* out);

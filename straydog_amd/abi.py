@@ -68,6 +68,8 @@ SIGNATURES = {
     "sd_op_index_candidates": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_void_p, c_u64]),
     "sd_op_index_select": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float, c_u64,
                                    c_void_p, c_void_p, c_void_p, c_u64, c_void_p, c_void_p, c_u64, c_u64]),
+    "sd_op_index_select_proj": (c_int, [c_void_p, c_void_p, c_int, c_u64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64,
+                                        c_float, c_u64, c_void_p, c_void_p, c_void_p, c_u64, c_void_p, c_void_p, c_u64, c_u64]),
     "sd_op_to_bf16": (c_int, [c_void_p, c_void_p, c_u64, c_void_p]),
     # straydog_gpu_ext.h
     "sd_op_dspark_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, ctypes.c_uint32, c_void_p, c_u64, c_void_p]),
@@ -102,6 +104,7 @@ SIGNATURES = {
                                        c_u64, c_u64, c_float, c_void_p, c_u64, c_u64, c_void_p, c_int, c_void_p, c_u64]),
     "sdx_qsa_decode_attend_scratch": (c_u64, [c_u64, c_u64, c_u64, c_u64]),
     "sdx_qsa_decode_attend": (c_int, [c_void_p, _P(QsaState), c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_void_p, c_u64, c_void_p]),
+    "sdx_index_projection": (c_int, [c_void_p, c_void_p, c_int, c_u64, c_void_p, c_u64, c_void_p]),
     "sdx_index_score_bounds": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float, c_void_p, c_void_p]),
     "sdx_index_top_k": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float, c_void_p,
                                 c_u64, c_void_p]),

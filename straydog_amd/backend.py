@@ -145,6 +145,17 @@ class Backend:
         self.check(self.lib.sd_op_index_select(self.handle, q, keys, weights, visible, rows, groups, heads, dim, scale, rope_dims,
                                                positions, frequencies, scores, k, out, candidates, blocks, block))
 
+    def index_projection(self, matrix, kind, cols, x, heads, weights):
+        self.check(self.lib.sdx_index_projection(self.handle, matrix, kind, cols, x, heads, weights))
+
+    def index_select_proj(self, proj, x, q, keys, weights, visible, groups, heads, dim, scale, rope, scores, k, out, within=None):
+        """ops.rs index_select_proj: proj = (matrix, kind, cols); one row."""
+        matrix, kind, cols = proj
+        rope_dims, positions, frequencies = rope if rope else (0, None, None)
+        candidates, blocks, block = within if within else (None, 0, 0)
+        self.check(self.lib.sd_op_index_select_proj(self.handle, matrix, kind, cols, x, q, keys, weights, visible, groups, heads, dim, scale,
+                                                    rope_dims, positions, frequencies, scores, k, out, candidates, blocks, block))
+
     def to_bf16(self, x, count, out):
         self.check(self.lib.sd_op_to_bf16(self.handle, x, count, out))
 

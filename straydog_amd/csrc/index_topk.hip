@@ -7,6 +7,7 @@
 // scale is applied last.  Top-k compares order-preserving integer keys, keeps the lowest indices among ties and
 // emits ascending indices.
 #include "device.hpp"
+#include <hip/hip_fp16.h>
 #include "../../include/straydog_gpu.h"
 #include "../../include/straydog_gpu_ext.h"
 
@@ -39,20 +40,41 @@ __global__ void to_bf16_kernel(const float* x, size_t count, uint16_t* out) {
     }
 }
 
-__global__ void compress_kernel(const float* kv, const float* gate, size_t groups, size_t ratio, size_t dim, float* out) {
-    const size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (index >= groups * dim) return;
-    const size_t group = index / dim, col = index % dim;
-    if (!gate) { out[index] = kv[group * dim + col]; return; }
-    float top = -INFINITY;
-    for (size_t r = 0; r < ratio; ++r) top = fmaxf(top, gate[(group * ratio + r) * dim + col]);
-    float sum = 0.0f, acc = 0.0f;
-    for (size_t r = 0; r < ratio; ++r) {
-        const float w = expf(gate[(group * ratio + r) * dim + col] - top);
-        sum += w;
-        acc += w * kv[(group * ratio + r) * dim + col];
+// Per-channel softmax pooling of `ratio` rows into one (reference op_compress_kernel, gpu/ops.hpp:1681-1694): out = sum_r
+// softmax_r(gate[r]) * kv[r] for each column on its own.  A thread takes V adjacent columns of a group (one 16-byte load of
+// the gates and one of the rows per pooled row when V = 4) and reads each of them ONCE: the maximum runs along with the sums,
+// which are scaled down whenever it grows (the usual online form; the quotient does not depend on it).
+template<int V> struct Lanes { float v[V]; };
+template<int V>
+__global__ void __launch_bounds__(256) compress_kernel(const float* kv, const float* gate, size_t pieces, size_t ratio, size_t dim, float* out) {
+    const size_t piece = size_t(blockIdx.x) * 256 + threadIdx.x;       // V columns of one group
+    if (piece >= pieces) return;
+    const size_t per_row = dim / V, group = piece / per_row, at = piece % per_row * V;
+    typedef Lanes<V> __attribute__((aligned(4 * V))) Piece;
+    if (!gate) {       // nothing to pool: row `group` as it is
+        *reinterpret_cast<Piece*>(out + group * dim + at) = *reinterpret_cast<const Piece*>(kv + group * dim + at);
+        return;
     }
-    out[index] = acc / sum;
+    float top[V], sum[V], acc[V];
+    #pragma unroll
+    for (int i = 0; i < V; ++i) { top[i] = -INFINITY; sum[i] = 0.0f; acc[i] = 0.0f; }
+    for (size_t r = 0; r < ratio; ++r) {
+        const size_t from = (group * ratio + r) * dim + at;
+        const Piece g = *reinterpret_cast<const Piece*>(gate + from), x = *reinterpret_cast<const Piece*>(kv + from);
+        #pragma unroll
+        for (int i = 0; i < V; ++i) {
+            const float higher = fmaxf(top[i], g.v[i]);
+            // (the first row, and a gate of -inf before any finite one, would give exp(-inf - -inf): nothing is kept then)
+            const float keep = top[i] == -INFINITY ? 0.0f : expf(top[i] - higher), w = higher == -INFINITY ? 0.0f : expf(g.v[i] - higher);
+            sum[i] = sum[i] * keep + w;
+            acc[i] = acc[i] * keep + w * x.v[i];
+            top[i] = higher;
+        }
+    }
+    Piece pooled;
+    #pragma unroll
+    for (int i = 0; i < V; ++i) pooled.v[i] = acc[i] / sum[i];
+    *reinterpret_cast<Piece*>(out + group * dim + at) = pooled;
 }
 
 // The last 2 * pairs values of each vector rotated in adjacent pairs by positions[row] * frequencies[pair]
@@ -86,11 +108,18 @@ __global__ void rope_kernel(const float* from, float* to, size_t count, size_t v
     to[at + 1] = float(a * s + b * c);
 }
 
-// A row's candidate group `v` (gpu/ops.hpp:1948-1951): groups of its candidate blocks in candidate order.
-__device__ __forceinline__ size_t candidate_group(const int32_t* candidates, size_t block, size_t v, size_t groups) {
-    const int32_t b = candidates[v / block];
-    return b < 0 ? groups : size_t(b) * block + v % block;
-}
+// The two-level indexer's numbering (reference gpu/ops.hpp:1942-1951): a row's candidate list names blocks of `block` groups,
+// in index order, -1 past the last; place p of the row's scores stands for group list[p / block] * block + p % block, and for
+// no group at all (the value `groups`) in an unused slot.
+struct CandidateMap {
+    const int32_t* list;
+    size_t block, groups;
+    __device__ __forceinline__ size_t group_at(size_t place) const {
+        const size_t slot = place / block;
+        const int32_t named = list[slot];
+        return named < 0 ? groups : size_t(named) * block + (place - slot * block);
+    }
+};
 
 // Indexer scores, a thread per scored group.  q is uniform over the workgroup, so its values arrive through
 // scalar loads and every fmaf is (scalar q, vector key, vector sum).  H = 32 or 64 heads are carried at once,
@@ -104,7 +133,7 @@ __global__ void __launch_bounds__(256) index_scores_kernel(const float* __restri
     const size_t row = blockIdx.y, place = size_t(blockIdx.x) * 256 + threadIdx.x;
     const size_t scored = candidates ? blocks * block : groups;
     const int32_t* row_candidates = candidates ? candidates + row * blocks : nullptr;
-    const size_t g = !row_candidates ? place : place < scored ? candidate_group(row_candidates, block, place, groups) : groups;
+    const size_t g = !row_candidates ? place : place < scored ? CandidateMap{row_candidates, block, groups}.group_at(place) : groups;
     const int32_t seen = visible[row];
     const size_t limit = min(groups, size_t(seen > 0 ? seen : 0));
     const size_t key_row = min(g, groups - 1);
@@ -161,9 +190,13 @@ __global__ void __launch_bounds__(256) index_scores_kernel(const float* __restri
 
 // ---- top-k -------------------------------------------------------------------------------------------------
 
+// A score as an unsigned key of the same order (the rule of reference gpu/ops.hpp:1766-1769): both zeros are one key, a
+// negative value has all its bits turned over, any other its sign bit set.  Integer work only: one mask from the sign.
 __device__ __forceinline__ uint32_t top_k_key(float value) {
-    const uint32_t bits = __float_as_uint(value == 0.0f ? 0.0f : value);   // -0 ties +0
-    return bits & 0x80000000u ? ~bits : bits | 0x80000000u;
+    uint32_t bits = __float_as_uint(value);
+    if (!(bits << 1)) bits = 0;
+    const uint32_t negative = uint32_t(int32_t(bits) >> 31);          // all ones below zero
+    return bits ^ (negative | 0x80000000u);
 }
 
 constexpr int TOPK_THREADS = 1024, TOPK_WAVES = TOPK_THREADS / 64, TOPK_RUN = 8;
@@ -269,22 +302,26 @@ __global__ void __launch_bounds__(TOPK_THREADS) top_k_kernel(const float* scores
 __global__ void __launch_bounds__(TOPK_THREADS) top_k_candidates_kernel(const float* scores, size_t score_stride, size_t groups, const int32_t* candidates,
                                                                         size_t blocks, size_t block, size_t k, int32_t* out) {
     const float* s = scores + size_t(blockIdx.x) * score_stride;
-    const int32_t* c = candidates + size_t(blockIdx.x) * blocks;
-    top_k_row([=](size_t v) { return candidate_group(c, block, v, groups) < groups ? s[v] : -INFINITY; },
-              [=](size_t v) { return int32_t(candidate_group(c, block, v, groups)); }, blocks * block, k, out + size_t(blockIdx.x) * k);
+    const CandidateMap map{candidates + size_t(blockIdx.x) * blocks, block, groups};
+    top_k_row([=](size_t place) { return map.group_at(place) < groups ? s[place] : -INFINITY; },
+              [=](size_t place) { return int32_t(map.group_at(place)); }, blocks * block, k, out + size_t(blockIdx.x) * k);
 }
 
-// Each block's highest score; the block of the row's last visible group is +inf (always kept).
+// What the candidate pick ranks blocks by (reference gpu/ops.hpp:1952-1965): a block's highest score, and +inf for the block
+// that holds the row's last visible group (the newest, partly filled block is always kept).  A wave per block: its lanes read
+// the block's scores side by side and the maximum is five lane exchanges; four blocks a workgroup.
 __global__ void __launch_bounds__(256) block_tops_kernel(const float* scores, const int32_t* visible, size_t groups, size_t block, size_t count,
                                                          float* tops) {
-    const size_t row = blockIdx.y, b = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t row = blockIdx.y, b = size_t(blockIdx.x) * 4 + threadIdx.x / 64;
     if (b >= count) return;
-    const float* s = scores + row * groups;
-    const int32_t raw = visible[row];
-    const size_t seen = min(groups, size_t(raw > 0 ? raw : 0));
-    float top = seen && b == (seen - 1) / block ? INFINITY : -INFINITY;
-    for (size_t g = b * block, end = min(groups, g + block); g < end; ++g) top = fmaxf(top, s[g]);
-    tops[row * count + b] = top;
+    const unsigned lane = threadIdx.x % 64;
+    const size_t begin = b * block, end = min(groups, begin + block);
+    float top = -INFINITY;
+    for (size_t g = begin + lane; g < end; g += 64) top = fmaxf(top, scores[row * groups + g]);
+    #pragma unroll
+    for (int offset = 32; offset; offset /= 2) top = fmaxf(top, __shfl_xor(top, offset));
+    const int64_t newest = min(int64_t(groups), int64_t(visible[row])) - 1;     // the row's last visible group, if it sees any
+    if (lane == 0) tops[row * count + b] = newest >= 0 && size_t(newest) / block == b ? INFINITY : top;
 }
 
 // ---- the sparse path's indexer on matrix cores --------------------------------------------------------------
@@ -695,6 +732,106 @@ void fast_index_top_k(Device& d, const FastIndexSpace& s, const void* q_index, c
     SD_CHECK(hipGetLastError());
 }
 
+
+// The indexer's projection (one decode row): weights[h] = row h of a heads x cols matrix . x, the matrix rows BF16 (kind 30) or
+// ggml Q8_0 blocks (kind 8: an FP16 scale d, then 32 int8; reference gpu/core.hpp:1290-1294).  The reference forms these with its
+// GEMV stack, whose summation order follows a per-device lane count (gpu/gemv_common.hpp:785-812, gpu/gemv.hpp:1-60); here the
+// order is fixed for wave64 and stated, so the bits are reproducible on the CPU: a wave per head; lane L takes the units L,
+// L + 64, ... (a unit = 8 BF16 columns, or one Q8_0 block of 32); a unit's value is one chain of fused multiply-adds over its
+// columns in order, started from zero (for Q8_0 over float(q) * x, the chain then multiplied by the block's scale); a lane adds
+// its units' values in order; the lanes' sums are added by exchanges at distances 32, 16, 8, 4, 2, 1.
+template<int KIND>
+__global__ void __launch_bounds__(256) index_projection_kernel(const uint8_t* matrix, size_t row_bytes, size_t cols, const float* x, size_t heads,
+                                                               float* weights) {
+    const size_t head = size_t(blockIdx.x) * 4 + threadIdx.x / 64;
+    if (head >= heads) return;
+    const unsigned lane = threadIdx.x % 64;
+    const uint8_t* row = matrix + head * row_bytes;
+    constexpr size_t UNIT = KIND == 30 ? 8 : 32;
+    float sum = 0.0f;
+    for (size_t unit = lane; unit < cols / UNIT; unit += 64) {
+        const float* in = x + unit * UNIT;
+        float chain = 0.0f;
+        if (KIND == 30) {
+            const uint4 packed = *reinterpret_cast<const uint4*>(row + unit * 16);
+            const uint32_t words[4] = {packed.x, packed.y, packed.z, packed.w};
+            #pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                chain = fmaf(__uint_as_float(words[i] << 16), in[2 * i], chain);
+                chain = fmaf(__uint_as_float(words[i] & 0xffff0000u), in[2 * i + 1], chain);
+            }
+        } else {
+            const uint8_t* blockp = row + unit * 34;
+            const float d = __half2float(*reinterpret_cast<const __half*>(blockp));
+            #pragma unroll
+            for (int i = 0; i < 32; ++i) chain = fmaf(float(reinterpret_cast<const int8_t*>(blockp + 2)[i]), in[i], chain);
+            chain *= d;
+        }
+        sum = rounded_sum(sum, chain);
+    }
+    #pragma unroll
+    for (int offset = 32; offset; offset /= 2) sum = rounded_sum(sum, __shfl_xor(sum, offset));
+    if (lane == 0) weights[head] = sum;
+}
+
+void index_projection(Device& value, const void* proj_weights, int proj_kind, uint64_t proj_cols, const float* x, uint64_t heads, float* weights) {
+    if (!proj_weights || !proj_cols || proj_cols > 8192 || !heads || heads > 64) throw std::runtime_error("invalid Straydog index shape");
+    if (proj_kind != 30 && proj_kind != 8) throw std::runtime_error("the index projection takes BF16 (kind 30) or Q8_0 (kind 8) rows");
+    if (proj_cols % (proj_kind == 30 ? 8 : 32)) throw std::runtime_error("invalid Straydog index shape");
+    const size_t row_bytes = proj_kind == 30 ? size_t(proj_cols) * 2 : size_t(proj_cols) / 32 * 34;
+    op_span(value, proj_weights, checked_product({heads, row_bytes}), "a weight matrix");
+    op_span(value, x, checked_floats({proj_cols}), "a linear input");
+    op_span(value, weights, checked_floats({heads}), "index weights");
+    if (proj_kind == 30 && reinterpret_cast<uintptr_t>(proj_weights) % 16) throw std::runtime_error("BF16 projection rows must be 16-byte aligned");
+    const unsigned grid = unsigned((heads + 3) / 4);
+    const auto* matrix = static_cast<const uint8_t*>(proj_weights);
+    if (proj_kind == 30) index_projection_kernel<30><<<grid, 256, 0, value.stream>>>(matrix, row_bytes, size_t(proj_cols), x, size_t(heads), weights);
+    else index_projection_kernel<8><<<grid, 256, 0, value.stream>>>(matrix, row_bytes, size_t(proj_cols), x, size_t(heads), weights);
+}
+
+void index_select(Device& value, const float* q, const float* keys, const float* weights, const int32_t* visible, uint64_t rows,
+                       uint64_t groups, uint64_t heads, uint64_t dim, float scale, uint64_t rope_dims, const int32_t* positions,
+                       const float* frequencies, float* scores, uint64_t k, int32_t* out, const int32_t* candidates, uint64_t blocks,
+                       uint64_t block) {
+    if (!rows || rows > 65535 || !groups || groups > (uint64_t(1) << 31) || !heads || heads > 64 || !dim || !k || k > (uint64_t(1) << 31) ||
+        rope_dims % 2 || rope_dims > dim || rope_dims > 128)
+        throw std::runtime_error("invalid Straydog index shape");
+    uint64_t scored = groups;
+    if (candidates) {
+        if (!blocks || !block || blocks > (uint64_t(1) << 20) || block > 4096) throw std::runtime_error("invalid Straydog index candidates");
+        op_span(value, candidates, checked_floats({rows, blocks}), "index candidates");
+        scored = blocks * block;
+    }
+    op_span(value, q, checked_floats({rows, heads, dim}), "index queries");
+    op_state_span(value, keys, checked_product({groups, dim}), "index keys");
+    op_span(value, weights, checked_floats({rows, heads}), "index weights");
+    op_span(value, visible, checked_floats({rows}), "visible counts");
+    op_span(value, positions, checked_floats({rows}), "query positions");
+    if (rope_dims) op_span(value, frequencies, checked_floats({rope_dims / 2}), "rope frequencies");
+    op_span(value, scores, checked_floats({rows, std::max(groups, scored)}), "index scores");
+    op_span(value, out, checked_floats({rows, k}), "top-k indices");
+    const float* rotated = q;
+    if (rope_dims) {
+        // q itself stays as it was: the rotated copy lives in the device's workspace
+        const size_t count = checked_product({rows, heads, dim});
+        float* copy = static_cast<float*>(workspace(value, count * 4));
+        rope_kernel<<<checked_blocks(count), 256, 0, value.stream>>>(q, copy, count, size_t(heads), size_t(dim), size_t(rope_dims / 2), positions,
+                                                                     frequencies, 0, 1);
+        SD_CHECK(hipGetLastError());
+        rotated = copy;
+    }
+    // scores rows are `scored` wide with candidates (candidate order), `groups` wide without
+    const size_t stride = candidates ? size_t(scored) : size_t(groups);
+    launch_scores(value, rotated, state_base(keys), state_bf16(keys), 0, weights, visible, size_t(rows), size_t(groups), size_t(heads), size_t(dim),
+                  scale, scores, stride, candidates, size_t(blocks), size_t(block ? block : 1));
+    if (candidates)
+        top_k_candidates_kernel<<<unsigned(rows), TOPK_THREADS, 0, value.stream>>>(scores, stride, size_t(groups), candidates, size_t(blocks),
+                                                                                   size_t(block), size_t(k), out);
+    else
+        top_k_kernel<<<unsigned(rows), TOPK_THREADS, 0, value.stream>>>(scores, size_t(groups), stride, size_t(k), out);
+    SD_CHECK(hipGetLastError());
+}
+
 }  // namespace
 
 extern "C" {
@@ -714,7 +851,12 @@ int sd_op_compress(void* handle, const float* kv, const float* gate, uint64_t gr
     op_span(value, kv, checked_floats({groups, ratio, dim}), "rows to compress");
     if (gate) op_span(value, gate, checked_floats({groups, ratio, dim}), "a compression gate");
     op_span(value, out, checked_floats({groups, dim}), "compressed rows");
-    compress_kernel<<<checked_blocks(checked_product({groups, dim})), 256, 0, value.stream>>>(kv, gate, size_t(groups), size_t(ratio), size_t(dim), out);
+    const size_t values = checked_product({groups, dim});
+    const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    if (dim % 4 == 0 && aligned(kv) && aligned(gate) && aligned(out))
+        compress_kernel<4><<<checked_blocks(values / 4), 256, 0, value.stream>>>(kv, gate, values / 4, size_t(ratio), size_t(dim), out);
+    else
+        compress_kernel<1><<<checked_blocks(values), 256, 0, value.stream>>>(kv, gate, values, size_t(ratio), size_t(dim), out);
     SD_OP_END
 }
 
@@ -766,7 +908,7 @@ int sd_op_index_candidates(void* handle, const float* scores, const int32_t* vis
     op_span(value, out, checked_floats({rows, blocks}), "index candidates");
     if (checked_floats({rows, count}) > scratch_bytes) throw std::runtime_error("Straydog index candidates need more scratch");
     op_span(value, scratch, checked_floats({rows, count}), "index candidates' scratch");
-    block_tops_kernel<<<dim3(checked_blocks(size_t(count)), unsigned(rows)), 256, 0, value.stream>>>(scores, visible, size_t(groups), size_t(block),
+    block_tops_kernel<<<dim3(checked_blocks(size_t(count), 4), unsigned(rows)), 256, 0, value.stream>>>(scores, visible, size_t(groups), size_t(block),
                                                                                                  size_t(count), scratch);
     SD_CHECK(hipGetLastError());
     top_k_kernel<<<unsigned(rows), TOPK_THREADS, 0, value.stream>>>(scratch, size_t(count), size_t(count), size_t(blocks), out);
@@ -778,42 +920,29 @@ int sd_op_index_select(void* handle, const float* q, const float* keys, const fl
                        const float* frequencies, float* scores, uint64_t k, int32_t* out, const int32_t* candidates, uint64_t blocks,
                        uint64_t block) {
     SD_OP_BEGIN
-    if (!rows || rows > 65535 || !groups || groups > (uint64_t(1) << 31) || !heads || heads > 64 || !dim || !k || k > (uint64_t(1) << 31) ||
-        rope_dims % 2 || rope_dims > dim || rope_dims > 128)
-        throw std::runtime_error("invalid Straydog index shape");
-    uint64_t scored = groups;
-    if (candidates) {
-        if (!blocks || !block || blocks > (uint64_t(1) << 20) || block > 4096) throw std::runtime_error("invalid Straydog index candidates");
-        op_span(value, candidates, checked_floats({rows, blocks}), "index candidates");
-        scored = blocks * block;
-    }
-    op_span(value, q, checked_floats({rows, heads, dim}), "index queries");
-    op_state_span(value, keys, checked_product({groups, dim}), "index keys");
-    op_span(value, weights, checked_floats({rows, heads}), "index weights");
-    op_span(value, visible, checked_floats({rows}), "visible counts");
-    op_span(value, positions, checked_floats({rows}), "query positions");
-    if (rope_dims) op_span(value, frequencies, checked_floats({rope_dims / 2}), "rope frequencies");
-    op_span(value, scores, checked_floats({rows, std::max(groups, scored)}), "index scores");
-    op_span(value, out, checked_floats({rows, k}), "top-k indices");
-    const float* rotated = q;
-    if (rope_dims) {
-        // q itself stays as it was: the rotated copy lives in the device's workspace
-        const size_t count = checked_product({rows, heads, dim});
-        float* copy = static_cast<float*>(workspace(value, count * 4));
-        rope_kernel<<<checked_blocks(count), 256, 0, value.stream>>>(q, copy, count, size_t(heads), size_t(dim), size_t(rope_dims / 2), positions,
-                                                                     frequencies, 0, 1);
-        SD_CHECK(hipGetLastError());
-        rotated = copy;
-    }
-    // scores rows are `scored` wide with candidates (candidate order), `groups` wide without
-    const size_t stride = candidates ? size_t(scored) : size_t(groups);
-    launch_scores(value, rotated, state_base(keys), state_bf16(keys), 0, weights, visible, size_t(rows), size_t(groups), size_t(heads), size_t(dim),
-                  scale, scores, stride, candidates, size_t(blocks), size_t(block ? block : 1));
-    if (candidates)
-        top_k_candidates_kernel<<<unsigned(rows), TOPK_THREADS, 0, value.stream>>>(scores, stride, size_t(groups), candidates, size_t(blocks),
-                                                                                   size_t(block), size_t(k), out);
-    else
-        top_k_kernel<<<unsigned(rows), TOPK_THREADS, 0, value.stream>>>(scores, size_t(groups), stride, size_t(k), out);
+    index_select(value, q, keys, weights, visible, rows, groups, heads, dim, scale, rope_dims, positions, frequencies, scores, k, out, candidates,
+                 blocks, block);
+    SD_OP_END
+}
+
+int sdx_index_projection(void* handle, const void* proj_weights, int proj_kind, uint64_t proj_cols, const float* x, uint64_t heads, float* weights) {
+    SD_OP_BEGIN
+    index_projection(value, proj_weights, proj_kind, proj_cols, x, heads, weights);
+    SD_OP_END
+}
+
+/* reference straydog_gpu.h:422 (gpu/kernels.cpp:5620-5667, kernel gpu/ops.hpp:2267-2300): one decode row's indexer with the
+ * projection of x into the heads' weights ahead of it; the weights are left in `weights`. */
+int sd_op_index_select_proj(void* handle, const void* proj_weights, int proj_kind, uint64_t proj_cols, const float* x, const float* q,
+                            const float* keys, float* weights, const int32_t* visible, uint64_t groups, uint64_t heads, uint64_t dim, float scale,
+                            uint64_t rope_dims, const int32_t* positions, const float* frequencies, float* scores, uint64_t k, int32_t* out,
+                            const int32_t* candidates, uint64_t blocks, uint64_t block) {
+    SD_OP_BEGIN
+    if (!heads || heads > 64) throw std::runtime_error("invalid Straydog index shape");
+    index_projection(value, proj_weights, proj_kind, proj_cols, x, heads, weights);
+    SD_CHECK(hipGetLastError());
+    index_select(value, q, keys, weights, visible, 1, groups, heads, dim, scale, rope_dims, positions, frequencies, scores, k, out, candidates, blocks,
+                 block);
     SD_OP_END
 }
 

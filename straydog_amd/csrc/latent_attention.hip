@@ -177,58 +177,100 @@ namespace {
 
 // DSpark's noncausal block attention (reference gpu/dspark_attention.hpp:1-101): every query of the block sees the history
 // positions [anchor - history, anchor) of the K = V ring of 128 rows and all the block's keys, 512 columns, scale 1/sqrt(512),
-// the head's sink in the maximum and the denominator only.  A workgroup per (query, head): at most 133 keys, so a wave takes
-// every fourth key with its lanes across the columns (two 16-byte loads a lane, a wave-wide sum), the weights are formed a
-// thread per key, and the output two columns a thread over the keys in order.
-constexpr size_t DSPARK_DIM = 512, DSPARK_RING = 128, DSPARK_MOST = DSPARK_RING + 5;
-__global__ void __launch_bounds__(256) dspark_attention_kernel(const float* q, const float* ring, const float* block, const float* sinks, size_t heads,
-                                                               size_t slots, uint32_t anchor, const int32_t* anchor_at, size_t window, float scale,
-                                                               float* out) {
-    __shared__ __align__(16) float qs[DSPARK_DIM];
-    __shared__ float scores[DSPARK_MOST];
-    const size_t row = blockIdx.x / heads, head = blockIdx.x % heads;
-    const unsigned t = threadIdx.x, lane = t % 64, wave = t / 64;
-    const int64_t p = int64_t(anchor_at ? anchor_at[0] : int32_t(anchor)) - 1;
-    const int64_t first = p - int64_t(window) + 1 < 0 ? 0 : p - int64_t(window) + 1;
-    const size_t raw_count = size_t(p - first + 1), total = raw_count + slots;
-    const float* query = q + (row * heads + head) * DSPARK_DIM;
-    for (size_t i = t; i < DSPARK_DIM; i += 256) qs[i] = query[i];
-    __syncthreads();
-    const auto key = [&](size_t index) {
-        return index < raw_count ? ring + size_t(first + int64_t(index)) % DSPARK_RING * DSPARK_DIM : block + (index - raw_count) * DSPARK_DIM;
+// the head's sink in the maximum and the denominator only.
+//
+// The keys are the same for every head and every slot of the block, so a workgroup serves ONE HEAD AND ALL ITS SLOTS (up to
+// five queries) and every key row it loads is used by all of them: a wave takes every fourth key, lanes across the 512 columns
+// (two 16-byte loads a lane), and forms the slots' dot products together, each a wave-wide sum; wave s then turns slot s's
+// scores into weights (lanes over the keys, maxima and sums by lane exchanges); the outputs are two columns a thread, one
+// value load feeding all the slots' sums.
+constexpr int DSPARK_DIM = 512, DSPARK_RING = 128, DSPARK_SLOTS = 5, DSPARK_KEYS = DSPARK_RING + DSPARK_SLOTS, DSPARK_WAVES = 4;
+struct DsparkArgs {
+    const float *q, *ring, *block, *sinks;
+    int heads, slots, history;
+    uint32_t anchor;
+    const int32_t* anchor_at;      // device-resident anchor, or null
+    float scale;
+    float* out;
+};
+__global__ void __launch_bounds__(DSPARK_WAVES * 64) dspark_attention_kernel(DsparkArgs a) {
+    __shared__ float weights[DSPARK_SLOTS][DSPARK_KEYS];
+    __shared__ float denominators[DSPARK_SLOTS];
+    const int head = blockIdx.x, t = threadIdx.x, lane = t % 64, wave = t / 64;
+    // ring keys: positions last - count + 1 .. last, last = anchor - 1, at most `history` of them and none below position 0
+    const long long last = (long long)(a.anchor_at ? a.anchor_at[0] : int32_t(a.anchor)) - 1;
+    const int ring_keys = int(min((long long)a.history, last + 1)), keys = ring_keys + a.slots;
+    const long long oldest = last - ring_keys + 1;
+    const auto row_of = [&](int key) -> const float* {
+        return key < ring_keys ? a.ring + size_t((oldest + key) % DSPARK_RING) * DSPARK_DIM : a.block + size_t(key - ring_keys) * DSPARK_DIM;
     };
-    for (size_t index = wave; index < total; index += 4) {
-        const float* k = key(index) + 8 * lane;
+    // the slots' queries of this head: a lane keeps its eight columns of each
+    float4 query[DSPARK_SLOTS][2];
+    #pragma unroll
+    for (int s = 0; s < DSPARK_SLOTS; ++s) {
+        const float* from = a.q + (size_t(min(s, a.slots - 1)) * a.heads + head) * DSPARK_DIM + 8 * lane;
+        query[s][0] = *reinterpret_cast<const float4*>(from);
+        query[s][1] = *reinterpret_cast<const float4*>(from + 4);
+    }
+    for (int key = wave; key < keys; key += DSPARK_WAVES) {
+        const float* k = row_of(key) + 8 * lane;
         const float4 k0 = *reinterpret_cast<const float4*>(k), k1 = *reinterpret_cast<const float4*>(k + 4);
-        const float4 q0 = *reinterpret_cast<const float4*>(qs + 8 * lane), q1 = *reinterpret_cast<const float4*>(qs + 8 * lane + 4);
-        float dot = q0.x * k0.x;
-        dot = fmaf(q0.y, k0.y, dot); dot = fmaf(q0.z, k0.z, dot); dot = fmaf(q0.w, k0.w, dot);
-        dot = fmaf(q1.x, k1.x, dot); dot = fmaf(q1.y, k1.y, dot); dot = fmaf(q1.z, k1.z, dot); dot = fmaf(q1.w, k1.w, dot);
         #pragma unroll
-        for (int offset = 32; offset; offset /= 2) dot += __shfl_xor(dot, offset);
-        if (lane == 0) scores[index] = dot * scale;
+        for (int s = 0; s < DSPARK_SLOTS; ++s) {
+            float dot = query[s][0].x * k0.x;
+            dot = fmaf(query[s][0].y, k0.y, dot); dot = fmaf(query[s][0].z, k0.z, dot); dot = fmaf(query[s][0].w, k0.w, dot);
+            dot = fmaf(query[s][1].x, k1.x, dot); dot = fmaf(query[s][1].y, k1.y, dot); dot = fmaf(query[s][1].z, k1.z, dot); dot = fmaf(query[s][1].w, k1.w, dot);
+            #pragma unroll
+            for (int offset = 32; offset; offset /= 2) dot += __shfl_xor(dot, offset);
+            if (lane == 0) weights[s][key] = dot * a.scale;
+        }
     }
     __syncthreads();
-    float top = sinks[head];
-    for (size_t index = 0; index < total; ++index) top = fmaxf(top, scores[index]);
-    __syncthreads();
-    if (t < total) scores[t] = scores[t] == -INFINITY ? 0.0f : expf(scores[t] - top);
-    __syncthreads();
-    float denominator = 0.0f;
-    for (size_t index = 0; index < total; ++index) denominator += scores[index];
-    denominator += expf(sinks[head] - top);
-    const size_t dim = 2 * size_t(t);
-    float a0 = 0.0f, a1 = 0.0f;
-    #pragma unroll 8
-    for (size_t index = 0; index < total; ++index) {
-        const float w = scores[index];
-        const float2 v = *reinterpret_cast<const float2*>(key(index) + dim);
-        a0 = w == 0.0f ? a0 : fmaf(w, v.x, a0);
-        a1 = w == 0.0f ? a1 : fmaf(w, v.y, a1);
+    // scores -> weights: wave s (and wave 0 again for a fifth slot) owns slot s; a lane holds keys lane, lane + 64, lane + 128
+    for (int s = wave; s < a.slots; s += DSPARK_WAVES) {
+        const float sink = a.sinks[head];
+        float score[3], top = sink;
+        #pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const int key = lane + 64 * i;
+            score[i] = key < keys ? weights[s][key] : -INFINITY;
+            top = fmaxf(top, score[i]);
+        }
+        #pragma unroll
+        for (int offset = 32; offset; offset /= 2) top = fmaxf(top, __shfl_xor(top, offset));
+        float sum = 0.0f;
+        #pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const int key = lane + 64 * i;
+            const float w = score[i] == -INFINITY ? 0.0f : expf(score[i] - top);
+            if (key < keys) weights[s][key] = w;
+            sum += w;
+        }
+        #pragma unroll
+        for (int offset = 32; offset; offset /= 2) sum += __shfl_xor(sum, offset);
+        if (lane == 0) denominators[s] = sum + expf(sink - top);
     }
-    float* o = out + (row * heads + head) * DSPARK_DIM;
-    o[dim] = a0 / denominator;
-    o[dim + 1] = a1 / denominator;
+    __syncthreads();
+    // outputs: columns 2t, 2t + 1 of every slot; a key whose weight is 0 in a slot adds nothing there
+    float2 sums[DSPARK_SLOTS];
+    #pragma unroll
+    for (int s = 0; s < DSPARK_SLOTS; ++s) sums[s] = make_float2(0.0f, 0.0f);
+    #pragma unroll 4
+    for (int key = 0; key < keys; ++key) {
+        const float2 v = *reinterpret_cast<const float2*>(row_of(key) + 2 * t);
+        #pragma unroll
+        for (int s = 0; s < DSPARK_SLOTS; ++s) {
+            const float w = weights[s][key];       // (slots past the block's last hold what the scores of its last slot left: unused)
+            sums[s].x = w == 0.0f ? sums[s].x : fmaf(w, v.x, sums[s].x);
+            sums[s].y = w == 0.0f ? sums[s].y : fmaf(w, v.y, sums[s].y);
+        }
+    }
+    #pragma unroll
+    for (int s = 0; s < DSPARK_SLOTS; ++s)
+        if (s < a.slots) {
+            const float denominator = denominators[s];
+            *reinterpret_cast<float2*>(a.out + (size_t(s) * a.heads + head) * DSPARK_DIM + 2 * t) = make_float2(sums[s].x / denominator, sums[s].y / denominator);
+        }
 }
 
 }  // namespace
@@ -238,17 +280,17 @@ extern "C" {
 int sd_op_dspark_attention(void* handle, const float* q, const float* ring, const float* block, const float* sinks, uint64_t heads, uint64_t slots,
                            uint32_t anchor, const int32_t* anchor_at, uint64_t history, float* out) {
     SD_OP_BEGIN
-    if (!heads || heads > 64 || !slots || slots > 5 || history > DSPARK_RING || anchor > uint32_t(INT32_MAX) || history > anchor)
+    if (!heads || heads > 64 || !slots || slots > uint64_t(DSPARK_SLOTS) || history > uint64_t(DSPARK_RING) || anchor > uint32_t(INT32_MAX) || history > anchor)
         throw std::runtime_error("invalid DSpark attention block or history range");
     op_span(value, q, checked_floats({slots, heads, uint64_t(DSPARK_DIM)}), "DSpark rotated queries");
-    op_span(value, ring, DSPARK_RING * DSPARK_DIM * 4, "DSpark history K ring");
+    op_span(value, ring, size_t(DSPARK_RING) * DSPARK_DIM * 4, "DSpark history K ring");
     op_span(value, block, checked_floats({slots, uint64_t(DSPARK_DIM)}), "DSpark rotated block keys");
     op_span(value, sinks, checked_floats({heads}), "DSpark attention sinks");
     op_span(value, out, checked_floats({slots, heads, uint64_t(DSPARK_DIM)}), "DSpark attention output");
     if (anchor_at) op_span(value, anchor_at, 4, "DSpark anchor position");
-    // p = anchor - 1 and a window of `history` give exactly [anchor - history, anchor); anchor = history = 0 gives no ring keys
-    dspark_attention_kernel<<<unsigned(slots * heads), 256, 0, value.stream>>>(q, ring, block, sinks, size_t(heads), size_t(slots), anchor, anchor_at,
-                                                                              size_t(history), 1.0f / sqrtf(float(DSPARK_DIM)), out);
+    // anchor = history = 0 gives no ring keys: the block's own keys are always seen
+    const DsparkArgs args{q, ring, block, sinks, int(heads), int(slots), int(history), anchor, anchor_at, 1.0f / sqrtf(float(DSPARK_DIM)), out};
+    dspark_attention_kernel<<<unsigned(heads), DSPARK_WAVES * 64, 0, value.stream>>>(args);
     SD_OP_END
 }
 

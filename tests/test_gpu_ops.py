@@ -234,7 +234,7 @@ def test_an_index_select_matches_rope_scores_and_top_k(gpu, oracle):
 
 
 def test_the_two_level_indexer_matches_its_reference(gpu, oracle):
-    # fused_gpu.rs:476-566 without the projection launch
+    # fused_gpu.rs:476-566
     rng = np.random.default_rng(0x1f83)
     heads, dim, k, blocks, block = 32, 128, 512, 2048, 8
     for rows, groups in [(1, 20000), (3, 23001)]:
@@ -269,8 +269,74 @@ def test_the_two_level_indexer_matches_its_reference(gpu, oracle):
             got = _read(gpu, o3, np.int32, rows * k).reshape(rows, k)
             assert np.array_equal(got, oracle.top_k(masked, k)), (rows, run)
             gpu.release(s3); gpu.release(o3)
+        if rows == 1:
+            # the decode launch (fused_gpu.rs:543-564): the projection of x into the weights, then the same choice among the candidates
+            width = 5120
+            x = (rng.random(width) * 4 - 2).astype(np.float32)
+            matrix = ((rng.random((heads, width)) * 0.1 - 0.05).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16).view(np.uint8).reshape(-1)
+            formed = oracle.index_projection(matrix, 30, width, x, heads)
+            masked = np.where(keep, oracle.index_scores(q2, keys, formed[None, :], seen, scale), -np.inf).astype(np.float32)
+            xb, mb = gpu.upload(x), gpu.upload(matrix)
+            for run in range(2):
+                s3, o3, w3 = gpu.buffer(max(groups, blocks * block) * 4), gpu.buffer(k * 4), gpu.buffer(heads * 4)
+                gpu.index_select_proj((mb.base(), 30, width), xb.base(), qb2.base(), kb.base(), w3.base(), vb.base(), groups, heads, dim, scale,
+                                      (0, vb.base(), None), s3.base(), k, o3.base(), (cand.base(), blocks, block))
+                assert np.array_equal(_read(gpu, o3, np.int32, k), oracle.top_k(masked, k).ravel()), f"run {run}: the decode launch's indices among the candidates"
+                for b in (s3, o3, w3):
+                    gpu.release(b)
+            gpu.release(xb); gpu.release(mb)
         for b in (kb, vb, qb, wb, scores, out, cand, scratch, qb2, wb2):
             gpu.release(b)
+
+
+def test_an_index_select_with_its_projection_matches_the_two_ops(gpu, oracle):
+    # fused_gpu.rs:430-474: the indexer's projection of x into its weights and the row's index select in one call give the
+    # weights, scores and indices of the two ops, bit for bit, twice in a row; BF16 rows and ggml Q8_0 rows.  The separate
+    # projection is sdx_index_projection (the reference's is sd_op_linear); its weights are also the oracle's, bit for bit.
+    from test_oracle_index_topk import _q8_0_rows
+    rng = np.random.default_rng(0x510e)
+    heads, dim, rope_dims, k, width, groups = 32, 128, 64, 512, 5120, 2500
+    frequencies = (np.float32(1.6e5) ** (-(2.0 * np.arange(rope_dims // 2, dtype=np.float32)) / np.float32(rope_dims))).astype(np.float32)
+    x = (rng.random(width) * 4 - 2).astype(np.float32)
+    q = (rng.random((heads, dim)) * 4 - 2).astype(np.float32)
+    keys = (rng.random((groups, dim)) * 2 - 1).astype(np.float32)
+    scale = float(1.0 / (np.sqrt(np.float32(dim)) * np.sqrt(np.float32(heads))))
+    fb, xb, qb, kb = (gpu.upload(a) for a in (frequencies, x, q, keys))
+    pb, vb = gpu.upload(np.array([31337], dtype=np.int32)), gpu.upload(np.array([groups - 5], dtype=np.int32))
+    bf16 = ((rng.random((heads, width)) * 0.1 - 0.05).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16).view(np.uint8).reshape(-1)
+    q8 = _q8_0_rows(rng, heads, width)[0]
+    rope = (rope_dims, pb.base(), fb.base())
+    for kind, matrix in ((30, bf16), (8, q8)):
+        mb = gpu.upload(matrix)
+        w1, s1, o1 = gpu.buffer(heads * 4), gpu.buffer(groups * 4), gpu.buffer(k * 4)
+        gpu.index_projection(mb.base(), kind, width, xb.base(), heads, w1.base())
+        gpu.index_select(qb.base(), kb.base(), w1.base(), vb.base(), 1, groups, heads, dim, scale, rope, s1.base(), k, o1.base())
+        weights_1, scores_1, out_1 = _read(gpu, w1, np.uint32, heads), _read(gpu, s1, np.uint32, groups), _read(gpu, o1, np.int32, k)
+        assert np.array_equal(weights_1, oracle.index_projection(matrix, kind, width, x, heads).view(np.uint32)), f"kind {kind}: weights vs oracle"
+        assert (out_1 >= 0).all() and len(set(out_1.tolist())) == k
+        for run in range(2):
+            w2, s2, o2 = gpu.buffer(heads * 4), gpu.buffer(groups * 4), gpu.buffer(k * 4)
+            gpu.index_select_proj((mb.base(), kind, width), xb.base(), qb.base(), kb.base(), w2.base(), vb.base(), groups, heads, dim, scale, rope,
+                                  s2.base(), k, o2.base())
+            assert np.array_equal(_read(gpu, w2, np.uint32, heads), weights_1), f"kind {kind}, run {run}: weights"
+            assert np.array_equal(_read(gpu, s2, np.uint32, groups), scores_1), f"kind {kind}, run {run}: scores"
+            assert np.array_equal(_read(gpu, o2, np.int32, k), out_1), f"kind {kind}, run {run}: indices"
+            for b in (w2, s2, o2):
+                gpu.release(b)
+        for b in (mb, w1, s1, o1):
+            gpu.release(b)
+    # refusals: a kind the projection does not take, columns that are not whole units
+    from straydog_amd.backend import StraydogError
+    mb = gpu.upload(bf16)
+    w, s, o = gpu.buffer(heads * 4), gpu.buffer(groups * 4), gpu.buffer(k * 4)
+    with pytest.raises(StraydogError, match="BF16 .kind 30. or Q8_0"):
+        gpu.index_select_proj((mb.base(), 12, width), xb.base(), qb.base(), kb.base(), w.base(), vb.base(), groups, heads, dim, scale, rope, s.base(), k, o.base())
+    with pytest.raises(StraydogError, match="invalid Straydog index shape"):
+        gpu.index_select_proj((mb.base(), 30, 5004), xb.base(), qb.base(), kb.base(), w.base(), vb.base(), groups, heads, dim, scale, rope, s.base(), k, o.base())
+    with pytest.raises(StraydogError, match="outside"):
+        gpu.index_select_proj((mb.base(), 30, width), xb.at(4 * 100), qb.base(), kb.base(), w.base(), vb.base(), groups, heads, dim, scale, rope, s.base(), k, o.base())
+    for b in (mb, w, s, o, fb, xb, qb, kb, pb, vb):
+        gpu.release(b)
 
 
 def test_sparse_attention_matches_the_oracle_and_bf16_rows_match_f32(gpu, oracle):

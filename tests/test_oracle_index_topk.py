@@ -178,3 +178,57 @@ def test_fill_normal_moments(oracle):
     assert np.array_equal(x, oracle.fill_normal(0x9e3779b97f4a7c15, 200000))
     u = oracle.fill_uniform(5, 100000)
     assert 0.0 <= u.min() and u.max() < 1.0 and abs(float(u.mean()) - 0.5) < 0.01
+
+
+def _q8_0_rows(rng, heads, cols):
+    """ggml Q8_0 rows as the reference's test draws them (fused_gpu.rs:448-455): an FP16 scale of moderate exponent, 32 int8."""
+    blocks = heads * cols // 32
+    out = np.zeros((blocks, 34), dtype=np.uint8)
+    bits = ((rng.integers(0, 2, blocks) << 15) | ((8 + rng.integers(0, 5, blocks)) << 10) | rng.integers(0, 1024, blocks)).astype(np.uint16)
+    out[:, 0] = bits & 0xff
+    out[:, 1] = bits >> 8
+    out[:, 2:] = rng.integers(0, 256, size=(blocks, 32), dtype=np.uint8)
+    return out.reshape(-1), bits.view(np.float16).astype(np.float64), out[:, 2:].view(np.int8).astype(np.float64)
+
+
+def test_index_projection_is_the_stated_order_and_a_dot_product(oracle):
+    rng = np.random.default_rng(31)
+    heads, cols = 5, 1024
+    x = (rng.random(cols) * 4 - 2).astype(np.float32)
+    # BF16 rows: against float64, and against the stated order written out with numpy float32 steps
+    w = (rng.standard_normal((heads, cols)) * 0.05).astype(np.float32)
+    bits = (w.view(np.uint32) >> 16).astype(np.uint16)
+    values = (bits.astype(np.uint32) << 16).view(np.float32)
+    got = oracle.index_projection(bits.view(np.uint8).reshape(-1), 30, cols, x, heads)
+    assert np.allclose(got, values.astype(np.float64) @ x.astype(np.float64), rtol=0, atol=2e-5)
+    import math
+    def f32(v):
+        return float(np.float32(v))
+    def fma(a, b, c):         # exact product and sum in Python floats are not exact; use fractions for the single rounding
+        from fractions import Fraction
+        return f32(Fraction(float(a)) * Fraction(float(b)) + Fraction(float(c)))
+    for h in range(2):
+        lanes = []
+        for lane in range(64):
+            total = 0.0
+            for u in range(lane, cols // 8, 64):
+                chain = 0.0
+                for i in range(8):
+                    chain = fma(values[h, u * 8 + i], x[u * 8 + i], chain)
+                total = f32(np.float32(total) + np.float32(chain))
+            lanes.append(total)
+        offset = 32
+        while offset:
+            lanes = [f32(np.float32(lanes[i]) + np.float32(lanes[i + offset])) for i in range(offset)]
+            offset //= 2
+        assert np.float32(lanes[0]).view(np.uint32) == got[h].view(np.uint32)
+    # Q8_0 rows: against float64 of d * q . x, a tiny case against the definition by hand, and block independence
+    raw, d, q = _q8_0_rows(rng, heads, cols)
+    got = oracle.index_projection(raw, 8, cols, x, heads)
+    want = ((d[:, None] * q).reshape(heads, cols) * x.astype(np.float64)).sum(axis=1)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-3 * np.abs(want).max())
+    one = np.zeros(34, dtype=np.uint8)
+    one[0:2] = np.frombuffer(np.float16(0.5).tobytes(), dtype=np.uint8)
+    one[2:5] = np.array([3, 0xfe, 127], dtype=np.uint8)          # 3, -2, 127
+    xs = np.zeros(32, dtype=np.float32); xs[:3] = [2.0, 4.0, 1.0]
+    assert oracle.index_projection(one, 8, 32, xs, 1)[0] == np.float32(0.5 * (6 - 8 + 127))
