@@ -24,9 +24,29 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense FP16/BF16 MFMA, published
 
-# HBM bytes per launch of the dominant kernel as rocprofv3's FETCH_SIZE (x 2.000) + WRITE_SIZE (x 1.000) counted them, the
-# scale factors being what the same counters read for the library's 1 GiB copy kernel.
-MEASURED_TRAFFIC = {"config1": 626.8e6, "config1_32k": 1147.4e6}
+# HBM bytes per launch of each workload's dominant kernel.  These are not measured in this run: they are the figures of the
+# rocprofv3 counter runs summarised under profiles/ (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors being what the same
+# counters read for the library's 1 GiB copy kernel), kept here so that the bench line carries them; `traffic_source` names the
+# summary.  A counter run cannot share a process with the timed passes.
+PROFILED_TRAFFIC = {
+    "config1": (626.8e6, "profiles/paged_attention_q8_d128_decode_config1.md"),
+    "config1_32k": (1147.4e6, "profiles/paged_attention_q8_d128_decode_config1_32k.md"),
+    "config0": (None, None),
+    "config3": (None, "profiles/paged_attention_q8_d128_verify_config3.md"),
+    "config2": (None, "profiles/prefill_dense_d128_config2.md"),
+    "config4": (None, "profiles/sparse_path_config4.md"),
+}
+
+
+def host_threads():
+    """(logical cores of this host, threads the CPU baselines use): the oracle runs OpenMP over (sequence, K/V head) or over
+    keys, on at most 16 threads (the box's CPU share for one GPU)."""
+    cores = os.cpu_count() or 1
+    try:
+        cores_allowed = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores_allowed = cores
+    return cores, min(cores_allowed, 16)
 
 
 def timed(gpu, step, steps, warmup):
@@ -116,7 +136,7 @@ def cpu_baseline_paged(work, sample_seqs, threads, budget_seconds=12.0):
         passes += 1
     rows = int(work.lengths[:sample_seqs].sum()) * work.kv_heads * 2 * work.row_bytes
     error = float(np.abs(got - want).max())
-    return {"value": rows / best / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+    return {"value": rows / best / 1e9, "unit": "GB/s", "cores": threads, "host_cores": host_threads()[0], "kind": "port",
             "sample": f"{sample_seqs} of {work.seqs} sequences of the same workload ({int(work.lengths[:sample_seqs].sum())} cached tokens, "
                       f"{rows / 1e6:.0f} MB of K/V rows), fastest of {passes} passes in {spent:.1f} s, OpenMP over (sequence, K/V head)",
             "tokens_per_s": sample_seqs * work.span / best}, error
@@ -156,43 +176,96 @@ def main():
     }
     copy_rate, read_rate = measured_ceilings(gpu)
 
-    def run_paged(name, with_cpu):
+    def run_paged(name, with_cpu, budget_seconds=12.0):
         work = builders[name]()
         result = paged_result(gpu, work, args.steps, args.warmup)
         baseline = None
         if with_cpu:
-            threads = min(os.cpu_count() or 1, 16)
-            sample = {"config1": 32, "config1_32k": 32, "config0": 1, "config3": 4}[name]
-            baseline, error = cpu_baseline_paged(work, min(sample, work.seqs), threads)
+            threads = host_threads()[1]
+            sample = {"config1": 32, "config1_32k": 4, "config0": 1, "config3": 1}[name]
+            baseline, error = cpu_baseline_paged(work, min(sample, work.seqs), threads, budget_seconds)
             result["max_abs_error_vs_oracle_on_sample"] = error
         work.release()
         return result, baseline
 
-    def run_sparse():
+    def cpu_baseline_sparse(work, b=0):
+        """The oracle on sequence b of the batch: canonical index scores over every key, the top-k rule, the gather attention.
+        One pass (about 131072 x 64 chains of 128 fused multiply-adds); also checks the GPU's indices and outputs of that sequence."""
+        import oracle
+        cores, threads = host_threads()
+        bf16 = lambda bits: (np.asarray(bits).astype(np.uint32) << 16).view(np.float32)
+        q = bf16(gpu.read_buffer(work.q_index, b * work.index_heads * work.index_dim * 2, np.uint16, work.index_heads * work.index_dim)).reshape(1, work.index_heads, -1)
+        keys = bf16(gpu.read_buffer(work.keys, b * work.context * work.index_dim * 2, np.uint16, work.context * work.index_dim)).reshape(work.context, -1)
+        weights = gpu.read_buffer(work.weights, b * work.index_heads * 4, np.float32, work.index_heads).reshape(1, -1)
+        aq = bf16(gpu.read_buffer(work.q, b * work.heads * work.kdim * 2, np.uint16, work.heads * work.kdim)).reshape(1, work.heads, work.kdim)
+        latents = gpu.read_buffer(work.latents, b * work.context * work.kdim * 2, np.uint16, work.context * work.kdim).reshape(work.context, work.kdim)
+        start = time.perf_counter()
+        scores = oracle.index_scores(q, keys, weights, np.array([work.context], np.int32), 1.0, threads=threads)
+        chosen = oracle.top_k(scores, work.k)
+        index_seconds = time.perf_counter() - start
+        want = oracle.latent_attention(aq, None, None, 0, latents, chosen, None, work.vdim, work.scale)
+        seconds = time.perf_counter() - start
+        got_indices = gpu.read_buffer(work.indices, b * work.k * 4, np.int32, work.k)
+        got = gpu.read_buffer(work.out, b * work.heads * work.vdim * 4, np.float32, work.heads * work.vdim).reshape(work.heads, work.vdim)
+        return {"value": seconds * work.batch * 1e6, "unit": "us/step", "cores": threads, "host_cores": cores, "kind": "port",
+                "sample": f"sequence {b} of {work.batch} (index scores over {work.context} keys in the canonical order, top-{work.k}, gather attention), one pass of "
+                          f"{seconds:.2f} s ({index_seconds:.2f} s of it the indexer), scaled by {work.batch} to the step; OpenMP over keys",
+                "indices_equal_oracle_on_sample": bool(np.array_equal(got_indices, chosen[0])),
+                "max_abs_error_vs_oracle_on_sample": float(np.abs(got - want[0]).max())}
+
+    def run_sparse(with_cpu=True):
         work = workloads.SparseWorkload(gpu)
         ms_index, bounds_ms = timed(gpu, work.step_index, max(args.steps // 5, 3), 2)
         ms_attention, gather_ms = timed(gpu, work.step_attention, max(args.steps // 5, 3), 2)
         size, keys = work.algorithmic_bytes(), work.batch * work.context * work.index_dim * 2
+        sparse_baseline = cpu_baseline_sparse(work) if with_cpu and not args.no_cpu else None
         work.release()
         total = ms_index + ms_attention
         # the timed launches: the score bounds over all keys (index_interval_kernel), the gather kernel
         return {"us_per_step": total * 1e3, "index_topk_us": ms_index * 1e3, "gather_attention_us": ms_attention * 1e3,
                 "kernel_us": None if bounds_ms is None else bounds_ms * 1e3, "key_bytes": keys,
                 "gather_kernel_us": None if gather_ms is None else gather_ms * 1e3,
-                "algorithmic_bytes": size, "gbps": size / total / 1e6, "frac_of_hbm_peak": size / total / 1e6 / HBM_PEAK_GBPS}
+                "algorithmic_bytes": size, "gbps": size / total / 1e6, "frac_of_hbm_peak": size / total / 1e6 / HBM_PEAK_GBPS,
+                "cpu_baseline": sparse_baseline}
 
-    def run_prefill():
+    def cpu_baseline_prefill(work, tokens=(2040, 4090, 6140, 8184), rows=8):
+        """The oracle on `rows` consecutive query tokens near the end of each chunk (each attends the cache up to its own position),
+        all heads: a stated part of the prompt's causal work, timed, and compared with the GPU's outputs of those tokens."""
+        import oracle
+        cores, threads = host_threads()
+        out = work.read(work.out, work.tokens * work.heads * work.dim).reshape(work.tokens, work.heads, work.dim)
+        q = work.read(work.q, work.tokens * work.heads * work.dim).reshape(work.tokens, work.heads, work.dim)
+        pool = gpu.read_buffer(work.pool_buffer, 0, np.uint8, work.pool_buffer.size)
+        wanted = [t + r for t in tokens for r in range(rows)]
+        # every sampled token as a sequence of its own over the same pages: the oracle's threads run over (sequence, K/V head)
+        table = np.repeat(work.table, len(wanted), axis=0)
+        best, error = None, 0.0
+        for _ in range(3):
+            start = time.perf_counter()
+            want = oracle.paged_attention(pool, work.row_bytes, work.page_tokens, work.kv_heads, work.dim, table, np.array(wanted, np.int32),
+                                          q[wanted][:, None], work.scale, threads=threads)
+            seconds = time.perf_counter() - start
+            best = seconds if best is None else min(best, seconds)
+        error = float(np.abs(out[wanted] - want[:, 0]).max())
+        flops = 4 * work.heads * work.dim * sum(t + 1 for t in wanted)
+        return {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "host_cores": cores, "kind": "port",
+                "sample": f"{len(wanted)} of {work.tokens} query tokens ({rows} at each of positions {list(tokens)}), all {work.heads} heads, {flops / 1e9:.2f} GFLOP of the "
+                          f"prompt's {work.flops() / 1e9:.0f}, fastest of 3 passes ({best:.2f} s), OpenMP over (token, K/V head)",
+                "max_abs_error_vs_oracle_on_sample": error}
+
+    def run_prefill(with_cpu=True):
         work = workloads.PrefillWorkload(gpu)
         steps = max(args.steps // 5, 3)
         ms, kernel_ms = timed(gpu, work.step, steps, 2)
         flops, size = work.flops(), work.algorithmic_bytes()
+        prefill_baseline = cpu_baseline_prefill(work) if with_cpu and not args.no_cpu else None
         work.release()
         # the timed kernel launches are the 4 attention kernels of a step (not the K/V writer, not the kernel that unpacks the tiles)
         return {"ms_per_step": ms, "us_per_step": ms * 1e3, "kernel_us": None if kernel_ms is None else kernel_ms * 4e3, "flops": flops,
                 "tflops": flops / ms / 1e9, "frac_of_mfma_peak": flops / ms / 1e9 / MFMA_PEAK_TFLOPS,
                 "kernel_tflops": None if kernel_ms is None else flops / (4 * kernel_ms) / 1e9,
                 "algorithmic_bytes": size, "gbps": size / ms / 1e6, "frac_of_hbm_peak": size / ms / 1e6 / HBM_PEAK_GBPS,
-                "tokens_per_s": work.tokens / (ms * 1e-3)}
+                "tokens_per_s": work.tokens / (ms * 1e-3), "cpu_baseline": prefill_baseline}
 
     def run_block_index():
         # Qwen's block indexer (scores + choice of 512 blocks) at 242K tokens: a decode row, and a prefill chunk of 256 rows
@@ -218,16 +291,20 @@ def main():
         return out
 
     if args.workload == "config4":
-        main_result, baseline = run_sparse(), None
+        main_result = run_sparse()
+        baseline = main_result.pop("cpu_baseline")
     elif args.workload == "config2":
-        main_result, baseline = run_prefill(), None
+        main_result = run_prefill()
+        baseline = main_result.pop("cpu_baseline")
     else:
         main_result, baseline = run_paged(args.workload, not args.no_cpu)
     also = {}
     if not args.no_also:
         for name in ("config1_32k", "config0", "config3"):
             if name != args.workload:
-                also[name], _ = run_paged(name, False)
+                # each config's CPU baseline beside it: the oracle on a stated part of the same workload, a few seconds each
+                also[name], also_baseline = run_paged(name, not args.no_cpu, budget_seconds=3.0)
+                also[name]["cpu_baseline"] = also_baseline
                 also[name]["workload"] = names[name]
         if args.workload != "config2":
             also["config2"] = run_prefill()
@@ -243,7 +320,7 @@ def main():
     kernel_us = main_result.get("kernel_us")
     achieved = main_result["algorithmic_bytes"] / (kernel_us * 1e-6) / 1e9 if kernel_us else main_result["gbps"]
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
-                "traffic": MEASURED_TRAFFIC.get(args.workload),
+                "traffic": PROFILED_TRAFFIC[args.workload][0], "traffic_source": PROFILED_TRAFFIC[args.workload][1],
                 "kernel": "paged_attention_kernel<128,3,Q8_0>" if args.workload == "config3" else "paged_attention_kernel<128,1,Q8_0>", "kernel_us": kernel_us, "measured_copy_gbps": copy_rate, "measured_read_gbps": read_rate}
     if args.workload == "config4" and kernel_us:
         # the dominant kernel reads every index key once: its algorithmic bytes are the keys
@@ -252,7 +329,7 @@ def main():
     if args.workload == "config2":
         achieved = main_result["kernel_tflops"] or main_result["tflops"]
         roofline = {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
-                    "traffic": None, "kernel": "prefill_dense_kernel<128,2>", "kernel_us": kernel_us,
+                    "traffic": PROFILED_TRAFFIC["config2"][0], "traffic_source": PROFILED_TRAFFIC["config2"][1], "kernel": "prefill_dense_kernel<128,2>", "kernel_us": kernel_us,
                     "measured_mfma_tflops": measured_mfma_ceiling(gpu, False),
                     "measured_mfma_tflops_live_operands": measured_mfma_ceiling(gpu, True)}
     line = {
@@ -262,7 +339,7 @@ def main():
         "config": {"workload": names[args.workload], "batch": 32 if args.workload.startswith("config1") else None},
         "tokens_per_s": main_result.get("tokens_per_s"), "frac_of_hbm_peak": main_result["frac_of_hbm_peak"],
         "roofline": roofline,
-        "cpu_baseline": baseline, "detail": main_result, "also": also,
+        "cpu_baseline": baseline, "host": {"cores": host_threads()[0], "cpu_threads_used": host_threads()[1]}, "detail": main_result, "also": also,
     }
     print(json.dumps(line))
     gpu.close()
