@@ -18,7 +18,7 @@ void select_thin_reserve(Device& d);     // block_index.hip
 // graphs recorded so far would replay on freed memory: they are dropped, sd_graph_run then answers 1 ("none stored under
 // this key") and the caller records again -- what the reference does when its K/V views change (kv_clear_graphs,
 // gpu/kv_stage.hpp:96-104).
-static void drop_graphs(Device& d) {
+void drop_recorded_graphs(Device& d) {
     for (auto& entry : d.graphs) {
         if (entry.second.executable) (void)hipGraphExecDestroy(entry.second.executable);
         if (entry.second.graph) (void)hipGraphDestroy(entry.second.graph);
@@ -107,7 +107,7 @@ void* workspace(Device& d, size_t bytes) {
     SD_CHECK(hipStreamIsCapturing(d.stream, &capturing));
     if (capturing != hipStreamCaptureStatusNone) throw std::runtime_error("Straydog attention workspace cannot grow while a graph is recorded");
     if (d.workspace) {
-        drop_graphs(d);
+        drop_recorded_graphs(d);
         release(d, d.workspace);
     }
     d.workspace = nullptr; d.workspace_bytes = 0;

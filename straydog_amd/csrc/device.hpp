@@ -63,6 +63,8 @@ struct Device {
     std::map<const void*, size_t> shared_limits;
     // This device's address of the partial-result area the library itself holds for sdx_paged_attention_static.
     float* paged_static = nullptr;
+    // The matrix-core indexer's radix histograms (index_topk.hip): all zero between calls.
+    uint32_t* index_bins = nullptr; size_t index_bins_rows = 0; bool index_bins_dirty = false;
     // The lists of a short span's thinned index rows (block_index.hip), allocated at the first such call and kept.
     void* select_thin = nullptr;
     // Page-locked host copies of sequence state (conversation checkpoints): pointer -> bytes.
@@ -111,6 +113,8 @@ void upload(Device& d, void* target, const void* data, size_t bytes);     // cal
 void download(Device& d, void* output, const void* source, size_t bytes);  // device -> caller memory, waits
 // A workspace of at least `bytes` that lives with the device; grows only outside graph capture.
 void* workspace(Device& d, size_t bytes);
+// Recorded graphs hold the addresses of the library's own buffers: when one of them moves, the graphs recorded so far go.
+void drop_recorded_graphs(Device& d);
 
 // [pointer, pointer + bytes) must lie inside one live allocation of this device.
 void op_span(Device& d, const void* pointer, size_t bytes, const char* what);

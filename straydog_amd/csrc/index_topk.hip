@@ -367,55 +367,32 @@ __device__ __forceinline__ void load_to_lds(const void* from, const void* to) {
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt\n\ts_mov_b32 m0, %0" : "=&s"(keep) : "v"(from), "s"(base) : "memory");
 }
 
-// Before the bounds, a few workgroups per row: the row's histograms zeroed, its queries widened to FP32 for the canonical
-// rescoring, and (the first of them) W of the margin: sum_h |w_h| |q_h| * |scale| * 2^-14, rounded up a little.
-__global__ void __launch_bounds__(256) index_prepare_kernel(const uint16_t* q, const float* weights, size_t heads, size_t dim, float scale, size_t rows,
-                                                            float* margin, float* wide_q, uint32_t* histogram) {
-    const size_t row = blockIdx.x;
-    const unsigned t = threadIdx.x, h = t / 4, part = t % 4, slice = blockIdx.y, slices = gridDim.y;
-    for (int level = 0; level < RADIX_LEVELS; ++level)
-        for (unsigned i = slice * 256 + t; i < unsigned(RADIX_BINS); i += slices * 256) histogram[(size_t(level) * rows + row) * RADIX_BINS + i] = 0u;
-    // (transposed, [column][head]: a lane per head then reads neighbouring words)
-    for (size_t i = slice * 256 + t; i < heads * dim; i += slices * 256) wide_q[row * heads * dim + (i % dim) * heads + i / dim] = bf16_value(q[row * heads * dim + i]);
-    if (slice) return;
-    // four lanes per head, 8 values a load
-    float square = 0.0f;
-    if (h < heads)
-        for (size_t d = 8 * part; d < dim; d += 32) {
-            const uint4 bits = *reinterpret_cast<const uint4*>(q + (row * heads + h) * dim + d);
-            const uint32_t words[4] = {bits.x, bits.y, bits.z, bits.w};
-            #pragma unroll
-            for (int i = 0; i < 4; ++i) { const float a = __uint_as_float(words[i] << 16), b = __uint_as_float(words[i] & 0xffff0000u); square += a * a + b * b; }
-        }
-    square += __shfl_xor(square, 1);
-    square += __shfl_xor(square, 2);
-    float total = h < heads && part == 0 ? fabsf(weights[row * heads + h]) * sqrtf(square) : 0.0f;
-    #pragma unroll
-    for (int d = 32; d; d >>= 1) total += __shfl_xor(total, d);
-    __shared__ float waves[4];
-    if ((t & 63) == 0) waves[t >> 6] = total;
-    __syncthreads();
-    if (t == 0) margin[row] = (waves[0] + waves[1] + waves[2] + waves[3]) * fabsf(scale) * (1.0f / 16384.0f) * 1.01f;
-}
-
 // Bounds of the scores of INTERVAL_KEYS groups per workgroup, 16 groups per MFMA tile and wave, and the first radix
 // histogram of the lower bounds.  S = Q . K^T with Q (heads x dim) as A operands from registers and K rows as B operands;
 // K . K^T from the same registers gives |k|^2 on its diagonal.  A tile's 16 rows are 4 KiB in one piece: they come HBM -> LDS
 // by four coalesced 1 KiB global->LDS loads into the wave's ring of stages, three tiles ahead of the one being computed
 // (two waves per SIMD leave room for that much in flight).  The loads place piece c of row r at position c ^ r of the row, so that the 16 lanes of an operand read (one
 // row each, the same piece) touch 16 different banks.
+// The histograms' place: [level][row][bin], and behind them the rows' largest margins (bits of a non-negative float, so that an
+// integer atomic maximum orders them).  `rows` = the rows the buffer was made for.
+__device__ __forceinline__ uint32_t* radix_bins(uint32_t* histogram, size_t rows, int level, size_t row) {
+    return histogram + (size_t(level) * rows + row) * RADIX_BINS;
+}
+__device__ __forceinline__ uint32_t* widest_margin(uint32_t* histogram, size_t rows, size_t row) { return histogram + size_t(RADIX_LEVELS) * rows * RADIX_BINS + row; }
+
 template<int HEADS>
 __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
-                                                             const int32_t* __restrict__ visible, const float* __restrict__ margin, size_t groups, float scale,
-                                                             float* __restrict__ lower, float* __restrict__ upper, uint32_t* __restrict__ histogram) {
+                                                             const int32_t* __restrict__ visible, size_t groups, float scale,
+                                                             float* __restrict__ lower, float* __restrict__ upper, uint32_t* __restrict__ histogram, size_t histogram_rows) {
     constexpr int DIM = 128, HT = HEADS / 16, KS = DIM / 32;
     const size_t row = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, g = lane >> 4;
     __shared__ uint32_t bins[RADIX_BINS];
     __shared__ __attribute__((aligned(16))) uint8_t stages[BRACKET_WAVES][BRACKET_RING][4096];
     for (int i = threadIdx.x; i < RADIX_BINS; i += BRACKET_WAVES * 64) bins[i] = 0;
+    float widest = 0.0f;            // the largest margin this lane has given a live group
     bf16x8 qa[HT][KS];
-    float w[HT][4];
+    float w[HT][4], own[HT];
     #pragma unroll
     for (int t = 0; t < HT; ++t) {
         #pragma unroll
@@ -423,12 +400,11 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
             qa[t][b] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(q + (row * HEADS + 16 * t + li) * DIM + 32 * b + 8 * g));
         #pragma unroll
         for (int r = 0; r < 4; ++r) w[t][r] = weights[row * HEADS + 16 * t + 4 * g + r];
+        own[t] = weights[row * HEADS + 16 * t + li];
     }
     const int32_t seen = visible[row];
     const size_t limit = min(groups, size_t(seen > 0 ? seen : 0));
-    const float bound = margin[row];
     const uint16_t* row_keys = keys + row * groups * DIM;
-    __syncthreads();
     const size_t first = size_t(blockIdx.x) * BRACKET_KEYS, end = min(first + BRACKET_KEYS, groups);
     const auto copy_in = [&](int buffer, size_t tile) {
         #pragma unroll
@@ -440,10 +416,32 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
     };
     constexpr size_t stride = 16 * BRACKET_WAVES;
     size_t tile = first + 16 * wave;
-    __builtin_amdgcn_s_waitcnt(0x0f70);      // the queries and weights are in: the compiler's wait for them stays out of the loop
+    // the first tiles are asked for before anything waits for the queries: they travel while the margin is worked out
     #pragma unroll
     for (int ahead = 0; ahead < BRACKET_RING - 1; ++ahead)
         if (tile + ahead * stride < end) copy_in(ahead, tile + ahead * stride);
+    // W of the margin, sum_h |w_h| |q_h|, by every wave for itself: a lane's 32 values of head 16t + li squared and summed, the
+    // four lane groups' parts added, the root times |w_h| added over the tile's 16 heads (lanes) and the tiles
+    float reach = 0.0f;
+    #pragma unroll
+    for (int t = 0; t < HT; ++t) {
+        float square = 0.0f;
+        #pragma unroll
+        for (int b = 0; b < KS; ++b) {
+            const uint4 bits = __builtin_bit_cast(uint4, qa[t][b]);
+            const uint32_t words[4] = {bits.x, bits.y, bits.z, bits.w};
+            #pragma unroll
+            for (int i = 0; i < 4; ++i) { const float lo = __uint_as_float(words[i] << 16), hi = __uint_as_float(words[i] & 0xffff0000u); square += lo * lo + hi * hi; }
+        }
+        reach += fabsf(own[t]) * sqrtf(quad_sum(square));
+    }
+    #pragma unroll
+    for (int d = 8; d; d >>= 1) reach += __shfl_xor(reach, d);
+    const float bound = reach * fabsf(scale) * (1.0f / 16384.0f) * 1.01f;      // 2^-14 |scale| W, rounded up a little
+    __syncthreads();                         // the histogram's bins are zero
+    // (the wait for the queries above was a wait for every load so far, the first tiles' among them: none of the compiler's
+    // own loads is outstanding, and the loop's waits count the tiles' loads alone)
+    __builtin_amdgcn_s_waitcnt(0x0f70);
     for (int buffer = 0; tile < end; tile += stride, buffer = (buffer + 1) % BRACKET_RING) {
         const size_t group = tile + li;
         if (tile + (BRACKET_RING - 1) * stride < end) copy_in((buffer + BRACKET_RING - 1) % BRACKET_RING, tile + (BRACKET_RING - 1) * stride);
@@ -478,27 +476,49 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
             lower[row * groups + group] = low;
             upper[row * groups + group] = high;
             const uint32_t key = top_k_key(low);
-            if (key > top_k_key(-INFINITY)) atomicAdd(&bins[radix_digit(key, 0)], 1u);
+            if (histogram && key > top_k_key(-INFINITY)) atomicAdd(&bins[radix_digit(key, 0)], 1u);
+            if (live) widest = fmaxf(widest, e);
         }
     }
+    if (!histogram) return;
+    #pragma unroll
+    for (int d = 32; d; d >>= 1) widest = fmaxf(widest, __shfl_xor(widest, d));
+    __shared__ uint32_t widest_of_all;
+    if (threadIdx.x == 0) widest_of_all = 0u;
     __syncthreads();
+    if (lane == 0 && widest > 0.0f) atomicMax(&widest_of_all, __float_as_uint(widest));
+    __syncthreads();
+    // (one atomic per workgroup and row: hundreds of waves on one address would queue up at the end of the kernel)
+    if (threadIdx.x == 0 && widest_of_all) atomicMax(widest_margin(histogram, histogram_rows, row), widest_of_all);
+    uint32_t* to = radix_bins(histogram, histogram_rows, 0, row);
     for (int i = threadIdx.x; i < RADIX_BINS; i += BRACKET_WAVES * 64)
-        if (bins[i]) atomicAdd(&histogram[row * RADIX_BINS + i], bins[i]);
+        if (bins[i]) atomicAdd(&to[i], bins[i]);
 }
 
 // Where the rank-th highest key lies, one digit at a time, from the levels' histograms (256 threads, every workgroup
 // that needs it finds it anew).  After `levels` digits: the key's leading digits and the rank among the keys that share
 // them; `everything` when fewer than rank keys are live at all.
 struct RadixPick { uint32_t prefix, rank; bool everything; };
-__device__ RadixPick radix_pick(const uint32_t* histogram /* [level][rows][RADIX_BINS] */, size_t rows, size_t row, int levels, uint32_t k) {
+__device__ RadixPick radix_pick(uint32_t* histogram, size_t rows, size_t row, int levels, uint32_t k) {
     __shared__ uint32_t wave_sums[4], found[2];
     RadixPick pick{0u, k, false};
     const unsigned t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    for (int level = 0; level < levels; ++level) {
-        const uint32_t* bins = histogram + (size_t(level) * rows + row) * RADIX_BINS;
-        // thread t owns the 8 bins below 2048 - 8t, highest first; a scan in thread order counts the keys in higher bins
+    // thread t owns the 8 bins below 2048 - 8t of every level, highest first; all levels are asked for at once (a level's histogram
+    // is one array whatever the digits before it turn out to be), so the levels cost one trip to memory, not one each
+    uint4 loaded[RADIX_LEVELS][2];
+    #pragma unroll
+    for (int level = 0; level < RADIX_LEVELS; ++level)
+        if (level < levels) {
+            const uint32_t* bins = radix_bins(histogram, rows, level, row);
+            loaded[level][0] = *reinterpret_cast<const uint4*>(bins + RADIX_BINS - 8 - 8 * t);
+            loaded[level][1] = *reinterpret_cast<const uint4*>(bins + RADIX_BINS - 4 - 8 * t);
+        }
+    #pragma unroll
+    for (int level = 0; level < RADIX_LEVELS; ++level) {
+        if (level >= levels) break;
+        // a scan in thread order counts the keys in higher bins
         uint32_t mine[8], sum = 0;
-        const uint4 a = *reinterpret_cast<const uint4*>(bins + RADIX_BINS - 8 - 8 * t), b = *reinterpret_cast<const uint4*>(bins + RADIX_BINS - 4 - 8 * t);
+        const uint4 a = loaded[level][0], b = loaded[level][1];
         mine[0] = b.w; mine[1] = b.z; mine[2] = b.y; mine[3] = b.x; mine[4] = a.w; mine[5] = a.z; mine[6] = a.y; mine[7] = a.x;
         #pragma unroll
         for (int i = 0; i < 8; ++i) sum += mine[i];
@@ -527,141 +547,276 @@ __device__ RadixPick radix_pick(const uint32_t* histogram /* [level][rows][RADIX
     return pick;
 }
 
-// The histogram of digit `level` over the keys that share the digits found so far.
-__global__ void __launch_bounds__(256) radix_histogram_kernel(const float* values, size_t groups, size_t rows, int level, uint32_t k, uint32_t* histogram) {
+// The second digit's histogram of the lower bounds, over the keys that share the first digit of the k-th highest.
+__global__ void __launch_bounds__(256) radix_histogram_kernel(const float* lower, size_t groups, size_t rows, uint32_t k, uint32_t* histogram) {
     const size_t row = blockIdx.y;
     __shared__ uint32_t bins[RADIX_BINS];
     for (int i = threadIdx.x; i < RADIX_BINS; i += 256) bins[i] = 0;
-    const RadixPick pick = radix_pick(histogram, rows, row, level, k);
+    // (the groups' values are asked for before the pick's own trip to memory ends)
+    const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS;
+    float values[INTERVAL_KEYS / 256];
+    #pragma unroll
+    for (int j = 0; j < INTERVAL_KEYS / 256; ++j) { const size_t group = first + threadIdx.x + 256 * j; values[j] = group < groups ? lower[row * groups + group] : -INFINITY; }
+    const RadixPick pick = radix_pick(histogram, rows, row, 1, k);
     __syncthreads();
     if (pick.everything) return;
-    const uint32_t mask = level == 1 ? 0xffe00000u : 0xfffffc00u;
-    const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS;
-    for (size_t group = first + threadIdx.x; group < min(first + INTERVAL_KEYS, groups); group += 256) {
-        const uint32_t key = top_k_key(values[row * groups + group]);
-        if ((key & mask) == pick.prefix) atomicAdd(&bins[radix_digit(key, level)], 1u);
+    #pragma unroll
+    for (int j = 0; j < INTERVAL_KEYS / 256; ++j) {
+        const uint32_t key = top_k_key(values[j]);
+        if ((key & 0xffe00000u) == pick.prefix && key > top_k_key(-INFINITY)) atomicAdd(&bins[radix_digit(key, 1)], 1u);
     }
     __syncthreads();
-    uint32_t* to = histogram + (size_t(level) * rows + row) * RADIX_BINS;
+    uint32_t* to = radix_bins(histogram, rows, 1, row);
     for (int i = threadIdx.x; i < RADIX_BINS; i += 256)
         if (bins[i]) atomicAdd(&to[i], bins[i]);
 }
 
-// Candidates: groups whose upper bound reaches the k-th highest lower bound (every live group when fewer than k are live).
-__device__ __forceinline__ bool is_candidate(float high, const RadixPick& pick) {
-    const uint32_t key = top_k_key(high);
-    return pick.everything ? key > top_k_key(-INFINITY) : key >= pick.prefix;
-}
-__global__ void __launch_bounds__(256) candidate_count_kernel(const float* upper, size_t groups, size_t rows, uint32_t k, const uint32_t* histogram,
-                                                              uint32_t* counts) {
+// Which groups can still matter, a workgroup per INTERVAL_KEYS groups of a row (a segment), listed in index order in the
+// segment's own stretch of `list` (no counting pass over the row first: a reader adds up the segments' counts).
+//   candidate   upper bound >= the k-th highest lower bound (its leading 22 bits): nobody else can be among the best k;
+//   certain     lower bound above L + 2 E, L the k-th highest lower bound (the next 22-bit step above it) and E the row's widest
+//               margin: no upper bound is more than 2 E above its lower bound, so the k-th highest upper bound is at most
+//               L + 2 E, fewer than k groups can score as high as this one, and it is among the best k whatever its exact
+//               score -- it is listed with the CERTAIN bit and needs no canonical score;
+//   the rest of the candidates are the band around the cut: only they are scored canonically.
+// With fewer than k live groups everything live is a certain candidate.
+constexpr uint32_t CERTAIN = 0x80000000u;
+__global__ void __launch_bounds__(256) candidate_segments_kernel(const float* lower, const float* upper, size_t groups, size_t rows, uint32_t k, uint32_t* histogram,
+                                                                 int32_t* list, uint32_t* counts) {
     const size_t row = blockIdx.y;
+    const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS + 4 * threadIdx.x;        // thread t owns 4 consecutive groups
+    // (the groups' bounds are asked for before the pick's own trip to memory ends)
+    float low[4], high[4];
+    if (first + 3 < groups && (row * groups) % 4 == 0) {
+        const float4 l4 = *reinterpret_cast<const float4*>(lower + row * groups + first), h4 = *reinterpret_cast<const float4*>(upper + row * groups + first);
+        low[0] = l4.x; low[1] = l4.y; low[2] = l4.z; low[3] = l4.w; high[0] = h4.x; high[1] = h4.y; high[2] = h4.z; high[3] = h4.w;
+    } else {
+        #pragma unroll
+        for (int i = 0; i < 4; ++i) { const bool in = first + i < groups; low[i] = in ? lower[row * groups + first + i] : -INFINITY; high[i] = in ? upper[row * groups + first + i] : -INFINITY; }
+    }
+    const float widest = __uint_as_float(*widest_margin(histogram, rows, row));
     const RadixPick pick = radix_pick(histogram, rows, row, RADIX_LEVELS, k);
-    __shared__ uint32_t total;
-    if (threadIdx.x == 0) total = 0;
-    __syncthreads();
-    const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS;
-    uint32_t mine = 0;
-    for (size_t group = first + threadIdx.x; group < min(first + INTERVAL_KEYS, groups); group += 256) mine += is_candidate(upper[row * groups + group], pick);
+    const uint32_t floor = top_k_key(-INFINITY);
+    // L's 22-bit step taken upwards as a value, 2 E added and the sum pushed up a little: a bound on the k-th highest upper bound
+    float certain_above = INFINITY;
+    if (!pick.everything && pick.prefix <= 0xffffffffu - 1024u) {
+        const uint32_t key = pick.prefix + 1024u, bits = key & 0x80000000u ? key ^ 0x80000000u : ~key;
+        const float sum = __uint_as_float(bits) + 2.0f * widest;
+        certain_above = sum + fabsf(sum) * 1.0e-6f;
+        if (!(certain_above == certain_above)) certain_above = INFINITY;      // a NaN in the bounds: nothing is certain
+    }
+    __shared__ uint32_t wave_sums[4];
+    uint32_t entry[4], mine = 0, band = 0;
     #pragma unroll
-    for (int d = 32; d; d >>= 1) mine += __shfl_xor(mine, d);
-    if ((threadIdx.x & 63) == 0) atomicAdd(&total, mine);
-    __syncthreads();
-    if (threadIdx.x == 0) counts[row * gridDim.x + blockIdx.x] = total;
-}
-// ... listed in index order: a workgroup's candidates follow those of the workgroups before it.
-__global__ void __launch_bounds__(256) candidate_list_kernel(const float* upper, size_t groups, size_t rows, uint32_t k, const uint32_t* histogram,
-                                                             const uint32_t* counts, int32_t* list, uint32_t* totals) {
-    const size_t row = blockIdx.y;
-    const RadixPick pick = radix_pick(histogram, rows, row, RADIX_LEVELS, k);
-    __shared__ uint32_t wave_sums[4], base;
-    uint32_t before = 0;
-    for (unsigned b = threadIdx.x; b < gridDim.x; b += 256) before += b < blockIdx.x ? counts[row * gridDim.x + b] : 0u;
-    #pragma unroll
-    for (int d = 32; d; d >>= 1) before += __shfl_xor(before, d);
-    if (threadIdx.x == 0) base = 0;
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) atomicAdd(&base, before);
-    __syncthreads();
-    // thread t owns 4 consecutive groups
-    const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS + 4 * threadIdx.x;
-    bool keep[4];
-    uint32_t mine = 0;
-    #pragma unroll
-    for (int i = 0; i < 4; ++i) { keep[i] = first + i < groups && is_candidate(upper[row * groups + first + i], pick); mine += keep[i]; }
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t high_key = top_k_key(high[i]);
+        const bool keep = first + i < groups && (pick.everything ? high_key > floor : high_key >= pick.prefix);
+        const bool certain = pick.everything || low[i] > certain_above;
+        entry[i] = keep ? uint32_t(first + i) | (certain ? CERTAIN : 0u) : 0xffffffffu;
+        mine += keep;
+        band += keep && !certain;
+    }
     const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    uint32_t inclusive = mine;
+    uint32_t packed = mine | (band << 16), inclusive = packed;        // both counts scanned at once (at most 1024 each)
     #pragma unroll
     for (unsigned offset = 1; offset < 64; offset *= 2) { const uint32_t other = __shfl_up(inclusive, offset); if (lane >= offset) inclusive += other; }
     if (lane == 63) wave_sums[wave] = inclusive;
     __syncthreads();
-    uint32_t at = base + inclusive - mine;
-    for (unsigned v = 0; v < wave; ++v) at += wave_sums[v];
+    uint32_t before = 0, all = 0;
+    for (unsigned v = 0; v < 4; ++v) { before += v < wave ? wave_sums[v] : 0u; all += wave_sums[v]; }
+    uint32_t at = ((before + inclusive - packed) & 0xffffu);
+    int32_t* out = list + row * groups + size_t(blockIdx.x) * INTERVAL_KEYS;
     #pragma unroll
-    for (int i = 0; i < 4; ++i) if (keep[i]) list[row * groups + at++] = int32_t(first + i);
-    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 255) totals[row] = at;
+    for (int i = 0; i < 4; ++i) if (entry[i] != 0xffffffffu) out[at++] = int32_t(entry[i]);
+    if (threadIdx.x == 0) counts[row * gridDim.x + blockIdx.x] = all;        // candidates | band members << 16
 }
 
-// The canonical score of every listed group: a wave takes a few groups at a time, a lane per head with the head's 128 query
+// The canonical score of the band's groups.  A wave takes a segment at a time (every SCORE_STRIDE-th one), finds the band
+// members among the segment's candidates by a ballot, and scores them a few at a time: a lane per head with the head's 128 query
 // values in its registers; a key row is 64 words, lane i fetches word i (one coalesced load, the next group's row on its
 // way while this one is used) and the words go round by v_readlane, so a group costs a wave 64 broadcasts and 128
 // multiply-adds in the canonical column order.  Then each group's 64 terms are added in head order -- lane c the terms of
-// group c, read from LDS, so the ordered sums run side by side.
+// group c, read from LDS, so the ordered sums run side by side.  A score lands at its group's place in the list.
 template<int HEADS>
-__global__ void __launch_bounds__(SCORE_WAVES * 64) candidate_score_kernel(const float* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
-                                                              size_t groups, float scale, const int32_t* __restrict__ list, const uint32_t* __restrict__ totals,
-                                                              float* __restrict__ scores) {
+__global__ void __launch_bounds__(SCORE_WAVES * 64) band_score_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
+                                                         size_t groups, float scale, const int32_t* __restrict__ list, const uint32_t* __restrict__ counts,
+                                                         size_t segments, float* __restrict__ scores, uint32_t* __restrict__ histogram, size_t histogram_rows) {
     constexpr int DIM = 128, BATCH = SCORE_BATCH;
     const size_t row = blockIdx.y;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // The histograms' last reader ran before this kernel: the row's first workgroup zeroes them (and the widest margin) for the
+    // next call, while everything below goes on.
+    if (blockIdx.x == 0) {
+        for (int level = 0; level < RADIX_LEVELS; ++level) {
+            uint32_t* bins = radix_bins(histogram, histogram_rows, level, row);
+            for (unsigned i = threadIdx.x; i < unsigned(RADIX_BINS); i += SCORE_WAVES * 64) bins[i] = 0u;
+        }
+        if (threadIdx.x == 0) *widest_margin(histogram, histogram_rows, row) = 0u;
+    }
     const int head = min(lane, HEADS - 1);
-    const uint32_t total = totals[row];
-    if (blockIdx.x * SCORE_WAVES * BATCH >= total) return;
     __shared__ float terms[SCORE_WAVES][BATCH][HEADS + 1];
+    __shared__ uint32_t places[SCORE_WAVES][64];
+    // the head's query values, widened (asked for at once: a wave with nothing to score has wasted a few loads from the cache)
     float mine[DIM];
     #pragma unroll
-    for (int d = 0; d < DIM; ++d) mine[d] = q[(row * DIM + d) * HEADS + head];          // [column][head]
+    for (int d = 0; d < DIM; d += 8) {
+        const uint4 bits = *reinterpret_cast<const uint4*>(q + (row * HEADS + head) * DIM + d);
+        const uint32_t words[4] = {bits.x, bits.y, bits.z, bits.w};
+        #pragma unroll
+        for (int i = 0; i < 4; ++i) { mine[d + 2 * i] = __uint_as_float(words[i] << 16); mine[d + 2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u); }
+    }
     const float weight = weights[row * HEADS + head];
     const uint32_t* row_keys = reinterpret_cast<const uint32_t*>(keys + row * groups * DIM);
-    for (uint32_t first = (blockIdx.x * SCORE_WAVES + wave) * BATCH; first < total; first += gridDim.x * SCORE_WAVES * BATCH) {
-        const int count = int(min(uint32_t(BATCH), total - first));
-        uint32_t words = row_keys[size_t(list[row * groups + first]) * (DIM / 2) + lane];
-        for (int c = 0; c < count; ++c) {
-            const uint32_t current = words;
-            if (c + 1 < count) words = row_keys[size_t(list[row * groups + first + c + 1]) * (DIM / 2) + lane];
-            float dot = 0.0f;
-            #pragma unroll
-            for (int d = 0; d < DIM; d += 2) {
-                const uint32_t pair = __builtin_amdgcn_readlane(current, d / 2);
-                dot = __builtin_fmaf(mine[d], __uint_as_float(pair << 16), dot);
-                dot = __builtin_fmaf(mine[d + 1], __uint_as_float(pair & 0xffff0000u), dot);
+    for (size_t segment = size_t(blockIdx.x) * SCORE_WAVES + wave; segment < segments; segment += size_t(gridDim.x) * SCORE_WAVES) {
+        const uint32_t count = counts[row * segments + segment];
+        if (!(count >> 16)) continue;                                  // no band member here (wave-uniform)
+        const int32_t* entries = list + row * groups + segment * INTERVAL_KEYS;
+        for (uint32_t base = 0; base < (count & 0xffffu); base += 64) {
+            const uint32_t entry = base + uint32_t(lane) < (count & 0xffffu) ? uint32_t(entries[base + lane]) : CERTAIN;
+            const uint64_t wanted = __ballot(!(entry & CERTAIN));
+            if (!wanted) continue;
+            // the band members' lanes in order: member m of this chunk sits at lane places[m]
+            const int members = __popcll(wanted);
+            if (!(entry & CERTAIN)) places[wave][__popcll(wanted & ((uint64_t(1) << lane) - 1))] = uint32_t(lane);
+            for (int done = 0; done < members; done += BATCH) {
+                const int batch = min(BATCH, members - done);
+                uint32_t words = row_keys[size_t(__shfl(entry, int(places[wave][done]))) * (DIM / 2) + lane];
+                for (int c = 0; c < batch; ++c) {
+                    const uint32_t current = words;
+                    if (c + 1 < batch) words = row_keys[size_t(__shfl(entry, int(places[wave][done + c + 1]))) * (DIM / 2) + lane];
+                    float dot = 0.0f;
+                    #pragma unroll
+                    for (int d = 0; d < DIM; d += 2) {
+                        const uint32_t pair = __builtin_amdgcn_readlane(current, d / 2);
+                        dot = __builtin_fmaf(mine[d], __uint_as_float(pair << 16), dot);
+                        dot = __builtin_fmaf(mine[d + 1], __uint_as_float(pair & 0xffff0000u), dot);
+                    }
+                    if (lane < HEADS) terms[wave][c][lane] = rounded_product(fmaxf(dot, 0.0f), weight);
+                }
+                // the wave's own writes, read back by the wave: LDS keeps a wave's accesses in order
+                if (lane < batch) {
+                    float sum = 0.0f;
+                    #pragma unroll
+                    for (int h = 0; h < HEADS; ++h) sum = rounded_sum(sum, terms[wave][lane][h]);
+                    scores[row * groups + segment * INTERVAL_KEYS + base + places[wave][done + lane]] = rounded_product(sum, scale);
+                }
             }
-            if (lane < HEADS) terms[wave][c][lane] = rounded_product(fmaxf(dot, 0.0f), weight);
-        }
-        // the wave's own writes, read back by the wave: LDS keeps a wave's accesses in order
-        if (lane < count) {
-            float sum = 0.0f;
-            #pragma unroll
-            for (int h = 0; h < HEADS; ++h) sum = rounded_sum(sum, terms[wave][lane][h]);
-            scores[row * groups + first + lane] = rounded_product(sum, scale);
         }
     }
 }
 
-// The exact top-k over a row's listed groups (scores in list order, which is index order).
-__global__ void __launch_bounds__(TOPK_THREADS) top_k_listed_kernel(const float* scores, const int32_t* list, const uint32_t* totals, size_t groups, size_t k,
-                                                                    int32_t* out) {
-    const float* s = scores + size_t(blockIdx.x) * groups;
-    const int32_t* c = list + size_t(blockIdx.x) * groups;
-    const uint32_t total = totals[blockIdx.x];
-    // the select passes over the scores five times: a list this short (k and a few) is read from memory once
-    constexpr uint32_t HELD = 6144;
+// The row's best k from its candidates, one workgroup per row: every certain candidate, and of the band the best by canonical
+// score (ties to the lowest index) for the places that are left; ascending indices, -1 past the last.  The segments' lists are
+// first laid end to end -- in LDS when they fit, else in `flat` (global) -- with one synthetic score each: +inf for a certain
+// candidate (above every band member, as it is known to be), the canonical score for a band member; the exact top-k over that
+// row is then the result.  A band of at most a thousand is ranked directly (every member counts who beats it, one thread
+// each); anything larger takes the general radix select.
+__global__ void __launch_bounds__(TOPK_THREADS) index_finish_kernel(const float* scores, const int32_t* list, const uint32_t* counts, size_t segments, size_t groups,
+                                                                    size_t k, float* flat_scores, int32_t* flat_list, int32_t* out) {
+    const size_t row = blockIdx.x;
+    const unsigned t = threadIdx.x;
+    constexpr uint32_t HELD = 6144, RANKED = 1024;
     __shared__ float held_scores[HELD];
     __shared__ int32_t held_list[HELD];
-    if (total <= HELD) {
-        for (uint32_t v = threadIdx.x; v < total; v += TOPK_THREADS) { held_scores[v] = s[v]; held_list[v] = c[v]; }
+    __shared__ uint32_t segment_base[TOPK_THREADS];
+    __shared__ __attribute__((aligned(16))) uint64_t band_order[RANKED + 2];     // a member's key above its place turned over: a higher value beats a lower one
+    __shared__ uint32_t wave_sums[TOPK_WAVES], band_filled;
+    // the candidates and band members of the row, and where each segment's candidates go in the flat list
+    uint32_t candidates = 0, band = 0;
+    for (size_t first = 0; first < segments; first += TOPK_THREADS) {
+        const uint32_t count = first + t < segments ? counts[row * segments + first + t] : 0u;
+        uint32_t all;
+        const uint32_t before = block_scan(count, wave_sums, all);       // (two 16-bit sums side by side: a row has fewer than 65536 of
+        if (first == 0) segment_base[t] = before & 0xffffu;               //  each only when it fits the fast path, which is checked below)
+        candidates += all & 0xffffu; band += all >> 16;
         __syncthreads();
-        top_k_row([&](size_t v) { return held_scores[v]; }, [&](size_t v) { return held_list[v]; }, total, k, out + size_t(blockIdx.x) * k);
-    } else top_k_row([=](size_t v) { return s[v]; }, [=](size_t v) { return c[v]; }, total, k, out + size_t(blockIdx.x) * k);
+    }
+    // exact counts for long rows (the packed sums above may have carried): recount separately when the row is large
+    if (segments > TOPK_THREADS || groups > 65535) {
+        uint32_t c = 0, b = 0;
+        for (size_t s = t; s < segments; s += TOPK_THREADS) { const uint32_t count = counts[row * segments + s]; c += count & 0xffffu; b += count >> 16; }
+        uint32_t all;
+        (void)block_scan(c, wave_sums, all); candidates = all; __syncthreads();
+        (void)block_scan(b, wave_sums, all); band = all; __syncthreads();
+    }
+    const bool held = candidates <= HELD && segments <= TOPK_THREADS;
+    float* const row_scores = held ? held_scores : flat_scores + row * groups;
+    int32_t* const row_list = held ? held_list : flat_list + row * groups;
+    if (t == 0) band_filled = 0;
+    if (held) {
+        // a thread per place of the flat list: the segment that holds it by bisection, then one trip to memory for all of them
+        __syncthreads();
+        for (uint32_t place = t; place < candidates; place += TOPK_THREADS) {
+            uint32_t segment = 0;
+            for (uint32_t step = TOPK_THREADS / 2; step; step /= 2)
+                if (segment + step < segments && segment_base[segment + step] <= place) segment += step;
+            // (segments without candidates share their base with the next one: move on to the one that really holds the place)
+            const size_t at = row * groups + size_t(segment) * INTERVAL_KEYS + (place - segment_base[segment]);
+            const uint32_t entry = uint32_t(list[at]);
+            const bool certain = entry & CERTAIN;
+            const float score = certain ? INFINITY : scores[at];
+            held_scores[place] = score;
+            held_list[place] = int32_t(entry & ~CERTAIN);
+            if (!certain && band <= RANKED) {
+                const uint32_t slot = atomicAdd(&band_filled, 1u);
+                band_order[slot] = (uint64_t(top_k_key(score)) << 32) | (0xffffffffu - place);
+            }
+        }
+        __syncthreads();
+    } else {
+        // the general way: one segment after the other through global memory, by the whole workgroup
+        uint32_t base = 0;
+        for (size_t segment = 0; segment < segments; ++segment) {
+            const uint32_t count = counts[row * segments + segment] & 0xffffu;
+            for (uint32_t i = t; i < count; i += TOPK_THREADS) {
+                const uint32_t entry = uint32_t(list[row * groups + segment * INTERVAL_KEYS + i]);
+                row_scores[base + i] = entry & CERTAIN ? INFINITY : scores[row * groups + segment * INTERVAL_KEYS + i];
+                row_list[base + i] = int32_t(entry & ~CERTAIN);
+            }
+            base += count;
+        }
+        __threadfence_block();
+        __syncthreads();
+    }
+    int32_t* const row_out = out + row * k;
+    const uint32_t certain = candidates - band;
+    if (held && band <= RANKED && certain <= k) {
+        // direct ranking: member i is kept when fewer than `room` members beat it (a higher key, or the same key earlier in the list)
+        const uint32_t room = uint32_t(min(size_t(band), k - certain)), floor = top_k_key(-INFINITY);
+        if (band & 1u) { if (t == 0) band_order[band] = 0; __syncthreads(); }        // (pairs are read: an odd band gets a member that beats nobody)
+        if (t < band) {
+            const uint64_t mine = band_order[t];
+            uint32_t beaten_by = 0;
+            const ulonglong2* pairs = reinterpret_cast<const ulonglong2*>(band_order);
+            #pragma unroll 8
+            for (uint32_t j = 0; j < (band + 1) / 2; ++j) { const ulonglong2 two = pairs[j]; beaten_by += (two.x > mine) + (two.y > mine); }
+            if (uint32_t(mine >> 32) <= floor || beaten_by >= room) held_list[0xffffffffu - uint32_t(mine)] = -1;      // not kept: a score of -inf never is
+        }
+        __syncthreads();
+        // ordered compaction of what is kept
+        uint32_t slot = 0;
+        for (uint32_t base = 0; base < candidates; base += TOPK_THREADS * 4) {
+            int32_t mine[4];
+            uint32_t kept = 0;
+            #pragma unroll
+            for (int i = 0; i < 4; ++i) { const uint32_t at = base + 4 * t + i; mine[i] = at < candidates ? held_list[at] : -1; kept += mine[i] >= 0; }
+            uint32_t all;
+            uint32_t at = slot + block_scan(kept, wave_sums, all);
+            #pragma unroll
+            for (int i = 0; i < 4; ++i) if (mine[i] >= 0) row_out[at++] = mine[i];
+            slot += all;
+            __syncthreads();
+        }
+        for (size_t i = slot + t; i < k; i += TOPK_THREADS) row_out[i] = -1;
+        return;
+    }
+    if (held) top_k_row([&](size_t v) { return held_scores[v]; }, [&](size_t v) { return held_list[v]; }, candidates, k, row_out);
+    else top_k_row([=](size_t v) { return row_scores[v]; }, [=](size_t v) { return row_list[v]; }, candidates, k, row_out);
+}
+
+// All of a row's histograms to zero: after a call that only wanted the bounds.
+__global__ void __launch_bounds__(256) radix_clear_kernel(uint32_t* histogram, size_t words) {
+    for (size_t i = size_t(blockIdx.x) * 256 + threadIdx.x; i < words; i += size_t(gridDim.x) * 256) histogram[i] = 0u;
 }
 
 __global__ void widen_bf16_kernel(const uint16_t* from, float* to, size_t count) {
@@ -690,46 +845,72 @@ void launch_scores(Device& d, const float* q, const void* keys, bool bf16, size_
 // The matrix-core indexer of the batched sparse path (scores are not returned by it): see the kernels above.
 bool index_fast_supported(uint64_t heads, uint64_t dim) { return dim == 128 && heads % 16 == 0 && heads >= 16 && heads <= 64; }
 
-struct FastIndexSpace { float *wide_q, *margin, *lower, *upper, *scores; uint32_t *histogram, *counts, *totals; int32_t* list; size_t blocks; };
-size_t fast_index_bytes(size_t batch, size_t groups, size_t heads, size_t dim) {
-    const size_t blocks = (groups + INTERVAL_KEYS - 1) / INTERVAL_KEYS;
-    return 4 * (batch * heads * dim + batch + 4 * batch * groups + RADIX_LEVELS * batch * RADIX_BINS + batch * blocks + batch) + 9 * 256;
+struct FastIndexSpace { float *lower, *upper, *scores, *flat_scores; uint32_t* counts; int32_t *list, *flat_list; size_t segments; };
+size_t fast_index_bytes(size_t batch, size_t groups) {
+    const size_t segments = (groups + INTERVAL_KEYS - 1) / INTERVAL_KEYS;
+    return 4 * (6 * batch * groups + batch * segments) + 8 * 256;
 }
-FastIndexSpace fast_index_space(void* base, size_t batch, size_t groups, size_t heads, size_t dim) {
+FastIndexSpace fast_index_space(void* base, size_t batch, size_t groups) {
     uint8_t* at = static_cast<uint8_t*>(base);
     const auto take = [&](size_t words) { void* p = at; at += (4 * words + 255) & ~size_t(255); return p; };
     FastIndexSpace s{};
-    s.blocks = (groups + INTERVAL_KEYS - 1) / INTERVAL_KEYS;
-    s.wide_q = static_cast<float*>(take(batch * heads * dim)); s.margin = static_cast<float*>(take(batch));
+    s.segments = (groups + INTERVAL_KEYS - 1) / INTERVAL_KEYS;
     s.lower = static_cast<float*>(take(batch * groups)); s.upper = static_cast<float*>(take(batch * groups));
     s.scores = static_cast<float*>(take(batch * groups)); s.list = static_cast<int32_t*>(take(batch * groups));
-    s.histogram = static_cast<uint32_t*>(take(RADIX_LEVELS * batch * RADIX_BINS)); s.counts = static_cast<uint32_t*>(take(batch * s.blocks));
-    s.totals = static_cast<uint32_t*>(take(batch));
+    s.flat_scores = static_cast<float*>(take(batch * groups)); s.flat_list = static_cast<int32_t*>(take(batch * groups));
+    s.counts = static_cast<uint32_t*>(take(batch * s.segments));
     return s;
 }
 
+// The radix histograms of the handle: [lower | upper][level][row][bin], all zero between calls (the kernel after their last reader zeroes them; a call that failed part-way leaves them marked, and the next call clears them first).  They
+// live apart from the workspace, which other ops overwrite.
+uint32_t* index_histograms(Device& d, size_t batch) {
+    const size_t words = size_t(RADIX_LEVELS) * RADIX_BINS + 1;        // a row's histograms and its widest margin
+    if (batch > d.index_bins_rows) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        SD_CHECK(hipStreamIsCapturing(d.stream, &capturing));
+        if (capturing != hipStreamCaptureStatusNone) throw std::runtime_error("Straydog index histograms cannot grow while a graph is recorded");
+        if (d.index_bins) {
+            drop_recorded_graphs(d);
+            release(d, d.index_bins);
+            d.index_bins = nullptr; d.index_bins_rows = 0;
+        }
+        d.index_bins = static_cast<uint32_t*>(allocate(d, words * batch * 4, true));
+        d.index_bins_rows = batch;
+        d.index_bins_dirty = false;
+    }
+    if (d.index_bins_dirty) {
+        radix_clear_kernel<<<64, 256, 0, d.stream>>>(d.index_bins, words * d.index_bins_rows);
+        SD_CHECK(hipGetLastError());
+        d.index_bins_dirty = false;
+    }
+    return d.index_bins;
+}
+
 template<int HEADS>
-void fast_index_bounds(Device& d, const FastIndexSpace& s, const void* q_index, const void* keys, const float* weights, const int32_t* visible, size_t batch,
-                       size_t groups, float scale) {
-    index_prepare_kernel<<<dim3(unsigned(batch), 8), 256, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), weights, HEADS, 128, scale, batch, s.margin, s.wide_q, s.histogram);
+void fast_index_bounds(Device& d, const void* q_index, const void* keys, const float* weights, const int32_t* visible, size_t batch, size_t groups, float scale,
+                       float* lower, float* upper, uint32_t* histogram) {
     timed_launch(d, &index_interval_kernel<HEADS>, dim3(unsigned((groups + BRACKET_KEYS - 1) / BRACKET_KEYS), unsigned(batch)), dim3(BRACKET_WAVES * 64), 0,
-                 static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys), weights, visible, s.margin, groups, scale, s.lower, s.upper, s.histogram);
+                 static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys), weights, visible, groups, scale, lower, upper, histogram, d.index_bins_rows);
     SD_CHECK(hipGetLastError());
 }
 
 template<int HEADS>
 void fast_index_top_k(Device& d, const FastIndexSpace& s, const void* q_index, const void* keys, const float* weights, const int32_t* visible, size_t batch,
                       size_t groups, float scale, size_t k, int32_t* indices) {
-    const dim3 grid(unsigned(s.blocks), unsigned(batch));
-    fast_index_bounds<HEADS>(d, s, q_index, keys, weights, visible, batch, groups, scale);
+    uint32_t* const histogram = index_histograms(d, batch);
+    d.index_bins_dirty = true;           // until the last kernel, which zeroes them again, is queued
+    const unsigned segments = unsigned(s.segments);
+    fast_index_bounds<HEADS>(d, q_index, keys, weights, visible, batch, groups, scale, s.lower, s.upper, histogram);
     const uint32_t rank = uint32_t(std::min<size_t>(k, 0xffffffffu));
-    radix_histogram_kernel<<<grid, 256, 0, d.stream>>>(s.lower, groups, batch, 1, rank, s.histogram);
-    candidate_count_kernel<<<grid, 256, 0, d.stream>>>(s.upper, groups, batch, rank, s.histogram, s.counts);
-    candidate_list_kernel<<<grid, 256, 0, d.stream>>>(s.upper, groups, batch, rank, s.histogram, s.counts, s.list, s.totals);
-    candidate_score_kernel<HEADS><<<dim3(unsigned((k + k / 8 + 64 + SCORE_WAVES * SCORE_BATCH - 1) / (SCORE_WAVES * SCORE_BATCH)), unsigned(batch)), SCORE_WAVES * 64, 0, d.stream>>>(s.wide_q, static_cast<const uint16_t*>(keys), weights, groups, scale, s.list, s.totals,
-                                                                                   s.scores);
-    top_k_listed_kernel<<<unsigned(batch), TOPK_THREADS, 0, d.stream>>>(s.scores, s.list, s.totals, groups, k, indices);
+    radix_histogram_kernel<<<dim3(segments, unsigned(batch)), 256, 0, d.stream>>>(s.lower, groups, d.index_bins_rows, rank, histogram);
+    candidate_segments_kernel<<<dim3(segments, unsigned(batch)), 256, 0, d.stream>>>(s.lower, s.upper, groups, d.index_bins_rows, rank, histogram, s.list, s.counts);
+    const unsigned score_groups = unsigned(std::min<size_t>((s.segments + SCORE_WAVES - 1) / SCORE_WAVES, 64));
+    band_score_kernel<HEADS><<<dim3(score_groups, unsigned(batch)), SCORE_WAVES * 64, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys), weights,
+                                                                                                 groups, scale, s.list, s.counts, s.segments, s.scores, histogram, d.index_bins_rows);
+    index_finish_kernel<<<unsigned(batch), TOPK_THREADS, 0, d.stream>>>(s.scores, s.list, s.counts, s.segments, groups, k, s.flat_scores, s.flat_list, indices);
     SD_CHECK(hipGetLastError());
+    d.index_bins_dirty = false;
 }
 
 
@@ -958,7 +1139,7 @@ int sdx_index_top_k(void* handle, const void* q_index, const void* keys, const f
     op_span(value, indices, checked_floats({batch, k}), "top-k indices");
     if (!scores && index_fast_supported(heads, dim)) {
         // the matrix cores bracket the scores; the canonical arithmetic runs on the few groups near the k-th only
-        const FastIndexSpace space = fast_index_space(workspace(value, fast_index_bytes(batch, groups, heads, dim)), batch, groups, heads, dim);
+        const FastIndexSpace space = fast_index_space(workspace(value, fast_index_bytes(batch, groups)), batch, groups);
         switch (heads) {
             case 16: fast_index_top_k<16>(value, space, q_index, keys, weights, visible, batch, groups, scale, k, indices); break;
             case 32: fast_index_top_k<32>(value, space, q_index, keys, weights, visible, batch, groups, scale, k, indices); break;
@@ -991,13 +1172,12 @@ int sdx_index_score_bounds(void* handle, const void* q_index, const void* keys, 
     op_span(value, visible, checked_floats({batch}), "visible counts");
     op_span(value, lower, checked_floats({batch, groups}), "score bounds");
     op_span(value, upper, checked_floats({batch, groups}), "score bounds");
-    FastIndexSpace space = fast_index_space(workspace(value, fast_index_bytes(batch, groups, heads, dim)), batch, groups, heads, dim);
-    space.lower = lower; space.upper = upper;
+    // (no histograms: the bounds alone)
     switch (heads) {
-        case 16: fast_index_bounds<16>(value, space, q_index, keys, weights, visible, batch, groups, scale); break;
-        case 32: fast_index_bounds<32>(value, space, q_index, keys, weights, visible, batch, groups, scale); break;
-        case 48: fast_index_bounds<48>(value, space, q_index, keys, weights, visible, batch, groups, scale); break;
-        default: fast_index_bounds<64>(value, space, q_index, keys, weights, visible, batch, groups, scale); break;
+        case 16: fast_index_bounds<16>(value, q_index, keys, weights, visible, batch, groups, scale, lower, upper, nullptr); break;
+        case 32: fast_index_bounds<32>(value, q_index, keys, weights, visible, batch, groups, scale, lower, upper, nullptr); break;
+        case 48: fast_index_bounds<48>(value, q_index, keys, weights, visible, batch, groups, scale, lower, upper, nullptr); break;
+        default: fast_index_bounds<64>(value, q_index, keys, weights, visible, batch, groups, scale, lower, upper, nullptr); break;
     }
     SD_OP_END
 }

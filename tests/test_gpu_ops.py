@@ -406,6 +406,35 @@ def test_matrix_core_indexer_brackets_and_selects_exactly(gpu, oracle, heads, gr
         gpu.release(b)
 
 
+def test_matrix_core_indexer_with_wide_bands_of_equal_scores(gpu, oracle):
+    # what the brackets cannot decide is scored canonically; here that band is large: a row whose keys are all the same (every group
+    # ties: the lowest indices win), a row where a few thousand identical keys straddle the cut, a row of zero keys (all scores 0,
+    # brackets of zero width), next to an ordinary row -- twice in a row, the histograms the call keeps being its own to reset
+    rng = np.random.default_rng(4242)
+    batch, heads, dim, groups, k = 4, 64, 128, 20000, 512
+    q_bits, q_vals = _bf16_round(oracle, rng.standard_normal((batch, heads, dim)).astype(np.float32))
+    keys = rng.standard_normal((batch, groups, dim)).astype(np.float32)
+    keys[0, :] = keys[0, 7]
+    best = np.argsort(-np.abs(keys[1]).sum(axis=1))[:1]
+    keys[1, 2000:5000] = keys[1, best[0]] * 3.0          # 3000 equal keys; whether they score high depends on q -- either way a wide tie
+    keys[2, :] = 0.0
+    key_bits, key_vals = _bf16_round(oracle, keys)
+    weights = rng.random((batch, heads)).astype(np.float32)
+    visible = np.array([groups, groups, groups - 11, groups], dtype=np.int32)
+    qb, kb, wb, vb = gpu.upload(q_bits), gpu.upload(key_bits), gpu.upload(weights), gpu.upload(visible)
+    indices = gpu.buffer(batch * k * 4)
+    want = [oracle.top_k(oracle.index_scores(q_vals[b:b + 1], key_vals[b], weights[b:b + 1], visible[b:b + 1], 1.0), k)[0] for b in range(batch)]
+    assert np.array_equal(want[0], np.arange(k)) and np.array_equal(want[2], np.arange(k))
+    for run in range(2):
+        gpu.write_buffer(indices, 0, np.full(batch * k, -7, np.int32))
+        gpu.index_top_k(qb.base(), kb.base(), wb.base(), vb.base(), batch, groups, heads, dim, 1.0, None, k, indices.base())
+        got = _read(gpu, indices, np.int32, batch * k).reshape(batch, k)
+        for b in range(batch):
+            assert np.array_equal(got[b], want[b]), (run, b)
+    for b in (qb, kb, wb, vb, indices):
+        gpu.release(b)
+
+
 def test_batched_sparse_path_small(gpu, oracle):
     # BASELINE config 4 in small: index scores -> top-k (bit-exact) -> gather attention over BF16 latents, per sequence
     rng = np.random.default_rng(12)
