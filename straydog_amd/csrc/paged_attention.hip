@@ -360,18 +360,21 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
     }
 }
 
-// One block per (sequence, span row, head): the segments' partial results merged and normalised (the algebra of the
-// reference's qsa_decode_merge, gpu/sparse_attention_compute.hpp:139-170).  The block's 256 threads are GROUPS groups of
-// DIM/2 threads; a group takes every GROUPS-th segment and a thread two columns, so all loads of a pass are in flight at
-// once; segments are taken 256 at a time with a running maximum.
+// A wave per (sequence, span row, head): the segments' partial results merged and normalised (the algebra of the
+// reference's qsa_decode_merge, gpu/sparse_attention_compute.hpp:139-170).  A lane takes two columns of every segment and
+// every lane reads the segments' maxima and sums for itself (one address a wave: a broadcast), so nothing is exchanged
+// between lanes and nothing waits on LDS or a barrier: the segments are asked for sixteen at a time, all loads in flight at
+// once, under a running maximum.  Four rows a workgroup.
 template<int DIM, bool F16_OUT>
-__global__ void __launch_bounds__(256) paged_merge_kernel(PagedArgs args, void* out) {
-    constexpr int STRIDE = DIM + 2, LANES = DIM / 2, GROUPS = 256 / LANES;
-    const unsigned item = blockIdx.x, head = item % args.heads, span_row = item / args.heads % args.span, seq = item / args.heads / args.span;
+__global__ void __launch_bounds__(256) paged_merge_kernel(PagedArgs args, void* out, unsigned outputs) {
+    constexpr int STRIDE = DIM + 2, PER = DIM / 128, AT_ONCE = 16;
+    static_assert(DIM % 128 == 0, "a lane takes two columns of every run of 128");
+    const unsigned item = blockIdx.x * 4 + threadIdx.x / 64;
+    if (item >= outputs) return;
+    const unsigned head = item % args.heads, span_row = item / args.heads % args.span, seq = item / args.heads / args.span;
     const unsigned kvh = head / args.group, row = span_row * args.group + head % args.group;
-    const unsigned tid = threadIdx.x, group = tid / LANES, col = 2 * (tid % LANES), wave = tid >> 6;
     // the workgroups whose shares met this sequence and K/V head
-    const int lane = int(tid & 63);
+    const int lane = int(threadIdx.x & 63);
     const Share share = batch_share(args, lane);
     unsigned before = 0;
     for (unsigned s = lane; s < seq; s += 64) before += unsigned(min(first_position(args.positions, s, args.max_context) + int(args.span), args.max_context) + int(UNIT) - 1) / UNIT;
@@ -382,60 +385,41 @@ __global__ void __launch_bounds__(256) paged_merge_kernel(PagedArgs args, void* 
     const unsigned used = share_owner(share, begin + units - 1) - owner + 1;
     const float* base = args.partial + (size_t(owner) + size_t(seq) * args.kv_heads + kvh) * args.rows * STRIDE + size_t(row) * STRIDE;
     const size_t step = size_t(args.rows) * STRIDE;
-    __shared__ float weights[256];
-    __shared__ float reduce[2][4];
-    __shared__ float2 sums[GROUPS][LANES];
     float top = NEG_BIG, sum = 0.0f;
-    float2 value = {0.0f, 0.0f};
-    for (unsigned first = 0; first < used; first += 256) {
-        const unsigned c = first + tid, count = min(used - first, 256u);
-        // eight of a group's partial results at a time: eight loads in flight, not one after the other; the first eight are
-        // asked for together with the maxima and sums their weights come from
-        constexpr unsigned AT_ONCE = 8;
-        float2 v[AT_ONCE];
-        if (group < count)
-            #pragma unroll
-            for (unsigned i = 0; i < AT_ONCE; ++i) v[i] = *reinterpret_cast<const float2*>(base + (first + min(group + i * GROUPS, count - 1)) * step + col);
-        float m = NEG_BIG, l = 0.0f;
-        if (c < used) { const float2 pair = *reinterpret_cast<const float2*>(base + c * step + DIM); m = pair.x; l = pair.y; }
-        float tile_top = m;
+    float2 value[PER];
+    #pragma unroll
+    for (int i = 0; i < PER; ++i) value[i] = make_float2(0.0f, 0.0f);
+    for (unsigned first = 0; first < used; first += AT_ONCE) {
+        float2 stats[AT_ONCE], v[AT_ONCE][PER];
         #pragma unroll
-        for (int d = 32; d; d >>= 1) tile_top = fmaxf(tile_top, __shfl_xor(tile_top, d));
-        if ((tid & 63) == 0) reduce[0][wave] = tile_top;
-        __syncthreads();
-        tile_top = fmaxf(fmaxf(reduce[0][0], reduce[0][1]), fmaxf(reduce[0][2], reduce[0][3]));
-        const float top_new = fmaxf(top, tile_top), keep = __builtin_amdgcn_exp2f(top - top_new);
-        const float w = __builtin_amdgcn_exp2f(m - top_new);
-        weights[tid] = w;
-        float part = l * w;
-        #pragma unroll
-        for (int d = 32; d; d >>= 1) part += __shfl_xor(part, d);
-        if ((tid & 63) == 0) reduce[1][wave] = part;
-        __syncthreads();
-        sum = sum * keep + (reduce[1][0] + reduce[1][1]) + (reduce[1][2] + reduce[1][3]);
-        value.x *= keep; value.y *= keep;
-        top = top_new;
-        for (unsigned k0 = group; k0 < count; k0 += AT_ONCE * GROUPS) {
-            if (k0 != group)
-                #pragma unroll
-                for (unsigned i = 0; i < AT_ONCE; ++i) v[i] = *reinterpret_cast<const float2*>(base + (first + min(k0 + i * GROUPS, count - 1)) * step + col);
+        for (int c = 0; c < AT_ONCE; ++c) {
+            const float* from = base + size_t(min(first + c, used - 1)) * step;
+            stats[c] = *reinterpret_cast<const float2*>(from + DIM);
             #pragma unroll
-            for (unsigned i = 0; i < AT_ONCE; ++i) {
-                const float w_k = k0 + i * GROUPS < count ? weights[k0 + i * GROUPS] : 0.0f;
-                value.x += v[i].x * w_k; value.y += v[i].y * w_k;
-            }
+            for (int i = 0; i < PER; ++i) v[c][i] = *reinterpret_cast<const float2*>(from + 128 * i + 2 * lane);
         }
-        __syncthreads();      // weights and reduce are rewritten by the next pass
-    }
-    sums[group][tid % LANES] = value;
-    __syncthreads();
-    if (group == 0) {
+        float higher = top;
         #pragma unroll
-        for (int g = 1; g < GROUPS; ++g) { value.x += sums[g][tid].x; value.y += sums[g][tid].y; }
-        value.x /= sum; value.y /= sum;
-        const size_t at = size_t(item) * DIM + col;
-        if (F16_OUT) *reinterpret_cast<__half2*>(static_cast<__half*>(out) + at) = __floats2half2_rn(value.x, value.y);
-        else *reinterpret_cast<float2*>(static_cast<float*>(out) + at) = value;
+        for (int c = 0; c < AT_ONCE; ++c) if (first + c < used) higher = fmaxf(higher, stats[c].x);
+        const float keep = __builtin_amdgcn_exp2f(top - higher);
+        top = higher;
+        sum *= keep;
+        #pragma unroll
+        for (int i = 0; i < PER; ++i) { value[i].x *= keep; value[i].y *= keep; }
+        #pragma unroll
+        for (int c = 0; c < AT_ONCE; ++c) {
+            const float w = first + c < used ? __builtin_amdgcn_exp2f(stats[c].x - top) : 0.0f;
+            sum += stats[c].y * w;
+            #pragma unroll
+            for (int i = 0; i < PER; ++i) { value[i].x += v[c][i].x * w; value[i].y += v[c][i].y * w; }
+        }
+    }
+    #pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const float2 result = make_float2(value[i].x / sum, value[i].y / sum);
+        const size_t at = size_t(item) * DIM + 128 * i + 2 * lane;
+        if (F16_OUT) *reinterpret_cast<__half2*>(static_cast<__half*>(out) + at) = __floats2half2_rn(result.x, result.y);
+        else *reinterpret_cast<float2*>(static_cast<float*>(out) + at) = result;
     }
 }
 
@@ -549,13 +533,13 @@ void paged_attention(Device& value, const sdx_kv_pool* pool, const int32_t* page
     if (pool->dim == 128) { if (q8) launch_tiles<128, true>(value, args, query_tiles, grid); else launch_tiles<128, false>(value, args, query_tiles, grid); }
     else { if (q8) launch_tiles<256, true>(value, args, query_tiles, grid); else launch_tiles<256, false>(value, args, query_tiles, grid); }
     SD_CHECK(hipGetLastError());
-    const unsigned outputs = unsigned(checked_product({seqs, span, heads}));
+    const unsigned outputs = unsigned(checked_product({seqs, span, heads})), merge_groups = (outputs + 3) / 4;
     if (pool->dim == 128) {
-        if (out_f16) paged_merge_kernel<128, true><<<outputs, 256, 0, value.stream>>>(args, out);
-        else paged_merge_kernel<128, false><<<outputs, 256, 0, value.stream>>>(args, out);
+        if (out_f16) paged_merge_kernel<128, true><<<merge_groups, 256, 0, value.stream>>>(args, out, outputs);
+        else paged_merge_kernel<128, false><<<merge_groups, 256, 0, value.stream>>>(args, out, outputs);
     } else {
-        if (out_f16) paged_merge_kernel<256, true><<<outputs, 256, 0, value.stream>>>(args, out);
-        else paged_merge_kernel<256, false><<<outputs, 256, 0, value.stream>>>(args, out);
+        if (out_f16) paged_merge_kernel<256, true><<<merge_groups, 256, 0, value.stream>>>(args, out, outputs);
+        else paged_merge_kernel<256, false><<<merge_groups, 256, 0, value.stream>>>(args, out, outputs);
     }
 }
 
