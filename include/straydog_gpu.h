@@ -87,6 +87,17 @@ int sd_state_copy(void* handle, void* state, uint64_t offset, uint64_t pitch, ui
 /* reference straydog_gpu.h:113 (gpu/kernels.cpp:4266-4274): the bytes of a K/V row of the Qwen state, 512 (FP16) or
  * 272 (Q8_0: 256 int8 then eight FP16 block scales, gpu/core.hpp:397-403).  Default 272. */
 int sd_kv_format(void* handle, uint32_t row);
+/* reference straydog_gpu.h:114 (gpu/kernels.cpp:4277-4290): registers an allocation of this device, exactly rows x 4096 bytes
+ * (rows <= 2^22, not a host state), as the VRAM stage that rows held in host memory are copied into to be attended from;
+ * "invalid Straydog K/V stage" otherwise.  What a former stage held is forgotten and recorded graphs are dropped.  The paged
+ * cache's `stage` / `unstage` (straydog_gpu_ext.h) are what fills and drains it. */
+int sd_kv_stage(void* handle, void* pointer, uint64_t rows);
+/* reference straydog_gpu.h:98 (gpu/kernels.cpp:3876-3903): `bytes` of zeroed, mapped, page-locked host memory that kernels read
+ * and write over the bus; owned like a device allocation (ops take pointers into it, sd_release frees it) but outside the VRAM
+ * budget.  Null on failure. */
+void* sd_host_state(void* handle, uint64_t bytes);
+/* reference straydog_gpu.h:112 (gpu/kernels.cpp:4292-4300): 1, host-resident state is supported. */
+int sd_host_state_supported(void* handle);
 
 /* ---- Attention ops ---- */
 /* reference straydog_gpu.h:528 (gpu/kernels.cpp:4387-4419, kernels :79-165): selection-list attention of `steps` rows at

@@ -60,6 +60,31 @@ int sdx_kv_cache_truncate(void* handle, void* cache, uint64_t sequence, uint64_t
 int sdx_kv_cache_fork(void* handle, void* cache, uint64_t from, uint64_t to, uint64_t tokens);
 int sdx_kv_cache_usage(void* handle, void* cache, uint64_t sequence, uint64_t* pages_held, uint64_t* pages_free);
 
+/* Rows that are not in HBM (the reference's host-resident K/V: gpu/kv_stage.hpp:4-184, sd_kv_stage gpu/kernels.cpp:4277-4290,
+ * sd_kv_grow :4048-4140), on the paged cache.  Pages move on a stream of their own behind the compute stream's queued work; the
+ * compute stream waits for them at its next call that touches K/V pages, not before (the prefetch between two layers).
+ *   host      gives the cache a tier of `host_pages` pages in page-locked host memory the library allocates (once)
+ *   park      the sequence's pages are copied to host pages and its HBM pages freed at once; it keeps its rows but can only be
+ *             staged, truncated or resumed
+ *   resume    a parked sequence takes HBM pages again and its rows are copied back ("out of pages" changes nothing)
+ *   stage     the first `tokens` positions of a parked sequence in the VRAM stage registered with sd_kv_stage: only the pages
+ *             the stage does not hold of it yet are copied; pool / page_table / table_stride are the view to attend through
+ *             (one sequence: row 0 of the table)
+ *   unstage   rows [first, first + count) that were written through the staged view go back to the sequence's host pages
+ *             (taking host pages as it grows)
+ *   grow      the pool becomes `pages` pages: a new allocation, the old pages copied on the device, the old one released (VRAM
+ *             for both during the copy); a view taken before is stale, recorded graphs are dropped.  A device without room
+ *             answers "not enough VRAM for the K/V of this sequence" and changes nothing
+ *   residency whether the sequence is parked, host pages free, pages of the sequence the stage holds */
+int sdx_kv_cache_host(void* handle, void* cache, uint64_t host_pages);
+int sdx_kv_cache_park(void* handle, void* cache, uint64_t sequence);
+int sdx_kv_cache_resume(void* handle, void* cache, uint64_t sequence);
+int sdx_kv_cache_stage(void* handle, void* cache, uint64_t sequence, uint64_t tokens, sdx_kv_pool* pool, const int32_t** page_table,
+                       uint64_t* table_stride);
+int sdx_kv_cache_unstage(void* handle, void* cache, uint64_t sequence, uint64_t first, uint64_t count);
+int sdx_kv_cache_grow(void* handle, void* cache, uint64_t pages);
+int sdx_kv_cache_residency(void* handle, void* cache, uint64_t sequence, uint64_t* parked, uint64_t* host_pages_free, uint64_t* staged_pages);
+
 /* Causal grouped-query attention over the paged cache: the attention step of a decode (span 1), a speculative
  * verify (span <= 8) or a prefill chunk (any span), i.e. qsa_decode_parts/qsa_decode_merge, qsa_flash and
  * qsa_prompt_attention of the reference (gpu/sparse_attention_compute.hpp:41-170, :176-279,

@@ -56,6 +56,9 @@ SIGNATURES = {
     "sd_state_copy": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_u64, c_int]),
     "sdx_checkpoint_release": (c_int, [c_void_p, c_void_p]),
     "sd_kv_format": (c_int, [c_void_p, c_u32]),
+    "sd_kv_stage": (c_int, [c_void_p, c_void_p, c_u64]),
+    "sd_host_state": (c_void_p, [c_void_p, c_u64]),
+    "sd_host_state_supported": (c_int, [c_void_p]),
     "sd_attention_sequence": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_u64, c_void_p, c_u64]),
     "sd_op_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float,
                                 c_void_p, c_void_p, c_u64, c_void_p]),
@@ -89,6 +92,13 @@ SIGNATURES = {
     "sdx_kv_cache_truncate": (c_int, [c_void_p, c_void_p, c_u64, c_u64]),
     "sdx_kv_cache_fork": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64]),
     "sdx_kv_cache_usage": (c_int, [c_void_p, c_void_p, c_u64, _P(c_u64), _P(c_u64)]),
+    "sdx_kv_cache_host": (c_int, [c_void_p, c_void_p, c_u64]),
+    "sdx_kv_cache_park": (c_int, [c_void_p, c_void_p, c_u64]),
+    "sdx_kv_cache_resume": (c_int, [c_void_p, c_void_p, c_u64]),
+    "sdx_kv_cache_stage": (c_int, [c_void_p, c_void_p, c_u64, c_u64, _P(KvPool), _P(c_void_p), _P(c_u64)]),
+    "sdx_kv_cache_unstage": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64]),
+    "sdx_kv_cache_grow": (c_int, [c_void_p, c_void_p, c_u64]),
+    "sdx_kv_cache_residency": (c_int, [c_void_p, c_void_p, c_u64, _P(c_u64), _P(c_u64), _P(c_u64)]),
     "sdx_kv_write": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_void_p, c_void_p, c_int, c_u64, c_u64]),
     "sdx_paged_attention_scratch": (c_u64, [c_u64, c_u64, c_u64, c_u64, c_u64]),
     "sdx_paged_attention": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_u64, c_void_p, c_int, c_u64, c_u64, c_u64,

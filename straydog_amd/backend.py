@@ -219,6 +219,50 @@ class Backend:
         self.check(self.lib.sdx_kv_cache_usage(self.handle, cache, sequence, ctypes.byref(held), ctypes.byref(free)))
         return held.value, free.value
 
+    def kv_cache_view(self, cache):
+        """(pool struct, device page table, table stride) as they are now (a growth moves the pool)."""
+        pool, table, stride = abi.KvPool(), ctypes.c_void_p(), abi.c_u64()
+        self.check(self.lib.sdx_kv_cache_view(self.handle, cache, ctypes.byref(pool), ctypes.byref(table), ctypes.byref(stride)))
+        return pool, table.value, stride.value
+
+    # ---- rows that are not in HBM: the cache's host tier, the VRAM stage, growth ----
+    def kv_cache_host(self, cache, host_pages):
+        self.check(self.lib.sdx_kv_cache_host(self.handle, cache, host_pages))
+
+    def kv_cache_park(self, cache, sequence):
+        self.check(self.lib.sdx_kv_cache_park(self.handle, cache, sequence))
+
+    def kv_cache_resume(self, cache, sequence):
+        self.check(self.lib.sdx_kv_cache_resume(self.handle, cache, sequence))
+
+    def kv_cache_stage(self, cache, sequence, tokens):
+        """(pool struct, device page table, table stride) of the sequence's first `tokens` positions in the VRAM stage."""
+        pool, table, stride = abi.KvPool(), ctypes.c_void_p(), abi.c_u64()
+        self.check(self.lib.sdx_kv_cache_stage(self.handle, cache, sequence, tokens, ctypes.byref(pool), ctypes.byref(table), ctypes.byref(stride)))
+        return pool, table.value, stride.value
+
+    def kv_cache_unstage(self, cache, sequence, first, count):
+        self.check(self.lib.sdx_kv_cache_unstage(self.handle, cache, sequence, first, count))
+
+    def kv_cache_grow(self, cache, pages):
+        self.check(self.lib.sdx_kv_cache_grow(self.handle, cache, pages))
+
+    def kv_cache_residency(self, cache, sequence=0):
+        """(parked, host pages free, pages of the sequence the stage holds)."""
+        parked, free, staged = abi.c_u64(), abi.c_u64(), abi.c_u64()
+        self.check(self.lib.sdx_kv_cache_residency(self.handle, cache, sequence, ctypes.byref(parked), ctypes.byref(free), ctypes.byref(staged)))
+        return bool(parked.value), free.value, staged.value
+
+    def kv_stage(self, pointer, rows):
+        self.check(self.lib.sd_kv_stage(self.handle, pointer, rows))
+
+    def host_state(self, size):
+        """A Buffer of `size` bytes in mapped, page-locked host memory (kernels reach it over the bus)."""
+        pointer = self.lib.sd_host_state(self.handle, size)
+        if not pointer:
+            raise StraydogError(self.error())
+        return Buffer(pointer, size)
+
     def kv_write(self, pool, page_table, table_stride, positions, keys, values, input_f16, seqs, span):
         self.check(self.lib.sdx_kv_write(self.handle, ctypes.byref(pool), page_table, table_stride, positions, keys, values,
                                          int(input_f16), seqs, span))

@@ -56,16 +56,26 @@ void* allocate(Device& d, size_t bytes, bool zero) {
 
 void release(Device& d, void* pointer) {
     size_t bytes = 0;
+    void* host = nullptr;
     {
         std::lock_guard<std::mutex> lock(d.mutex);
         const auto found = d.allocations.find(static_cast<const uint8_t*>(pointer));
         if (found == d.allocations.end()) throw std::runtime_error("Straydog release: not an allocation of this device");
         bytes = found->second;
         d.allocations.erase(found);
-        d.used -= bytes + allocation_tail;
+        const auto state = d.host_states.find(pointer);
+        if (state != d.host_states.end()) { host = state->second; d.host_states.erase(state); }
+        else d.used -= bytes + allocation_tail;
     }
     SD_CHECK(hipStreamSynchronize(d.stream));
-    SD_CHECK(hipFree(pointer));
+    if (d.kv_stream) SD_CHECK(hipStreamSynchronize(d.kv_stream));
+    if (pointer == d.kv_stage) {
+        // (the stage's address is in recorded graphs that attend from it)
+        drop_recorded_graphs(d);
+        d.kv_stage = nullptr; d.kv_stage_bytes = 0; d.kv_stage_owner = nullptr; d.kv_stage_pages = 0;
+    }
+    if (host) SD_CHECK(hipHostFree(host));
+    else SD_CHECK(hipFree(pointer));
 }
 
 // Caller memory goes through the page-locked arena a half at a time, so the caller's buffer is free on return and
@@ -199,7 +209,12 @@ void sd_destroy(void* handle) {
         if (entry.second.executable) (void)hipGraphExecDestroy(entry.second.executable);
         if (entry.second.graph) (void)hipGraphDestroy(entry.second.graph);
     }
+    if (d->kv_stream) (void)hipStreamSynchronize(d->kv_stream);
+    for (const auto& entry : d->host_states) { d->allocations.erase(static_cast<const uint8_t*>(entry.first)); (void)hipHostFree(entry.second); }
     for (const auto& entry : d->allocations) (void)hipFree(const_cast<uint8_t*>(entry.first));
+    if (d->kv_released) (void)hipEventDestroy(d->kv_released);
+    if (d->kv_moved) (void)hipEventDestroy(d->kv_moved);
+    if (d->kv_stream) (void)hipStreamDestroy(d->kv_stream);
     for (auto& event : d->events) if (event) (void)hipEventDestroy(event);
     for (auto& event : d->profile_events) (void)hipEventDestroy(event);
     for (const auto& entry : d->checkpoints) (void)hipHostFree(entry.first);
@@ -421,6 +436,56 @@ int sd_kv_format(void* handle, uint32_t row) {
     } catch (const std::exception& e) { last_error = e.what(); return -1; }
 }
 
+// Sequence state in mapped, page-locked host memory that kernels read and write over the bus (reference gpu/kernels.cpp:3876-3903
+// sd_host_state, :4292-4300 sd_host_state_supported): owned like a device allocation -- ops take pointers into it, sd_release
+// frees it -- but outside the VRAM budget.  A K/V pool may live there whole; the paged cache's host tier (kv_cache.hip) is the
+// faster way to hold rows that are not being attended to.
+void* sd_host_state(void* handle, uint64_t bytes) {
+    try {
+        Device& d = device(handle);
+        if (!bytes || bytes > (uint64_t(1) << 48)) throw std::runtime_error("invalid Straydog host state");
+        void* host = nullptr;
+        SD_CHECK(hipHostMalloc(&host, size_t(bytes) + allocation_tail, hipHostMallocMapped));
+        try {
+            std::memset(host, 0, size_t(bytes) + allocation_tail);
+            void* pointer = nullptr;
+            SD_CHECK(hipHostGetDevicePointer(&pointer, host, 0));
+            std::lock_guard<std::mutex> lock(d.mutex);
+            d.allocations.emplace(static_cast<const uint8_t*>(pointer), size_t(bytes));
+            try { d.host_states.emplace(pointer, host); }
+            catch (...) { d.allocations.erase(static_cast<const uint8_t*>(pointer)); throw; }
+            return pointer;
+        } catch (...) { (void)hipHostFree(host); throw; }
+    } catch (const std::exception& e) { last_error = e.what(); return nullptr; }
+}
+
+int sd_host_state_supported(void* handle) {
+    try { (void)device(handle); return 1; }
+    catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+// The VRAM stage (reference gpu/kernels.cpp:4277-4290): an allocation of the caller's, `rows` x 4096 bytes, that rows held in host
+// memory are copied into to be attended from.  Registering it forgets what a former stage held and the graphs recorded so far.
+int sd_kv_stage(void* handle, void* pointer, uint64_t rows) {
+    try {
+        Device& d = device(handle);
+        {
+            std::lock_guard<std::mutex> lock(d.mutex);
+            const auto found = d.allocations.find(static_cast<const uint8_t*>(pointer));
+            if (!rows || rows > (uint64_t(1) << 22) || found == d.allocations.end() || found->second != size_t(rows) * 1024 * 4 ||
+                d.host_states.count(pointer))
+                throw std::runtime_error("invalid Straydog K/V stage");
+        }
+        if (d.recording) throw std::runtime_error("invalid Straydog K/V stage");
+        if (d.kv_stream) SD_CHECK(hipStreamSynchronize(d.kv_stream));
+        d.kv_moving = false;
+        drop_recorded_graphs(d);
+        d.kv_stage = pointer; d.kv_stage_bytes = size_t(rows) * 1024 * 4;
+        d.kv_stage_owner = nullptr; d.kv_stage_pages = 0;
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
 // ---- graphs of ops (reference gpu/kernels.cpp:4765-4813) ----
 // Between begin and end the ops queued on the device's stream are recorded rather than run.  Only ops that take no host data and
 // allocate nothing may be recorded; the ops that keep a workspace (see the extension header) are called once before.
@@ -431,6 +496,7 @@ int sd_graph_begin(void* handle) {
         if (d.recording) throw std::runtime_error("a Straydog graph is already being recorded");
         // (made here, not by the op that uses it: a capture takes no allocation; reference gpu/kernels.cpp:4769-4773)
         try { select_thin_reserve(d); } catch (const std::exception&) {}
+        kv_settle(d);
         SD_CHECK(hipStreamBeginCapture(d.stream, hipStreamCaptureModeThreadLocal));
         d.recording = true;
         return 0;

@@ -67,6 +67,19 @@ struct Device {
     uint32_t* index_bins = nullptr; size_t index_bins_rows = 0; bool index_bins_dirty = false;
     // The lists of a short span's thinned index rows (block_index.hip), allocated at the first such call and kept.
     void* select_thin = nullptr;
+    // Sequence state in mapped, page-locked host memory (sd_host_state): device pointer -> host pointer.  They are listed in
+    // `allocations` too, so ops take them, but not counted in the VRAM budget.
+    std::map<const void*, void*> host_states;
+    // The VRAM stage the host registered (sd_kv_stage) and whose rows it holds: a K/V cache, one of its sequences, and how many
+    // of that sequence's pages from the first on are in it.
+    void* kv_stage = nullptr; size_t kv_stage_bytes = 0;
+    const void* kv_stage_owner = nullptr; size_t kv_stage_sequence = 0, kv_stage_pages = 0;
+    // K/V pages move between HBM and host memory on a stream of their own (same priority), behind `kv_released` of the
+    // compute stream; `kv_moved` marks the last move queued, and the compute stream waits for it before the next work
+    // that touches pages (kv_settle).
+    hipStream_t kv_stream = nullptr;
+    hipEvent_t kv_released = nullptr, kv_moved = nullptr;
+    bool kv_moving = false;
     // Page-locked host copies of sequence state (conversation checkpoints): pointer -> bytes.
     std::map<void*, size_t> checkpoints;
     // Recorded graphs of ops (sd_graph_begin / _end / _run), by the caller's key.
@@ -104,6 +117,14 @@ inline void raise_shared_limit(Device& d, const void* kernel, size_t bytes) {
     const hipError_t error = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes));
     if (error != hipSuccess) throw std::runtime_error(std::string("Straydog op: ") + gpu_error_text(error));
     have = bytes;
+}
+
+// Work on the compute stream that reads or writes K/V pages comes after the page moves queued so far.  (A recording takes no
+// wait on an event from outside it: sd_graph_begin settles first, and no move is queued while a graph is recorded.)
+inline void kv_settle(Device& d) {
+    if (!d.kv_moving) return;
+    SD_CHECK(hipStreamWaitEvent(d.stream, d.kv_moved, 0));
+    d.kv_moving = false;
 }
 
 Device& device(void* handle);                         // sets the HIP device of the handle; throws on null

@@ -140,6 +140,7 @@ void validate_pool(Device& d, const sdx_kv_pool* pool) {
         (pool->dim != 128 && pool->dim != 256) || (pool->row_bytes != pool->dim + pool->dim / 16 && pool->row_bytes != 2 * pool->dim))
         throw std::runtime_error("invalid Straydog K/V pool");
     op_span(d, pool->pages, checked_product({pool->page_count, 2, pool->kv_heads, pool->page_tokens, pool->row_bytes}), "a K/V pool");
+    kv_settle(d);       // (every op that reads or writes pages passes here: it runs after the page moves queued so far)
 }
 }  // namespace sd
 

@@ -267,6 +267,35 @@ def test_selected_attention(gpu, oracle, row_bytes, paged):
         gpu.release(b)
 
 
+def test_selected_attention_of_a_prompt_chunk(gpu, oracle):
+    # what the prompt path does from position 8192 on (gpu/qsa_prompt_attention.hpp:218-234, gpu/sparse_attention_compute.hpp:589-608):
+    # a chunk of 256 rows, each with its own selection list, over Q8_0 rows behind a shuffled page table, gated, FP16 in and out
+    from gpu_util import close_enough
+    rng = np.random.default_rng(256)
+    context, base, steps, selected, row_bytes = 12288, 9000, 256, 2052, 272
+    state, q, indices, counts, want = _qwen_case(oracle, rng, row_bytes, context, base, steps, selected)
+    planes = state.reshape(4, context, row_bytes)
+    page_tokens, pages = 256, context // 256
+    order = rng.permutation(pages + 2)[:pages].astype(np.int32)
+    host = np.zeros((pages + 2, 4, page_tokens, row_bytes), dtype=np.uint8)
+    for p in range(pages):
+        host[order[p]] = planes[:, p * page_tokens:(p + 1) * page_tokens]
+    pool, buffer = gpu.kv_pool(pages + 2, page_tokens, 2, 256, row_bytes)
+    table = gpu.upload(order)
+    gpu.write_buffer(buffer, 0, host.reshape(-1))
+    gate = rng.standard_normal((steps, 24, 512)).astype(np.float32) * 2
+    ib, cb, gb, qb = gpu.upload(indices), gpu.upload(counts), gpu.upload(gate), gpu.upload(q.astype(np.float16))
+    scratch = gpu.buffer(gpu.selected_attention_scratch(steps, 2, selected))
+    out = gpu.buffer(steps * 24 * 256 * 2)
+    gpu.selected_attention(pool, table.base(), context, base, ib.base(), selected, cb.base(), qb.base(), True, steps, 24, 0.0625, out.base(), True,
+                           scratch, gate=gb.at(256 * 4), gate_stride=512)
+    got = _read(gpu, out, np.float16, steps * 24 * 256).astype(np.float32).reshape(steps, 24, 256)
+    expect = want * (1.0 / (1.0 + np.exp(-gate[:, :, 256:].astype(np.float64))))
+    close_enough(got, expect, "a chunk of 256 rows")
+    for b in (ib, cb, gb, qb, scratch, out, buffer, table):
+        gpu.release(b)
+
+
 def test_index_then_attend_on_the_device(gpu, oracle):
     # the two stages chained on the device, as a decode pass runs them: sdx_qsa_index's lists feed sdx_selected_attention unchanged
     from gpu_util import close_enough
