@@ -276,6 +276,18 @@ def main():
             out[name] = {"us_per_call": ms * 1e3, "us_per_token": ms * 1e3 / rows, "scores_kernel_us": None if kernel_ms is None else kernel_ms * 1e3,
                          "scores_gbps": None if kernel_ms is None else work.complete() * 512 / kernel_ms / 1e6,
                          "scores_fp32_tflops": None if kernel_ms is None else work.flops() / kernel_ms / 1e9}
+            if rows > 8:
+                # the same selection by intervals (sdx_qsa_index_interval): FP16 matrix products bound every score, only the blocks
+                # around the 512th best are scored exactly; the second figure keeps the packed keys from the call before, as the
+                # chunks of one prompt do
+                work.with_interval()
+                ms, kernel_ms = timed(gpu, work.step_interval, max(args.steps // 5, 3), 2)
+                undecided = work.undecided()
+                kept_ms, _ = timed(gpu, lambda: work.step_interval(True), max(args.steps // 5, 3), 2)
+                out[name].update({"interval_us_per_call": ms * 1e3, "interval_us_per_token": ms * 1e3 / rows,
+                                  "interval_scan_kernel_us": None if kernel_ms is None else kernel_ms * 1e3,
+                                  "interval_scan_fp16_tflops": None if kernel_ms is None else work.flops() / kernel_ms / 1e9,
+                                  "interval_kept_operands_us_per_call": kept_ms * 1e3, "interval_rows_left_to_exact_kernels": undecided})
             if True:
                 # the attention over the rows' selections (24q/2kv heads, 256 columns, Q8_0 rows in the reference's state layout);
                 # the 256 rows of a prompt chunk select overlapping rows, so their figure counts bytes the caches serve

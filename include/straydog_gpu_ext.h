@@ -135,6 +135,22 @@ int sdx_qsa_pool(void* handle, const float* incoming, float* history, const floa
 int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, const float* blocks, uint64_t pool, uint64_t base,
                   const uint32_t* dynamic_base, uint64_t steps, uint64_t selected, float* scores, float* indices, float* counts);
 
+/* sdx_qsa_index_interval = the reference's selection by intervals for prompt chunks (gpu/qsa_interval.hpp:1-36 the bound, :601-626
+ * qsa_iv_chunk): the same indices and counts as sdx_qsa_index, block for block, from FP16 matrix products with a proven error
+ * bound; only the blocks whose bound straddles the 512th best score are scored exactly.  A row the scheme cannot decide (its
+ * guessed threshold too high, too many blocks near the 512th, an input beyond FP16 or not a number) is decided by sdx_qsa_index's
+ * kernels in the same call: more time, never a different result.  Spans below position 32768 go to sdx_qsa_index as they are.
+ * scores: steps x pool floats of scratch (afterwards: matrix-unit scores at the kept blocks, exact ones for undecided rows).
+ * scratch: sdx_qsa_index_interval_scratch(steps, pool) bytes.  valid (host, may be null): in, the number of blocks whose packed
+ * operands `scratch` still holds from the previous call on the same keys (0 when the keys' earlier blocks changed or the scratch
+ * was used otherwise); out, this call's.  No device-resident position: the scheme serves chunks, not recorded decode steps. */
+uint64_t sdx_qsa_index_interval_scratch(uint64_t steps, uint64_t pool);
+int sdx_qsa_index_interval(void* handle, const float* queries, uint64_t query_stride, const float* blocks, uint64_t pool, uint64_t base, uint64_t steps,
+                           uint64_t selected, float* scores, float* indices, float* counts, void* scratch, uint64_t scratch_bytes, uint64_t* valid);
+/* For harnesses: how many rows the last sdx_qsa_index_interval on this scratch (same steps and pool) left to the exact kernels
+ * (waits for the device). */
+int sdx_qsa_index_interval_undecided(void* handle, const void* scratch, uint64_t steps, uint64_t pool, uint64_t* rows);
+
 /* The attention stage of a Qwen decode or verification pass in one call: the reference's qsa_decode_attend / qsa_decode_attend_rows
  * (gpu/qsa_decode.hpp:28-44, 113-129; kernel qsa_normalize_rows :86-111).  For rows r < steps (1..8) at the consecutive positions
  * positions[r] with rope positions ropes[r], both device-resident (a recorded pass replays at the next position):

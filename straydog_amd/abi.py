@@ -108,6 +108,10 @@ SIGNATURES = {
                                            c_float, c_void_p, c_int]),
     "sdx_qsa_normalize": (c_int, [c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_u64, c_void_p]),
     "sdx_qsa_pool": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_void_p]),
+    "sdx_qsa_index_interval_scratch": (c_u64, [c_u64, c_u64]),
+    "sdx_qsa_index_interval": (c_int, [c_void_p, c_void_p, c_u64, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_void_p, c_void_p, c_void_p, c_u64,
+                                       _P(c_u64)]),
+    "sdx_qsa_index_interval_undecided": (c_int, [c_void_p, c_void_p, c_u64, c_u64, _P(c_u64)]),
     "sdx_qsa_index": (c_int, [c_void_p, c_void_p, c_u64, c_void_p, c_u64, c_u64, c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_void_p]),
     "sdx_selected_attention_scratch": (c_u64, [c_u64, c_u64, c_u64]),
     "sdx_selected_attention": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_u64, c_void_p, c_void_p, c_int,

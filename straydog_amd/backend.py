@@ -322,6 +322,22 @@ class Backend:
         self.check(self.lib.sdx_qsa_index(self.handle, queries, query_stride, blocks, pool, base, dynamic_base, steps, selected, scores,
                                           indices, counts))
 
+    def qsa_index_interval_scratch(self, steps, pool):
+        return self.lib.sdx_qsa_index_interval_scratch(steps, pool)
+
+    def qsa_index_interval(self, queries, query_stride, blocks, pool, base, steps, selected, scores, indices, counts, scratch, valid=None):
+        """The chunk's selection by intervals; `valid` is a one-element list holding the blocks the scratch still has packed (in and out)."""
+        held = abi.c_u64(valid[0] if valid else 0)
+        self.check(self.lib.sdx_qsa_index_interval(self.handle, queries, query_stride, blocks, pool, base, steps, selected, scores, indices,
+                                                   counts, scratch.base(), scratch.size, ctypes.byref(held) if valid is not None else None))
+        if valid is not None:
+            valid[0] = held.value
+
+    def qsa_index_interval_undecided(self, scratch, steps, pool):
+        rows = abi.c_u64()
+        self.check(self.lib.sdx_qsa_index_interval_undecided(self.handle, scratch.base(), steps, pool, ctypes.byref(rows)))
+        return rows.value
+
     def latent_attention(self, q, latents, selected, batch, groups, k, heads, kdim, vdim, scale, out):
         self.check(self.lib.sdx_latent_attention(self.handle, q, latents, selected, batch, groups, k, heads, kdim, vdim, scale, out))
 

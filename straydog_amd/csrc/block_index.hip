@@ -137,12 +137,20 @@ __global__ void __launch_bounds__(64 * HEADS) scores_rows_kernel(const float* __
 constexpr int TILE_ROWS = 32, TILE_BLOCKS = 256, TILE_COLUMNS = 16, TILE_THREADS = 512, QUERY_PITCH = TILE_ROWS * HEADS + 4;
 __global__ void __launch_bounds__(TILE_THREADS) scores_tiled_kernel(const float* __restrict__ queries, size_t query_stride,
                                                                     const float* __restrict__ blocks, size_t pool, size_t base, size_t steps,
-                                                                    float* __restrict__ scores) {
+                                                                    float* __restrict__ scores, const uint32_t* __restrict__ only, unsigned gate) {
     __shared__ __align__(16) float keys[2][TILE_COLUMNS][TILE_BLOCKS];
     __shared__ __align__(16) float query[2][TILE_COLUMNS][QUERY_PITCH];
-    const size_t first_row = size_t(blockIdx.y) * TILE_ROWS, first_block = size_t(blockIdx.x) * TILE_BLOCKS;
+    const size_t first_row = size_t(blockIdx.y) * TILE_ROWS;
+    if (only) {         // (behind the interval selection: the tiles of the rows it left undecided; only[gate] counts those rows)
+        if (!only[gate]) return;
+        bool any = false;
+        for (size_t r = first_row; r < min(steps, first_row + TILE_ROWS); ++r) any |= only[r] != 0;
+        if (!any) return;
+    }
     const size_t most = min((base + min(steps, first_row + TILE_ROWS)) / 4, pool);        // complete blocks of the tile's last row
-    if (most <= KEEP || first_block >= most) return;
+    if (most <= KEEP) return;
+    // (a launch may have fewer workgroups than tiles of blocks: each takes every gridDim.x-th)
+    for (size_t first_block = size_t(blockIdx.x) * TILE_BLOCKS; first_block < most; first_block += size_t(gridDim.x) * TILE_BLOCKS) {
     const unsigned t = threadIdx.x, lane = t % 64, wave = t / 64;
     constexpr int KEY_LOADS = TILE_COLUMNS * TILE_BLOCKS / TILE_THREADS, QUERY_LOADS = TILE_COLUMNS * TILE_ROWS * HEADS / TILE_THREADS;
     float key_next[KEY_LOADS], query_next[QUERY_LOADS];
@@ -202,6 +210,7 @@ __global__ void __launch_bounds__(TILE_THREADS) scores_tiled_kernel(const float*
             const float dot[HEADS] = {sums[i][0][b], sums[i][1][b], sums[i][2][b], sums[i][3][b]};
             if (block < complete) scores[row * pool + block] = positive_sum(dot);
         }
+    }
     }
 }
 
@@ -403,8 +412,9 @@ template<int REGS>
 __global__ void __launch_bounds__(SELECT_THREADS) select_kernel(const float* __restrict__ scores, size_t pool, size_t base, const uint32_t* dynamic,
                                                                 size_t selected, unsigned held_runs, float* __restrict__ indices,
                                                                 float* __restrict__ counts, const uint2* __restrict__ thinned,
-                                                                const uint32_t* __restrict__ thinned_counts) {
+                                                                const uint32_t* __restrict__ thinned_counts, const uint32_t* __restrict__ only) {
     extern __shared__ uint32_t held[];                       // [run][1024]
+    if (only && !only[blockIdx.x]) return;
     __shared__ SelectShared sh;
     __shared__ uint2 list[LIST];                             // (score bits, block) of the values that reach the guess
     if (dynamic) base = *dynamic;
@@ -551,11 +561,11 @@ __global__ void __launch_bounds__(SELECT_THREADS) select_kernel(const float* __r
 
 template<int REGS>
 void launch_select(Device& d, const float* scores, size_t pool, size_t base, const uint32_t* dynamic, size_t selected, size_t most, unsigned rows,
-                   float* indices, float* counts, const uint2* thinned, const uint32_t* thinned_counts) {
+                   float* indices, float* counts, const uint2* thinned, const uint32_t* thinned_counts, const uint32_t* only = nullptr) {
     const unsigned held_runs = unsigned(std::min<size_t>((most + SELECT_THREADS - 1) / SELECT_THREADS, LDS_RUNS));
     const size_t shared = size_t(std::max(held_runs, 1u)) * SELECT_THREADS * 4;
     if (shared > 48 * 1024) raise_shared_limit(d, reinterpret_cast<const void*>(&select_kernel<REGS>), LDS_RUNS * SELECT_THREADS * 4);
-    select_kernel<REGS><<<rows, SELECT_THREADS, shared, d.stream>>>(scores, pool, base, dynamic, selected, held_runs, indices, counts, thinned, thinned_counts);
+    select_kernel<REGS><<<rows, SELECT_THREADS, shared, d.stream>>>(scores, pool, base, dynamic, selected, held_runs, indices, counts, thinned, thinned_counts, only);
 }
 
 // ---- a decode or verification pass's inputs in one launch --------------------------------------------------------------
@@ -633,6 +643,12 @@ void launch_rows(Device& d, const float* queries, size_t stride, const float* bl
 }  // namespace
 
 namespace sd {
+// block_interval.hip
+size_t interval_scratch_bytes(size_t steps, size_t pool);
+bool interval_serves(size_t base);
+const uint32_t* interval_select(Device& d, const float* queries, size_t stride, const float* blocks, size_t pool, size_t base, size_t steps,
+                                size_t selected, float* scores, float* indices, float* counts, void* scratch, uint64_t* valid, unsigned* gate);
+size_t interval_undecided(Device& d, const void* scratch, size_t steps, size_t pool);
 // The lists of a short span's thinned rows: allocated once per handle, never while a graph is being recorded (sd_graph_begin
 // calls this first, so that a recorded pass takes the same path as an eager one).
 constexpr size_t thin_list_bytes = size_t(THIN_ROWS) * THIN_SEGMENTS * THIN_CAP * sizeof(uint2);
@@ -697,7 +713,7 @@ int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, con
             else {
                 if (dynamic_base) throw std::runtime_error("sdx_qsa_index: a device-resident position serves spans of up to 8 rows");
                 timed_launch(value, &scores_tiled_kernel, dim3(checked_blocks(most, TILE_BLOCKS), checked_blocks(steps, TILE_ROWS)), dim3(TILE_THREADS), 0,
-                             queries, query_stride, blocks, pool, base, steps, scores);
+                             queries, query_stride, blocks, pool, base, steps, scores, static_cast<const uint32_t*>(nullptr), 0u);
             }
         }
     }
@@ -718,6 +734,50 @@ int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, con
     }
     if (most <= size_t(LDS_RUNS) * SELECT_THREADS) launch_select<0>(value, scores, pool, base, dynamic_base, selected, most, rows, indices, counts, thinned, thinned_counts);
     else launch_select<33>(value, scores, pool, base, dynamic_base, selected, most, rows, indices, counts, thinned, thinned_counts);
+    SD_OP_END
+}
+
+uint64_t sdx_qsa_index_interval_scratch(uint64_t steps, uint64_t pool) {
+    try { return interval_scratch_bytes(size_t(checked_product({steps, 1})), size_t(checked_product({pool, 1}))); } catch (const std::exception&) { return 0; }
+}
+
+int sdx_qsa_index_interval(void* handle, const float* queries, uint64_t query_stride, const float* blocks, uint64_t pool, uint64_t base, uint64_t steps,
+                           uint64_t selected, float* scores, float* indices, float* counts, void* scratch, uint64_t scratch_bytes, uint64_t* valid) {
+    if (handle && !interval_serves(size_t(base))) {
+        // a short context: the exact kernels' time is small, and a sample of it says little
+        if (valid) *valid = 0;
+        return sdx_qsa_index(handle, queries, query_stride, blocks, pool, base, nullptr, steps, selected, scores, indices, counts);
+    }
+    SD_OP_BEGIN
+    if (!steps || steps > 4096 || !pool || query_stride < HEADS * COLUMNS) throw std::runtime_error("sdx_qsa_index_interval: 1 to 4096 steps, pool >= 1, query stride >= 512");
+    if (pool > size_t(64) * SELECT_THREADS + 1) throw std::runtime_error("sdx_qsa_index_interval: a pool of more than 65537 blocks (a context beyond 262144)");
+    if ((base + steps) / 4 > pool || base + steps > 4 * pool) throw std::runtime_error("sdx_qsa_index_interval: the span's blocks must fit the pool");
+    if (selected < 2052) throw std::runtime_error("sdx_qsa_index_interval: `selected` is smaller than a row's selection can be");
+    op_span(value, queries, checked_floats({steps - 1, query_stride}) + HEADS * COLUMNS * 4, "sdx_qsa_index_interval queries");
+    op_span(value, blocks, checked_floats({pool, uint64_t(COLUMNS)}), "sdx_qsa_index_interval blocks");
+    op_span(value, scores, checked_floats({steps, pool}), "sdx_qsa_index_interval scores");
+    op_span(value, indices, checked_floats({steps, selected}), "sdx_qsa_index_interval indices");
+    op_span(value, counts, checked_floats({steps}), "sdx_qsa_index_interval counts");
+    const size_t need = interval_scratch_bytes(steps, pool);
+    if (scratch_bytes < need) throw std::runtime_error("sdx_qsa_index_interval: scratch too small (see sdx_qsa_index_interval_scratch)");
+    op_span(value, scratch, need, "sdx_qsa_index_interval scratch");
+    unsigned gate = 0;
+    const uint32_t* undecided = interval_select(value, queries, query_stride, blocks, pool, base, steps, selected, scores, indices, counts, scratch, valid, &gate);
+    // the rows the intervals left undecided, by the exact kernels (workgroups of other rows leave at once)
+    const size_t most = size_t((base + steps) / 4);
+    scores_tiled_kernel<<<dim3(std::min(checked_blocks(most, TILE_BLOCKS), 128u), checked_blocks(steps, TILE_ROWS)), TILE_THREADS, 0, value.stream>>>(
+        queries, query_stride, blocks, pool, base, steps, scores, undecided, gate);
+    const unsigned rows = checked_blocks(steps, 1);
+    if (most <= size_t(LDS_RUNS) * SELECT_THREADS) launch_select<0>(value, scores, pool, base, nullptr, selected, most, rows, indices, counts, nullptr, nullptr, undecided);
+    else launch_select<33>(value, scores, pool, base, nullptr, selected, most, rows, indices, counts, nullptr, nullptr, undecided);
+    SD_OP_END
+}
+
+int sdx_qsa_index_interval_undecided(void* handle, const void* scratch, uint64_t steps, uint64_t pool, uint64_t* rows) {
+    SD_OP_BEGIN
+    if (!rows || !steps || steps > 4096 || !pool) throw std::runtime_error("sdx_qsa_index_interval_undecided: steps, pool, rows");
+    op_span(value, scratch, interval_scratch_bytes(steps, pool), "sdx_qsa_index_interval scratch");
+    *rows = interval_undecided(value, scratch, steps, pool);
     SD_OP_END
 }
 

@@ -210,6 +210,21 @@ class BlockIndexWorkload:
         self.gpu.qsa_index(self.queries.base(), 512, self.blocks.base(), self.pool, self.base, self.steps, 2052, self.scores.base(),
                            self.indices.base(), self.counts.base())
 
+    def with_interval(self):
+        """Adds the selection by intervals (sdx_qsa_index_interval): its scratch, and the packed keys kept from call to call."""
+        self.interval_scratch = self.gpu.buffer(self.gpu.qsa_index_interval_scratch(self.steps, self.pool))
+        self.valid = [0]
+        return self
+
+    def step_interval(self, keep_operands=False):
+        if not keep_operands:
+            self.valid[0] = 0
+        self.gpu.qsa_index_interval(self.queries.base(), 512, self.blocks.base(), self.pool, self.base, self.steps, 2052, self.scores.base(),
+                                    self.indices.base(), self.counts.base(), self.interval_scratch, self.valid)
+
+    def undecided(self):
+        return self.gpu.qsa_index_interval_undecided(self.interval_scratch, self.steps, self.pool)
+
     def with_attention(self, heads=24, kv_heads=2, row_bytes=272, seed=7):
         """Adds the attention over each row's selection: Q8_0 rows of 256 columns in the reference's state layout."""
         gpu, context = self.gpu, (self.pool - 1) * 4
@@ -253,6 +268,8 @@ class BlockIndexWorkload:
         if hasattr(self, "kv_buffer"):
             for b in (self.kv_buffer, self.q, self.out, self.scratch):
                 self.gpu.release(b)
+        if hasattr(self, "interval_scratch"):
+            self.gpu.release(self.interval_scratch)
 
 
 class QwenStageWorkload:

@@ -115,6 +115,114 @@ def test_block_scores_and_selection(gpu, oracle, mode, base, steps, context, str
     _check(oracle, queries, blocks, base, selected, _run_index(gpu, queries, blocks, base, selected))
 
 
+def _run_interval(gpu, queries, blocks, base, selected, state=None):
+    """sdx_qsa_index_interval on host arrays; `state` keeps the key buffer, scratch and packed-operand count between calls."""
+    steps, stride = queries.shape
+    pool = blocks.shape[1]
+    qb = gpu.upload(queries)
+    if state is None or "keys" not in state:
+        held = {"keys": gpu.upload(blocks), "scratch": gpu.buffer(gpu.qsa_index_interval_scratch(steps, pool)), "valid": [0]}
+        if state is not None:
+            state.update(held)
+    else:
+        held = state
+    scores = gpu.buffer(steps * pool * 4)
+    indices = gpu.upload(np.full(steps * selected + 8, CANARY, dtype=np.float32))
+    counts = gpu.upload(np.full(steps, CANARY, dtype=np.float32))
+    gpu.qsa_index_interval(qb.base(), stride, held["keys"].base(), pool, base, steps, selected, scores.base(), indices.base(), counts.base(),
+                           held["scratch"], held["valid"])
+    out = (_read(gpu, indices, np.float32, steps * selected + 8), _read(gpu, counts, np.float32, steps),
+           gpu.qsa_index_interval_undecided(held["scratch"], steps, pool))
+    for b in (qb, scores, indices, counts) + (() if state is not None else (held["keys"], held["scratch"])):
+        gpu.release(b)
+    return out
+
+
+def _check_selection(oracle, queries, blocks, base, selected, indices, counts):
+    steps = queries.shape[0]
+    want_scores = oracle.qsa_block_scores(queries, np.nan_to_num(blocks), base)
+    assert np.all(indices[steps * selected:] == CANARY)
+    for r in range(steps):
+        want = oracle.qsa_select(want_scores[r], base + r)
+        assert counts[r] == float(len(want)), f"row {r}: count {counts[r]} != {len(want)}"
+        row = indices[r * selected:(r + 1) * selected]
+        assert np.array_equal(row[:len(want)], want), f"row {r}: selection"
+        assert np.all(row[len(want):] == CANARY), f"row {r}: entries past the count are not touched"
+
+
+@pytest.mark.parametrize("mode,base,steps,context,decided", [
+    ("g", 40000, 37, 65536, True),       # gaussian keys: the intervals decide every row
+    ("t", 100000, 130, 131072, True),    # clustered scores, two row groups, rows of different complete counts
+    ("d", 60000, 20, 65536, True),       # exact ties where the cut falls: the band's order and ties are the exact kernels'
+    ("z", 40000, 6, 65536, False),       # zero queries on every other row: every block ties, the exact kernels take those rows
+    ("s", 50000, 9, 65536, None),        # magnitudes around the smallest normal FP16: wide bounds, whoever decides
+])
+def test_interval_selection_is_the_exact_one(gpu, oracle, mode, base, steps, context, decided):
+    # the reference's qsa_interval_test.cpp cases (:71-93 inputs, :95-140 "the selection is qsa_select_rows', block for block")
+    pool = context // 4 + 1
+    queries, blocks = _case(oracle, mode, base, steps, pool, 512, seed=base + steps)
+    indices, counts, undecided = _run_interval(gpu, queries, blocks, base, 2052)
+    _check_selection(oracle, queries, blocks, base, 2052, indices, counts)
+    if decided is True:
+        assert undecided == 0, f"{undecided} rows went to the exact kernels"
+    if decided is False:
+        assert undecided == (steps + 1) // 2
+
+
+def test_interval_selection_with_inputs_beyond_fp16_and_kept_operands(gpu, oracle):
+    base, steps, pool = 50000, 24, 65536 // 4 + 1
+    queries, blocks = _case(oracle, "g", base, 2 * steps, pool, 512, seed=9)
+    state = {}
+    first = _run_interval(gpu, queries[:steps], blocks, base, 2052, state)
+    _check_selection(oracle, queries[:steps], blocks, base, 2052, first[0], first[1])
+    assert first[2] == 0 and state["valid"][0] == (base + steps) // 4
+    # the next chunk packs only the new blocks' operands
+    second = _run_interval(gpu, queries[steps:], blocks, base + steps, 2052, state)
+    _check_selection(oracle, queries[steps:], blocks, base + steps, 2052, second[0], second[1])
+    assert second[2] == 0 and state["valid"][0] == (base + 2 * steps) // 4
+    for b in (state["keys"], state["scratch"]):
+        gpu.release(b)
+    # a key element beyond FP16 leaves every row that sees its block to the exact kernels; a query row beyond it, that row
+    wild = blocks.copy()
+    wild[7, 300] = 1.0e6
+    got = _run_interval(gpu, queries[:steps], wild, base, 2052)
+    _check_selection(oracle, queries[:steps], wild, base, 2052, got[0], got[1])
+    assert got[2] == steps
+    loud = queries[:steps].copy()
+    loud[5, 130] = -7.0e4
+    got = _run_interval(gpu, loud, blocks, base, 2052)
+    _check_selection(oracle, loud, blocks, base, 2052, got[0], got[1])
+    assert got[2] == 1
+    # below position 32768 the call is sdx_qsa_index
+    queries, blocks = _case(oracle, "g", 9000, 5, 16384 // 4 + 1, 512, seed=10)
+    got = _run_interval(gpu, queries, blocks, 9000, 2052)
+    _check_selection(oracle, queries, blocks, 9000, 2052, got[0], got[1])
+
+
+def test_interval_selection_of_a_chunk_at_242k_tokens(gpu):
+    # the bench's shape: 256 rows at position 242000 of a 262144-token context, against the exact kernels on the same device data
+    steps, base, pool = 256, 242000, 262144 // 4 + 1
+    queries, blocks = gpu.buffer(steps * 512 * 4), gpu.buffer(128 * pool * 4)
+    gpu.fill_normal(queries.base(), steps * 512, 61, 0)
+    gpu.fill_normal(blocks.base(), 128 * pool, 62, 0)
+    outs = []
+    scores = gpu.buffer(steps * pool * 4)
+    scratch = gpu.buffer(gpu.qsa_index_interval_scratch(steps, pool))
+    for interval in (False, True):
+        indices, counts = gpu.buffer(steps * 2052 * 4), gpu.buffer(steps * 4)
+        if interval:
+            gpu.qsa_index_interval(queries.base(), 512, blocks.base(), pool, base, steps, 2052, scores.base(), indices.base(), counts.base(), scratch)
+        else:
+            gpu.qsa_index(queries.base(), 512, blocks.base(), pool, base, steps, 2052, scores.base(), indices.base(), counts.base())
+        outs.append((_read(gpu, indices, np.float32, steps * 2052), _read(gpu, counts, np.float32, steps)))
+        gpu.release(indices); gpu.release(counts)
+    assert np.array_equal(outs[0][1], outs[1][1])
+    assert np.array_equal(outs[0][0], outs[1][0])
+    assert gpu.qsa_index_interval_undecided(scratch, steps, pool) <= 2
+    for b in (queries, blocks, scores, scratch):
+        gpu.release(b)
+
+
 def test_device_resident_position(gpu, oracle):
     # the replayable form: the position is read on the device, the launch shape does not depend on it
     base, steps, context = 12345, 4, 32768
