@@ -29,12 +29,12 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense FP16/BF16 MFMA, published
 # counters read for the library's 1 GiB copy kernel), kept here so that the bench line carries them; `traffic_source` names the
 # summary.  A counter run cannot share a process with the timed passes.
 PROFILED_TRAFFIC = {
-    "config1": (626.8e6, "profiles/paged_attention_q8_d128_decode_config1.md"),
-    "config1_32k": (1147.4e6, "profiles/paged_attention_q8_d128_decode_config1_32k.md"),
-    "config0": (None, None),
-    "config3": (None, "profiles/paged_attention_q8_d128_verify_config3.md"),
-    "config2": (None, "profiles/prefill_dense_d128_config2.md"),
-    "config4": (None, "profiles/sparse_path_config4.md"),
+    "config1": (626.9e6, "profiles/paged_attention_q8_d128_decode_config1.md"),
+    "config1_32k": (1147.5e6, "profiles/paged_attention_q8_d128_decode_config1_32k.md"),
+    "config0": (2.61e6, "profiles/paged_attention_q8_d128_decode_config0.md"),
+    "config3": (1157.7e6, "profiles/paged_attention_q8_d128_verify_config3.md"),
+    "config2": (117.1e6, "profiles/prefill_dense_d128_config2.md"),        # prefill_dense_kernel, averaged over a prompt's four launches
+    "config4": (278.0e6, "profiles/sparse_path_config4.md"),               # index_interval_kernel
 }
 
 
@@ -303,6 +303,11 @@ def main():
                 stage.release()
         return out
 
+    if args.workload == "block_index":
+        # the Qwen block indexer alone (what profiles/block_index_242k.md traces): not a BASELINE config, no headline metric
+        print(json.dumps({"workload": "Qwen block indexer at 242K tokens", "steps": args.steps, **run_block_index()}))
+        gpu.close()
+        return
     if args.workload == "config4":
         main_result = run_sparse()
         baseline = main_result.pop("cpu_baseline")
@@ -319,14 +324,17 @@ def main():
                 also[name], also_baseline = run_paged(name, not args.no_cpu, budget_seconds=3.0)
                 also[name]["cpu_baseline"] = also_baseline
                 also[name]["workload"] = names[name]
+                also[name]["traffic"], also[name]["traffic_source"] = PROFILED_TRAFFIC[name]
         if args.workload != "config2":
             also["config2"] = run_prefill()
             also["config2"]["workload"] = names["config2"]
+            also["config2"]["traffic"], also["config2"]["traffic_source"] = PROFILED_TRAFFIC["config2"]
             also["config2"]["measured_mfma_tflops"] = measured_mfma_ceiling(gpu, False)
             also["config2"]["measured_mfma_tflops_live_operands"] = measured_mfma_ceiling(gpu, True)
         if args.workload != "config4":
             also["config4"] = run_sparse()
             also["config4"]["workload"] = names["config4"]
+            also["config4"]["traffic"], also["config4"]["traffic_source"] = PROFILED_TRAFFIC["config4"]
         also["block_index_242k"] = run_block_index()
         also["block_index_242k"]["workload"] = "Qwen block indexer: 4x128 index heads, 60.5K complete blocks of a 262144-token context, top 512 blocks"
 
