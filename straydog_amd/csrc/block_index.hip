@@ -135,22 +135,10 @@ __global__ void __launch_bounds__(64 * HEADS) scores_rows_kernel(const float* __
 // bank conflicts, the query read is wave-uniform.  The next sixteen columns travel from global memory into registers while
 // the current ones are multiplied.
 constexpr int TILE_ROWS = 32, TILE_BLOCKS = 256, TILE_COLUMNS = 16, TILE_THREADS = 512, QUERY_PITCH = TILE_ROWS * HEADS + 4;
-__global__ void __launch_bounds__(TILE_THREADS) scores_tiled_kernel(const float* __restrict__ queries, size_t query_stride,
-                                                                    const float* __restrict__ blocks, size_t pool, size_t base, size_t steps,
-                                                                    float* __restrict__ scores, const uint32_t* __restrict__ only, unsigned gate) {
-    __shared__ __align__(16) float keys[2][TILE_COLUMNS][TILE_BLOCKS];
-    __shared__ __align__(16) float query[2][TILE_COLUMNS][QUERY_PITCH];
-    const size_t first_row = size_t(blockIdx.y) * TILE_ROWS;
-    if (only) {         // (behind the interval selection: the tiles of the rows it left undecided; only[gate] counts those rows)
-        if (!only[gate]) return;
-        bool any = false;
-        for (size_t r = first_row; r < min(steps, first_row + TILE_ROWS); ++r) any |= only[r] != 0;
-        if (!any) return;
-    }
-    const size_t most = min((base + min(steps, first_row + TILE_ROWS)) / 4, pool);        // complete blocks of the tile's last row
-    if (most <= KEEP) return;
-    // (a launch may have fewer workgroups than tiles of blocks: each takes every gridDim.x-th)
-    for (size_t first_block = size_t(blockIdx.x) * TILE_BLOCKS; first_block < most; first_block += size_t(gridDim.x) * TILE_BLOCKS) {
+// One tile of 32 rows x 256 blocks (every thread of the workgroup calls it; `most`: the complete blocks of the tile's last row).
+__device__ __forceinline__ void scores_tile(const float* __restrict__ queries, size_t query_stride, const float* __restrict__ blocks, size_t pool,
+                                            size_t base, size_t steps, float* __restrict__ scores, size_t first_row, size_t first_block,
+                                            float (&keys)[2][TILE_COLUMNS][TILE_BLOCKS], float (&query)[2][TILE_COLUMNS][QUERY_PITCH]) {
     const unsigned t = threadIdx.x, lane = t % 64, wave = t / 64;
     constexpr int KEY_LOADS = TILE_COLUMNS * TILE_BLOCKS / TILE_THREADS, QUERY_LOADS = TILE_COLUMNS * TILE_ROWS * HEADS / TILE_THREADS;
     float key_next[KEY_LOADS], query_next[QUERY_LOADS];
@@ -211,6 +199,30 @@ __global__ void __launch_bounds__(TILE_THREADS) scores_tiled_kernel(const float*
             if (block < complete) scores[row * pool + block] = positive_sum(dot);
         }
     }
+}
+
+// ONLY = false: a workgroup per tile.  ONLY = true (behind the interval selection): the tiles of the rows it left undecided, which
+// only[row] marks and only[gate] counts; a launch has fewer workgroups than tiles of blocks, each takes every gridDim.x-th, and
+// every workgroup leaves at once when no row is marked.
+template<bool ONLY>
+__global__ void __launch_bounds__(TILE_THREADS) scores_tiled_kernel(const float* __restrict__ queries, size_t query_stride,
+                                                                    const float* __restrict__ blocks, size_t pool, size_t base, size_t steps,
+                                                                    float* __restrict__ scores, const uint32_t* __restrict__ only, unsigned gate) {
+    __shared__ __align__(16) float keys[2][TILE_COLUMNS][TILE_BLOCKS];
+    __shared__ __align__(16) float query[2][TILE_COLUMNS][QUERY_PITCH];
+    const size_t first_row = size_t(blockIdx.y) * TILE_ROWS;
+    const size_t most = min((base + min(steps, first_row + TILE_ROWS)) / 4, pool);        // complete blocks of the tile's last row
+    if (most <= KEEP) return;
+    if (ONLY) {
+        if (!only[gate]) return;
+        bool any = false;
+        for (size_t r = first_row; r < min(steps, first_row + TILE_ROWS); ++r) any |= only[r] != 0;
+        if (!any) return;
+        for (size_t first_block = size_t(blockIdx.x) * TILE_BLOCKS; first_block < most; first_block += size_t(gridDim.x) * TILE_BLOCKS)
+            scores_tile(queries, query_stride, blocks, pool, base, steps, scores, first_row, first_block, keys, query);
+    } else {
+        const size_t first_block = size_t(blockIdx.x) * TILE_BLOCKS;
+        if (first_block < most) scores_tile(queries, query_stride, blocks, pool, base, steps, scores, first_row, first_block, keys, query);
     }
 }
 
@@ -712,7 +724,7 @@ int sdx_qsa_index(void* handle, const float* queries, uint64_t query_stride, con
             else if (steps <= 8) launch_rows<8>(value, queries, query_stride, blocks, pool, base, dynamic_base, steps, most, scores);
             else {
                 if (dynamic_base) throw std::runtime_error("sdx_qsa_index: a device-resident position serves spans of up to 8 rows");
-                timed_launch(value, &scores_tiled_kernel, dim3(checked_blocks(most, TILE_BLOCKS), checked_blocks(steps, TILE_ROWS)), dim3(TILE_THREADS), 0,
+                timed_launch(value, &scores_tiled_kernel<false>, dim3(checked_blocks(most, TILE_BLOCKS), checked_blocks(steps, TILE_ROWS)), dim3(TILE_THREADS), 0,
                              queries, query_stride, blocks, pool, base, steps, scores, static_cast<const uint32_t*>(nullptr), 0u);
             }
         }
@@ -765,7 +777,7 @@ int sdx_qsa_index_interval(void* handle, const float* queries, uint64_t query_st
     const uint32_t* undecided = interval_select(value, queries, query_stride, blocks, pool, base, steps, selected, scores, indices, counts, scratch, valid, &gate);
     // the rows the intervals left undecided, by the exact kernels (workgroups of other rows leave at once)
     const size_t most = size_t((base + steps) / 4);
-    scores_tiled_kernel<<<dim3(std::min(checked_blocks(most, TILE_BLOCKS), 128u), checked_blocks(steps, TILE_ROWS)), TILE_THREADS, 0, value.stream>>>(
+    scores_tiled_kernel<true><<<dim3(std::min(checked_blocks(most, TILE_BLOCKS), 128u), checked_blocks(steps, TILE_ROWS)), TILE_THREADS, 0, value.stream>>>(
         queries, query_stride, blocks, pool, base, steps, scores, undecided, gate);
     const unsigned rows = checked_blocks(steps, 1);
     if (most <= size_t(LDS_RUNS) * SELECT_THREADS) launch_select<0>(value, scores, pool, base, nullptr, selected, most, rows, indices, counts, nullptr, nullptr, undecided);
