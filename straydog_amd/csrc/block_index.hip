@@ -777,7 +777,7 @@ int sdx_qsa_index_interval(void* handle, const float* queries, uint64_t query_st
     const uint32_t* undecided = interval_select(value, queries, query_stride, blocks, pool, base, steps, selected, scores, indices, counts, scratch, valid, &gate);
     // the rows the intervals left undecided, by the exact kernels (workgroups of other rows leave at once)
     const size_t most = size_t((base + steps) / 4);
-    scores_tiled_kernel<true><<<dim3(std::min(checked_blocks(most, TILE_BLOCKS), 128u), checked_blocks(steps, TILE_ROWS)), TILE_THREADS, 0, value.stream>>>(
+    scores_tiled_kernel<true><<<dim3(std::min(checked_blocks(most, TILE_BLOCKS), 64u), checked_blocks(steps, TILE_ROWS)), TILE_THREADS, 0, value.stream>>>(
         queries, query_stride, blocks, pool, base, steps, scores, undecided, gate);
     const unsigned rows = checked_blocks(steps, 1);
     if (most <= size_t(LDS_RUNS) * SELECT_THREADS) launch_select<0>(value, scores, pool, base, nullptr, selected, most, rows, indices, counts, nullptr, nullptr, undecided);
