@@ -295,6 +295,17 @@ def main():
                 ms, kernel_ms = timed(gpu, work.step_attention, max(args.steps // 5, 3), 2)
                 out[name].update({"selected_attention_us": ms * 1e3, "selected_attention_kernel_us": None if kernel_ms is None else kernel_ms * 1e3,
                                   "selected_attention_gbps": work.attention_bytes() / ms / 1e6})
+                if rows > 8:
+                    # the same attention as a union walk (sdx_selected_attention_union), on these selections (independent queries:
+                    # nothing to share) and on selections that overlap as consecutive prompt tokens' do (runs of 16 similar queries)
+                    work.with_union()
+                    ms, _ = timed(gpu, work.step_attention_union, 3, 1)
+                    out[name]["selected_attention_union_us"] = ms * 1e3
+                    work.similar_queries()
+                    work.step()
+                    ms, _ = timed(gpu, work.step_attention, 3, 1)
+                    union_ms, _ = timed(gpu, work.step_attention_union, 3, 1)
+                    out[name].update({"similar_queries_selected_attention_us": ms * 1e3, "similar_queries_selected_attention_union_us": union_ms * 1e3})
             work.release()
             if rows <= 8:
                 stage = workloads.QwenStageWorkload(gpu, rows)

@@ -192,6 +192,18 @@ int sdx_selected_attention(void* handle, const sdx_kv_pool* pool, const int32_t*
                            const uint32_t* dynamic_base, const float* indices, uint64_t selected, const float* counts, const void* q, int q_f16,
                            uint64_t rows, uint64_t heads, float scale, const float* gate, uint64_t gate_stride, uint64_t gate_row_stride, void* out, int out_f16,
                            void* scratch, uint64_t scratch_bytes);
+/* The same attention for the rows of a prompt chunk as a union walk (the reference's qsa_flash_wmma over qsa_mark_blocks /
+ * qsa_union_blocks, gpu/sparse_attention_compute.hpp:744-755, 841-896, 906-1041): the tokens whose query rows share a tile of 64
+ * rows walk the union of their selections once, a K/V row converted once for all of them, a bit per (entry, token) masking what a
+ * token did not select.  It pays when consecutive tokens select mostly the same positions, as the rows of a real prompt do; on
+ * selections that do not overlap it gains nothing over sdx_selected_attention.  Same arguments (no device-resident position),
+ * same rule for entries that count; an entry a row names twice counts once; a row with no entry that counts gives zeros.
+ * scratch: sdx_selected_attention_union_scratch(rows, heads, kv_heads, selected, context) bytes (a word per position and tile). */
+uint64_t sdx_selected_attention_union_scratch(uint64_t rows, uint64_t heads, uint64_t kv_heads, uint64_t selected, uint64_t context);
+int sdx_selected_attention_union(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t context, uint64_t base,
+                                 const float* indices, uint64_t selected, const float* counts, const void* q, int q_f16, uint64_t rows, uint64_t heads,
+                                 float scale, const float* gate, uint64_t gate_stride, uint64_t gate_row_stride, void* out, int out_f16, void* scratch,
+                                 uint64_t scratch_bytes);
 
 /* Top-k indexed sparse attention over BF16 latent K/V for a batch of sequences (one decode row each):
  * stage 1+2 = sd_op_index_scores + sd_op_top_k per sequence (gpu/ops.hpp:1700-1739, 1766-1941) with each sequence's own

@@ -116,6 +116,9 @@ SIGNATURES = {
     "sdx_selected_attention_scratch": (c_u64, [c_u64, c_u64, c_u64]),
     "sdx_selected_attention": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_u64, c_void_p, c_void_p, c_int,
                                        c_u64, c_u64, c_float, c_void_p, c_u64, c_u64, c_void_p, c_int, c_void_p, c_u64]),
+    "sdx_selected_attention_union_scratch": (c_u64, [c_u64, c_u64, c_u64, c_u64, c_u64]),
+    "sdx_selected_attention_union": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_u64, c_void_p, c_u64, c_void_p, c_void_p, c_int,
+                                             c_u64, c_u64, c_float, c_void_p, c_u64, c_u64, c_void_p, c_int, c_void_p, c_u64]),
     "sdx_qsa_decode_attend_scratch": (c_u64, [c_u64, c_u64, c_u64, c_u64]),
     "sdx_qsa_decode_attend": (c_int, [c_void_p, _P(QsaState), c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_void_p, c_u64, c_void_p]),
     "sdx_index_projection": (c_int, [c_void_p, c_void_p, c_int, c_u64, c_void_p, c_u64, c_void_p]),

@@ -291,6 +291,15 @@ class Backend:
                                                    counts, q, int(q_f16), rows, heads, scale, gate, gate_stride, gate_row_stride, out, int(out_f16),
                                                    scratch.pointer, scratch.size))
 
+    def selected_attention_union_scratch(self, rows, heads, kv_heads, selected, context):
+        return int(self.lib.sdx_selected_attention_union_scratch(rows, heads, kv_heads, selected, context))
+
+    def selected_attention_union(self, pool, page_table, context, base, indices, selected, counts, q, q_f16, rows, heads, scale, out, out_f16,
+                                 scratch, gate=None, gate_stride=0, gate_row_stride=0):
+        self.check(self.lib.sdx_selected_attention_union(self.handle, ctypes.byref(pool), page_table, context, base, indices, selected, counts, q,
+                                                         int(q_f16), rows, heads, scale, gate, gate_stride, gate_row_stride, out, int(out_f16),
+                                                         scratch.pointer, scratch.size))
+
     def qsa_state(self, pool, page_table, context, blocks, history, q_norm, k_norm, index_q_norm, index_k_norm, heads):
         """An sdx_qsa_state over device pointers (the pool struct is kept alive by the returned object)."""
         state = abi.QsaState(ctypes.pointer(pool), page_table, context, blocks, history, q_norm, k_norm, index_q_norm, index_k_norm, heads)

@@ -51,9 +51,20 @@ struct PrefillArgs {
     unsigned page_last;    // the pool's last page (table entries outside the pool are taken as the nearest page of it)
     void* out;
     int out_f16;
+    // The union walk (UNION kernels only): each tile of query rows walks the list of positions that some token of the tile
+    // selected, union_pos[tile][entry] in ascending order, union_count[tile] of them; bit (token - the tile's first token) of
+    // union_mask[tile][entry] says whether that token selected the entry.  One sequence, whose first row is at `base`; a null
+    // page table means one page holds the context.  gate (or null): the output is multiplied by sigmoid(gate[token][head][column]).
+    const int32_t* union_pos;
+    const uint32_t* union_mask;
+    const uint32_t* union_count;
+    unsigned union_cap;
+    int base;
+    const float* gate;
+    size_t gate_stride, gate_row_stride;
 };
 
-template<int DIM, int QT, bool Q8, int OCC>
+template<int DIM, int QT, bool Q8, int OCC, bool UNION = false>
 __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) prefill_attention_kernel(PrefillArgs args) {
     constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, BLOCKS = DIM / 32, W = DIM / 16, TILES = DIM / 16;
     constexpr int SLAB = WALK * ROW, UNITS = (SLAB + 1023) / 1024;     // a slab is copied 1 KiB (one instruction of a wave) at a time
@@ -61,15 +72,19 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     static_assert(STAGES >= 2, "a step is copied while the one before is computed");
     const int tile = int(gridDim.x) - 1 - int(blockIdx.x), kvh = blockIdx.y, seq = blockIdx.z;   // later rows walk further: first
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), li = lane & 15, g = lane >> 4;
-    const int position = first_position(args.positions, unsigned(seq), args.max_context);
-    const int cached = min(position + int(args.span), args.max_context);          // rows of the sequence the cache holds
+    const int position = UNION ? args.base : first_position(args.positions, unsigned(seq), args.max_context);
+    // rows of the sequence the cache holds; of a union walk: the entries of the tile's list, which `keys` then counts
+    const int cached = UNION ? int(args.union_count[tile]) : min(position + int(args.span), args.max_context);
     const int quarter = wave % GROUPS, half = wave / GROUPS;                      // waves w and w + 4 share a SIMD and the rows
     const int row0 = tile * GROUP_ROWS + quarter * WAVE_ROWS;                     // the wave's first query row
     const int group_last = min(int(args.rows), (tile + 1) * GROUP_ROWS) - 1;
-    const int keys = min(position + group_last / int(args.group) + 1, cached);    // the workgroup walks keys 0..keys-1
+    const int keys = UNION ? cached : min(position + group_last / int(args.group) + 1, cached);    // the workgroup walks keys 0..keys-1
     const bool idle = row0 >= int(args.rows);                                     // a wave past the last row only helps copying
-    const int wave_first = position + row0 / int(args.group);                      // the smallest and largest position of
-    const int wave_last = position + (min(int(args.rows), row0 + WAVE_ROWS) - 1) / int(args.group);   // the wave's rows
+    const int wave_first = UNION ? -1 : position + row0 / int(args.group);        // the smallest and largest position of
+    const int wave_last = UNION ? 0x7fffffff : position + (min(int(args.rows), row0 + WAVE_ROWS) - 1) / int(args.group);   // the wave's rows
+    const int tile_token = tile * GROUP_ROWS / int(args.group);                  // (union walk) the first token with a row in the tile
+    const int32_t* const listed = UNION ? args.union_pos + size_t(tile) * args.union_cap : nullptr;
+    const uint32_t* const marks = UNION ? args.union_mask + size_t(tile) * args.union_cap : nullptr;
     const table_ptr table = (table_ptr)(args.page_table + size_t(seq) * args.table_stride);
     const size_t plane_bytes = size_t(args.page_tokens) * ROW;
     extern __shared__ uint8_t stages[];                                           // [STAGES][K slab | V slab]
@@ -79,7 +94,7 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     // The step's two slabs into a stage: 2 * UNITS pieces of 1 KiB, every fourth one by this wave.
     // (Pages of fewer tokens than a step: the step's rows lie in two pages, and every lane looks up the page of its own
     // 16 bytes; rows past the cached ones are the last cached row again, and never read.)
-    const bool split_pages = args.page_tokens % WALK != 0;
+    const bool split_pages = UNION || args.page_tokens % WALK != 0;
     const auto copy_in = [&](int buffer, int token0) {
         uint8_t* stage = stages + buffer * (2 * SLAB);
         if (split_pages) {
@@ -87,8 +102,10 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
             for (int k = 0; k < MOST; ++k) {
                 const int unit = wave + TEAM * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS, at = 16 * lane + 1024 * j;
                 if (unit < 2 * UNITS && at < SLAB) {
-                    const int token = min(token0 + at / ROW, cached - 1);
-                    const int page = pool_page(args.page_table[size_t(seq) * args.table_stride + token / int(args.page_tokens)], args.page_last);
+                    // (union walk: the step's rows are the list's entries; entries past the last are the last again, masked)
+                    const int token = UNION ? listed[min(token0 + at / ROW, cached - 1)] : min(token0 + at / ROW, cached - 1);
+                    const int page = UNION && !args.page_table ? 0 :
+                        pool_page(args.page_table[size_t(seq) * args.table_stride + token / int(args.page_tokens)], args.page_last);
                     const uint8_t* from = args.pages + (size_t(page) * 2 * args.kv_heads + (part ? args.kv_heads : 0) + kvh) * plane_bytes +
                                           size_t(token % int(args.page_tokens)) * ROW + at % ROW;
                     __builtin_amdgcn_global_load_lds((global_ptr)from, (lds_ptr)(stage + part * SLAB + 1024 * j), 16, 0, 0);
@@ -121,7 +138,8 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
         const int row = row0 + qt * 16 + li;
         const bool real = row < int(args.rows);
         const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
-        limit[qt] = real ? position + span_row : 0x7fffffff;
+        // (union walk: the bit of the row's token in an entry's mask; a padding row has none)
+        limit[qt] = UNION ? (real ? span_row - tile_token : 31) : real ? position + span_row : 0x7fffffff;
         const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
         #pragma unroll
         for (int b = 0; b < BLOCKS; ++b) {
@@ -152,7 +170,7 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
         __syncthreads();                             // ... and everybody's; the stage of the step before is no longer being read
         copy_in(buffer == 0 ? STAGES - 1 : buffer - 1, min(walk0 + (STAGES - 1) * WALK, last_step));
         uint8_t* stage = stages + buffer * (2 * SLAB);
-        if (cached - walk0 < WALK) {
+        if (!UNION && cached - walk0 < WALK) {
             // the sequence's last rows: the stage's tail holds whatever the page held.  It is cleared (those scores are masked,
             // but a stray scale must not meet a zero weight).
             #pragma unroll
@@ -179,7 +197,18 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
             }
         }
         // Scores stay unscaled; the scale goes into the exponent's multiply-add.  m is a row's reference maximum in unscaled units.
-        if (token0 + STEP - 1 > wave_first) {          // wave-uniform: some token of the step is past some row's position
+        if (UNION) {
+            // an entry counts for a row when the row's token selected it: the lane's eight entries' masks, the row's bit
+            const uint4 low = *reinterpret_cast<const uint4*>(marks + token0 + 4 * g), high = *reinterpret_cast<const uint4*>(marks + token0 + 16 + 4 * g);
+            const uint32_t mask[2][4] = {{low.x, low.y, low.z, low.w}, {high.x, high.y, high.z, high.w}};
+            #pragma unroll
+            for (int qt = 0; qt < QT; ++qt)
+                #pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    #pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (token0 + 16 * t + 4 * g + r >= keys || !((mask[t][r] >> limit[qt]) & 1u)) s[qt][t][r] = -INFINITY;
+        } else if (token0 + STEP - 1 > wave_first) {          // wave-uniform: some token of the step is past some row's position
             #pragma unroll
             for (int qt = 0; qt < QT; ++qt)
                 #pragma unroll
@@ -270,9 +299,19 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     for (int qt = 0; qt < QT; ++qt) {
         const int row = row0 + qt * 16 + li;
         if (row >= int(args.rows)) continue;
-        const float inverse = 1.0f / l[qt];
+        const float inverse = UNION && !(l[qt] > 0.0f) ? 0.0f : 1.0f / l[qt];     // (a row whose list names no position it may see: zeros)
         const int span_row = row / int(args.group), head = kvh * int(args.group) + row % int(args.group);
         const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
+        if (UNION && args.gate) {
+            #pragma unroll
+            for (int r = 0; r < 4; ++r)
+                #pragma unroll
+                for (int jj = 0; jj < TILES; ++jj) {
+                    const float x = args.gate[size_t(span_row) * args.gate_row_stride + size_t(head) * args.gate_stride + W * (4 * g + r) + jj];
+                    const float e = expf(-fabsf(x));
+                    acc[qt][jj][r] *= x >= 0.0f ? 1.0f / (1.0f + e) : e / (1.0f + e);
+                }
+        }
         #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const size_t first = at + W * (4 * g + r);
@@ -674,6 +713,35 @@ void prefill_attention(Device& d, const sdx_kv_pool* pool, const int32_t* page_t
     const bool q8 = pool->row_bytes != 2 * pool->dim;
     if (pool->dim == 128) { if (q8) launch_dense<128, 2, true>(d, args, unsigned(seqs)); else launch_dense<128, 2, false>(d, args, unsigned(seqs)); }
     else { if (q8) launch<256, 1, true, 2>(d, args, unsigned(seqs)); else launch<256, 1, false, 2>(d, args, unsigned(seqs)); }
+}
+
+// The union walk of a prompt chunk (256 columns): `tokens` rows of one sequence from position `base`, each tile of 64 query rows
+// (16 x the heads of a K/V head) walking its own list of positions (see PrefillArgs).  Lists and masks are device memory.
+unsigned union_tile_rows() { return GROUPS * 16; }
+void prefill_union(Device& d, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t base, const void* q, int q_f16, uint64_t tokens,
+                   uint64_t heads, float scale, const float* gate, uint64_t gate_stride, uint64_t gate_row_stride, void* out, int out_f16,
+                   const int32_t* union_pos, const uint32_t* union_mask, const uint32_t* union_count, unsigned union_cap) {
+    PrefillArgs args{};
+    args.pages = static_cast<const uint8_t*>(pool->pages);
+    args.page_tokens = pool->page_tokens; args.kv_heads = pool->kv_heads; args.heads = unsigned(heads);
+    args.group = unsigned(heads / pool->kv_heads); args.span = unsigned(tokens);
+    args.page_table = page_table; args.table_stride = 0; args.positions = nullptr;
+    args.q = q; args.q_f16 = q_f16; args.scale_log2 = scale * 1.44269504088896341f;
+    args.rows = unsigned(tokens * args.group); args.max_context = 0;
+    args.page_last = unsigned(std::min<uint64_t>(pool->page_count - 1, 0x7fffffffu));
+    args.out = out; args.out_f16 = out_f16;
+    args.union_pos = union_pos; args.union_mask = union_mask; args.union_count = union_count; args.union_cap = union_cap;
+    args.base = int(base); args.gate = gate; args.gate_stride = size_t(gate_stride); args.gate_row_stride = size_t(gate_row_stride);
+    const bool q8 = pool->row_bytes != 2 * pool->dim;
+    const auto go = [&](auto kernel, size_t stage_bytes) {
+        const size_t merge = size_t(GROUPS) * (256 / 16 * 4 + 2) * 64 * 4, ring = stages_for(int(stage_bytes)) * stage_bytes;
+        const size_t shared = ring > merge ? ring : merge;
+        if (shared > 64 * 1024) raise_shared_limit(d, reinterpret_cast<const void*>(kernel), shared);
+        const unsigned tiles = (args.rows + GROUPS * 16 - 1) / (GROUPS * 16);
+        timed_launch(d, kernel, dim3(tiles, args.kv_heads, 1), dim3(TEAM * 64), shared, args);
+    };
+    if (q8) go(&prefill_attention_kernel<256, 1, true, 2, true>, size_t(2) * WALK * (256 + 16));
+    else go(&prefill_attention_kernel<256, 1, false, 2, true>, size_t(2) * WALK * 512);
 }
 
 }  // namespace sd

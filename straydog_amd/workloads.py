@@ -248,6 +248,24 @@ class BlockIndexWorkload:
         self.gpu.selected_attention(self.kv, None, (self.pool - 1) * 4, self.base, self.indices.base(), 2052, self.counts.base(), self.q.base(), True,
                                     self.steps, self.heads, 0.0625, self.out.base(), True, self.scratch)
 
+    def with_union(self):
+        """Adds the union walk over the same selections (sdx_selected_attention_union); call after with_attention."""
+        context = (self.pool - 1) * 4
+        self.union_scratch = self.gpu.buffer(self.gpu.selected_attention_union_scratch(self.steps, self.heads, self.kv_heads, 2052, context))
+        return self
+
+    def step_attention_union(self):
+        self.gpu.selected_attention_union(self.kv, None, (self.pool - 1) * 4, self.base, self.indices.base(), 2052, self.counts.base(), self.q.base(), True,
+                                          self.steps, self.heads, 0.0625, self.out.base(), True, self.union_scratch)
+
+    def similar_queries(self, alike=16, noise=0.05, seed=9):
+        """Index queries as consecutive tokens of a prompt have them: runs of `alike` rows share a query up to a little noise, so
+        their selections overlap; call step() afterwards to select with them."""
+        rng = np.random.default_rng(seed)
+        shared = rng.standard_normal(((self.steps + alike - 1) // alike, 512)).astype(np.float32)
+        rows = np.repeat(shared, alike, axis=0)[:self.steps] + noise * rng.standard_normal((self.steps, 512)).astype(np.float32)
+        self.gpu.write_buffer(self.queries, 0, rows.astype(np.float32).reshape(-1))
+
     def attention_bytes(self):
         # the selected rows of both planes of every K/V head, once per row
         return self.steps * 2051 * self.kv_heads * 2 * self.row_bytes
@@ -270,6 +288,8 @@ class BlockIndexWorkload:
                 self.gpu.release(b)
         if hasattr(self, "interval_scratch"):
             self.gpu.release(self.interval_scratch)
+        if hasattr(self, "union_scratch"):
+            self.gpu.release(self.union_scratch)
 
 
 class QwenStageWorkload:

@@ -404,6 +404,45 @@ def test_selected_attention_of_a_prompt_chunk(gpu, oracle):
         gpu.release(b)
 
 
+@pytest.mark.parametrize("row_bytes,paged,steps", [(272, True, 40), (512, False, 23), (272, False, 7)])
+def test_selected_attention_as_a_union_walk(gpu, oracle, row_bytes, paged, steps):
+    # the rows of a chunk sharing one walk over the union of their selections (the reference's qsa_flash_wmma over qsa_union_blocks,
+    # gpu/sparse_attention_compute.hpp:841-1041): the same outputs as the per-row form, against the oracle; lists with entries that do
+    # not count, Q8_0 and FP16 rows, the state layout and a shuffled page table, the gate, FP16 in and out
+    from gpu_util import close_enough
+    rng = np.random.default_rng(1000 + row_bytes + steps)
+    context, base, selected = 4096, 2900, 2052
+    state, q, indices, counts, want = _qwen_case(oracle, rng, row_bytes, context, base, steps, selected)
+    planes = state.reshape(4, context, row_bytes)
+    if paged:
+        page_tokens, pages = 256, context // 256
+        order = rng.permutation(pages + 3)[:pages].astype(np.int32)
+        host = np.zeros((pages + 3, 4, page_tokens, row_bytes), dtype=np.uint8)
+        for p in range(pages):
+            host[order[p]] = planes[:, p * page_tokens:(p + 1) * page_tokens]
+        pool, buffer = gpu.kv_pool(pages + 3, page_tokens, 2, 256, row_bytes)
+        table = gpu.upload(order)
+    else:
+        host = planes
+        pool, buffer = gpu.kv_pool(1, context, 2, 256, row_bytes)
+        table = None
+    gpu.write_buffer(buffer, 0, np.ascontiguousarray(host).reshape(-1))
+    gate = rng.standard_normal((steps, 24, 512)).astype(np.float32) * 2
+    ib, cb, gb = gpu.upload(indices), gpu.upload(counts), gpu.upload(gate)
+    scratch = gpu.buffer(gpu.selected_attention_union_scratch(steps, 24, 2, selected, context))
+    for q_f16, out_f16, gated in ((False, False, False), (True, True, True)):
+        qb = gpu.upload(q.astype(np.float16) if q_f16 else q)
+        out = gpu.buffer(steps * 24 * 256 * (2 if out_f16 else 4))
+        gpu.selected_attention_union(pool, table.base() if paged else None, context, base, ib.base(), selected, cb.base(), qb.base(), q_f16, steps, 24,
+                                     0.0625, out.base(), out_f16, scratch, gate=gb.at(256 * 4) if gated else None, gate_stride=512)
+        got = _read(gpu, out, np.float16 if out_f16 else np.float32, steps * 24 * 256).astype(np.float32).reshape(steps, 24, 256)
+        expect = want * (1.0 / (1.0 + np.exp(-gate[:, :, 256:].astype(np.float64)))) if gated else want
+        close_enough(got, expect, f"union walk f16={q_f16} gated={gated}")
+        gpu.release(qb); gpu.release(out)
+    for b in (ib, cb, gb, scratch, buffer) + ((table,) if paged else ()):
+        gpu.release(b)
+
+
 def test_index_then_attend_on_the_device(gpu, oracle):
     # the two stages chained on the device, as a decode pass runs them: sdx_qsa_index's lists feed sdx_selected_attention unchanged
     from gpu_util import close_enough
