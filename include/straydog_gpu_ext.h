@@ -195,7 +195,7 @@ int sdx_selected_attention(void* handle, const sdx_kv_pool* pool, const int32_t*
 /* The same attention for the rows of a prompt chunk as a union walk (the reference's qsa_flash_wmma over qsa_mark_blocks /
  * qsa_union_blocks, gpu/sparse_attention_compute.hpp:744-755, 841-896, 906-1041): the tokens whose query rows share a tile of 64
  * rows walk the union of their selections once, a K/V row converted once for all of them, a bit per (entry, token) masking what a
- * token did not select.  It pays when consecutive tokens select mostly the same positions, as the rows of a real prompt do; on
+ * token did not select (2 to 16 heads a K/V head).  It pays when consecutive tokens select mostly the same positions, as the rows of a real prompt do; on
  * selections that do not overlap it gains nothing over sdx_selected_attention.  Same arguments (no device-resident position),
  * same rule for entries that count; an entry a row names twice counts once; a row with no entry that counts gives zeros.
  * scratch: sdx_selected_attention_union_scratch(rows, heads, kv_heads, selected, context) bytes (a word per position and tile). */

@@ -166,9 +166,10 @@ int sdx_selected_attention_union(void* handle, const sdx_kv_pool* pool, const in
     SD_OP_BEGIN
     validate_pool(value, pool);
     if (pool->dim != 256) throw std::runtime_error("sdx_selected_attention_union: rows of 256 columns");
-    if (!(scale > 0.0f) || !rows || rows > 65535 || !heads || heads % pool->kv_heads || heads / pool->kv_heads > 16 || !selected || !context ||
-        context > (uint64_t(1) << 24) || pool->kv_heads > 65535 || selected > (uint64_t(1) << 20))
-        throw std::runtime_error("sdx_selected_attention_union: rows, heads (a multiple of the K/V heads, at most 16 each), selected and context >= 1, scale > 0");
+    // (a tile of 64 query rows holds 64 / group tokens, and an entry's mask has 32 bits)
+    if (!(scale > 0.0f) || !rows || rows > 65535 || !heads || heads % pool->kv_heads || heads / pool->kv_heads > 16 || heads / pool->kv_heads < 2 ||
+        !selected || !context || context > (uint64_t(1) << 24) || pool->kv_heads > 65535 || selected > (uint64_t(1) << 20))
+        throw std::runtime_error("sdx_selected_attention_union: rows, heads (a multiple of the K/V heads, 2 to 16 each), selected and context >= 1, scale > 0");
     const uint64_t pages = (context + pool->page_tokens - 1) / pool->page_tokens;
     if (page_table) op_span(value, page_table, checked_floats({pages}), "a page table");
     else if (pool->page_tokens < context) throw std::runtime_error("sdx_selected_attention_union: without a page table one page must hold the context");
