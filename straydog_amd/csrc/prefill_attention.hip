@@ -95,17 +95,37 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     // (Pages of fewer tokens than a step: the step's rows lie in two pages, and every lane looks up the page of its own
     // 16 bytes; rows past the cached ones are the last cached row again, and never read.)
     const bool split_pages = UNION || args.page_tokens % WALK != 0;
-    const auto copy_in = [&](int buffer, int token0) {
+    // (union walk) where the rows of the wave's pieces of one step lie, in 16-byte units from the pool's start (K plane of K/V
+    // head 0): read from the list a step before the pieces themselves are asked for, so that the wait for them does not also
+    // wait for the copies in flight.  Entries past the list's last are the last again (masked).
+    uint32_t held[MOST] = {};
+    const auto look_up = [&](int token0, uint32_t (&places)[MOST]) {
+        #pragma unroll
+        for (int k = 0; k < MOST; ++k) {
+            const int unit = wave + TEAM * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS, at = 16 * lane + 1024 * j;
+            places[k] = unit < 2 * UNITS && at < SLAB ? uint32_t(listed[min(token0 + at / ROW, cached - 1)]) : 0u;
+        }
+    };
+    const auto copy_in = [&](int buffer, int token0, const uint32_t (&places)[MOST] = {}) {
         uint8_t* stage = stages + buffer * (2 * SLAB);
+        if (UNION) {
+            #pragma unroll
+            for (int k = 0; k < MOST; ++k) {
+                const int unit = wave + TEAM * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS, at = 16 * lane + 1024 * j;
+                if (unit < 2 * UNITS && at < SLAB) {
+                    const uint8_t* from = args.pages + size_t(places[k]) * 16 + (size_t(part ? args.kv_heads : 0) + kvh) * plane_bytes + at % ROW;
+                    __builtin_amdgcn_global_load_lds((global_ptr)from, (lds_ptr)(stage + part * SLAB + 1024 * j), 16, 0, 0);
+                }
+            }
+            return;
+        }
         if (split_pages) {
             #pragma unroll
             for (int k = 0; k < MOST; ++k) {
                 const int unit = wave + TEAM * k, part = unit >= UNITS ? 1 : 0, j = unit - part * UNITS, at = 16 * lane + 1024 * j;
                 if (unit < 2 * UNITS && at < SLAB) {
-                    // (union walk: the step's rows are the list's entries; entries past the last are the last again, masked)
-                    const int token = UNION ? listed[min(token0 + at / ROW, cached - 1)] : min(token0 + at / ROW, cached - 1);
-                    const int page = UNION && !args.page_table ? 0 :
-                        pool_page(args.page_table[size_t(seq) * args.table_stride + token / int(args.page_tokens)], args.page_last);
+                    const int token = min(token0 + at / ROW, cached - 1);
+                    const int page = pool_page(args.page_table[size_t(seq) * args.table_stride + token / int(args.page_tokens)], args.page_last);
                     const uint8_t* from = args.pages + (size_t(page) * 2 * args.kv_heads + (part ? args.kv_heads : 0) + kvh) * plane_bytes +
                                           size_t(token % int(args.page_tokens)) * ROW + at % ROW;
                     __builtin_amdgcn_global_load_lds((global_ptr)from, (lds_ptr)(stage + part * SLAB + 1024 * j), 16, 0, 0);
@@ -127,7 +147,11 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     // is the same at every step.
     const int last_step = (keys - 1) / WALK * WALK;
     #pragma unroll
-    for (int ahead = 0; ahead < STAGES - 1; ++ahead) copy_in(ahead, min(ahead * WALK, last_step));
+    for (int ahead = 0; ahead < STAGES - 1; ++ahead) {
+        if (UNION) look_up(min(ahead * WALK, last_step), held);
+        copy_in(ahead, min(ahead * WALK, last_step), held);
+    }
+    if (UNION) look_up(min((STAGES - 1) * WALK, last_step), held);
 
     // Query rows: row = span_row * group + head_in_group; a lane holds row row0 + qt*16 + li as B operands.  A row past the
     // last real one holds zeros and is never stored.
@@ -166,8 +190,19 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
 
     for (int walk0 = 0, buffer = 0; walk0 < keys; walk0 += WALK, buffer = buffer + 1 == STAGES ? 0 : buffer + 1) {
         // this wave's pieces of the step have landed when only the later steps' are outstanding
-        if (most) wait_loads<MOST * (STAGES - 2)>(); else wait_loads<LEAST * (STAGES - 2)>();
+        // (union walk: between two steps' copies lie the look-ups of the step after them, as many loads again)
+        constexpr int BETWEEN = UNION ? 2 : 1;
+        if (most) wait_loads<BETWEEN * MOST * (STAGES - 2)>(); else wait_loads<BETWEEN * LEAST * (STAGES - 2)>();
         __syncthreads();                             // ... and everybody's; the stage of the step before is no longer being read
+        if (UNION) {
+            // the copies of the step three ahead use the places looked up a step ago; the next step's are looked up first, so
+            // that waiting for them later leaves these copies in flight
+            uint32_t next[MOST];
+            look_up(min(walk0 + STAGES * WALK, last_step), next);
+            copy_in(buffer == 0 ? STAGES - 1 : buffer - 1, 0, held);
+            #pragma unroll
+            for (int k = 0; k < MOST; ++k) held[k] = next[k];
+        } else
         copy_in(buffer == 0 ? STAGES - 1 : buffer - 1, min(walk0 + (STAGES - 1) * WALK, last_step));
         uint8_t* stage = stages + buffer * (2 * SLAB);
         if (!UNION && cached - walk0 < WALK) {

@@ -35,7 +35,7 @@ constexpr int SEGMENT = 4096, PER_THREAD = SEGMENT / 256;
 struct UnionSpace {
     uint32_t* marks;        // [tiles][context rounded up to segments]
     uint32_t* segment;      // [tiles][segments] marked positions of a segment
-    int32_t* pos;           // [tiles][cap]
+    int32_t* pos;           // [tiles][cap] where the entry's K row (K/V head 0) lies in the pool, in 16-byte units
     uint32_t* mask;         // [tiles][cap]
     uint32_t* count;        // [tiles]
     size_t tiles, segments, cap, bytes;
@@ -96,8 +96,9 @@ __global__ void __launch_bounds__(256) union_count_kernel(const uint32_t* __rest
 // The lists in position order: a workgroup per (tile, segment) knows how many marked positions lie before its segment, a thread
 // how many before its 16 positions.  A tile without any entry gets one that nobody selected (the walk needs a row to read).
 __global__ void __launch_bounds__(256) union_list_kernel(const uint32_t* __restrict__ marks, size_t stride, unsigned segments, const uint32_t* __restrict__ segment,
-                                                         size_t cap, size_t base, int32_t* __restrict__ pos, uint32_t* __restrict__ mask,
-                                                         uint32_t* __restrict__ count) {
+                                                         size_t cap, size_t base, const int32_t* __restrict__ page_table, unsigned page_tokens,
+                                                         unsigned page_last, size_t plane16, unsigned row16, unsigned kv_heads,
+                                                         int32_t* __restrict__ pos, uint32_t* __restrict__ mask, uint32_t* __restrict__ count) {
     __shared__ uint32_t sums[4], before_segment, total;
     const unsigned tile = blockIdx.y, seg = blockIdx.x, t = threadIdx.x, lane = t % 64, wave = t / 64;
     {
@@ -114,9 +115,14 @@ __global__ void __launch_bounds__(256) union_list_kernel(const uint32_t* __restr
         if (t == 0) total = sums[0] + sums[1] + sums[2] + sums[3];
         __syncthreads();
     }
+    // a position's place: its page's K plane of K/V head 0, its row in the page (16-byte units; a row is 17 or 32 of them)
+    const auto place = [&](size_t position) {
+        const size_t page = page_table ? size_t(min(unsigned(page_table[position / page_tokens]), page_last)) : 0, in_page = page_table ? position % page_tokens : position;
+        return int32_t(page * 2 * kv_heads * plane16 + in_page * row16);
+    };
     if (seg == 0 && t == 0) {
         count[tile] = max(total, 1u);
-        if (total == 0) { pos[size_t(tile) * cap] = int32_t(base); mask[size_t(tile) * cap] = 0u; }
+        if (total == 0) { pos[size_t(tile) * cap] = place(base); mask[size_t(tile) * cap] = 0u; }
     }
     const uint32_t* from = marks + size_t(tile) * stride + size_t(seg) * SEGMENT + t * PER_THREAD;
     uint32_t held[PER_THREAD], mine = 0;
@@ -141,7 +147,7 @@ __global__ void __launch_bounds__(256) union_list_kernel(const uint32_t* __restr
     #pragma unroll
     for (int i = 0; i < PER_THREAD; ++i)
         if (held[i] != 0 && at < cap) {
-            pos[size_t(tile) * cap + at] = int32_t(size_t(seg) * SEGMENT + t * PER_THREAD + i);
+            pos[size_t(tile) * cap + at] = place(size_t(seg) * SEGMENT + t * PER_THREAD + i);
             mask[size_t(tile) * cap + at] = held[i];
             ++at;
         }
@@ -191,8 +197,12 @@ int sdx_selected_attention_union(void* handle, const sdx_kv_pool* pool, const in
     union_clear_kernel<<<unsigned(std::min<size_t>(s.tiles * stride / 4 / 256 + 1, 4096)), 256, 0, value.stream>>>(reinterpret_cast<uint4*>(s.marks), s.tiles * stride / 4);
     union_mark_kernel<<<unsigned(rows), 256, 0, value.stream>>>(indices, selected, counts, base, context, unsigned(group), union_tile_rows(), stride, s.marks);
     union_count_kernel<<<dim3(unsigned(s.segments), unsigned(s.tiles)), 256, 0, value.stream>>>(s.marks, stride, unsigned(s.segments), s.segment);
-    union_list_kernel<<<dim3(unsigned(s.segments), unsigned(s.tiles)), 256, 0, value.stream>>>(s.marks, stride, unsigned(s.segments), s.segment, s.cap, base,
-                                                                                                 s.pos, s.mask, s.count);
+    const size_t row_bytes = pool->row_bytes, plane_bytes = size_t(pool->page_tokens) * row_bytes;
+    if (checked_product({pool->page_count, 2, pool->kv_heads, uint64_t(plane_bytes)}) / 16 > 0x7fffffffu)
+        throw std::runtime_error("sdx_selected_attention_union: a pool of more than 32 GiB");
+    union_list_kernel<<<dim3(unsigned(s.segments), unsigned(s.tiles)), 256, 0, value.stream>>>(
+        s.marks, stride, unsigned(s.segments), s.segment, s.cap, base, page_table, pool->page_tokens,
+        unsigned(std::min<uint64_t>(pool->page_count - 1, 0x7fffffffu)), plane_bytes / 16, unsigned(row_bytes / 16), pool->kv_heads, s.pos, s.mask, s.count);
     SD_CHECK(hipGetLastError());
     prefill_union(value, pool, page_table, base, q, q_f16, rows, heads, scale, gate, gate_stride, gate_row_stride, out, out_f16, s.pos, s.mask, s.count,
                   unsigned(s.cap));
