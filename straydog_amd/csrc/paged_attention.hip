@@ -249,17 +249,20 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
                     for (int r = 0; r < 4; ++r)
                         if (token0 + 16 * t + 4 * g + r > limit[qt]) s[qt][t][r] = -INFINITY;
         }
+        // (whether a row has outgrown its reference is seen by the lane that holds its largest score: the row's four lanes
+        // compare their own eight scores, and only a step that moves a reference reduces the maxima across them)
         float top[QT];
         bool grown = false;
         #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
-            top[qt] = row_max(fmaxf(fmaxf(fmaxf(s[qt][0][0], s[qt][0][1]), fmaxf(s[qt][0][2], s[qt][0][3])),
-                                    fmaxf(fmaxf(s[qt][1][0], s[qt][1][1]), fmaxf(s[qt][1][2], s[qt][1][3]))));
+            top[qt] = fmaxf(fmaxf(fmaxf(s[qt][0][0], s[qt][0][1]), fmaxf(s[qt][0][2], s[qt][0][3])),
+                            fmaxf(fmaxf(s[qt][1][0], s[qt][1][1]), fmaxf(s[qt][1][2], s[qt][1][3])));
             grown |= (top[qt] - m[qt]) * args.scale_log2 > SLACK;
         }
         if (__any(grown)) {
             #pragma unroll
             for (int qt = 0; qt < QT; ++qt) {
+                top[qt] = row_max(top[qt]);
                 const float m_new = fmaxf(m[qt], top[qt]);
                 const float alpha = __builtin_amdgcn_exp2f((m[qt] - m_new) * args.scale_log2);
                 m[qt] = m_new;
