@@ -248,16 +248,17 @@ __global__ void __launch_bounds__(64 * SCAN_WAVES) interval_scan_kernel(const ui
     float4* row_info = reinterpret_cast<float4*>(staged + ROWS_OPS);
     const unsigned t = threadIdx.x, lane = t % 64, wave = t / 64, first_row = blockIdx.y * ROWS;
     const unsigned tiles = (min(steps - first_row, unsigned(ROWS)) + 15) / 16;
+    // the wave's keys are asked for first: their trip overlaps the staging of the queries
+    const unsigned group = blockIdx.x * SCAN_WAVES + wave;
+    ScanTask task;
+    load_task(task, key_ops, key_stats, min(group, tasks - 1), lane);
     {
         const uint4* source = query_ops + size_t(blockIdx.y) * ROWS_OPS;
         for (unsigned i = t; i < tiles * 16 * 64; i += 64 * SCAN_WAVES) staged[i] = source[i];
         if (t < ROWS) row_info[t] = info[first_row + t];
     }
     __syncthreads();
-    const unsigned group = blockIdx.x * SCAN_WAVES + wave;
     if (group >= tasks) return;
-    ScanTask task;
-    load_task(task, key_ops, key_stats, group, lane);
     #pragma unroll 1
     for (unsigned j = 0; j < tiles; ++j) {
         floatx4 acc[4][HEADS];
@@ -303,9 +304,9 @@ __global__ void __launch_bounds__(64 * SCAN_WAVES) interval_scan_kernel(const ui
     }
 }
 
-// ---- pieces of the per-row kernels: 256 threads --------------------------------------------------------------------------------
+// ---- pieces of the per-row kernels (256 or 512 threads) --------------------------------------------------------------------------------
 // The sum of `value` over the threads before this one; the workgroup's total in `total`.  `sums` is 8 words, free to rewrite
-// after the next barrier of the caller.
+// after the next barrier of the caller (up to 16 waves).
 __device__ __forceinline__ uint32_t before_me(uint32_t value, uint32_t* sums, uint32_t& total) {
     const unsigned lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     uint32_t running = value;
@@ -319,8 +320,7 @@ __device__ __forceinline__ uint32_t before_me(uint32_t value, uint32_t* sums, ui
     __syncthreads();
     uint32_t before = 0;
     total = 0;
-    #pragma unroll
-    for (unsigned w = 0; w < 4; ++w) { before += w < wave ? sums[w] : 0u; total += sums[w]; }
+    for (unsigned w = 0; w < blockDim.x / 64; ++w) { before += w < wave ? sums[w] : 0u; total += sums[w]; }
     return before + running - value;
 }
 
@@ -353,33 +353,35 @@ __device__ uint32_t kth_highest(const uint32_t* keys, unsigned n, unsigned k, ui
 
 // The first 22 bits (the rest zero) of the k-th highest of a[] and of b[] (n keys each, in LDS), found in step: two passes of
 // eleven bits over two histograms of 2048 counts; a thread owns eight neighbouring counts of each, from the highest down.
+template<int THREADS>
 __device__ void kth_pair(const uint32_t* a, const uint32_t* b, unsigned n, unsigned k, uint32_t (*bins)[2048], uint32_t* state, uint32_t* sums,
                          uint32_t& found_a, uint32_t& found_b) {
     const unsigned t = threadIdx.x;
     uint32_t prefix_a = 0, prefix_b = 0, mask = 0, want_a = k, want_b = k;
     for (unsigned pass = 0; pass < 2; ++pass) {
         const unsigned shift = pass ? 10 : 21;
+        constexpr unsigned MINE = 2048 / THREADS;      // neighbouring counts a thread owns
         #pragma unroll
-        for (unsigned i = 0; i < 8; ++i) { bins[0][t * 8 + i] = 0; bins[1][t * 8 + i] = 0; }
+        for (unsigned i = 0; i < MINE; ++i) { bins[0][t * MINE + i] = 0; bins[1][t * MINE + i] = 0; }
         __syncthreads();
-        for (unsigned i = t; i < n; i += 256) {
+        for (unsigned i = t; i < n; i += THREADS) {
             const uint32_t x = a[i], y = b[i];
             if ((x & mask) == prefix_a) atomicAdd(&bins[0][(x >> shift) & 2047], 1u);
             if ((y & mask) == prefix_b) atomicAdd(&bins[1][(y >> shift) & 2047], 1u);
         }
         __syncthreads();
-        uint32_t mine_a[8], mine_b[8], sum = 0;
+        uint32_t mine_a[MINE], mine_b[MINE], sum = 0;
         #pragma unroll
-        for (unsigned i = 0; i < 8; ++i) {
-            mine_a[i] = bins[0][2047 - (t * 8 + i)]; mine_b[i] = bins[1][2047 - (t * 8 + i)];
+        for (unsigned i = 0; i < MINE; ++i) {
+            mine_a[i] = bins[0][2047 - (t * MINE + i)]; mine_b[i] = bins[1][2047 - (t * MINE + i)];
             sum += mine_a[i] | mine_b[i] << 16;         // (two counts of at most CAP each, scanned in one)
         }
         uint32_t total;
         const uint32_t above = before_me(sum, sums, total);
         uint32_t above_a = above & 0xffffu, above_b = above >> 16;
         #pragma unroll
-        for (unsigned i = 0; i < 8; ++i) {
-            const uint32_t bin = 2047 - (t * 8 + i);
+        for (unsigned i = 0; i < MINE; ++i) {
+            const uint32_t bin = 2047 - (t * MINE + i);
             if (above_a < want_a && above_a + mine_a[i] >= want_a) { state[0] = prefix_a | bin << shift; state[1] = want_a - above_a; }
             if (above_b < want_b && above_b + mine_b[i] >= want_b) { state[2] = prefix_b | bin << shift; state[3] = want_b - above_b; }
             above_a += mine_a[i]; above_b += mine_b[i];
@@ -404,7 +406,8 @@ __global__ void __launch_bounds__(256) interval_threshold_kernel(const float* __
 }
 
 // ---- the selection of a row ----------------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(256) interval_select_kernel(const float* __restrict__ queries, size_t stride, const float* __restrict__ blocks, size_t pool,
+constexpr int SELECT = 512;         // threads of a row's selection
+__global__ void __launch_bounds__(SELECT) interval_select_kernel(const float* __restrict__ queries, size_t stride, const float* __restrict__ blocks, size_t pool,
                                                               size_t base, size_t selected, const float* __restrict__ scores, const float* __restrict__ copy,
                                                               const float2* __restrict__ key_stats, const float4* __restrict__ info,
                                                               const uint64_t* __restrict__ kept, const uint64_t* __restrict__ sure, unsigned words,
@@ -414,7 +417,7 @@ __global__ void __launch_bounds__(256) interval_select_kernel(const float* __res
     __shared__ uint32_t exact[BAND];
     __shared__ uint16_t band_of[BAND];
     __shared__ float query[HEADS * COLUMNS];
-    __shared__ uint32_t bins[2][2048], state[4], sums[8];
+    __shared__ uint32_t bins[2][2048], state[4], sums[16];
     const unsigned t = threadIdx.x, row = blockIdx.x;
     if (flags[row]) {           // (a query element beyond FP16 or not a number)
         if (t == 0) atomicAdd(&flags[gate], 1u);
@@ -423,9 +426,9 @@ __global__ void __launch_bounds__(256) interval_select_kernel(const float* __res
     const float4 mine = info[row];
     const unsigned complete = __float_as_uint(mine.w);
     const size_t position = base + row;
-    for (unsigned i = t; i < HEADS * COLUMNS; i += 256) query[i] = queries[size_t(row) * stride + i];
+    for (unsigned i = t; i < HEADS * COLUMNS; i += SELECT) query[i] = queries[size_t(row) * stride + i];
     // the kept blocks in block order: a run of words per thread
-    const unsigned used = (complete + GROUP - 1) / GROUP, per = (used + 255) / 256;
+    const unsigned used = (complete + GROUP - 1) / GROUP, per = (used + SELECT - 1) / SELECT;
     const unsigned first_word = min(t * per, used), last_word = min(first_word + per, used);
     uint32_t mine_kept = 0, mine_sure = 0;
     for (unsigned w = first_word; w < last_word; ++w) {
@@ -449,7 +452,7 @@ __global__ void __launch_bounds__(256) interval_select_kernel(const float* __res
     __syncthreads();
     bool odd = false;
     #pragma unroll 6
-    for (unsigned i = t; i < n; i += 256) {
+    for (unsigned i = t; i < n; i += SELECT) {
         const unsigned block = block_of[i];
         const float score = scores[size_t(row) * pool + block];
         const float2 norms = key_stats[block];
@@ -463,10 +466,10 @@ __global__ void __launch_bounds__(256) interval_select_kernel(const float* __res
     }
     // to 22 bits: the 512th highest lower bound rounded down, the 512th highest upper bound rounded up (either way the safe side)
     uint32_t low_kth, high_kth;
-    kth_pair(low, high, n, KEEP, bins, state, sums, low_kth, high_kth);
+    kth_pair<SELECT>(low, high, n, KEEP, bins, state, sums, low_kth, high_kth);
     high_kth |= 0x3ffu;
     // a run of kept blocks per thread: certain ones counted, the band listed in block order
-    const unsigned run = (n + 255) / 256, c0 = min(t * run, n), c1 = min(c0 + run, n);
+    const unsigned run = (n + SELECT - 1) / SELECT, c0 = min(t * run, n), c1 = min(c0 + run, n);
     uint32_t my_certain = 0, my_band = 0;
     for (unsigned c = c0; c < c1; ++c) {
         if (low[c] > high_kth) ++my_certain;
@@ -484,7 +487,7 @@ __global__ void __launch_bounds__(256) interval_select_kernel(const float* __res
     __syncthreads();
     // the band's exact scores: four neighbouring lanes take a block's four heads, each its chain of 128 fused multiply-adds in
     // column order; the first of them adds the positive parts in head order
-    for (unsigned i = t / 4; i < ((band + 63) & ~63u); i += 64) {
+    for (unsigned i = t / 4; i < ((band + SELECT / 4 - 1) / (SELECT / 4)) * (SELECT / 4); i += SELECT / 4) {
         const unsigned head = t % 4;
         float dot = 0.0f;
         if (i < band) {
@@ -507,7 +510,7 @@ __global__ void __launch_bounds__(256) interval_select_kernel(const float* __res
     __syncthreads();
     // the (512 - certain)th highest of the band's exact scores, by counting: the band is short
     const uint32_t need = unsigned(KEEP) - certain;
-    for (unsigned i = t; i < band; i += 256) {
+    for (unsigned i = t; i < band; i += SELECT) {
         const uint32_t x = exact[i];
         uint32_t higher = 0, same = 0;
         for (unsigned j = 0; j < band; ++j) { const uint32_t y = exact[j]; higher += y > x; same += y == x; }
@@ -516,7 +519,7 @@ __global__ void __launch_bounds__(256) interval_select_kernel(const float* __res
     __syncthreads();
     const uint32_t limit = state[0];
     uint32_t my_above = 0;
-    for (unsigned i = t; i < band; i += 256) my_above += exact[i] > limit;
+    for (unsigned i = t; i < band; i += SELECT) my_above += exact[i] > limit;
     uint32_t above;
     (void)before_me(my_above, sums, above);
     const uint32_t ties = need - above;         // blocks at the limit that are taken: the earliest
@@ -558,7 +561,7 @@ __global__ void __launch_bounds__(256) interval_select_kernel(const float* __res
         }
     }
     const size_t head = size_t(KEEP) * 4;
-    for (size_t i = t; size_t(complete) * 4 + i <= position; i += 256) out[head + i] = float(size_t(complete) * 4 + i);
+    for (size_t i = t; size_t(complete) * 4 + i <= position; i += SELECT) out[head + i] = float(size_t(complete) * 4 + i);
     if (t == 0) counts_out[row] = float(head + position + 1 - size_t(complete) * 4);
 }
 
@@ -619,7 +622,7 @@ const uint32_t* interval_select(Device& d, const float* queries, size_t stride, 
     interval_threshold_kernel<<<unsigned(steps), 256, 0, d.stream>>>(s.sample, sampled, s.info);
     timed_launch(d, &interval_scan_kernel, dim3((tasks + SCAN_WAVES - 1) / SCAN_WAVES, row_groups), dim3(64 * SCAN_WAVES), shared,
                  s.key_ops, s.key_stats, s.query_ops, s.info, tasks, unsigned(steps), pool, scores, s.kept, s.sure, words);
-    interval_select_kernel<<<unsigned(steps), 256, 0, d.stream>>>(queries, stride, blocks, pool, base, selected, scores, s.copy, s.key_stats, s.info, s.kept,
+    interval_select_kernel<<<unsigned(steps), SELECT, 0, d.stream>>>(queries, stride, blocks, pool, base, selected, scores, s.copy, s.key_stats, s.info, s.kept,
                                                                   s.sure, words, s.flags, rows, indices, counts);
     SD_CHECK(hipGetLastError());
     *gate = rows;
