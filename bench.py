@@ -162,9 +162,9 @@ def main():
     lengths = workloads.config1_lengths()
     builders = {
         "config1": lambda: workloads.PagedWorkload(gpu, lengths, seed=1),
-        "config1_32k": lambda: workloads.PagedWorkload(gpu, [32768] * 32, seed=2),
-        "config0": lambda: workloads.PagedWorkload(gpu, [4096], heads=16, kv_heads=2, seed=3, q_f16=False, out_f16=False),
-        "config3": lambda: workloads.PagedWorkload(gpu, [65536 + 5] * 16, span=5, seed=5),
+        "config1_32k": lambda: workloads.PagedWorkload(gpu, [32768] * 32, seed=0x101),
+        "config0": lambda: workloads.PagedWorkload(gpu, [4096], heads=16, kv_heads=2, seed=0, q_f16=False, out_f16=False),
+        "config3": lambda: workloads.PagedWorkload(gpu, [65536 + 5] * 16, span=5, seed=3),
     }
     names = {
         "config1": "configs[1]: 32 seqs, len~U[1024,32768], 32q/4kv heads, d128, Q8_0 pages of 256, fp16 q/out",

@@ -245,6 +245,9 @@ int sdx_device_compute_units(void* handle);
  * (sd_graph_begin .. sd_graph_end) are not timed. */
 int sdx_profile(void* handle, int enable);
 int sdx_profile_read(void* handle, double* milliseconds, uint64_t* launches);
+/* Seeded N(0,1) values as the reference's tests draw them: one xorshift64 stream from `seed` (0: 0x9e3779b97f4a7c15), two draws a
+ * Box-Muller pair in double precision, value i of the stream at out[i] (crates/straydog-engine/tests/fused_gpu.rs:39-53,
+ * gpu/tests/qsa_interval_test.cpp:12-18).  The threads reach their stretches of the stream by jumping (the generator is linear). */
 int sdx_fill_normal(void* handle, void* out, uint64_t count, uint64_t seed, int out_kind /* 0 f32, 1 f16, 2 bf16 */);
 int sdx_fill_uniform(void* handle, float* out, uint64_t count, uint64_t seed, float lo, float hi);
 int sdx_copy(void* handle, void* target, const void* source, uint64_t bytes);

@@ -46,32 +46,79 @@ __global__ void __launch_bounds__(256) kv_write_kernel(uint8_t* pages, size_t pa
     kv_store_quad(out, unsigned(quad), dim, row_bytes != 2 * dim, x, stored);
 }
 
-__device__ __forceinline__ uint64_t mix64(uint64_t z) {   // splitmix64 finaliser
-    z += 0x9e3779b97f4a7c15ull;
-    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
-    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
-    return z ^ (z >> 31);
+// Seeded normal values as the reference's tests draw them: one xorshift64 stream (x ^= x << 13; x ^= x >> 7; x ^= x << 17, e.g.
+// crates/straydog-engine/tests/fused_gpu.rs:39-53), two draws a Box-Muller pair (gpu/tests/qsa_interval_test.cpp:12-18), in double
+// precision, value i of the stream at out[i].  The stream is sequential; the generator is linear over GF(2), so a thread reaches
+// its own stretch of RUN pairs by jumping: jump[b] holds the matrix of 2 * RUN * 2^b steps as 64 columns, and the bits of the
+// thread's number say which to apply.
+constexpr int RUN = 64;                       // pairs a thread draws
+__constant__ uint64_t jump[32][64];
+
+__host__ __device__ inline uint64_t xorshift64(uint64_t x) { x ^= x << 13; x ^= x >> 7; x ^= x << 17; return x; }
+
+// The state of the stream 2 * RUN * stretch steps after `seed`.
+__device__ __forceinline__ uint64_t jumped(uint64_t seed, size_t stretch) {
+    uint64_t state = seed;
+    for (int b = 0; b < 32 && stretch >> b; ++b) {
+        if (!((stretch >> b) & 1)) continue;
+        uint64_t moved = 0;
+        #pragma unroll 8
+        for (int j = 0; j < 64; ++j) moved ^= (0 - ((state >> j) & 1)) & jump[b][j];
+        state = moved;
+    }
+    return state;
 }
 
-__global__ void fill_normal_kernel(void* out, size_t count, uint64_t seed, int kind) {
-    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) {
-        const uint64_t bits = mix64(seed ^ (i * 0xd1342543de82ef95ull));
-        const float u = (float(uint32_t(bits >> 40)) + 0.5f) * (1.0f / 16777216.0f);
-        const float v = (float(uint32_t(bits) >> 8) + 0.5f) * (1.0f / 16777216.0f);
-        const float value = sqrtf(-2.0f * logf(u)) * cosf(6.2831853f * v);
+__global__ void __launch_bounds__(256) fill_normal_kernel(void* out, size_t count, uint64_t seed, int kind) {
+    const size_t thread = size_t(blockIdx.x) * blockDim.x + threadIdx.x, first = thread * (2 * RUN);
+    if (first >= count) return;
+    uint64_t state = jumped(seed, thread);
+    const auto store = [&](size_t i, double x) {
+        const float value = float(x);
         if (kind == 0) static_cast<float*>(out)[i] = value;
         else if (kind == 1) static_cast<__half*>(out)[i] = __float2half_rn(value);
         else {
-            const uint32_t b = __float_as_uint(value);
-            static_cast<uint16_t*>(out)[i] = uint16_t((b + 0x7fffu + ((b >> 16) & 1u)) >> 16);
+            const uint32_t bits = __float_as_uint(value);
+            static_cast<uint16_t*>(out)[i] = uint16_t((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
         }
+    };
+    for (size_t i = first; i < min(count, first + 2 * RUN); i += 2) {
+        state = xorshift64(state);
+        const double u = (double(state >> 11) + 0.5) / 9007199254740992.0;
+        state = xorshift64(state);
+        const double v = (double(state >> 11) + 0.5) / 9007199254740992.0;
+        const double r = sqrt(-2.0 * log(u));
+        store(i, r * cos(6.283185307179586 * v));
+        if (i + 1 < count) store(i + 1, r * sin(6.283185307179586 * v));
     }
 }
 
-__global__ void fill_uniform_kernel(float* out, size_t count, uint64_t seed, float lo, float hi) {
-    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += size_t(gridDim.x) * blockDim.x) {
-        const uint64_t bits = mix64(seed ^ (i * 0xd1342543de82ef95ull));
-        out[i] = lo + (hi - lo) * (float(uint32_t(bits >> 40)) * (1.0f / 16777216.0f));
+// The jump matrices, worked out once a device: a matrix is its 64 columns (the images of the unit vectors).
+void fill_normal_setup(Device& d) {
+    static std::mutex mutex;
+    static std::map<int, bool> ready;
+    std::lock_guard<std::mutex> lock(mutex);
+    if (ready[d.ordinal]) return;
+    typedef std::vector<uint64_t> Matrix;
+    const auto apply = [](const Matrix& m, uint64_t x) { uint64_t y = 0; for (int j = 0; j < 64; ++j) if ((x >> j) & 1) y ^= m[j]; return y; };
+    const auto squared = [&](const Matrix& m) { Matrix r(64); for (int j = 0; j < 64; ++j) r[j] = apply(m, m[j]); return r; };
+    Matrix m(64);
+    for (int j = 0; j < 64; ++j) m[j] = xorshift64(uint64_t(1) << j);
+    for (int steps = 1; steps < 2 * RUN; steps *= 2) m = squared(m);        // 2 * RUN steps: one thread's stretch
+    std::vector<uint64_t> all;
+    for (int b = 0; b < 32; ++b) { all.insert(all.end(), m.begin(), m.end()); m = squared(m); }
+    SD_CHECK(hipMemcpyToSymbol(HIP_SYMBOL(jump), all.data(), all.size() * sizeof(uint64_t)));
+    ready[d.ordinal] = true;
+}
+
+// Uniform values of the same stream, one draw each: lo + (hi - lo) * (x >> 40) / 2^24.
+__global__ void __launch_bounds__(256) fill_uniform_kernel(float* out, size_t count, uint64_t seed, float lo, float hi) {
+    const size_t thread = size_t(blockIdx.x) * blockDim.x + threadIdx.x, first = thread * (2 * RUN);
+    if (first >= count) return;
+    uint64_t state = jumped(seed, thread);
+    for (size_t i = first; i < min(count, first + 2 * RUN); ++i) {
+        state = xorshift64(state);
+        out[i] = __fadd_rn(lo, __fmul_rn(hi - lo, float(double(state >> 40) / 16777216.0)));    // (two roundings, as the host's)
     }
 }
 
@@ -171,7 +218,10 @@ int sdx_fill_normal(void* handle, void* out, uint64_t count, uint64_t seed, int 
     SD_OP_BEGIN
     if (!count || out_kind < 0 || out_kind > 2) throw std::runtime_error("invalid Straydog fill");
     op_span(value, out, checked_product({count, out_kind == 0 ? 4u : 2u}), "a filled buffer");
-    fill_normal_kernel<<<unsigned(std::min<size_t>(checked_blocks(size_t(count)), 65536)), 256, 0, value.stream>>>(out, size_t(count), seed, out_kind);
+    if (count > (uint64_t(1) << 38)) throw std::runtime_error("invalid Straydog fill");
+    fill_normal_setup(value);
+    fill_normal_kernel<<<checked_blocks((size_t(count) + 2 * RUN - 1) / (2 * RUN)), 256, 0, value.stream>>>(out, size_t(count),
+                                                                                                      seed ? seed : 0x9e3779b97f4a7c15ull, out_kind);
     SD_OP_END
 }
 
@@ -179,7 +229,10 @@ int sdx_fill_uniform(void* handle, float* out, uint64_t count, uint64_t seed, fl
     SD_OP_BEGIN
     if (!count) throw std::runtime_error("invalid Straydog fill");
     op_span(value, out, checked_floats({count}), "a filled buffer");
-    fill_uniform_kernel<<<unsigned(std::min<size_t>(checked_blocks(size_t(count)), 65536)), 256, 0, value.stream>>>(out, size_t(count), seed, lo, hi);
+    if (count > (uint64_t(1) << 38)) throw std::runtime_error("invalid Straydog fill");
+    fill_normal_setup(value);
+    fill_uniform_kernel<<<checked_blocks((size_t(count) + 2 * RUN - 1) / (2 * RUN)), 256, 0, value.stream>>>(out, size_t(count),
+                                                                                                       seed ? seed : 0x9e3779b97f4a7c15ull, lo, hi);
     SD_OP_END
 }
 

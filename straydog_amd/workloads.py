@@ -6,6 +6,12 @@ import numpy as np
 ROW_Q8 = {128: 136, 256: 272}
 
 
+def stream(seed, index):
+    """The seed of tensor `index` of a workload: every tensor is its own xorshift64 stream, (0x9e3779b97f4a7c15 ^ seed) + index,
+    `seed` being the BASELINE config's number (the reference's habit, crates/straydog-engine/tests/attention_gpu.rs:91)."""
+    return ((0x9e3779b97f4a7c15 ^ seed) + index) & 0xffffffffffffffff
+
+
 class PagedWorkload:
     """A batch of sequences in a shuffled paged Q8_0 cache, with `span` query rows each."""
 
@@ -39,8 +45,8 @@ class PagedWorkload:
         zero = gpu.upload(np.zeros(1, dtype=np.int32))
         for s in range(self.seqs):
             n = int(self.lengths[s])
-            gpu.fill_normal(stage_k.base(), n * kv_heads * dim, seed * 1000003 + 2 * s, 0)
-            gpu.fill_normal(stage_v.base(), n * kv_heads * dim, seed * 1000003 + 2 * s + 1, 0)
+            gpu.fill_normal(stage_k.base(), n * kv_heads * dim, stream(seed, 2 * s + 1), 0)
+            gpu.fill_normal(stage_v.base(), n * kv_heads * dim, stream(seed, 2 * s + 2), 0)
             gpu.kv_write(self.pool, self.table_buffer.at(s * self.table_stride * 4), self.table_stride, zero.base(), stage_k.base(),
                          stage_v.base(), False, 1, n)
         gpu.synchronize()
@@ -48,7 +54,7 @@ class PagedWorkload:
             gpu.release(b)
         count = self.seqs * span * heads * dim
         self.q_buffer = gpu.buffer(count * (2 if q_f16 else 4))
-        gpu.fill_normal(self.q_buffer.base(), count, seed * 7919 + 5, 1 if q_f16 else 0)
+        gpu.fill_normal(self.q_buffer.base(), count, stream(seed, 0), 1 if q_f16 else 0)
         self.out_buffer = gpu.buffer(count * (2 if out_f16 else 4))
         self.scratch = gpu.buffer(max(gpu.paged_attention_scratch(self.seqs, span, heads, dim, self.max_context), 4))
         gpu.synchronize()
@@ -108,9 +114,9 @@ class PrefillWorkload:
         self.v = gpu.buffer(tokens * kv_heads * dim * 2)
         self.q = gpu.buffer(tokens * heads * dim * 2)
         self.out = gpu.buffer(tokens * heads * dim * 2)
-        gpu.fill_normal(self.k.base(), tokens * kv_heads * dim, seed * 13 + 1, 1)
-        gpu.fill_normal(self.v.base(), tokens * kv_heads * dim, seed * 13 + 2, 1)
-        gpu.fill_normal(self.q.base(), tokens * heads * dim, seed * 13 + 3, 1)
+        gpu.fill_normal(self.k.base(), tokens * kv_heads * dim, stream(seed, 1), 1)
+        gpu.fill_normal(self.v.base(), tokens * kv_heads * dim, stream(seed, 2), 1)
+        gpu.fill_normal(self.q.base(), tokens * heads * dim, stream(seed, 3), 1)
         self.scratch = gpu.buffer(max(gpu.paged_attention_scratch(1, chunk, heads, dim, tokens), 4))
         gpu.synchronize()
 
@@ -158,11 +164,11 @@ class SparseWorkload:
         self.q = gpu.buffer(batch * heads * kdim * 2)
         self.latents = gpu.buffer(batch * context * kdim * 2)
         self.out = gpu.buffer(batch * heads * vdim * 4)
-        gpu.fill_normal(self.q_index.base(), batch * index_heads * index_dim, seed * 11 + 1, 2)
-        gpu.fill_normal(self.keys.base(), batch * context * index_dim, seed * 11 + 2, 2)
-        gpu.fill_uniform(self.weights.base(), batch * index_heads, seed * 11 + 3, 0.0, 1.0)
-        gpu.fill_normal(self.q.base(), batch * heads * kdim, seed * 11 + 4, 2)
-        gpu.fill_normal(self.latents.base(), batch * context * kdim, seed * 11 + 5, 2)
+        gpu.fill_normal(self.q_index.base(), batch * index_heads * index_dim, stream(seed, 1), 2)
+        gpu.fill_normal(self.keys.base(), batch * context * index_dim, stream(seed, 2), 2)
+        gpu.fill_uniform(self.weights.base(), batch * index_heads, stream(seed, 3), 0.0, 1.0)
+        gpu.fill_normal(self.q.base(), batch * heads * kdim, stream(seed, 4), 2)
+        gpu.fill_normal(self.latents.base(), batch * context * kdim, stream(seed, 5), 2)
         gpu.synchronize()
 
     def step_index(self, keep_scores=False):
@@ -202,8 +208,8 @@ class BlockIndexWorkload:
         self.scores = gpu.buffer(steps * self.pool * 4)
         self.indices = gpu.buffer(steps * 2052 * 4)
         self.counts = gpu.buffer(steps * 4)
-        gpu.fill_normal(self.queries.base(), steps * 512, seed * 11 + 1, 0)
-        gpu.fill_normal(self.blocks.base(), 128 * self.pool, seed * 11 + 2, 0)
+        gpu.fill_normal(self.queries.base(), steps * 512, stream(seed, 1), 0)
+        gpu.fill_normal(self.blocks.base(), 128 * self.pool, stream(seed, 2), 0)
         gpu.synchronize()
 
     def step(self):
@@ -231,13 +237,13 @@ class BlockIndexWorkload:
         self.heads, self.kv_heads, self.row_bytes = heads, kv_heads, row_bytes
         self.kv, self.kv_buffer = gpu.kv_pool(1, context, kv_heads, 256, row_bytes)
         k, table = gpu.buffer(8192 * kv_heads * 256 * 2), gpu.upload(np.zeros(1, dtype=np.int32))
-        gpu.fill_normal(k.base(), 8192 * kv_heads * 256, seed * 11 + 3, 1)
+        gpu.fill_normal(k.base(), 8192 * kv_heads * 256, stream(seed, 3), 1)
         for first in range(0, context, 8192):                # the cache is filled through the library's own writer
             start = gpu.upload(np.array([first], dtype=np.int32))
             gpu.kv_write(self.kv, table.base(), 1, start.base(), k.base(), k.base(), True, 1, 8192)
             gpu.release(start)
         self.q = gpu.buffer(self.steps * heads * 256 * 2)
-        gpu.fill_normal(self.q.base(), self.steps * heads * 256, seed * 11 + 4, 1)
+        gpu.fill_normal(self.q.base(), self.steps * heads * 256, stream(seed, 4), 1)
         self.out = gpu.buffer(self.steps * heads * 256 * 2)
         self.scratch = gpu.buffer(gpu.selected_attention_scratch(self.steps, kv_heads, 2052))
         gpu.synchronize()
@@ -302,7 +308,7 @@ class QwenStageWorkload:
         self.stride = heads * 512 + kv_heads * 512 + 640
         self.kv, self.kv_buffer = gpu.kv_pool(1, context, kv_heads, 256, row_bytes)
         k, table = gpu.buffer(8192 * kv_heads * 256 * 2), gpu.upload(np.zeros(1, dtype=np.int32))
-        gpu.fill_normal(k.base(), 8192 * kv_heads * 256, seed * 11 + 3, 1)
+        gpu.fill_normal(k.base(), 8192 * kv_heads * 256, stream(seed, 3), 1)
         for first in range(0, context, 8192):
             start = gpu.upload(np.array([first], dtype=np.int32))
             gpu.kv_write(self.kv, table.base(), 1, start.base(), k.base(), k.base(), True, 1, 8192)
@@ -310,10 +316,10 @@ class QwenStageWorkload:
         self.projections = gpu.buffer(steps * self.stride * 4)
         self.blocks, self.history = gpu.buffer(128 * pool * 4), gpu.buffer(16 * 128 * 4)
         self.norms = [gpu.buffer(n * 4) for n in (256, 256, 128, 128)]
-        gpu.fill_normal(self.projections.base(), steps * self.stride, seed * 11 + 1, 0)
-        gpu.fill_normal(self.blocks.base(), 128 * pool, seed * 11 + 2, 0)
+        gpu.fill_normal(self.projections.base(), steps * self.stride, stream(seed, 1), 0)
+        gpu.fill_normal(self.blocks.base(), 128 * pool, stream(seed, 2), 0)
         for i, n in enumerate((256, 256, 128, 128)):
-            gpu.fill_uniform(self.norms[i].base(), n, seed * 11 + 5 + i, 0.5, 1.5)
+            gpu.fill_uniform(self.norms[i].base(), n, stream(seed, 5 + i), 0.5, 1.5)
         self.positions = gpu.upload(np.arange(base, base + steps, dtype=np.uint32))
         self.state = gpu.qsa_state(self.kv, None, context, self.blocks.base(), self.history.base(), *[n.base() for n in self.norms], heads)
         self.scratch = gpu.buffer(gpu.qsa_decode_attend_scratch(steps, heads, kv_heads, context))

@@ -521,3 +521,23 @@ def test_dspark_block_attention(gpu, oracle):
         _dspark_check(f"sink={sink}", constant(), np.full(q.size, expected))
     for b in (qb, rb, bb, sb, out, anchor):
         gpu.release(b)
+
+
+def test_device_normal_values_are_the_xorshift_box_muller_stream(gpu, oracle):
+    # the harness fills its workloads on the device with the generator the reference's tests use (xorshift64, two draws a Box-Muller
+    # pair): the device reaches every stretch of the one stream by jumping, and the values are the host stream's (the double-precision
+    # logarithm and sine of the two libraries may differ in the last place, which a float rarely shows)
+    for seed, count in ((0x9e3779b97f4a7c15 ^ 1, 300001), (7, 129), (0, 2)):
+        out = gpu.buffer(count * 4)
+        gpu.fill_normal(out.base(), count, seed, 0)
+        got = _read(gpu, out, np.float32, count)
+        want = oracle.fill_normal(seed, count)
+        differ = np.flatnonzero(got != want)
+        assert len(differ) <= max(2, count // 100000), f"{len(differ)} of {count} values differ"
+        assert np.allclose(got, want, rtol=3e-7, atol=1e-9)
+        gpu.release(out)
+    out = gpu.buffer(5000 * 4)
+    gpu.fill_uniform(out.base(), 5000, 11, -0.5, 1.5)
+    assert np.array_equal(_read(gpu, out, np.float32, 5000), oracle.fill_uniform(11, 5000, -0.5, 1.5))
+    gpu.release(out)
+
