@@ -96,6 +96,9 @@ int sd_kv_stage(void* handle, void* pointer, uint64_t rows);
  * and write over the bus; owned like a device allocation (ops take pointers into it, sd_release frees it) but outside the VRAM
  * budget.  Null on failure. */
 void* sd_host_state(void* handle, uint64_t bytes);
+/* reference straydog_gpu.h:99 (gpu/kernels.cpp:3824-3847): page-locks and zeroes host states of these sizes on a thread of its
+ * own; sd_host_state then takes one of the right size (in any order) once the thread is done.  One prefetch at a time. */
+int sd_host_states_prefetch(void* handle, const uint64_t* sizes, uint64_t count);
 /* reference straydog_gpu.h:112 (gpu/kernels.cpp:4292-4300): 1, host-resident state is supported. */
 int sd_host_state_supported(void* handle);
 

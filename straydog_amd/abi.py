@@ -59,6 +59,7 @@ SIGNATURES = {
     "sd_kv_stage": (c_int, [c_void_p, c_void_p, c_u64]),
     "sd_host_state": (c_void_p, [c_void_p, c_u64]),
     "sd_host_state_supported": (c_int, [c_void_p]),
+    "sd_host_states_prefetch": (c_int, [c_void_p, _P(c_u64), c_u64]),
     "sd_attention_sequence": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_void_p, c_u64, c_void_p, c_u64]),
     "sd_op_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float,
                                 c_void_p, c_void_p, c_u64, c_void_p]),

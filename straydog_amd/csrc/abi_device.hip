@@ -210,6 +210,8 @@ void sd_destroy(void* handle) {
         if (entry.second.graph) (void)hipGraphDestroy(entry.second.graph);
     }
     if (d->kv_stream) (void)hipStreamSynchronize(d->kv_stream);
+    if (d->host_prefetch.joinable()) d->host_prefetch.join();
+    for (const auto& held : d->host_ready) (void)hipHostFree(held.second);
     for (const auto& entry : d->host_states) { d->allocations.erase(static_cast<const uint8_t*>(entry.first)); (void)hipHostFree(entry.second); }
     for (const auto& entry : d->allocations) (void)hipFree(const_cast<uint8_t*>(entry.first));
     if (d->kv_released) (void)hipEventDestroy(d->kv_released);
@@ -440,14 +442,48 @@ int sd_kv_format(void* handle, uint32_t row) {
 // sd_host_state, :4292-4300 sd_host_state_supported): owned like a device allocation -- ops take pointers into it, sd_release
 // frees it -- but outside the VRAM budget.  A K/V pool may live there whole; the paged cache's host tier (kv_cache.hip) is the
 // faster way to hold rows that are not being attended to.
+// Page-locks and zeroes host states of these sizes on a thread of their own (reference gpu/kernels.cpp:3824-3847): sd_host_state then
+// takes one of the right size, in any order, once the thread is done.
+int sd_host_states_prefetch(void* handle, const uint64_t* sizes, uint64_t count) {
+    try {
+        Device& d = device(handle);
+        if (!sizes || count > 4096 || d.host_prefetch.joinable() || !d.host_ready.empty()) throw std::runtime_error("invalid Straydog host state prefetch");
+        std::vector<size_t> wanted(sizes, sizes + count);
+        for (const size_t bytes : wanted) if (!bytes || bytes > (size_t(1) << 48)) throw std::runtime_error("invalid Straydog host state prefetch");
+        const int ordinal = d.ordinal;
+        d.host_prefetch_error.clear();
+        d.host_prefetch = std::thread([&d, wanted, ordinal]() {
+            try {
+                SD_CHECK(hipSetDevice(ordinal));
+                for (const size_t bytes : wanted) {
+                    void* host = nullptr;
+                    SD_CHECK(hipHostMalloc(&host, bytes + allocation_tail, hipHostMallocMapped));
+                    d.host_ready.emplace_back(bytes, host);
+                    std::memset(host, 0, bytes + allocation_tail);
+                }
+            } catch (const std::exception& e) { d.host_prefetch_error = e.what(); }
+        });
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
 void* sd_host_state(void* handle, uint64_t bytes) {
     try {
         Device& d = device(handle);
         if (!bytes || bytes > (uint64_t(1) << 48)) throw std::runtime_error("invalid Straydog host state");
+        if (d.host_prefetch.joinable()) d.host_prefetch.join();
+        if (!d.host_prefetch_error.empty()) {
+            const std::string error = d.host_prefetch_error;
+            d.host_prefetch_error.clear();
+            throw std::runtime_error(error);
+        }
         void* host = nullptr;
-        SD_CHECK(hipHostMalloc(&host, size_t(bytes) + allocation_tail, hipHostMallocMapped));
+        const auto ready = std::find_if(d.host_ready.begin(), d.host_ready.end(), [&](const auto& held) { return held.first == size_t(bytes); });
+        const bool zeroed = ready != d.host_ready.end();            // (the prefetch zeroed it)
+        if (zeroed) { host = ready->second; d.host_ready.erase(ready); }
+        else SD_CHECK(hipHostMalloc(&host, size_t(bytes) + allocation_tail, hipHostMallocMapped));
         try {
-            std::memset(host, 0, size_t(bytes) + allocation_tail);
+            if (!zeroed) std::memset(host, 0, size_t(bytes) + allocation_tail);
             void* pointer = nullptr;
             SD_CHECK(hipHostGetDevicePointer(&pointer, host, 0));
             std::lock_guard<std::mutex> lock(d.mutex);

@@ -14,6 +14,8 @@
 #include <mutex>
 #include <stdexcept>
 #include <string>
+#include <thread>
+#include <utility>
 #include <vector>
 
 namespace sd {
@@ -70,6 +72,10 @@ struct Device {
     // Sequence state in mapped, page-locked host memory (sd_host_state): device pointer -> host pointer.  They are listed in
     // `allocations` too, so ops take them, but not counted in the VRAM budget.
     std::map<const void*, void*> host_states;
+    // Host states page-locked and zeroed ahead of their use on a thread of their own (sd_host_states_prefetch): (bytes, host pointer).
+    std::thread host_prefetch;
+    std::vector<std::pair<size_t, void*>> host_ready;
+    std::string host_prefetch_error;
     // The VRAM stage the host registered (sd_kv_stage) and whose rows it holds: a K/V cache, one of its sequences, and how many
     // of that sequence's pages from the first on are in it.
     void* kv_stage = nullptr; size_t kv_stage_bytes = 0;

@@ -235,3 +235,12 @@ def test_a_pool_in_mapped_host_memory_attends_to_the_same_bits(gpu, oracle):
     for b in (tb, kb, vb, zero, qb, pb, buffer, state):
         gpu.release(b)
     assert gpu.memory()[0] == used
+    # states page-locked ahead of time on a thread are taken by size, zeroed; another size is allocated on the spot
+    import ctypes
+    sizes = (ctypes.c_uint64 * 2)(4096, 1 << 20)
+    assert gpu.lib.sd_host_states_prefetch(gpu.handle, sizes, 2) == 0
+    assert gpu.lib.sd_host_states_prefetch(gpu.handle, sizes, 2) == -1 and "prefetch" in gpu.error()
+    large, other, small = gpu.host_state(1 << 20), gpu.host_state(12345), gpu.host_state(4096)
+    assert not gpu.read_buffer(large, 0, np.uint8, 1 << 20).any() and not gpu.read_buffer(small, 0, np.uint8, 4096).any()
+    for b in (large, other, small):
+        gpu.release(b)
