@@ -339,16 +339,28 @@ def main():
                 also[name]["cpu_baseline"] = also_baseline
                 also[name]["workload"] = names[name]
                 also[name]["traffic"], also[name]["traffic_source"] = PROFILED_TRAFFIC[name]
+                kernel = also[name]["kernel_us"] or also[name]["us_per_step"]
+                also[name]["roofline"] = {"bound": "hbm", "achieved": also[name]["algorithmic_bytes"] / kernel / 1e3, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                          "frac": also[name]["algorithmic_bytes"] / kernel / 1e3 / HBM_PEAK_GBPS, "traffic": PROFILED_TRAFFIC[name][0],
+                                          "kernel": "paged_attention_kernel<128,3,Q8_0>" if name == "config3" else "paged_attention_kernel<128,1,Q8_0>",
+                                          "kernel_us": also[name]["kernel_us"]}
         if args.workload != "config2":
             also["config2"] = run_prefill()
             also["config2"]["workload"] = names["config2"]
             also["config2"]["traffic"], also["config2"]["traffic_source"] = PROFILED_TRAFFIC["config2"]
+            achieved = also["config2"]["kernel_tflops"] or also["config2"]["tflops"]
+            also["config2"]["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
+                                           "traffic": PROFILED_TRAFFIC["config2"][0], "kernel": "prefill_dense_kernel<128,2>", "kernel_us": also["config2"]["kernel_us"]}
             also["config2"]["measured_mfma_tflops"] = measured_mfma_ceiling(gpu, False)
             also["config2"]["measured_mfma_tflops_live_operands"] = measured_mfma_ceiling(gpu, True)
         if args.workload != "config4":
             also["config4"] = run_sparse()
             also["config4"]["workload"] = names["config4"]
             also["config4"]["traffic"], also["config4"]["traffic_source"] = PROFILED_TRAFFIC["config4"]
+            if also["config4"]["kernel_us"]:
+                achieved = also["config4"]["key_bytes"] / also["config4"]["kernel_us"] / 1e3
+                also["config4"]["roofline"] = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
+                                               "traffic": PROFILED_TRAFFIC["config4"][0], "kernel": "index_interval_kernel<64>", "kernel_us": also["config4"]["kernel_us"]}
         also["block_index_242k"] = run_block_index()
         also["block_index_242k"]["workload"] = "Qwen block indexer: 4x128 index heads, 60.5K complete blocks of a 262144-token context, top 512 blocks"
 
