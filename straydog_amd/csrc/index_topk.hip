@@ -344,7 +344,6 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int RADIX_BINS = 2048, RADIX_LEVELS = 2, INTERVAL_KEYS = 1024;   // digits of 11 and 11 bits (the cut is the k-th highest lower bound's leading 22 bits: the
                                                                            // last 10 would spare a candidate in a thousand and cost a pass over the bounds); groups per workgroup
-constexpr int SCORE_WAVES = 4, SCORE_BATCH = 8;                             // the rescoring kernel: waves per workgroup, groups a wave takes at a time
 constexpr int BRACKET_WAVES = 8, BRACKET_KEYS = 4096, BRACKET_RING = 4;     // the bracket kernel: waves, groups per workgroup, stages per wave
 __device__ __forceinline__ uint32_t radix_digit(uint32_t key, int level) { return level == 0 ? key >> 21 : level == 1 ? (key >> 10) & 2047u : key & 1023u; }
 
@@ -365,6 +364,31 @@ __device__ __forceinline__ void load_to_lds(const void* from, const void* to) {
     const uint32_t base = __builtin_amdgcn_readfirstlane(uint32_t(uintptr_t((lds_bytes)to)));
     uint32_t keep;      // M0 names the LDS address; it is put back for whatever else the compiler keeps there
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt\n\ts_mov_b32 m0, %0" : "=&s"(keep) : "v"(from), "s"(base) : "memory");
+}
+
+// The same from a base address that the whole wave shares (in scalar registers) and a lane's 32-bit offset from it: a loop that
+// walks through memory then moves the base with scalar arithmetic and spends no vector instruction on addresses.
+__device__ __forceinline__ void load_to_lds(const void* shared_base, uint32_t offset, const void* to) {
+    typedef __attribute__((address_space(3))) const uint8_t* lds_bytes;
+    const uint32_t base = __builtin_amdgcn_readfirstlane(uint32_t(uintptr_t((lds_bytes)to)));
+    const uint64_t from = uint64_t(uintptr_t(shared_base));
+    const uint64_t uniform = uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(from))))) |
+                             uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(from >> 32))))) << 32;      // (the builtin gives a signed int)
+    uint32_t keep;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %3 nt\n\ts_mov_b32 m0, %0" : "=&s"(keep) : "v"(offset), "s"(base), "s"(uniform) : "memory");
+}
+
+// max(x, 0) as one instruction, an integer maximum of the bits: a negative number, a negative zero or a NaN with the sign set
+// gives 0; a NaN without it stays (fmaxf would give 0, and cost an instruction more, which first quiets x).  For brackets
+// only: a NaN or an infinity among the inputs reaches the bracket's margin as well, which is then no number either way.
+__device__ __forceinline__ float positive_part(float x) { return __int_as_float(max(__float_as_int(x), 0)); }
+
+// A square root good to a few units in the last place (the hardware's, with the scaling that keeps tiny arguments out of the
+// flushed range): for bounds that carry a margin of their own.
+__device__ __forceinline__ float rough_sqrt(float x) {
+    const bool tiny = x < 0x1p-96f;
+    const float root = __builtin_amdgcn_sqrtf(tiny ? x * 0x1p+32f : x);
+    return tiny ? root * 0x1p-16f : root;
 }
 
 // Bounds of the scores of INTERVAL_KEYS groups per workgroup, 16 groups per MFMA tile and wave, and the first radix
@@ -406,12 +430,21 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
     const size_t limit = min(groups, size_t(seen > 0 ? seen : 0));
     const uint16_t* row_keys = keys + row * groups * DIM;
     const size_t first = size_t(blockIdx.x) * BRACKET_KEYS, end = min(first + BRACKET_KEYS, groups);
+    uint32_t place[4];                  // where in a tile's 4 KiB this lane's four pieces lie
+    #pragma unroll
+    for (int j = 0; j < 4; ++j) { const int r = 4 * j + g; place[j] = uint32_t(r * 256 + (li ^ r) * 16); }
     const auto copy_in = [&](int buffer, size_t tile) {
-        #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int r = 4 * j + (lane >> 4), c = (lane & 15) ^ r;
-            const uint16_t* from = row_keys + min(tile + r, groups - 1) * DIM + 8 * c;
-            load_to_lds(from, stages[wave][buffer] + 1024 * j);
+        if (tile + 16 <= groups) {
+            #pragma unroll
+            for (int j = 0; j < 4; ++j) load_to_lds(row_keys + tile * DIM, place[j], stages[wave][buffer] + 1024 * j);
+        } else {
+            // the row's last tile: the rows past the end read the last one again
+            #pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int r = 4 * j + g, c = li ^ r;
+                const uint16_t* from = row_keys + min(tile + r, groups - 1) * DIM + 8 * c;
+                load_to_lds(from, stages[wave][buffer] + 1024 * j);
+            }
         }
     };
     constexpr size_t stride = 16 * BRACKET_WAVES;
@@ -447,8 +480,10 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
         if (tile + (BRACKET_RING - 1) * stride < end) copy_in((buffer + BRACKET_RING - 1) % BRACKET_RING, tile + (BRACKET_RING - 1) * stride);
         // this tile has landed when only the tiles after it (at most three, four loads each) are outstanding
         const size_t after = (end - tile - 1) / stride;
-        if (after >= 3) __builtin_amdgcn_s_waitcnt(0x0f70 | 12); else if (after == 2) __builtin_amdgcn_s_waitcnt(0x0f70 | 8);
-        else if (after == 1) __builtin_amdgcn_s_waitcnt(0x0f70 | 4); else __builtin_amdgcn_s_waitcnt(0x0f70);
+        // (and the bounds of the three tiles before, two stores each, issued between those loads: memory operations finish in the
+        // order issued, so a count that left them out would wait for a later tile as well)
+        if (after >= 3) __builtin_amdgcn_s_waitcnt(0x4f72); else if (after == 2) __builtin_amdgcn_s_waitcnt(0x0f7e);       // 18, 14
+        else if (after == 1) __builtin_amdgcn_s_waitcnt(0x0f7a); else __builtin_amdgcn_s_waitcnt(0x0f76);                  // 10, 6
         bf16x8 kb[KS];
         #pragma unroll
         for (int b = 0; b < KS; ++b) kb[b] = *reinterpret_cast<const bf16x8*>(stages[wave][buffer] + li * 256 + 16 * ((4 * b + g) ^ li));
@@ -463,14 +498,14 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
             #pragma unroll
             for (int b = 0; b < KS; ++b) dots = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[t][b], kb[b], dots, 0, 0, 0);
             #pragma unroll
-            for (int r = 0; r < 4; ++r) total = fmaf(fmaxf(dots[r], 0.0f), w[t][r], total);
+            for (int r = 0; r < 4; ++r) total = fmaf(positive_part(dots[r]), w[t][r], total);
         }
         total = quad_sum(total) * scale;
         // the diagonal of K . K^T: row 4g + r = column li
         const int r = li & 3;
         const float square = r == 0 ? norms[0] : r == 1 ? norms[1] : r == 2 ? norms[2] : norms[3];
         if (g == (li >> 2) && group < groups) {
-            const float e = bound * sqrtf(square);
+            const float e = bound * rough_sqrt(square);
             const bool live = group < limit;
             const float low = live ? total - e : -INFINITY, high = live ? total + e : -INFINITY;
             lower[row * groups + group] = low;
@@ -580,12 +615,22 @@ __global__ void __launch_bounds__(256) radix_histogram_kernel(const float* lower
 //               score -- it is listed with the CERTAIN bit and needs no canonical score;
 //   the rest of the candidates are the band around the cut: only they are scored canonically.
 // With fewer than k live groups everything live is a certain candidate.
+//
+// The band members of the segment get their canonical score here as well, a wave a member (the workgroup's four waves take the
+// members in turn): a lane per head; the head's 128 query values come from LDS, where the row's queries were put on the way in
+// (a head every 272 bytes, so that sixteen lanes' 16-byte reads fall in different banks); a key row is 64 words, lane i
+// fetches word i (one coalesced load, the next member's row on its way while this one is used) and the words go round by
+// v_readlane, so a member costs a wave 64 broadcasts and 128 multiply-adds in the canonical column order.  Then the member's
+// terms are added in head order by one lane, read from LDS.  A score lands at its group's place in the list.
 constexpr uint32_t CERTAIN = 0x80000000u;
-__global__ void __launch_bounds__(256) candidate_segments_kernel(const float* lower, const float* upper, size_t groups, size_t rows, uint32_t k, uint32_t* histogram,
-                                                                 int32_t* list, uint32_t* counts) {
+template<int HEADS>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
+candidate_segments_kernel(const float* lower, const float* upper, size_t groups, size_t rows, uint32_t k, uint32_t* histogram, int32_t* list, uint32_t* counts,
+                          const uint16_t* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights, float scale, float* __restrict__ scores) {
+    constexpr int DIM = 128;
     const size_t row = blockIdx.y;
     const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS + 4 * threadIdx.x;        // thread t owns 4 consecutive groups
-    // (the groups' bounds are asked for before the pick's own trip to memory ends)
+    // (the groups' bounds and the row's queries are asked for before the pick's own trip to memory ends)
     float low[4], high[4];
     if (first + 3 < groups && (row * groups) % 4 == 0) {
         const float4 l4 = *reinterpret_cast<const float4*>(lower + row * groups + first), h4 = *reinterpret_cast<const float4*>(upper + row * groups + first);
@@ -606,6 +651,8 @@ __global__ void __launch_bounds__(256) candidate_segments_kernel(const float* lo
         if (!(certain_above == certain_above)) certain_above = INFINITY;      // a NaN in the bounds: nothing is certain
     }
     __shared__ uint32_t wave_sums[4];
+    __shared__ uint32_t band_members[INTERVAL_KEYS];              // place in the segment's list << 10 | group within the segment
+    __shared__ float terms[4][HEADS + 1];
     uint32_t entry[4], mine = 0, band = 0;
     #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -616,91 +663,64 @@ __global__ void __launch_bounds__(256) candidate_segments_kernel(const float* lo
         mine += keep;
         band += keep && !certain;
     }
-    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     uint32_t packed = mine | (band << 16), inclusive = packed;        // both counts scanned at once (at most 1024 each)
     #pragma unroll
-    for (unsigned offset = 1; offset < 64; offset *= 2) { const uint32_t other = __shfl_up(inclusive, offset); if (lane >= offset) inclusive += other; }
+    for (int offset = 1; offset < 64; offset *= 2) { const uint32_t other = __shfl_up(inclusive, offset); if (lane >= offset) inclusive += other; }
     if (lane == 63) wave_sums[wave] = inclusive;
     __syncthreads();
     uint32_t before = 0, all = 0;
-    for (unsigned v = 0; v < 4; ++v) { before += v < wave ? wave_sums[v] : 0u; all += wave_sums[v]; }
-    uint32_t at = ((before + inclusive - packed) & 0xffffu);
+    for (int v = 0; v < 4; ++v) { before += v < wave ? wave_sums[v] : 0u; all += wave_sums[v]; }
+    uint32_t at = (before + inclusive - packed) & 0xffffu, band_at = (before + inclusive - packed) >> 16;
     int32_t* out = list + row * groups + size_t(blockIdx.x) * INTERVAL_KEYS;
     #pragma unroll
-    for (int i = 0; i < 4; ++i) if (entry[i] != 0xffffffffu) out[at++] = int32_t(entry[i]);
-    if (threadIdx.x == 0) counts[row * gridDim.x + blockIdx.x] = all;        // candidates | band members << 16
-}
-
-// The canonical score of the band's groups.  A wave takes a segment at a time (every SCORE_STRIDE-th one), finds the band
-// members among the segment's candidates by a ballot, and scores them a few at a time: a lane per head with the head's 128 query
-// values in its registers; a key row is 64 words, lane i fetches word i (one coalesced load, the next group's row on its
-// way while this one is used) and the words go round by v_readlane, so a group costs a wave 64 broadcasts and 128
-// multiply-adds in the canonical column order.  Then each group's 64 terms are added in head order -- lane c the terms of
-// group c, read from LDS, so the ordered sums run side by side.  A score lands at its group's place in the list.
-template<int HEADS>
-__global__ void __launch_bounds__(SCORE_WAVES * 64) band_score_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ keys, const float* __restrict__ weights,
-                                                         size_t groups, float scale, const int32_t* __restrict__ list, const uint32_t* __restrict__ counts,
-                                                         size_t segments, float* __restrict__ scores, uint32_t* __restrict__ histogram, size_t histogram_rows) {
-    constexpr int DIM = 128, BATCH = SCORE_BATCH;
-    const size_t row = blockIdx.y;
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    // The histograms' last reader ran before this kernel: the row's first workgroup zeroes them (and the widest margin) for the
-    // next call, while everything below goes on.
-    if (blockIdx.x == 0) {
-        for (int level = 0; level < RADIX_LEVELS; ++level) {
-            uint32_t* bins = radix_bins(histogram, histogram_rows, level, row);
-            for (unsigned i = threadIdx.x; i < unsigned(RADIX_BINS); i += SCORE_WAVES * 64) bins[i] = 0u;
+    for (int i = 0; i < 4; ++i)
+        if (entry[i] != 0xffffffffu) {
+            if (!(entry[i] & CERTAIN)) band_members[band_at++] = (at << 10) | (4 * threadIdx.x + i);
+            out[at++] = int32_t(entry[i]);
         }
-        if (threadIdx.x == 0) *widest_margin(histogram, histogram_rows, row) = 0u;
-    }
+    if (threadIdx.x == 0) counts[row * gridDim.x + blockIdx.x] = all;        // candidates | band members << 16
+    const int members = int(all >> 16);
+    if (!members) return;
+    __syncthreads();
+    if (wave >= members) return;
     const int head = min(lane, HEADS - 1);
-    __shared__ float terms[SCORE_WAVES][BATCH][HEADS + 1];
-    __shared__ uint32_t places[SCORE_WAVES][64];
-    // the head's query values, widened (asked for at once: a wave with nothing to score has wasted a few loads from the cache)
-    float mine[DIM];
-    #pragma unroll
-    for (int d = 0; d < DIM; d += 8) {
-        const uint4 bits = *reinterpret_cast<const uint4*>(q + (row * HEADS + head) * DIM + d);
-        const uint32_t words[4] = {bits.x, bits.y, bits.z, bits.w};
-        #pragma unroll
-        for (int i = 0; i < 4; ++i) { mine[d + 2 * i] = __uint_as_float(words[i] << 16); mine[d + 2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u); }
-    }
     const float weight = weights[row * HEADS + head];
-    const uint32_t* row_keys = reinterpret_cast<const uint32_t*>(keys + row * groups * DIM);
-    for (size_t segment = size_t(blockIdx.x) * SCORE_WAVES + wave; segment < segments; segment += size_t(gridDim.x) * SCORE_WAVES) {
-        const uint32_t count = counts[row * segments + segment];
-        if (!(count >> 16)) continue;                                  // no band member here (wave-uniform)
-        const int32_t* entries = list + row * groups + segment * INTERVAL_KEYS;
-        for (uint32_t base = 0; base < (count & 0xffffu); base += 64) {
-            const uint32_t entry = base + uint32_t(lane) < (count & 0xffffu) ? uint32_t(entries[base + lane]) : CERTAIN;
-            const uint64_t wanted = __ballot(!(entry & CERTAIN));
-            if (!wanted) continue;
-            // the band members' lanes in order: member m of this chunk sits at lane places[m]
-            const int members = __popcll(wanted);
-            if (!(entry & CERTAIN)) places[wave][__popcll(wanted & ((uint64_t(1) << lane) - 1))] = uint32_t(lane);
-            for (int done = 0; done < members; done += BATCH) {
-                const int batch = min(BATCH, members - done);
-                uint32_t words = row_keys[size_t(__shfl(entry, int(places[wave][done]))) * (DIM / 2) + lane];
-                for (int c = 0; c < batch; ++c) {
-                    const uint32_t current = words;
-                    if (c + 1 < batch) words = row_keys[size_t(__shfl(entry, int(places[wave][done + c + 1]))) * (DIM / 2) + lane];
-                    float dot = 0.0f;
-                    #pragma unroll
-                    for (int d = 0; d < DIM; d += 2) {
-                        const uint32_t pair = __builtin_amdgcn_readlane(current, d / 2);
-                        dot = __builtin_fmaf(mine[d], __uint_as_float(pair << 16), dot);
-                        dot = __builtin_fmaf(mine[d + 1], __uint_as_float(pair & 0xffff0000u), dot);
-                    }
-                    if (lane < HEADS) terms[wave][c][lane] = rounded_product(fmaxf(dot, 0.0f), weight);
-                }
-                // the wave's own writes, read back by the wave: LDS keeps a wave's accesses in order
-                if (lane < batch) {
-                    float sum = 0.0f;
-                    #pragma unroll
-                    for (int h = 0; h < HEADS; ++h) sum = rounded_sum(sum, terms[wave][lane][h]);
-                    scores[row * groups + segment * INTERVAL_KEYS + base + places[wave][done + lane]] = rounded_product(sum, scale);
-                }
+    // the head's query values, two to a word (a lane reads its own head's 256 bytes: every load spreads over 64 lines, and
+    // the many waves that read the same row at the same time do not crowd on one of them)
+    uint4 query[DIM / 8];
+    #pragma unroll
+    for (int j = 0; j < DIM / 8; ++j) query[j] = reinterpret_cast<const uint4*>(q + (row * HEADS + head) * DIM)[j];
+    const uint32_t* segment_keys = reinterpret_cast<const uint32_t*>(keys + (row * groups + size_t(blockIdx.x) * INTERVAL_KEYS) * DIM);
+    uint32_t member = band_members[wave];
+    uint32_t words = segment_keys[size_t(member & 1023u) * (DIM / 2) + lane];
+    for (int m = wave; m < members; m += 4) {
+        const uint32_t current = words, place = member >> 10;
+        if (m + 4 < members) {
+            member = band_members[m + 4];
+            words = segment_keys[size_t(member & 1023u) * (DIM / 2) + lane];
+        }
+        float dot = 0.0f;
+        #pragma unroll
+        for (int d = 0; d < DIM; d += 8) {
+            uint32_t pairs[4] = {query[d / 8].x, query[d / 8].y, query[d / 8].z, query[d / 8].w};
+            // (widened again for every member: 128 widened values held across the loop would cost a wave of occupancy)
+            #pragma unroll
+            for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(pairs[i]));
+            #pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t pair = __builtin_amdgcn_readlane(current, d / 2 + i);
+                dot = __builtin_fmaf(__uint_as_float(pairs[i] << 16), __uint_as_float(pair << 16), dot);
+                dot = __builtin_fmaf(__uint_as_float(pairs[i] & 0xffff0000u), __uint_as_float(pair & 0xffff0000u), dot);
             }
+        }
+        if (lane < HEADS) terms[wave][lane] = rounded_product(fmaxf(dot, 0.0f), weight);
+        // the wave's own writes, read back by the wave: LDS keeps a wave's accesses in order
+        if (lane == 0) {
+            float sum = 0.0f;
+            #pragma unroll 4
+            for (int h = 0; h < HEADS; ++h) sum = rounded_sum(sum, terms[wave][h]);
+            scores[row * groups + size_t(blockIdx.x) * INTERVAL_KEYS + place] = rounded_product(sum, scale);
         }
     }
 }
@@ -712,9 +732,16 @@ __global__ void __launch_bounds__(SCORE_WAVES * 64) band_score_kernel(const uint
 // row is then the result.  A band of at most a thousand is ranked directly (every member counts who beats it, one thread
 // each); anything larger takes the general radix select.
 __global__ void __launch_bounds__(TOPK_THREADS) index_finish_kernel(const float* scores, const int32_t* list, const uint32_t* counts, size_t segments, size_t groups,
-                                                                    size_t k, float* flat_scores, int32_t* flat_list, int32_t* out) {
+                                                                    size_t k, float* flat_scores, int32_t* flat_list, int32_t* out, uint32_t* histogram,
+                                                                    size_t histogram_rows) {
     const size_t row = blockIdx.x;
     const unsigned t = threadIdx.x;
+    // The histograms' last reader ran before this kernel: the row's are zeroed (and its widest margin) for the next call.
+    for (int level = 0; level < RADIX_LEVELS; ++level) {
+        uint32_t* bins = radix_bins(histogram, histogram_rows, level, row);
+        for (unsigned i = t; i < unsigned(RADIX_BINS); i += TOPK_THREADS) bins[i] = 0u;
+    }
+    if (t == 0) *widest_margin(histogram, histogram_rows, row) = 0u;
     constexpr uint32_t HELD = 6144, RANKED = 1024;
     __shared__ float held_scores[HELD];
     __shared__ int32_t held_list[HELD];
@@ -904,11 +931,11 @@ void fast_index_top_k(Device& d, const FastIndexSpace& s, const void* q_index, c
     fast_index_bounds<HEADS>(d, q_index, keys, weights, visible, batch, groups, scale, s.lower, s.upper, histogram);
     const uint32_t rank = uint32_t(std::min<size_t>(k, 0xffffffffu));
     radix_histogram_kernel<<<dim3(segments, unsigned(batch)), 256, 0, d.stream>>>(s.lower, groups, d.index_bins_rows, rank, histogram);
-    candidate_segments_kernel<<<dim3(segments, unsigned(batch)), 256, 0, d.stream>>>(s.lower, s.upper, groups, d.index_bins_rows, rank, histogram, s.list, s.counts);
-    const unsigned score_groups = unsigned(std::min<size_t>((s.segments + SCORE_WAVES - 1) / SCORE_WAVES, 64));
-    band_score_kernel<HEADS><<<dim3(score_groups, unsigned(batch)), SCORE_WAVES * 64, 0, d.stream>>>(static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys), weights,
-                                                                                                 groups, scale, s.list, s.counts, s.segments, s.scores, histogram, d.index_bins_rows);
-    index_finish_kernel<<<unsigned(batch), TOPK_THREADS, 0, d.stream>>>(s.scores, s.list, s.counts, s.segments, groups, k, s.flat_scores, s.flat_list, indices);
+    candidate_segments_kernel<HEADS><<<dim3(segments, unsigned(batch)), 256, 0, d.stream>>>(s.lower, s.upper, groups, d.index_bins_rows, rank, histogram, s.list, s.counts,
+                                                                                          static_cast<const uint16_t*>(q_index), static_cast<const uint16_t*>(keys), weights,
+                                                                                          scale, s.scores);
+    index_finish_kernel<<<unsigned(batch), TOPK_THREADS, 0, d.stream>>>(s.scores, s.list, s.counts, s.segments, groups, k, s.flat_scores, s.flat_list, indices, histogram,
+                                                                        d.index_bins_rows);
     SD_CHECK(hipGetLastError());
     d.index_bins_dirty = false;
 }
