@@ -448,11 +448,14 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
         }
     };
     constexpr size_t stride = 16 * BRACKET_WAVES;
-    size_t tile = first + 16 * wave;
+    // the wave's tiles, `count` of them, one every `stride` groups
+    const size_t mine = first + 16 * wave;
+    const int count = mine < end ? int((end - mine + stride - 1) / stride) : 0;
+    const auto tile_at = [&](int turn) { return mine + size_t(turn) * stride; };
     // the first tiles are asked for before anything waits for the queries: they travel while the margin is worked out
     #pragma unroll
-    for (int ahead = 0; ahead < BRACKET_RING - 1; ++ahead)
-        if (tile + ahead * stride < end) copy_in(ahead, tile + ahead * stride);
+    for (int ahead = 0; ahead < BRACKET_RING; ++ahead)
+        if (ahead < count) copy_in(ahead, tile_at(ahead));
     // W of the margin, sum_h |w_h| |q_h|, by every wave for itself: a lane's 32 values of head 16t + li squared and summed, the
     // four lane groups' parts added, the root times |w_h| added over the tile's 16 heads (lanes) and the tiles
     float reach = 0.0f;
@@ -475,31 +478,10 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
     // (the wait for the queries above was a wait for every load so far, the first tiles' among them: none of the compiler's
     // own loads is outstanding, and the loop's waits count the tiles' loads alone)
     __builtin_amdgcn_s_waitcnt(0x0f70);
-    for (int buffer = 0; tile < end; tile += stride, buffer = (buffer + 1) % BRACKET_RING) {
+    // Two tiles a turn, so that one's matrix products run under the other's arithmetic: the pair's operands are read from their
+    // stages, the stages take the copies of the pair two turns on, and both tiles are worked out side by side.
+    const auto finish = [&](size_t tile, float total, const floatx4& norms) {
         const size_t group = tile + li;
-        if (tile + (BRACKET_RING - 1) * stride < end) copy_in((buffer + BRACKET_RING - 1) % BRACKET_RING, tile + (BRACKET_RING - 1) * stride);
-        // this tile has landed when only the tiles after it (at most three, four loads each) are outstanding
-        const size_t after = (end - tile - 1) / stride;
-        // (and the bounds of the three tiles before, two stores each, issued between those loads: memory operations finish in the
-        // order issued, so a count that left them out would wait for a later tile as well)
-        if (after >= 3) __builtin_amdgcn_s_waitcnt(0x4f72); else if (after == 2) __builtin_amdgcn_s_waitcnt(0x0f7e);       // 18, 14
-        else if (after == 1) __builtin_amdgcn_s_waitcnt(0x0f7a); else __builtin_amdgcn_s_waitcnt(0x0f76);                  // 10, 6
-        bf16x8 kb[KS];
-        #pragma unroll
-        for (int b = 0; b < KS; ++b) kb[b] = *reinterpret_cast<const bf16x8*>(stages[wave][buffer] + li * 256 + 16 * ((4 * b + g) ^ li));
-        __builtin_amdgcn_s_waitcnt(0xc07f);          // the operands are in registers: the stage is free for the copy issued next
-        floatx4 norms = {0.0f, 0.0f, 0.0f, 0.0f};
-        #pragma unroll
-        for (int b = 0; b < KS; ++b) norms = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[b], kb[b], norms, 0, 0, 0);
-        float total = 0.0f;
-        #pragma unroll
-        for (int t = 0; t < HT; ++t) {
-            floatx4 dots = {0.0f, 0.0f, 0.0f, 0.0f};
-            #pragma unroll
-            for (int b = 0; b < KS; ++b) dots = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[t][b], kb[b], dots, 0, 0, 0);
-            #pragma unroll
-            for (int r = 0; r < 4; ++r) total = fmaf(positive_part(dots[r]), w[t][r], total);
-        }
         total = quad_sum(total) * scale;
         // the diagonal of K . K^T: row 4g + r = column li
         const int r = li & 3;
@@ -514,6 +496,43 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
             if (histogram && key > top_k_key(-INFINITY)) atomicAdd(&bins[radix_digit(key, 0)], 1u);
             if (live) widest = fmaxf(widest, e);
         }
+    };
+    for (int turn = 0, buffer = 0; turn < count; turn += 2, buffer ^= 2) {
+        // The pair has landed when only what was issued after its second copy is outstanding: the bounds of the two pairs before
+        // (two stores a tile, issued between the copies; memory operations finish in the order issued) and the copies of the
+        // pair after this one, four loads a tile.  (The first two pairs had landed before the loop.)
+        const int after = count - 1 - turn;                        // tiles after the pair's first
+        const bool second = after >= 1;
+        if (after >= 3) __builtin_amdgcn_s_waitcnt(0x4f70); else if (after == 2) __builtin_amdgcn_s_waitcnt(0x0f7c);       // 16, 12
+        else __builtin_amdgcn_s_waitcnt(0x0f78);                                                                           // 8
+        bf16x8 kb[2][KS];
+        #pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            #pragma unroll
+            for (int b = 0; b < KS; ++b) kb[u][b] = *reinterpret_cast<const bf16x8*>(stages[wave][buffer + u] + li * 256 + 16 * ((4 * b + g) ^ li));
+        }
+        __builtin_amdgcn_s_waitcnt(0xc07f);          // the operands are in registers: the stages are free for the next copies
+        if (turn + 4 < count) copy_in(buffer, tile_at(turn + 4));
+        if (turn + 5 < count) copy_in(buffer + 1, tile_at(turn + 5));
+        floatx4 norms[2];
+        float total[2];
+        #pragma unroll
+        for (int u = 0; u < 2; ++u) {          // (the second of a lone tile's pair works on whatever its stage holds, and is dropped)
+            norms[u] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            #pragma unroll
+            for (int b = 0; b < KS; ++b) norms[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[u][b], kb[u][b], norms[u], 0, 0, 0);
+            total[u] = 0.0f;
+            #pragma unroll
+            for (int t = 0; t < HT; ++t) {
+                floatx4 dots = {0.0f, 0.0f, 0.0f, 0.0f};
+                #pragma unroll
+                for (int b = 0; b < KS; ++b) dots = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[t][b], kb[u][b], dots, 0, 0, 0);
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) total[u] = fmaf(positive_part(dots[r]), w[t][r], total[u]);
+            }
+        }
+        finish(tile_at(turn), total[0], norms[0]);
+        if (second) finish(tile_at(turn + 1), total[1], norms[1]);
     }
     if (!histogram) return;
     #pragma unroll
