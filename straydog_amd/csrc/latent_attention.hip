@@ -336,7 +336,7 @@ int sdx_latent_attention(void* handle, const void* q, const void* latents, const
     op_span(value, latents, checked_product({batch, groups, kdim, 2}), "latent rows");
     op_span(value, selected, checked_floats({batch, k}), "selected rows");
     op_span(value, out, checked_floats({batch, heads, vdim}), "an attention output");
-    if (latent_gather_supported(kdim, vdim) && groups < (uint64_t(1) << 31) && k < (uint64_t(1) << 31)) {
+    if (latent_gather_supported(kdim, vdim) && groups * kdim * 2 < (uint64_t(1) << 32) && k < (uint64_t(1) << 31)) {      // (a sequence's rows within 32-bit offsets)
         // the matrix-core path; its chunk partials live in the device's workspace (grown outside graph capture)
         float* partial = static_cast<float*>(workspace(value, latent_gather_scratch(batch, k, heads, vdim)));
         latent_gather(value, q, latents, selected, batch, groups, k, heads, scale, out, partial);

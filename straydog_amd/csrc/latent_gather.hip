@@ -4,7 +4,10 @@
 // sums, as the reference's WMMA prompt path does it (gpu/ds_attention_wmma.hpp:26-340).
 //
 // Shape of the work on gfx950 (wave64, v_mfma_f32_16x16x32_bf16):
-//   * a workgroup (4 waves) owns one sequence, 128 of its selected rows and 64 heads, a wave 16 of the heads;
+//   * a workgroup (4 waves) owns one sequence, 64 or 128 of its selected rows and 32 heads; a wave takes 16 of the heads and
+//     half of the value columns (the two waves of a head tile form the same scores and weights, each for itself: the partial
+//     results, and not the products, are what this kernel's time goes into, and 32 heads a workgroup let a chunk be twice as
+//     long, and the partial results half as many, with the same number of workgroups);
 //   * 32 rows at a time are gathered (16-byte pieces, every row whole) into a padded K tile in LDS and from there
 //     transposed into a V tile, both read without bank conflicts as MFMA operands by all four waves;
 //   * S^T = K . Q^T (rows x heads) leaves the weights in the B-operand layout of O^T += V^T . P^T, so they never move
@@ -19,13 +22,13 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-constexpr int CHUNK = 64;           // selected rows per workgroup
+constexpr int CHUNK = 64, CHUNK_MAX = 128, BLOCK_HEADS = 32;           // selected rows per workgroup (the shorter kind, the longer), heads
 
 struct GatherArgs {
     const uint16_t* q;              // [batch][heads][kdim] BF16
     const uint16_t* latents;        // [batch][groups][kdim] BF16
     const int32_t* selected;        // [batch][k], entries outside 0..groups-1 are skipped
-    unsigned groups, k, heads, chunks;
+    unsigned groups, k, heads, chunks, chunk_rows;
     float scale_log2;
     float* partial;                 // [batch][chunk][heads][vdim + 2]
     float* out;                     // [batch][heads][vdim]
@@ -42,16 +45,17 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
     constexpr int KSTEPS = KDIM / 32, TILES = VDIM / 16, KP = 2 * KDIM + 16, VP = 2 * STEP + 8, PIECES = KDIM / 8;
     const int chunk = blockIdx.x, batch = blockIdx.z, thread = threadIdx.x;
     const int lane = thread & 63, wave = __builtin_amdgcn_readfirstlane(thread >> 6), li = lane & 15, g = lane >> 4;
-    const int head = int(blockIdx.y) * 64 + wave * 16 + li;
+    const int tile_of_heads = wave & 1, half = wave >> 1;                                  // the wave's 16 heads and its half of the columns
+    const int head = int(blockIdx.y) * BLOCK_HEADS + tile_of_heads * 16 + li;
     const bool real = head < int(a.heads);
     extern __shared__ uint8_t lds[];
     uint8_t* ktile = lds;                                     // [32 rows][KP]
     uint8_t* vtile = ktile + STEP * KP;                       // [VDIM columns][VP]
     uint32_t* seen = reinterpret_cast<uint32_t*>(vtile + VDIM * VP);   // [32]: 1 where the step's row exists
-    int32_t* chosen = reinterpret_cast<int32_t*>(seen + STEP);         // [CHUNK]: the workgroup's selected rows, -1 where there is none
-    const int first = chunk * CHUNK, last = min(int(a.k), first + CHUNK);
+    int32_t* chosen = reinterpret_cast<int32_t*>(seen + STEP);         // [CHUNK_MAX]: the workgroup's selected rows, -1 where there is none
+    const int first = chunk * int(a.chunk_rows), last = min(int(a.k), first + int(a.chunk_rows));
     // the selection is read once, ahead of everything else: a step's rows then wait for one load, not for two in a row
-    if (thread < CHUNK) chosen[thread] = first + thread < last ? a.selected[size_t(batch) * a.k + first + thread] : -1;
+    if (thread < CHUNK_MAX) chosen[thread] = first + thread < last ? a.selected[size_t(batch) * a.k + first + thread] : -1;
 
     bf16x8 qf[KSTEPS];
     #pragma unroll
@@ -60,17 +64,21 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
         if (real) bits = *reinterpret_cast<const uint4*>(a.q + (size_t(batch) * a.heads + head) * KDIM + 32 * b + 8 * g);
         qf[b] = __builtin_bit_cast(bf16x8, bits);
     }
-    floatx4 acc[TILES];
+    constexpr int MY_TILES = TILES / 2;
+    floatx4 acc[MY_TILES];
     #pragma unroll
-    for (int jj = 0; jj < TILES; ++jj) acc[jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int j = 0; j < MY_TILES; ++j) acc[j] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     float m = NEG_BIG, l = 0.0f;
 
     __syncthreads();
     // gather: a row is PIECES pieces of 16 bytes, a thread takes every 256th piece of a step; a missing row is read from row 0
-    // and masked.  The pieces of the step after this one are fetched into registers before this one is multiplied.
+    // and masked.  The pieces of the step after this one are fetched into registers before this one is multiplied.  (Two steps
+    // ahead was measured and is slower: the registers it takes cost more than the trip to memory it hides.)
     constexpr int MINE = (STEP * PIECES + 255) / 256;
     uint4 fetched[MINE];
     uint32_t present = 0;                                     // bit j: the row of the thread's j-th piece exists
+    // (the sequence's rows from an address all lanes share and a 32-bit offset a lane: two vector instructions an address)
+    const uint8_t* rows = reinterpret_cast<const uint8_t*>(a.latents + size_t(batch) * a.groups * KDIM);
     const auto fetch = [&](int key0) {
         present = 0;
         #pragma unroll
@@ -78,10 +86,9 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
             const int piece = thread + 256 * j, row = piece / PIECES, part = piece % PIECES;
             fetched[j] = uint4{0u, 0u, 0u, 0u};
             if (piece < STEP * PIECES) {
- 
-                const int index = chosen[key0 - first + row];
-                const bool exists = index >= 0 && index < int(a.groups);
-                fetched[j] = *reinterpret_cast<const uint4*>(a.latents + (size_t(batch) * a.groups + (exists ? index : 0)) * KDIM + 8 * part);
+                const uint32_t index = uint32_t(chosen[key0 - first + row]);
+                const bool exists = index < a.groups;                       // (a negative entry is a large unsigned one)
+                fetched[j] = *reinterpret_cast<const uint4*>(rows + size_t((exists ? index : 0u) * uint32_t(2 * KDIM) + uint32_t(16 * part)));
                 present |= exists ? 1u << j : 0u;
             }
         }
@@ -145,7 +152,7 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
             m = m_new;
             l *= alpha;
             #pragma unroll
-            for (int jj = 0; jj < TILES; ++jj) acc[jj] *= alpha;
+            for (int j = 0; j < MY_TILES; ++j) acc[j] *= alpha;
         }
         const float offset = -m * a.scale_log2;
         float w[8], sum = 0.0f;
@@ -164,22 +171,22 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
         const uint4 high = {bf16_pair(w[0], w[1]), bf16_pair(w[2], w[3]), bf16_pair(w[4], w[5]), bf16_pair(w[6], w[7])};
         const uint4 low = {bf16_pair(rest[0], rest[1]), bf16_pair(rest[2], rest[3]), bf16_pair(rest[4], rest[5]), bf16_pair(rest[6], rest[7])};
         const bf16x8 pb = __builtin_bit_cast(bf16x8, high), pl = __builtin_bit_cast(bf16x8, low);
-        // O^T tiles: columns (16 jj + 4 g + r) x heads
+        // O^T tiles: columns (16 jj + 4 g + r) x heads, the wave's half of them
         #pragma unroll
-        for (int jj = 0; jj < TILES; ++jj) {
-            const uint8_t* from = vtile + (16 * jj + li) * VP + 8 * g;
+        for (int j = 0; j < MY_TILES; ++j) {
+            const uint8_t* from = vtile + (16 * (half * MY_TILES + j) + li) * VP + 8 * g;
             const uint2 near = *reinterpret_cast<const uint2*>(from), far = *reinterpret_cast<const uint2*>(from + 32);
             const uint4 both = {near.x, near.y, far.x, far.y};
-            acc[jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb, acc[jj], 0, 0, 0);
-            acc[jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pl, acc[jj], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb, acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pl, acc[j], 0, 0, 0);
         }
     }
     l = row_sum(l);
     if (!real) return;
     float* to = a.partial + ((size_t(batch) * a.chunks + chunk) * a.heads + head) * (VDIM + 2);
     #pragma unroll
-    for (int jj = 0; jj < TILES; ++jj) *reinterpret_cast<floatx4*>(to + 16 * jj + 4 * g) = acc[jj];
-    if (g == 0) { to[VDIM] = m; to[VDIM + 1] = l; }
+    for (int j = 0; j < MY_TILES; ++j) *reinterpret_cast<floatx4*>(to + 16 * (half * MY_TILES + j) + 4 * g) = acc[j];
+    if (g == 0 && half == 0) { to[VDIM] = m; to[VDIM + 1] = l; }
 }
 
 // One block per (sequence, head): the chunks merged under their common maximum and normalised; a head none of whose
@@ -237,11 +244,15 @@ void latent_gather(Device& d, const void* q, const void* latents, const int32_t*
     constexpr int KDIM = 576, VDIM = 512;
     GatherArgs args{};
     args.q = static_cast<const uint16_t*>(q); args.latents = static_cast<const uint16_t*>(latents); args.selected = selected;
-    args.groups = unsigned(groups); args.k = unsigned(k); args.heads = unsigned(heads); args.chunks = unsigned((k + CHUNK - 1) / CHUNK);
+    args.groups = unsigned(groups); args.k = unsigned(k); args.heads = unsigned(heads);
+    // the longer chunks when they still give every compute unit a workgroup: half the partial results to write and to merge
+    const uint64_t head_parts = (heads + BLOCK_HEADS - 1) / BLOCK_HEADS;
+    args.chunk_rows = batch * ((k + CHUNK_MAX - 1) / CHUNK_MAX) * head_parts >= uint64_t(d.compute_units) ? CHUNK_MAX : CHUNK;
+    args.chunks = unsigned((k + args.chunk_rows - 1) / args.chunk_rows);
     args.scale_log2 = scale * 1.44269504088896341f; args.partial = partial; args.out = out;
-    constexpr size_t shared = size_t(STEP) * (2 * KDIM + 16) + size_t(VDIM) * (2 * STEP + 8) + STEP * 4 + CHUNK * 4;
+    constexpr size_t shared = size_t(STEP) * (2 * KDIM + 16) + size_t(VDIM) * (2 * STEP + 8) + STEP * 4 + CHUNK_MAX * 4;
     raise_shared_limit(d, reinterpret_cast<const void*>(&latent_gather_kernel<KDIM, VDIM>), shared);
-    timed_launch(d, &latent_gather_kernel<KDIM, VDIM>, dim3(args.chunks, unsigned((heads + 63) / 64), unsigned(batch)), dim3(256), shared, args);
+    timed_launch(d, &latent_gather_kernel<KDIM, VDIM>, dim3(args.chunks, unsigned(head_parts), unsigned(batch)), dim3(256), shared, args);
     SD_CHECK(hipGetLastError());
     latent_merge_kernel<VDIM><<<unsigned(batch * heads), VDIM / 4, 0, d.stream>>>(args);
 }

@@ -469,6 +469,35 @@ def test_batched_sparse_path_small(gpu, oracle):
         gpu.release(b)
 
 
+def test_latent_gather_long_chunks(gpu, oracle):
+    # enough (sequence, chunk, head part) workgroups for every compute unit: the gather takes its longer chunks of 128 rows; a
+    # selection that is no multiple of the chunk, padded with -1 and with rows out of range, and a head count that fills the
+    # last head part only half
+    rng = np.random.default_rng(77)
+    batch, groups, k, heads, kdim, vdim = 16, 2500, 1000, 48, 576, 512
+    aq_bits, aq = _bf16_round(oracle, rng.standard_normal((batch, heads, kdim)).astype(np.float32))
+    lat_bits, lat = _bf16_round(oracle, rng.standard_normal((batch, groups, kdim)).astype(np.float32))
+    selected = np.stack([rng.permutation(groups)[:k] for _ in range(batch)]).astype(np.int32)
+    selected[1, 900:] = -1                              # a short list
+    selected[2, ::3] = -1                               # holes
+    selected[3, 5] = groups + 7                         # out of range: skipped here (the reference would read past its rows)
+    selected[4, :] = -1                                 # nothing selected: zeros
+    ab, lb, sb, out = gpu.upload(aq_bits), gpu.upload(lat_bits), gpu.upload(selected), gpu.buffer(batch * heads * vdim * 4)
+    scale = float(1.0 / np.sqrt(kdim))
+    gpu.latent_attention(ab.base(), lb.base(), sb.base(), batch, groups, k, heads, kdim, vdim, scale, out.base())
+    got = _read(gpu, out, np.float32, batch * heads * vdim).reshape(batch, heads, vdim)
+    for b in range(batch):
+        if b == 4:
+            continue                                    # (0 / 0 in the reference's arithmetic; zeros here, checked below)
+        listed = np.where(selected[b:b + 1] >= groups, -1, selected[b:b + 1]).astype(np.int32)
+        want = oracle.latent_attention(aq[b:b + 1], None, None, 0, lat_bits[b], listed, None, vdim, scale)
+        close_enough(got[b], want[0], f"sequence {b}")
+        assert np.abs(got[b] - want[0]).max() < 5e-5
+    assert not got[4].any()
+    for b in (ab, lb, sb, out):
+        gpu.release(b)
+
+
 def _dspark_check(label, actual, expected):
     # the reference's own bar (dspark_attention_gpu.rs:41-50): |a - b| / (1 + |b|) <= 2e-5
     error = np.abs(actual.astype(np.float64) - expected) / (1.0 + np.abs(expected))
