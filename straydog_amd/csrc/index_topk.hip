@@ -224,6 +224,29 @@ __device__ __forceinline__ uint32_t block_scan(uint32_t value, uint32_t* wave_su
     return before + inclusive - value;
 }
 
+// The same for two values at once (the exclusive prefix of the first is returned): one pair of barriers for both.
+__device__ __forceinline__ uint32_t block_scan_pair(uint32_t first, uint32_t second, uint2* wave_sums, uint32_t& total_first, uint32_t& total_second) {
+    const unsigned lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    uint32_t inclusive = first, other_inclusive = second;
+    #pragma unroll
+    for (unsigned offset = 1; offset < 64; offset *= 2) {
+        const uint32_t a = __shfl_up(inclusive, offset), b = __shfl_up(other_inclusive, offset);
+        if (lane >= offset) { inclusive += a; other_inclusive += b; }
+    }
+    __syncthreads();
+    if (lane == 63) wave_sums[wave] = uint2{inclusive, other_inclusive};
+    __syncthreads();
+    uint32_t before = 0, sum = 0, other_sum = 0;
+    #pragma unroll
+    for (int w = 0; w < TOPK_WAVES; ++w) {
+        const uint2 c = wave_sums[w];
+        before += unsigned(w) < wave ? c.x : 0u;
+        sum += c.x; other_sum += c.y;
+    }
+    total_first = sum; total_second = other_sum;
+    return before + inclusive - first;
+}
+
 // One workgroup per row.  The k-th highest key by four 8-bit radix passes (MSB first, a 256-bin histogram per pass
 // in LDS), then one ordered pass: thread t owns runs of TOPK_RUN consecutive places so a workgroup scan of the kept
 // counts gives every kept place its slot in ascending index order.  score(place) and index(place) let the same code
@@ -768,22 +791,15 @@ __global__ void __launch_bounds__(TOPK_THREADS) index_finish_kernel(const float*
     __shared__ __attribute__((aligned(16))) uint64_t band_order[RANKED + 2];     // a member's key above its place turned over: a higher value beats a lower one
     __shared__ uint32_t wave_sums[TOPK_WAVES], band_filled;
     // the candidates and band members of the row, and where each segment's candidates go in the flat list
+    __shared__ uint2 wave_pairs[TOPK_WAVES];
     uint32_t candidates = 0, band = 0;
     for (size_t first = 0; first < segments; first += TOPK_THREADS) {
         const uint32_t count = first + t < segments ? counts[row * segments + first + t] : 0u;
-        uint32_t all;
-        const uint32_t before = block_scan(count, wave_sums, all);       // (two 16-bit sums side by side: a row has fewer than 65536 of
-        if (first == 0) segment_base[t] = before & 0xffffu;               //  each only when it fits the fast path, which is checked below)
-        candidates += all & 0xffffu; band += all >> 16;
+        uint32_t all, all_band;
+        const uint32_t before = block_scan_pair(count & 0xffffu, count >> 16, wave_pairs, all, all_band);
+        if (first == 0) segment_base[t] = before;
+        candidates += all; band += all_band;
         __syncthreads();
-    }
-    // exact counts for long rows (the packed sums above may have carried): recount separately when the row is large
-    if (segments > TOPK_THREADS || groups > 65535) {
-        uint32_t c = 0, b = 0;
-        for (size_t s = t; s < segments; s += TOPK_THREADS) { const uint32_t count = counts[row * segments + s]; c += count & 0xffffu; b += count >> 16; }
-        uint32_t all;
-        (void)block_scan(c, wave_sums, all); candidates = all; __syncthreads();
-        (void)block_scan(b, wave_sums, all); band = all; __syncthreads();
     }
     const bool held = candidates <= HELD && segments <= TOPK_THREADS;
     float* const row_scores = held ? held_scores : flat_scores + row * groups;
@@ -799,8 +815,9 @@ __global__ void __launch_bounds__(TOPK_THREADS) index_finish_kernel(const float*
             // (segments without candidates share their base with the next one: move on to the one that really holds the place)
             const size_t at = row * groups + size_t(segment) * INTERVAL_KEYS + (place - segment_base[segment]);
             const uint32_t entry = uint32_t(list[at]);
+            const float scored = scores[at];               // (asked for beside the entry, whether it will count or not: one trip, not two)
             const bool certain = entry & CERTAIN;
-            const float score = certain ? INFINITY : scores[at];
+            const float score = certain ? INFINITY : scored;
             held_scores[place] = score;
             held_list[place] = int32_t(entry & ~CERTAIN);
             if (!certain && band <= RANKED) {
@@ -830,14 +847,20 @@ __global__ void __launch_bounds__(TOPK_THREADS) index_finish_kernel(const float*
         // direct ranking: member i is kept when fewer than `room` members beat it (a higher key, or the same key earlier in the list)
         const uint32_t room = uint32_t(min(size_t(band), k - certain)), floor = top_k_key(-INFINITY);
         if (band & 1u) { if (t == 0) band_order[band] = 0; __syncthreads(); }        // (pairs are read: an odd band gets a member that beats nobody)
-        if (t < band) {
-            const uint64_t mine = band_order[t];
-            uint32_t beaten_by = 0;
+        // (a short band is shared out over more threads: 2, 4 or 8 of them count a member's betters, each its share of the pairs)
+        const uint32_t parts = band <= 128 ? 8u : band <= 256 ? 4u : band <= 512 ? 2u : 1u;
+        const uint32_t member = t / parts, part = t % parts;
+        uint64_t mine = 0;
+        uint32_t beaten_by = 0;
+        if (member < band) {
+            mine = band_order[member];
             const ulonglong2* pairs = reinterpret_cast<const ulonglong2*>(band_order);
-            #pragma unroll 8
-            for (uint32_t j = 0; j < (band + 1) / 2; ++j) { const ulonglong2 two = pairs[j]; beaten_by += (two.x > mine) + (two.y > mine); }
-            if (uint32_t(mine >> 32) <= floor || beaten_by >= room) held_list[0xffffffffu - uint32_t(mine)] = -1;      // not kept: a score of -inf never is
+            #pragma unroll 4
+            for (uint32_t j = part; j < (band + 1) / 2; j += parts) { const ulonglong2 two = pairs[j]; beaten_by += (two.x > mine) + (two.y > mine); }
         }
+        for (uint32_t offset = 1; offset < parts; offset *= 2) beaten_by += __shfl_xor(beaten_by, int(offset));
+        if (member < band && part == 0 && (uint32_t(mine >> 32) <= floor || beaten_by >= room))
+            held_list[0xffffffffu - uint32_t(mine)] = -1;                          // not kept: a score of -inf never is
         __syncthreads();
         // ordered compaction of what is kept
         uint32_t slot = 0;
