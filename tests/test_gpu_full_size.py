@@ -113,3 +113,24 @@ def test_config4_sparse_path_full_size(gpu, oracle):
     want_out = oracle.latent_attention(aq, None, None, 0, lat, exact[b:b + 1], None, work.vdim, work.scale)
     close_enough(out, want_out[0], "gather attention")
     work.release()
+
+
+def test_indexer_rows_longer_than_a_million_groups(gpu):
+    # more segments a row than the finishing workgroup has threads (1024 segments of 1024 groups): its counts, lists and top-k go
+    # the general way through global memory.  At this length the check is the size-independent one: the matrix-core path picks
+    # the indices of the all-canonical path (whose scores the oracle pins at the smaller sizes), bit for bit.
+    batch, groups, heads, dim, k = 2, 1_200_000, 16, 128, 2048
+    q, keys, weights = gpu.buffer(batch * heads * dim * 2), gpu.buffer(batch * groups * dim * 2), gpu.buffer(batch * heads * 4)
+    gpu.fill_normal(q.base(), batch * heads * dim, 31, 2)
+    gpu.fill_normal(keys.base(), batch * groups * dim, 32, 2)
+    gpu.fill_uniform(weights.base(), batch * heads, 33)
+    visible = gpu.upload(np.array([groups, groups - 12345], dtype=np.int32))
+    scores, exact, fast = gpu.buffer(batch * groups * 4), gpu.buffer(batch * k * 4), gpu.buffer(batch * k * 4)
+    gpu.index_top_k(q.base(), keys.base(), weights.base(), visible.base(), batch, groups, heads, dim, 0.25, scores.base(), k, exact.base())
+    gpu.index_top_k(q.base(), keys.base(), weights.base(), visible.base(), batch, groups, heads, dim, 0.25, None, k, fast.base())
+    want = gpu.read_buffer(exact, 0, np.int32, batch * k).reshape(batch, k)
+    got = gpu.read_buffer(fast, 0, np.int32, batch * k).reshape(batch, k)
+    assert np.array_equal(got, want)
+    assert np.all(np.diff(want, axis=1) > 0) and want.min() >= 0 and want[1].max() < groups - 12345
+    for b in (q, keys, weights, visible, scores, exact, fast):
+        gpu.release(b)
