@@ -8,8 +8,10 @@
 //     half of the value columns (the two waves of a head tile form the same scores and weights, each for itself: the partial
 //     results, and not the products, are what this kernel's time goes into, and 32 heads a workgroup let a chunk be twice as
 //     long, and the partial results half as many, with the same number of workgroups);
-//   * 32 rows at a time are gathered (16-byte pieces, every row whole) into a padded K tile in LDS and from there
-//     transposed into a V tile, both read without bank conflicts as MFMA operands by all four waves;
+//   * 32 rows at a time are gathered (16-byte pieces, every row whole) into a padded tile in LDS, two tiles in turn, read
+//     without bank conflicts as MFMA operands by all four waves: as rows for the scores, and for the values a lane takes
+//     eight neighbouring columns of its eight rows (16 bytes each) and sorts them into eight operands with v_perm -- which
+//     value column a lane's place in an operand stands for is free to choose, so nothing is transposed through LDS;
 //   * S^T = K . Q^T (rows x heads) leaves the weights in the B-operand layout of O^T += V^T . P^T, so they never move
 //     between lanes (the layout notes of paged_rows.hpp apply);
 //   * the chunks' (maximum, sum, unnormalised output) are merged by a second kernel.
@@ -30,7 +32,7 @@ struct GatherArgs {
     const int32_t* selected;        // [batch][k], entries outside 0..groups-1 are skipped
     unsigned groups, k, heads, chunks, chunk_rows;
     float scale_log2;
-    float* partial;                 // [batch][chunk][heads][vdim + 2]
+    float* partial;                 // [batch][chunk][heads][vdim], then [batch][chunk][heads] (maximum, sum)
     float* out;                     // [batch][heads][vdim]
 };
 
@@ -42,17 +44,16 @@ __device__ __forceinline__ uint32_t bf16_pair(float low, float high) {
 
 template<int KDIM, int VDIM>
 __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
-    constexpr int KSTEPS = KDIM / 32, TILES = VDIM / 16, KP = 2 * KDIM + 16, VP = 2 * STEP + 8, PIECES = KDIM / 8;
+    constexpr int KSTEPS = KDIM / 32, TILES = VDIM / 16, KP = 2 * KDIM + 16, PIECES = KDIM / 8;
     const int chunk = blockIdx.x, batch = blockIdx.z, thread = threadIdx.x;
     const int lane = thread & 63, wave = __builtin_amdgcn_readfirstlane(thread >> 6), li = lane & 15, g = lane >> 4;
     const int tile_of_heads = wave & 1, half = wave >> 1;                                  // the wave's 16 heads and its half of the columns
     const int head = int(blockIdx.y) * BLOCK_HEADS + tile_of_heads * 16 + li;
     const bool real = head < int(a.heads);
     extern __shared__ uint8_t lds[];
-    uint8_t* ktile = lds;                                     // [32 rows][KP]
-    uint8_t* vtile = ktile + STEP * KP;                       // [VDIM columns][VP]
-    uint32_t* seen = reinterpret_cast<uint32_t*>(vtile + VDIM * VP);   // [32]: 1 where the step's row exists
-    int32_t* chosen = reinterpret_cast<int32_t*>(seen + STEP);         // [CHUNK_MAX]: the workgroup's selected rows, -1 where there is none
+    uint8_t* tiles = lds;                                     // two of [32 rows][KP]
+    uint32_t* seen = reinterpret_cast<uint32_t*>(tiles + 2 * STEP * KP);   // two of [32]: 1 where the step's row exists
+    int32_t* chosen = reinterpret_cast<int32_t*>(seen + 2 * STEP);         // [CHUNK_MAX]: the workgroup's selected rows, -1 where there is none
     const int first = chunk * int(a.chunk_rows), last = min(int(a.k), first + int(a.chunk_rows));
     // the selection is read once, ahead of everything else: a step's rows then wait for one load, not for two in a row
     if (thread < CHUNK_MAX) chosen[thread] = first + thread < last ? a.selected[size_t(batch) * a.k + first + thread] : -1;
@@ -94,33 +95,19 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
         }
     };
     if (first < last) fetch(first);
-    for (int key0 = first; key0 < last; key0 += STEP) {
-        __syncthreads();                                      // the tiles of the step before are done with
+    for (int key0 = first, turn = 0; key0 < last; key0 += STEP, turn ^= 1) {
+        // (the tile of the step before last is done with: every wave has passed the barrier of the step between)
+        uint8_t* ktile = tiles + turn * STEP * KP;
+        uint32_t* here = seen + turn * STEP;
         #pragma unroll
         for (int j = 0; j < MINE; ++j) {
             const int piece = thread + 256 * j, row = piece / PIECES, part = piece % PIECES;
             if (piece < STEP * PIECES) {
                 *reinterpret_cast<uint4*>(ktile + row * KP + 16 * part) = fetched[j];
-                if (part == 0) seen[row] = (present >> j) & 1u;
+                if (part == 0) here[row] = (present >> j) & 1u;
             }
         }
         if (key0 + STEP < last) fetch(key0 + STEP);
-        __syncthreads();
-        // V tile: 4 rows x 4 columns at a time, transposed
-        for (int block = thread; block < (STEP / 4) * (VDIM / 4); block += 256) {
-            const int rows4 = block % (STEP / 4), cols4 = block / (STEP / 4);
-            uint2 words[4];
-            #pragma unroll
-            for (int e = 0; e < 4; ++e) words[e] = *reinterpret_cast<const uint2*>(ktile + (4 * rows4 + e) * KP + 8 * cols4);
-            #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
-                uint2 packed;
-                packed.x = byte_perm(c < 2 ? words[1].x : words[1].y, c < 2 ? words[0].x : words[0].y, sel);
-                packed.y = byte_perm(c < 2 ? words[3].x : words[3].y, c < 2 ? words[2].x : words[2].y, sel);
-                *reinterpret_cast<uint2*>(vtile + (4 * cols4 + c) * VP + 8 * rows4) = packed;
-            }
-        }
         __syncthreads();
         // S^T tiles: rows of the step (4 per lane group) x heads (lane li)
         floatx4 s[2] = {floatx4{0.0f, 0.0f, 0.0f, 0.0f}, floatx4{0.0f, 0.0f, 0.0f, 0.0f}};
@@ -134,7 +121,7 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
         float top = NEG_BIG;
         #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const uint4 flags = *reinterpret_cast<const uint4*>(seen + 16 * t + 4 * g);
+            const uint4 flags = *reinterpret_cast<const uint4*>(here + 16 * t + 4 * g);
             const uint32_t flag[4] = {flags.x, flags.y, flags.z, flags.w};
             #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -171,22 +158,56 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
         const uint4 high = {bf16_pair(w[0], w[1]), bf16_pair(w[2], w[3]), bf16_pair(w[4], w[5]), bf16_pair(w[6], w[7])};
         const uint4 low = {bf16_pair(rest[0], rest[1]), bf16_pair(rest[2], rest[3]), bf16_pair(rest[4], rest[5]), bf16_pair(rest[6], rest[7])};
         const bf16x8 pb = __builtin_bit_cast(bf16x8, high), pl = __builtin_bit_cast(bf16x8, low);
-        // O^T tiles: columns (16 jj + 4 g + r) x heads, the wave's half of them
+        // O^T tiles, the wave's half of them.  The lane's place li in an A operand stands for value column
+        // 128 (2 half + q) + 8 li + c in tile 8 q + c: its eight k-slots are that column of the lane's rows {4g..4g+3, 16+4g..}, and
+        // one 16-byte read a row brings the eight columns c = 0..7 at once.
         #pragma unroll
-        for (int j = 0; j < MY_TILES; ++j) {
-            const uint8_t* from = vtile + (16 * (half * MY_TILES + j) + li) * VP + 8 * g;
-            const uint2 near = *reinterpret_cast<const uint2*>(from), far = *reinterpret_cast<const uint2*>(from + 32);
-            const uint4 both = {near.x, near.y, far.x, far.y};
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pb, acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pl, acc[j], 0, 0, 0);
+        for (int q = 0; q < MY_TILES / 8; ++q) {
+            uint4 rows8[8];
+            #pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int row = 4 * g + (e < 4 ? e : 12 + e);
+                rows8[e] = *reinterpret_cast<const uint4*>(ktile + row * KP + 2 * (128 * (2 * half + q) + 8 * li));
+            }
+            #pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+                uint32_t words[4];
+                #pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const uint4 &low = rows8[2 * w], &high = rows8[2 * w + 1];
+                    const uint32_t lo = c / 2 == 0 ? low.x : c / 2 == 1 ? low.y : c / 2 == 2 ? low.z : low.w;
+                    const uint32_t hi = c / 2 == 0 ? high.x : c / 2 == 1 ? high.y : c / 2 == 2 ? high.z : high.w;
+                    words[w] = byte_perm(hi, lo, sel);
+                }
+                const bf16x8 va = __builtin_bit_cast(bf16x8, uint4{words[0], words[1], words[2], words[3]});
+                acc[8 * q + c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb, acc[8 * q + c], 0, 0, 0);
+                acc[8 * q + c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pl, acc[8 * q + c], 0, 0, 0);
+            }
         }
     }
     l = row_sum(l);
-    if (!real) return;
-    float* to = a.partial + ((size_t(batch) * a.chunks + chunk) * a.heads + head) * (VDIM + 2);
+    // The partial results leave through LDS: an accumulator's four values are columns 8 apart (rows 4g + r of the tile are the
+    // places li = 4g + r of the A operand), and a store should be a stretch of one head's row.  A wave uses a stretch of LDS of
+    // its own, written and read back by itself; the barrier is for the tiles that the stretches lie over.
+    constexpr int MY_COLUMNS = VDIM / 2, ROW_WORDS = MY_COLUMNS + 4;
+    static_assert(MY_COLUMNS == 4 * 64 && MY_TILES == 16, "a lane stores 16 bytes of a head's half row");
+    __syncthreads();
+    float* mine = reinterpret_cast<float*>(lds) + wave * 16 * ROW_WORDS;
     #pragma unroll
-    for (int j = 0; j < MY_TILES; ++j) *reinterpret_cast<floatx4*>(to + 16 * (half * MY_TILES + j) + 4 * g) = acc[j];
-    if (g == 0 && half == 0) { to[VDIM] = m; to[VDIM + 1] = l; }
+    for (int j = 0; j < MY_TILES; ++j)
+        #pragma unroll
+        for (int r = 0; r < 4; ++r) mine[li * ROW_WORDS + 128 * (j / 8) + 8 * (4 * g + r) + j % 8] = acc[j][r];
+    const size_t item = (size_t(batch) * a.chunks + chunk) * a.heads;
+    const int head0 = int(blockIdx.y) * BLOCK_HEADS + tile_of_heads * 16;
+    #pragma unroll 4
+    for (int h = 0; h < 16; ++h)
+        if (head0 + h < int(a.heads))
+            *reinterpret_cast<floatx4*>(a.partial + (item + head0 + h) * VDIM + half * MY_COLUMNS + 4 * lane) = *reinterpret_cast<const floatx4*>(mine + h * ROW_WORDS + 4 * lane);
+    if (real && g == 0 && half == 0) {
+        float* stats = a.partial + size_t(gridDim.z) * a.chunks * a.heads * VDIM + (item + head) * 2;
+        stats[0] = m; stats[1] = l;
+    }
 }
 
 // One block per (sequence, head): the chunks merged under their common maximum and normalised; a head none of whose
@@ -194,14 +215,15 @@ __global__ void __launch_bounds__(256) latent_gather_kernel(GatherArgs a) {
 template<int VDIM>
 __global__ void __launch_bounds__(VDIM / 4) latent_merge_kernel(GatherArgs a) {
     const size_t item = blockIdx.x, batch = item / a.heads, head = item % a.heads;
-    const float* base = a.partial + (batch * a.chunks * a.heads + head) * (VDIM + 2);
-    const size_t step = size_t(a.heads) * (VDIM + 2);
+    const float* base = a.partial + (batch * a.chunks * a.heads + head) * VDIM;
+    const float* stats = a.partial + size_t(gridDim.x) * a.chunks * VDIM + (batch * a.chunks * a.heads + head) * 2;      // (behind all the values)
+    const size_t step = size_t(a.heads) * VDIM, stats_step = size_t(a.heads) * 2;
     constexpr unsigned AT_ONCE = 8;
     float top = NEG_BIG;
     for (unsigned c0 = 0; c0 < a.chunks; c0 += AT_ONCE) {
         float tops[AT_ONCE];
         #pragma unroll
-        for (unsigned i = 0; i < AT_ONCE; ++i) tops[i] = base[min(c0 + i, a.chunks - 1) * step + VDIM];
+        for (unsigned i = 0; i < AT_ONCE; ++i) tops[i] = stats[min(c0 + i, a.chunks - 1) * stats_step];
         #pragma unroll
         for (unsigned i = 0; i < AT_ONCE; ++i) top = fmaxf(top, tops[i]);
     }
@@ -212,10 +234,10 @@ __global__ void __launch_bounds__(VDIM / 4) latent_merge_kernel(GatherArgs a) {
         float tops[AT_ONCE], sums[AT_ONCE];
         #pragma unroll
         for (unsigned i = 0; i < AT_ONCE; ++i) {
-            const size_t at = min(c0 + i, a.chunks - 1) * step;
-            values[i] = *reinterpret_cast<const floatx4*>(base + at + 4 * threadIdx.x);
-            tops[i] = base[at + VDIM];
-            sums[i] = base[at + VDIM + 1];
+            const size_t chunk = min(c0 + i, a.chunks - 1);
+            values[i] = *reinterpret_cast<const floatx4*>(base + chunk * step + 4 * threadIdx.x);
+            tops[i] = stats[chunk * stats_step];
+            sums[i] = stats[chunk * stats_step + 1];
         }
         #pragma unroll
         for (unsigned i = 0; i < AT_ONCE; ++i) {
@@ -250,7 +272,7 @@ void latent_gather(Device& d, const void* q, const void* latents, const int32_t*
     args.chunk_rows = batch * ((k + CHUNK_MAX - 1) / CHUNK_MAX) * head_parts >= uint64_t(d.compute_units) ? CHUNK_MAX : CHUNK;
     args.chunks = unsigned((k + args.chunk_rows - 1) / args.chunk_rows);
     args.scale_log2 = scale * 1.44269504088896341f; args.partial = partial; args.out = out;
-    constexpr size_t shared = size_t(STEP) * (2 * KDIM + 16) + size_t(VDIM) * (2 * STEP + 8) + STEP * 4 + CHUNK_MAX * 4;
+    constexpr size_t shared = 2 * size_t(STEP) * (2 * KDIM + 16) + 2 * STEP * 4 + CHUNK_MAX * 4;
     raise_shared_limit(d, reinterpret_cast<const void*>(&latent_gather_kernel<KDIM, VDIM>), shared);
     timed_launch(d, &latent_gather_kernel<KDIM, VDIM>, dim3(args.chunks, unsigned(head_parts), unsigned(batch)), dim3(256), shared, args);
     SD_CHECK(hipGetLastError());
