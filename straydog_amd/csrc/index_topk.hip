@@ -503,14 +503,24 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
     __builtin_amdgcn_s_waitcnt(0x0f70);
     // Two tiles a turn, so that one's matrix products run under the other's arithmetic: the pair's operands are read from their
     // stages, the stages take the copies of the pair two turns on, and both tiles are worked out side by side.
-    const auto finish = [&](size_t tile, float total, const floatx4& norms) {
-        const size_t group = tile + li;
-        total = quad_sum(total) * scale;
+    // A tile's 16 groups are finished by 16 lanes (lane group g = li / 4 holds group li's squared norm on the diagonal of
+    // K . K^T); the pair's second tile goes to the lanes 32 further on, so one pass of this arithmetic, and one pair of
+    // stores, serves both tiles.
+    const auto finish = [&](size_t tile0, size_t tile1, bool second, float total0, float total1, const floatx4& norms0, const floatx4& norms1) {
+        total0 = quad_sum(total0) * scale;
+        total1 = quad_sum(total1) * scale;
         // the diagonal of K . K^T: row 4g + r = column li
         const int r = li & 3;
-        const float square = r == 0 ? norms[0] : r == 1 ? norms[1] : r == 2 ? norms[2] : norms[3];
-        if (g == (li >> 2) && group < groups) {
-            const float e = bound * rough_sqrt(square);
+        const float square0 = r == 0 ? norms0[0] : r == 1 ? norms0[1] : r == 2 ? norms0[2] : norms0[3];
+        const float square1 = r == 0 ? norms1[0] : r == 1 ? norms1[1] : r == 2 ? norms1[2] : norms1[3];
+        float low_half = square1, high_half = square1;        // after the swap: the lower lanes' value in both halves / the upper lanes'
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(low_half), "+v"(high_half));
+        const float across = lane < 32 ? high_half : low_half;      // square1 of the lane 32 away
+        const bool own = g == (li >> 2), other = g == ((li >> 2) ^ 2);
+        const size_t group = (own ? tile0 : tile1) + li;
+        if ((own || (other && second)) && group < groups) {
+            const float total = own ? total0 : total1;
+            const float e = bound * rough_sqrt(own ? square0 : across);
             const bool live = group < limit;
             const float low = live ? total - e : -INFINITY, high = live ? total + e : -INFINITY;
             lower[row * groups + group] = low;
@@ -522,12 +532,12 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
     };
     for (int turn = 0, buffer = 0; turn < count; turn += 2, buffer ^= 2) {
         // The pair has landed when only what was issued after its second copy is outstanding: the bounds of the two pairs before
-        // (two stores a tile, issued between the copies; memory operations finish in the order issued) and the copies of the
+        // (two stores a pair, issued between the copies; memory operations finish in the order issued) and the copies of the
         // pair after this one, four loads a tile.  (The first two pairs had landed before the loop.)
         const int after = count - 1 - turn;                        // tiles after the pair's first
         const bool second = after >= 1;
-        if (after >= 3) __builtin_amdgcn_s_waitcnt(0x4f70); else if (after == 2) __builtin_amdgcn_s_waitcnt(0x0f7c);       // 16, 12
-        else __builtin_amdgcn_s_waitcnt(0x0f78);                                                                           // 8
+        if (after >= 3) __builtin_amdgcn_s_waitcnt(0x0f7c); else if (after == 2) __builtin_amdgcn_s_waitcnt(0x0f78);       // 12, 8
+        else __builtin_amdgcn_s_waitcnt(0x0f74);                                                                           // 4
         bf16x8 kb[2][KS];
         #pragma unroll
         for (int u = 0; u < 2; ++u) {
@@ -554,8 +564,7 @@ __global__ void __launch_bounds__(BRACKET_WAVES * 64) index_interval_kernel(cons
                 for (int r = 0; r < 4; ++r) total[u] = fmaf(positive_part(dots[r]), w[t][r], total[u]);
             }
         }
-        finish(tile_at(turn), total[0], norms[0]);
-        if (second) finish(tile_at(turn + 1), total[1], norms[1]);
+        finish(tile_at(turn), tile_at(turn + 1), second, total[0], total[1], norms[0], norms[1]);
     }
     if (!histogram) return;
     #pragma unroll
