@@ -20,6 +20,12 @@ def _read(gpu, buffer, dtype, count):
     return gpu.read_buffer(buffer, 0, dtype, count)
 
 
+def _bf16_pair(oracle, values):
+    """(BF16 bit patterns, the FP32 values they stand for)."""
+    bits = oracle.to_bf16(values)
+    return bits, (bits.astype(np.uint32) << 16).view(np.float32).reshape(values.shape)
+
+
 def test_graph_bookkeeping(gpu):
     from straydog_amd.backend import StraydogError
     assert not gpu.graph_run(12345), "no graph is stored under that key"
@@ -195,4 +201,51 @@ def test_graphs_are_dropped_when_the_workspace_moves(gpu, oracle):
     assert gpu.graph_run(21)
     assert np.array_equal(_read(gpu, small_out, np.float32, 64 * 512), eager)
     for b in small_buffers + large_buffers:
+        gpu.release(b)
+
+
+def test_batched_sparse_step_recorded(gpu, oracle):
+    # the batched sparse path -- matrix-core indexer with its histograms, top-k, gather attention over the selection -- recorded
+    # once and replayed with other queries and other visible lengths: the histograms one replay leaves must be what the next one
+    # expects, and every replay picks the indices and gives the outputs of the same work run eagerly
+    rng = np.random.default_rng(41)
+    batch, groups, iheads, idim, k, heads, kdim, vdim = 4, 9000, 64, 128, 512, 32, 576, 512
+    key_bits, key_vals = _bf16_pair(oracle, rng.standard_normal((batch, groups, idim)).astype(np.float32))
+    lat_bits, _ = _bf16_pair(oracle, rng.standard_normal((batch, groups, kdim)).astype(np.float32))
+    kb, lb = gpu.upload(key_bits), gpu.upload(lat_bits)
+    qb, wb, vb = gpu.buffer(batch * iheads * idim * 2), gpu.buffer(batch * iheads * 4), gpu.buffer(batch * 4)
+    ab, indices, out = gpu.buffer(batch * heads * kdim * 2), gpu.buffer(batch * k * 4), gpu.buffer(batch * heads * vdim * 4)
+    scale = float(1.0 / np.sqrt(kdim))
+
+    def load(turn):
+        q_bits, q_vals = _bf16_pair(oracle, rng.standard_normal((batch, iheads, idim)).astype(np.float32))
+        a_bits, a_vals = _bf16_pair(oracle, rng.standard_normal((batch, heads, kdim)).astype(np.float32))
+        weights = rng.random((batch, iheads)).astype(np.float32)
+        visible = np.array([groups, groups - 1000 * turn, 300 + turn, max(1, groups // (turn + 1))], dtype=np.int32)   # (row 2: fewer than k)
+        for b, a in ((qb, q_bits), (wb, weights), (vb, visible), (ab, a_bits)):
+            gpu.write_buffer(b, 0, a)
+        return q_vals, a_vals, weights, visible
+
+    def step():
+        gpu.index_top_k(qb.base(), kb.base(), wb.base(), vb.base(), batch, groups, iheads, idim, 0.5, None, k, indices.base())
+        gpu.latent_attention(ab.base(), lb.base(), indices.base(), batch, groups, k, heads, kdim, vdim, scale, out.base())
+    load(0)
+    step()                                  # once eagerly: whatever a first call sets up is set up outside the recording
+    gpu.graph_begin()
+    step()
+    gpu.graph_end(11)
+    for turn in range(4):
+        q_vals, a_vals, weights, visible = load(turn)
+        assert gpu.graph_run(11)
+        got_indices = _read(gpu, indices, np.int32, batch * k).reshape(batch, k)
+        got = _read(gpu, out, np.float32, batch * heads * vdim).reshape(batch, heads, vdim)
+        for b in range(batch):
+            scores = oracle.index_scores(q_vals[b:b + 1], key_vals[b], weights[b:b + 1], visible[b:b + 1], 0.5)
+            assert np.array_equal(got_indices[b], oracle.top_k(scores, k)[0]), f"replay {turn}, sequence {b}"
+            want = oracle.latent_attention(a_vals[b:b + 1], None, None, 0, lat_bits[b], got_indices[b:b + 1], None, vdim, scale)
+            close_enough(got[b], want[0], f"replay {turn}, sequence {b}")
+        if turn == 1:
+            step()                          # eager work between replays, through the same histograms and workspace
+            gpu.synchronize()
+    for b in (kb, lb, qb, wb, vb, ab, indices, out):
         gpu.release(b)
