@@ -1215,7 +1215,8 @@ int sdx_index_top_k(void* handle, const void* q_index, const void* keys, const f
     op_span(value, weights, checked_floats({batch, heads}), "index weights");
     op_span(value, visible, checked_floats({batch}), "visible counts");
     op_span(value, indices, checked_floats({batch, k}), "top-k indices");
-    if (!scores && index_fast_supported(heads, dim)) {
+    const bool whole_pieces = (uintptr_t(q_index) | uintptr_t(keys)) % 16 == 0;        // the matrix-core path reads 16 bytes at a time
+    if (!scores && index_fast_supported(heads, dim) && whole_pieces) {
         // the matrix cores bracket the scores; the canonical arithmetic runs on the few groups near the k-th only
         const FastIndexSpace space = fast_index_space(workspace(value, fast_index_bytes(batch, groups)), batch, groups);
         switch (heads) {
@@ -1244,6 +1245,7 @@ int sdx_index_score_bounds(void* handle, const void* q_index, const void* keys, 
     SD_OP_BEGIN
     if (!batch || batch > 65535 || !groups || groups > (uint64_t(1) << 31) || !index_fast_supported(heads, dim))
         throw std::runtime_error("invalid Straydog index shape");
+    if ((uintptr_t(q_index) | uintptr_t(keys)) % 16) throw std::runtime_error("Straydog index queries and keys must lie on 16-byte boundaries here");
     op_span(value, q_index, checked_product({batch, heads, dim, 2}), "index queries");
     op_span(value, keys, checked_product({batch, groups, dim, 2}), "index keys");
     op_span(value, weights, checked_floats({batch, heads}), "index weights");

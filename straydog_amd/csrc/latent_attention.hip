@@ -336,7 +336,8 @@ int sdx_latent_attention(void* handle, const void* q, const void* latents, const
     op_span(value, latents, checked_product({batch, groups, kdim, 2}), "latent rows");
     op_span(value, selected, checked_floats({batch, k}), "selected rows");
     op_span(value, out, checked_floats({batch, heads, vdim}), "an attention output");
-    if (latent_gather_supported(kdim, vdim) && groups * kdim * 2 < (uint64_t(1) << 32) && k < (uint64_t(1) << 31)) {      // (a sequence's rows within 32-bit offsets)
+    const bool whole_pieces = (uintptr_t(q) | uintptr_t(latents) | uintptr_t(out)) % 16 == 0;       // the matrix-core kernels move 16 bytes at a time
+    if (latent_gather_supported(kdim, vdim) && whole_pieces && groups * kdim * 2 < (uint64_t(1) << 32) && k < (uint64_t(1) << 31)) {      // (a sequence's rows within 32-bit offsets)
         // the matrix-core path; its chunk partials live in the device's workspace (grown outside graph capture)
         float* partial = static_cast<float*>(workspace(value, latent_gather_scratch(batch, k, heads, vdim)));
         latent_gather(value, q, latents, selected, batch, groups, k, heads, scale, out, partial);

@@ -570,3 +570,35 @@ def test_device_normal_values_are_the_xorshift_box_muller_stream(gpu, oracle):
     assert np.array_equal(_read(gpu, out, np.float32, 5000), oracle.fill_uniform(11, 5000, -0.5, 1.5))
     gpu.release(out)
 
+
+
+def test_sparse_path_operands_off_16_byte_boundaries(gpu, oracle):
+    # queries and keys that start 2 bytes off a 16-byte boundary: the matrix-core kernels read whole 16-byte pieces, so such
+    # operands take the general kernels -- the same indices and outputs
+    rng = np.random.default_rng(91)
+    batch, groups, heads, dim, k = 2, 3000, 64, 128, 256
+    q_bits, q_vals = _bf16_round(oracle, rng.standard_normal((batch, heads, dim)).astype(np.float32))
+    key_bits, key_vals = _bf16_round(oracle, rng.standard_normal((batch, groups, dim)).astype(np.float32))
+    weights = rng.random((batch, heads)).astype(np.float32)
+    visible = np.array([groups, groups - 9], dtype=np.int32)
+    qb, kb = gpu.buffer(q_bits.size * 2 + 16), gpu.buffer(key_bits.size * 2 + 16)
+    gpu.write_buffer(qb, 2, q_bits); gpu.write_buffer(kb, 2, key_bits)
+    wb, vb, indices = gpu.upload(weights), gpu.upload(visible), gpu.buffer(batch * k * 4)
+    gpu.index_top_k(qb.at(2), kb.at(2), wb.base(), vb.base(), batch, groups, heads, dim, 1.0, None, k, indices.base())
+    got = _read(gpu, indices, np.int32, batch * k).reshape(batch, k)
+    for b in range(batch):
+        want = oracle.index_scores(q_vals[b:b + 1], key_vals[b], weights[b:b + 1], visible[b:b + 1], 1.0)
+        assert np.array_equal(got[b], oracle.top_k(want, k)[0])
+    kdim, vdim, aheads = 576, 512, 32
+    a_bits, a_vals = _bf16_round(oracle, rng.standard_normal((batch, aheads, kdim)).astype(np.float32))
+    lat_bits, _ = _bf16_round(oracle, rng.standard_normal((batch, groups, kdim)).astype(np.float32))
+    ab, lb, out = gpu.upload(a_bits), gpu.buffer(lat_bits.size * 2 + 16), gpu.buffer(batch * aheads * vdim * 4)
+    gpu.write_buffer(lb, 2, lat_bits)
+    scale = float(1.0 / np.sqrt(kdim))
+    gpu.latent_attention(ab.base(), lb.at(2), indices.base(), batch, groups, k, aheads, kdim, vdim, scale, out.base())
+    result = _read(gpu, out, np.float32, batch * aheads * vdim).reshape(batch, aheads, vdim)
+    for b in range(batch):
+        want = oracle.latent_attention(a_vals[b:b + 1], None, None, 0, lat_bits[b], got[b:b + 1], None, vdim, scale)
+        close_enough(result[b], want[0], f"sequence {b}")
+    for b in (qb, kb, wb, vb, indices, ab, lb, out):
+        gpu.release(b)
