@@ -8,7 +8,7 @@ shuffled page table, FP16 queries and outputs.  The one JSON line also carries, 
 of the same shape (the north-star target), config 0, the chunked prefill of config 2 (MFMA-bound: TFLOP/s against the
 dense FP16 peak), the verify span of config 3 and the sparse path of config 4.
 
-    python bench.py --gpus 1 --steps 50 --warmup 10 [--workload config1|config1_32k|config0|config2|config3|config4]
+    python bench.py --gpus 1 --steps 100 --warmup 200 [--workload config1|config1_32k|config0|config2|config3|config4]
 """
 import argparse
 import json
@@ -145,8 +145,10 @@ def cpu_baseline_paged(work, sample_seqs, threads, budget_seconds=12.0):
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=50)
-    parser.add_argument("--warmup", type=int, default=10)
+    # (the defaults: 200 untimed steps are ~25 ms of the same load -- the memory and fabric clocks of the box take tens of
+    # milliseconds of sustained traffic to settle, and a pass timed after 10 steps reads 1.5-4 % low)
+    parser.add_argument("--steps", type=int, default=100)
+    parser.add_argument("--warmup", type=int, default=200)
     parser.add_argument("--workload", default="config1")
     parser.add_argument("--no-also", action="store_true", help="measure only the named workload")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")

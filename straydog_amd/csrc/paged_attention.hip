@@ -130,32 +130,6 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
     const table_ptr table = (table_ptr)(args.page_table + size_t(seq) * args.table_stride);
     const size_t plane_bytes = size_t(args.page_tokens) * ROW;
 
-    // Query rows of this K/V head: row = span_row * group + head_in_group; a lane holds row qt*16 + li as B operands.
-    // A row past the last real one holds zeros (its scores are never stored).
-    half8 qf[QT][BLOCKS];
-    int limit[QT];
-    #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-        const int row = qt * 16 + li;
-        const bool real = row < int(args.rows);
-        const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
-        limit[qt] = real ? position + span_row : 0x7fffffff;
-        const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
-        #pragma unroll
-        for (int b = 0; b < BLOCKS; ++b) {
-            half8 value = {};
-            if (real) {
-                if (args.q_f16) value = *reinterpret_cast<const half8*>(static_cast<const _Float16*>(args.q) + at + 32 * b + 8 * g);
-                else {
-                    const float* from = static_cast<const float*>(args.q) + at + 32 * b + 8 * g;
-                    #pragma unroll
-                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)from[i];
-                }
-            }
-            qf[qt][b] = value;
-        }
-    }
-
     floatx4 acc[QT][TILES];
     float m[QT], l[QT];
     #pragma unroll
@@ -202,12 +176,42 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         in_page += STEP * WAVES;
         while (in_page >= int(args.page_tokens)) { in_page -= int(args.page_tokens); ++page_index; }
     };
+    // The first steps' copies are asked for first, then the queries: both are on their way together, and one wait for every
+    // load so far stands before the loop (the compiler's own wait for the queries would otherwise sit at their first use
+    // inside the loop and wait for the copies issued by then as well).
     settle_loads();
     #pragma unroll
     for (int ahead = 0; ahead < DEPTH; ++ahead) {
         if (token0 + ahead * STEP * WAVES < segment_end) copy_in(stages + ahead * (2 * SLAB), table[min(page_index, last_page)], in_page);
         advance();
     }
+    // Query rows of this K/V head: row = span_row * group + head_in_group; a lane holds row qt*16 + li as B operands.
+    // A row past the last real one holds zeros (its scores are never stored).
+    half8 qf[QT][BLOCKS];
+    int limit[QT];
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int row = qt * 16 + li;
+        const bool real = row < int(args.rows);
+        const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
+        limit[qt] = real ? position + span_row : 0x7fffffff;
+        const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
+        #pragma unroll
+        for (int b = 0; b < BLOCKS; ++b) {
+            half8 value = {};
+            if (real) {
+                if (args.q_f16) value = *reinterpret_cast<const half8*>(static_cast<const _Float16*>(args.q) + at + 32 * b + 8 * g);
+                else {
+                    const float* from = static_cast<const float*>(args.q) + at + 32 * b + 8 * g;
+                    #pragma unroll
+                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)from[i];
+                }
+            }
+            qf[qt][b] = value;
+        }
+    }
+
+    settle_loads();
     int page_ahead = table[min(page_index, last_page)];
     for (int buffer = 0; token0 < segment_end; token0 += STEP * WAVES, buffer = DEPTH == 2 ? buffer ^ 1 : 0) {
         uint8_t* const stage = stages + buffer * (2 * SLAB);
