@@ -177,6 +177,7 @@ def main():
         "config4": "configs[4]: batch 8, ctx 131072, 64x128 bf16 indexer, top-2048, 64 heads over bf16 latents 576/512",
     }
     copy_rate, read_rate = measured_ceilings(gpu)
+    short_warmup = max(args.warmup // 5, 2)       # for the workloads whose steps are long or many launches: the same settling, fewer steps
 
     def run_paged(name, with_cpu, budget_seconds=12.0, warmup=None):
         work = builders[name]()
@@ -218,8 +219,8 @@ def main():
 
     def run_sparse(with_cpu=True):
         work = workloads.SparseWorkload(gpu)
-        ms_index, bounds_ms = timed(gpu, work.step_index, max(args.steps // 5, 3), 2)
-        ms_attention, gather_ms = timed(gpu, work.step_attention, max(args.steps // 5, 3), 2)
+        ms_index, bounds_ms = timed(gpu, work.step_index, max(args.steps // 5, 3), short_warmup)
+        ms_attention, gather_ms = timed(gpu, work.step_attention, max(args.steps // 5, 3), short_warmup)
         size, keys = work.algorithmic_bytes(), work.batch * work.context * work.index_dim * 2
         sparse_baseline = cpu_baseline_sparse(work) if with_cpu and not args.no_cpu else None
         work.release()
@@ -259,7 +260,7 @@ def main():
     def run_prefill(with_cpu=True):
         work = workloads.PrefillWorkload(gpu)
         steps = max(args.steps // 5, 3)
-        ms, kernel_ms = timed(gpu, work.step, steps, 2)
+        ms, kernel_ms = timed(gpu, work.step, steps, short_warmup)
         flops, size = work.flops(), work.algorithmic_bytes()
         prefill_baseline = cpu_baseline_prefill(work) if with_cpu and not args.no_cpu else None
         work.release()
