@@ -183,6 +183,17 @@ def main():
         work = builders[name]()
         result = paged_result(gpu, work, args.steps, args.warmup if warmup is None else warmup)
         result["warmup"] = args.warmup if warmup is None else warmup
+        # what the same pool gives to the decode kernel's order of asking with the arithmetic left out (the pool holds a little
+        # more than the batch's rows: whole pages)
+        for _ in range(3):
+            gpu.paged_stream_probe(work.pool)
+        gpu.synchronize()
+        begin = gpu.event()
+        for _ in range(10):
+            read = gpu.paged_stream_probe(work.pool)
+        end = gpu.event()
+        result["paged_stream_probe_gbps"] = read / (gpu.elapsed_ms(begin, end) / 10) / 1e6
+        gpu.events_clear()
         baseline = None
         if with_cpu:
             threads = host_threads()[1]
@@ -371,7 +382,8 @@ def main():
     achieved = main_result["algorithmic_bytes"] / (kernel_us * 1e-6) / 1e9 if kernel_us else main_result["gbps"]
     roofline = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS,
                 "traffic": PROFILED_TRAFFIC[args.workload][0], "traffic_source": PROFILED_TRAFFIC[args.workload][1],
-                "kernel": "paged_attention_kernel<128,3,Q8_0>" if args.workload == "config3" else "paged_attention_kernel<128,1,Q8_0>", "kernel_us": kernel_us, "measured_copy_gbps": copy_rate, "measured_read_gbps": read_rate}
+                "kernel": "paged_attention_kernel<128,3,Q8_0>" if args.workload == "config3" else "paged_attention_kernel<128,1,Q8_0>", "kernel_us": kernel_us, "measured_copy_gbps": copy_rate, "measured_read_gbps": read_rate,
+                "measured_paged_stream_gbps": main_result.get("paged_stream_probe_gbps")}
     if args.workload == "config4" and kernel_us:
         # the dominant kernel reads every index key once: its algorithmic bytes are the keys
         achieved = main_result["key_bytes"] / (kernel_us * 1e-6) / 1e9

@@ -255,6 +255,11 @@ int sdx_copy(void* handle, void* target, const void* source, uint64_t bytes);
 int sdx_checkpoint_release(void* handle, void* buffer);
 /* Read-only streaming probe (16-byte loads, `unroll` per lane per trip, `blocks_per_cu` workgroups per compute unit). */
 int sdx_read_probe(void* handle, const void* source, uint64_t bytes, uint32_t blocks_per_cu, uint32_t unroll);
+/* The decode kernel's way through a pool with the arithmetic left out (no counterpart in the reference: a harness probe): every
+ * K and V plane of every page read once in the decode kernel's order -- a workgroup of four waves per K/V head of a run of pages,
+ * the waves taking alternate 32-token steps, a step's two slabs by 1 KiB global->LDS loads.  *bytes receives what the launch reads;
+ * time it with the events above: what the pool's layout and that order of asking give by themselves. */
+int sdx_paged_stream_probe(void* handle, const sdx_kv_pool* pool, uint64_t* bytes);
 /* Matrix-core probe: eight waves per compute unit, each `trips` x 32 independent v_mfma_f32_16x16x32_f16; *flops receives the
  * floating-point operations the launch performs (time it with the events above).  live = 0: tame constant operands, the
  * rate at the clock the box holds for them; live = 1: pseudo-random operands that change from product to product, as real

@@ -139,6 +139,7 @@ SIGNATURES = {
     "sdx_fill_uniform": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_float, c_float]),
     "sdx_copy": (c_int, [c_void_p, c_void_p, c_void_p, c_u64]),
     "sdx_read_probe": (c_int, [c_void_p, c_void_p, c_u64, c_u32, c_u32]),
+    "sdx_paged_stream_probe": (c_int, [c_void_p, _P(KvPool), _P(c_u64)]),
     "sdx_mfma_probe": (c_int, [c_void_p, c_u32, c_int, _P(ctypes.c_double)]),
 }
 

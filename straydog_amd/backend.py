@@ -426,5 +426,11 @@ class Backend:
     def read_probe(self, source, size, blocks_per_cu=8, unroll=4):
         self.check(self.lib.sdx_read_probe(self.handle, source, size, blocks_per_cu, unroll))
 
+    def paged_stream_probe(self, pool):
+        """Queues the loads-only walk of the pool in the decode kernel's order; returns the bytes it reads."""
+        size = abi.c_u64()
+        self.check(self.lib.sdx_paged_stream_probe(self.handle, ctypes.byref(pool), ctypes.byref(size)))
+        return size.value
+
     def copy(self, target, source, size):
         self.check(self.lib.sdx_copy(self.handle, target, source, size))

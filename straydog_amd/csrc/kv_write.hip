@@ -145,6 +145,38 @@ __global__ void __launch_bounds__(256) read_probe_kernel(const probe_u4* __restr
     if (fold == 0x9e3779b9u && sink) *sink = fold;
 }
 
+// The decode kernel's way through a pool, loads only: a workgroup of four waves takes one K/V head of a run of pages; on each
+// page its waves take alternate steps of 32 tokens, a step's K slab and V slab (32 rows of a plane each, contiguous) copied by
+// 1 KiB global->LDS loads into the wave's one stage, one word of the stage read back, then the next step.  What the pool's
+// layout and this order of asking are worth by themselves, with no arithmetic and no operand reads beside them.
+__global__ void __launch_bounds__(256) paged_stream_probe_kernel(const uint8_t* __restrict__ pages, unsigned page_count, unsigned page_tokens, unsigned kv_heads,
+                                                                 unsigned row_bytes, unsigned pages_per_group, uint32_t* sink) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t probe_stage[];
+    typedef __attribute__((address_space(3))) uint8_t* lds_bytes;
+    const unsigned lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const unsigned kvh = blockIdx.x % kv_heads, first_page = (blockIdx.x / kv_heads) * pages_per_group;
+    const unsigned slab = 32 * row_bytes, pieces = (slab + 1023) / 1024, steps_per_page = page_tokens / 32;
+    const size_t plane = size_t(page_tokens) * row_bytes;
+    const uint32_t mine = __builtin_amdgcn_readfirstlane(uint32_t(uintptr_t((lds_bytes)probe_stage))) + wave * 2 * slab;     // (a slab is whole 16-byte pieces)
+    uint32_t fold = 0;
+    for (unsigned page = first_page; page < min(first_page + pages_per_group, page_count); ++page)
+        for (unsigned step = wave; step < steps_per_page; step += 4) {
+            const uint8_t* k = pages + (size_t(page) * 2 * kv_heads + kvh) * plane + size_t(step) * slab + 16 * lane;
+            for (unsigned part = 0; part < 2; ++part) {
+                const uint8_t* from = k + (part ? size_t(kv_heads) * plane : 0);
+                for (unsigned j = 0; j < pieces; ++j)
+                    if (16 * lane + 1024 * j < slab) {
+                        const uint32_t to = mine + part * slab + j * 1024;
+                        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" :: "v"(from + 1024 * j), "s"(to) : "memory");
+                    }
+            }
+            uint32_t word;
+            asm volatile("s_waitcnt vmcnt(0)\n\tds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(word) : "v"(mine + lane * 4) : "memory");
+            fold ^= word;
+        }
+    if (fold == 0x9e3779b9u && sink) *sink = fold;
+}
+
 // Matrix-core probe: every wave keeps eight independent chains of v_mfma_f32_16x16x32_f16 going on operands it holds in
 // registers, two waves a SIMD, nothing else in the loop: the dense FP16 ceiling of the box at the clock it holds under
 // that load.  The clock depends on the operands: with LIVE ones (pseudo-random values, another pair of registers for every
@@ -245,6 +277,24 @@ int sdx_read_probe(void* handle, const void* source, uint64_t bytes, uint32_t bl
     if (unroll >= 8) read_probe_kernel<8><<<grid, 256, 0, value.stream>>>(static_cast<const probe_u4*>(source), size_t(bytes / 16), sink);
     else if (unroll >= 4) read_probe_kernel<4><<<grid, 256, 0, value.stream>>>(static_cast<const probe_u4*>(source), size_t(bytes / 16), sink);
     else read_probe_kernel<2><<<grid, 256, 0, value.stream>>>(static_cast<const probe_u4*>(source), size_t(bytes / 16), sink);
+    SD_OP_END
+}
+
+int sdx_paged_stream_probe(void* handle, const sdx_kv_pool* pool, uint64_t* bytes) {
+    SD_OP_BEGIN
+    validate_pool(value, pool);
+    if (pool->page_count > (uint64_t(1) << 31)) throw std::runtime_error("invalid Straydog read probe");
+    // as many workgroups as the decode kernel keeps resident (four a compute unit), each a K/V head of a run of pages
+    const unsigned groups = std::max(1u, value.compute_units * 4 / pool->kv_heads);
+    const unsigned pages_per_group = unsigned((pool->page_count + groups - 1) / groups);
+    const unsigned grid = unsigned((pool->page_count + pages_per_group - 1) / pages_per_group) * pool->kv_heads;
+    const size_t shared = size_t(4) * 2 * 32 * pool->row_bytes;
+    uint32_t* sink = static_cast<uint32_t*>(workspace(value, 256));
+    if (shared > 64 * 1024) raise_shared_limit(value, reinterpret_cast<const void*>(&paged_stream_probe_kernel), shared);
+    paged_stream_probe_kernel<<<grid, 256, shared, value.stream>>>(static_cast<const uint8_t*>(pool->pages), unsigned(pool->page_count), pool->page_tokens, pool->kv_heads,
+                                                                 pool->row_bytes, pages_per_group, sink);
+    SD_CHECK(hipGetLastError());
+    if (bytes) *bytes = pool->page_count * 2 * pool->kv_heads * pool->page_tokens * pool->row_bytes;
     SD_OP_END
 }
 

@@ -506,3 +506,18 @@ def test_table_entries_outside_the_pool_read_inside_it(gpu, oracle):
         close_enough(got[s], want[s], f"sequence {s}")
     for b in (buffer, tb, bb):
         gpu.release(b)
+
+
+@pytest.mark.parametrize("pages,page_tokens,kv_heads,dim,row_bytes", [(37, 64, 2, 128, 136), (5, 256, 4, 128, 136), (3, 32, 1, 256, 272), (9, 64, 3, 128, 256),
+                                                                      (4, 32, 2, 256, 512)])
+def test_paged_stream_probe_reads_the_whole_pool(gpu, pages, page_tokens, kv_heads, dim, row_bytes):
+    # the harness probe that walks a pool in the decode kernel's order: every layout the pools take, pools smaller than the
+    # launch has workgroups; it reports the pool's bytes and leaves the pool as it was
+    pool, buffer = gpu.kv_pool(pages, page_tokens, kv_heads, dim, row_bytes)
+    size = pages * 2 * kv_heads * page_tokens * row_bytes
+    before = np.random.default_rng(pages).integers(0, 256, size=size, dtype=np.uint8)
+    gpu.write_buffer(buffer, 0, before)
+    assert gpu.paged_stream_probe(pool) == size
+    gpu.synchronize()
+    assert np.array_equal(gpu.read_buffer(buffer, 0, np.uint8, size), before)
+    gpu.release(buffer)
