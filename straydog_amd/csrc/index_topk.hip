@@ -668,11 +668,12 @@ __global__ void __launch_bounds__(256) radix_histogram_kernel(const float* lower
 // With fewer than k live groups everything live is a certain candidate.
 //
 // The band members of the segment get their canonical score here as well, a wave a member (the workgroup's four waves take the
-// members in turn): a lane per head; the head's 128 query values come from LDS, where the row's queries were put on the way in
-// (a head every 272 bytes, so that sixteen lanes' 16-byte reads fall in different banks); a key row is 64 words, lane i
+// members in turn): a lane per head; a wave that has a member reads its head's 128 query values itself, two to a word (a lane
+// its own 256 bytes: a load spreads over 64 lines -- staged through LDS by coalesced loads in every workgroup, the same 16 KB a
+// row made a thousand workgroups ask for the same lines at the same moment and cost 13 us); a key row is 64 words, lane i
 // fetches word i (one coalesced load, the next member's row on its way while this one is used) and the words go round by
 // v_readlane, so a member costs a wave 64 broadcasts and 128 multiply-adds in the canonical column order.  Then the member's
-// terms are added in head order by one lane, read from LDS.  A score lands at its group's place in the list.
+// terms are added in head order, a broadcast and an addition a head.  A score lands at its group's place in the list.
 constexpr uint32_t CERTAIN = 0x80000000u;
 template<int HEADS>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4)))
@@ -703,7 +704,6 @@ candidate_segments_kernel(const float* lower, const float* upper, size_t groups,
     }
     __shared__ uint32_t wave_sums[4];
     __shared__ uint32_t band_members[INTERVAL_KEYS];              // place in the segment's list << 10 | group within the segment
-    __shared__ float terms[4][HEADS + 1];
     uint32_t entry[4], mine = 0, band = 0;
     #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -765,14 +765,13 @@ candidate_segments_kernel(const float* lower, const float* upper, size_t groups,
                 dot = __builtin_fmaf(__uint_as_float(pairs[i] & 0xffff0000u), __uint_as_float(pair & 0xffff0000u), dot);
             }
         }
-        if (lane < HEADS) terms[wave][lane] = rounded_product(fmaxf(dot, 0.0f), weight);
-        // the wave's own writes, read back by the wave: LDS keeps a wave's accesses in order
-        if (lane == 0) {
-            float sum = 0.0f;
-            #pragma unroll 4
-            for (int h = 0; h < HEADS; ++h) sum = rounded_sum(sum, terms[wave][h]);
-            scores[row * groups + size_t(blockIdx.x) * INTERVAL_KEYS + place] = rounded_product(sum, scale);
-        }
+        // the heads' terms added in head order: lane h holds head h's, every lane adds them all (a broadcast and an addition a
+        // head, nothing through LDS)
+        const float term = rounded_product(fmaxf(dot, 0.0f), weight);
+        float sum = 0.0f;
+        #pragma unroll
+        for (int h = 0; h < HEADS; ++h) sum = rounded_sum(sum, __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(term), h)));
+        if (lane == 0) scores[row * groups + size_t(blockIdx.x) * INTERVAL_KEYS + place] = rounded_product(sum, scale);
     }
 }
 
