@@ -751,18 +751,19 @@ candidate_segments_kernel(const float* lower, const float* upper, size_t groups,
             member = band_members[m + 4];
             words = segment_keys[size_t(member & 1023u) * (DIM / 2) + lane];
         }
+        // (the queries are widened again for every member -- 128 widened values held across the loop would cost a wave of
+        // occupancy -- which the shift and the mask being unknown to the compiler sees to)
+        uint32_t up = 16u, high_half = 0xffff0000u;
+        asm volatile("" : "+s"(up), "+s"(high_half));
         float dot = 0.0f;
         #pragma unroll
         for (int d = 0; d < DIM; d += 8) {
-            uint32_t pairs[4] = {query[d / 8].x, query[d / 8].y, query[d / 8].z, query[d / 8].w};
-            // (widened again for every member: 128 widened values held across the loop would cost a wave of occupancy)
-            #pragma unroll
-            for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(pairs[i]));
+            const uint32_t pairs[4] = {query[d / 8].x, query[d / 8].y, query[d / 8].z, query[d / 8].w};
             #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const uint32_t pair = __builtin_amdgcn_readlane(current, d / 2 + i);
-                dot = __builtin_fmaf(__uint_as_float(pairs[i] << 16), __uint_as_float(pair << 16), dot);
-                dot = __builtin_fmaf(__uint_as_float(pairs[i] & 0xffff0000u), __uint_as_float(pair & 0xffff0000u), dot);
+                dot = __builtin_fmaf(__uint_as_float(pairs[i] << up), __uint_as_float(pair << 16), dot);
+                dot = __builtin_fmaf(__uint_as_float(pairs[i] & high_half), __uint_as_float(pair & 0xffff0000u), dot);
             }
         }
         // the heads' terms added in head order: lane h holds head h's, every lane adds them all (a broadcast and an addition a
