@@ -682,7 +682,7 @@ candidate_segments_kernel(const float* lower, const float* upper, size_t groups,
     constexpr int DIM = 128;
     const size_t row = blockIdx.y;
     const size_t first = size_t(blockIdx.x) * INTERVAL_KEYS + 4 * threadIdx.x;        // thread t owns 4 consecutive groups
-    // (the groups' bounds and the row's queries are asked for before the pick's own trip to memory ends)
+    // (the groups' bounds are asked for before the pick's own trip to memory ends)
     float low[4], high[4];
     if (first + 3 < groups && (row * groups) % 4 == 0) {
         const float4 l4 = *reinterpret_cast<const float4*>(lower + row * groups + first), h4 = *reinterpret_cast<const float4*>(upper + row * groups + first);
@@ -780,8 +780,8 @@ candidate_segments_kernel(const float* lower, const float* upper, size_t groups,
 // score (ties to the lowest index) for the places that are left; ascending indices, -1 past the last.  The segments' lists are
 // first laid end to end -- in LDS when they fit, else in `flat` (global) -- with one synthetic score each: +inf for a certain
 // candidate (above every band member, as it is known to be), the canonical score for a band member; the exact top-k over that
-// row is then the result.  A band of at most a thousand is ranked directly (every member counts who beats it, one thread
-// each); anything larger takes the general radix select.
+// row is then the result.  A band of at most a thousand is ranked directly (every member counts who beats it, one to eight
+// threads a member); anything larger takes the general radix select.
 __global__ void __launch_bounds__(TOPK_THREADS) index_finish_kernel(const float* scores, const int32_t* list, const uint32_t* counts, size_t segments, size_t groups,
                                                                     size_t k, float* flat_scores, int32_t* flat_list, int32_t* out, uint32_t* histogram,
                                                                     size_t histogram_rows) {
