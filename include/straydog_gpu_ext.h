@@ -239,15 +239,20 @@ int64_t sdx_event_record(void* handle);
 int sdx_event_elapsed(void* handle, int64_t begin, int64_t end, float* milliseconds);
 int sdx_events_clear(void* handle);
 int sdx_device_compute_units(void* handle);
+/* For harnesses that check what a call allocates: values[0..3] = the device's free and total memory as the driver reports them
+ * (hipMemGetInfo), the bytes of the handle's workspace, and the number of timing events sdx_profile has recorded. */
+int sdx_device_state(void* handle, uint64_t* values);
 /* Kernel timing for benchmarks: while enabled, each op launches its dominant kernel through the extended launch, whose two
  * events take the kernel's own start and end on the handle's stream; sdx_profile_read waits for the stream and returns the
  * summed kernel time and the launch count.  sdx_profile(handle, 0|1) clears what was recorded.  Launches recorded into a graph
  * (sd_graph_begin .. sd_graph_end) are not timed. */
 int sdx_profile(void* handle, int enable);
 int sdx_profile_read(void* handle, double* milliseconds, uint64_t* launches);
-/* Seeded N(0,1) values as the reference's tests draw them: one xorshift64 stream from `seed` (0: 0x9e3779b97f4a7c15), two draws a
- * Box-Muller pair in double precision, value i of the stream at out[i] (crates/straydog-engine/tests/fused_gpu.rs:39-53,
- * gpu/tests/qsa_interval_test.cpp:12-18).  The threads reach their stretches of the stream by jumping (the generator is linear). */
+/* Seeded N(0,1) values from the generator family of the reference's tests (crates/straydog-engine/tests/fused_gpu.rs:39-53,
+ * gpu/tests/qsa_interval_test.cpp:12-18): one xorshift64 stream from `seed` (0: 0x9e3779b97f4a7c15), two draws a Box-Muller
+ * pair in double precision, uniforms ((x >> 11) + 0.5) / 2^53, cosine and sine both kept, value i of the stream at out[i].  The
+ * same family, not those tests' values: their seeding and their uniforms differ, so no fixture of the reference is reproduced.
+ * The threads reach their stretches of the stream by jumping (the generator is linear). */
 int sdx_fill_normal(void* handle, void* out, uint64_t count, uint64_t seed, int out_kind /* 0 f32, 1 f16, 2 bf16 */);
 int sdx_fill_uniform(void* handle, float* out, uint64_t count, uint64_t seed, float lo, float hi);
 int sdx_copy(void* handle, void* target, const void* source, uint64_t bytes);

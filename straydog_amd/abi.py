@@ -133,6 +133,7 @@ SIGNATURES = {
     "sdx_event_elapsed": (c_int, [c_void_p, c_i64, c_i64, _P(c_float)]),
     "sdx_events_clear": (c_int, [c_void_p]),
     "sdx_device_compute_units": (c_int, [c_void_p]),
+    "sdx_device_state": (c_int, [c_void_p, c_void_p]),
     "sdx_profile": (c_int, [c_void_p, c_int]),
     "sdx_profile_read": (c_int, [c_void_p, _P(ctypes.c_double), _P(c_u64)]),
     "sdx_fill_normal": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_int]),

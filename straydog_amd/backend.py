@@ -65,6 +65,12 @@ class Backend:
         self.close()
 
     # ---- allocations and transfers -------------------------------------------------
+    def device_state(self):
+        """(free device bytes, total device bytes, the handle's workspace bytes, timing events recorded)."""
+        values = (abi.c_u64 * 4)()
+        self.check(self.lib.sdx_device_state(self.handle, values))
+        return tuple(int(v) for v in values)
+
     def memory(self):
         used, budget = abi.c_u64(), abi.c_u64()
         self.check(self.lib.sd_memory(self.handle, ctypes.byref(used), ctypes.byref(budget)))

@@ -12,6 +12,7 @@ namespace sd {
 
 thread_local std::string last_error;
 void paged_attention_setup(Device& d);   // paged_attention.hip
+void harness_setup(Device& d);           // harness.hip
 void select_thin_reserve(Device& d);     // block_index.hip
 
 // Recorded graphs hold the addresses their ops were given.  When a buffer the library owns moves (the workspace grows), the
@@ -84,6 +85,7 @@ void upload(Device& d, void* target, const void* data, size_t bytes) {
     const size_t half = io_arena_bytes / 2;
     const uint8_t* from = static_cast<const uint8_t*>(data);
     uint8_t* to = static_cast<uint8_t*>(target);
+    kv_settle(d);       // (the target may be pages a queued move still reads or writes)
     static thread_local int turn = 0;
     while (bytes) {
         const size_t part = std::min(bytes, half);
@@ -100,6 +102,8 @@ void upload(Device& d, void* target, const void* data, size_t bytes) {
 void download(Device& d, void* output, const void* source, size_t bytes) {
     uint8_t* to = static_cast<uint8_t*>(output);
     const uint8_t* from = static_cast<const uint8_t*>(source);
+    // the bytes may be pages still on their way from host memory on the page stream
+    kv_settle(d);
     // both halves may hold an upload in flight: wait for the stream once, then the arena is ours
     SD_CHECK(hipStreamSynchronize(d.stream));
     while (bytes) {
@@ -192,6 +196,7 @@ void* sd_create(int ordinal, uint64_t budget) {
         d->events.resize(2);
         for (auto& event : d->events) { SD_CHECK(hipEventCreateWithFlags(&event, hipEventDisableTiming)); SD_CHECK(hipEventRecord(event, d->stream)); }
         paged_attention_setup(*d);
+        harness_setup(*d);
         return d;
     } catch (const std::exception& e) {
         last_error = e.what();
@@ -381,6 +386,7 @@ int sd_checkpoint_copy(void* handle, int save, void* const* states, uint64_t cou
             }
         }
         auto* host = static_cast<uint8_t*>(buffer);
+        kv_settle(d);
         for (uint64_t i = 0; i < count; ++i) {
             if (save) SD_CHECK(hipMemcpyAsync(host, states[i], sizes[i], hipMemcpyDeviceToHost, d.stream));
             else SD_CHECK(hipMemcpyAsync(states[i], host, sizes[i], hipMemcpyHostToDevice, d.stream));
@@ -422,6 +428,7 @@ int sd_state_copy(void* handle, void* state, uint64_t offset, uint64_t pitch, ui
         if (offset > floats || height - 1 > (floats - offset) / pitch || width > floats - offset - (height - 1) * pitch)
             throw std::runtime_error("Straydog state copy outside its state");
         float* base = static_cast<float*>(state) + offset;
+        kv_settle(d);
         if (save) SD_CHECK(hipMemcpy2DAsync(host, width * 4, base, pitch * 4, width * 4, height, hipMemcpyDeviceToHost, d.stream));
         else SD_CHECK(hipMemcpy2DAsync(base, pitch * 4, host, width * 4, width * 4, height, hipMemcpyHostToDevice, d.stream));
         SD_CHECK(hipStreamSynchronize(d.stream));
@@ -568,6 +575,8 @@ int sd_graph_run(void* handle, uint64_t key) {
         Device& d = device(handle);
         const auto found = d.graphs.find(key);
         if (found == d.graphs.end()) return 1;
+        // page moves queued since the recording (a resume, a stage) come first: the graph's ops read the pages they fill
+        kv_settle(d);
         SD_CHECK(hipGraphLaunch(found->second.executable, d.stream));
         return 0;
     } catch (const std::exception& e) { last_error = e.what(); return -1; }
@@ -634,6 +643,17 @@ int sdx_profile_read(void* handle, double* milliseconds, uint64_t* launches) {
         }
         if (milliseconds) *milliseconds = total;
         if (launches) *launches = d.profile_events.size() / 2;
+        return 0;
+    } catch (const std::exception& e) { last_error = e.what(); return -1; }
+}
+
+int sdx_device_state(void* handle, uint64_t* values) {
+    try {
+        Device& d = device(handle);
+        if (!values) throw std::runtime_error("invalid Straydog device query");
+        size_t free_bytes = 0, total_bytes = 0;
+        SD_CHECK(hipMemGetInfo(&free_bytes, &total_bytes));
+        values[0] = free_bytes; values[1] = total_bytes; values[2] = d.workspace_bytes; values[3] = d.profile_events.size();
         return 0;
     } catch (const std::exception& e) { last_error = e.what(); return -1; }
 }

@@ -1033,7 +1033,8 @@ __global__ void __launch_bounds__(256) index_projection_kernel(const uint8_t* ma
     if (lane == 0) weights[head] = sum;
 }
 
-void index_projection(Device& value, const void* proj_weights, int proj_kind, uint64_t proj_cols, const float* x, uint64_t heads, float* weights) {
+// Every check of the projection's arguments; returns the bytes of a weight row.
+size_t index_projection_check(Device& value, const void* proj_weights, int proj_kind, uint64_t proj_cols, const float* x, uint64_t heads, float* weights) {
     if (!proj_weights || !proj_cols || proj_cols > 8192 || !heads || heads > 64) throw std::runtime_error("invalid Straydog index shape");
     if (proj_kind != 30 && proj_kind != 8) throw std::runtime_error("the index projection takes BF16 (kind 30) or Q8_0 (kind 8) rows");
     if (proj_cols % (proj_kind == 30 ? 8 : 32)) throw std::runtime_error("invalid Straydog index shape");
@@ -1042,16 +1043,27 @@ void index_projection(Device& value, const void* proj_weights, int proj_kind, ui
     op_span(value, x, checked_floats({proj_cols}), "a linear input");
     op_span(value, weights, checked_floats({heads}), "index weights");
     if (proj_kind == 30 && reinterpret_cast<uintptr_t>(proj_weights) % 16) throw std::runtime_error("BF16 projection rows must be 16-byte aligned");
+    return row_bytes;
+}
+
+void index_projection_launch(Device& value, const void* proj_weights, int proj_kind, uint64_t proj_cols, const float* x, uint64_t heads, float* weights,
+                             size_t row_bytes) {
     const unsigned grid = unsigned((heads + 3) / 4);
     const auto* matrix = static_cast<const uint8_t*>(proj_weights);
     if (proj_kind == 30) index_projection_kernel<30><<<grid, 256, 0, value.stream>>>(matrix, row_bytes, size_t(proj_cols), x, size_t(heads), weights);
     else index_projection_kernel<8><<<grid, 256, 0, value.stream>>>(matrix, row_bytes, size_t(proj_cols), x, size_t(heads), weights);
 }
 
-void index_select(Device& value, const float* q, const float* keys, const float* weights, const int32_t* visible, uint64_t rows,
-                       uint64_t groups, uint64_t heads, uint64_t dim, float scale, uint64_t rope_dims, const int32_t* positions,
-                       const float* frequencies, float* scores, uint64_t k, int32_t* out, const int32_t* candidates, uint64_t blocks,
-                       uint64_t block) {
+void index_projection(Device& value, const void* proj_weights, int proj_kind, uint64_t proj_cols, const float* x, uint64_t heads, float* weights) {
+    index_projection_launch(value, proj_weights, proj_kind, proj_cols, x, heads, weights,
+                            index_projection_check(value, proj_weights, proj_kind, proj_cols, x, heads, weights));
+}
+
+// Every check of the fused indexer's arguments (nothing is queued before all of them have passed, as gpu/kernels.cpp:5626-5640).
+void index_select_check(Device& value, const float* q, const float* keys, const float* weights, const int32_t* visible, uint64_t rows,
+                        uint64_t groups, uint64_t heads, uint64_t dim, uint64_t rope_dims, const int32_t* positions,
+                        const float* frequencies, float* scores, uint64_t k, int32_t* out, const int32_t* candidates, uint64_t blocks,
+                        uint64_t block) {
     if (!rows || rows > 65535 || !groups || groups > (uint64_t(1) << 31) || !heads || heads > 64 || !dim || !k || k > (uint64_t(1) << 31) ||
         rope_dims % 2 || rope_dims > dim || rope_dims > 128)
         throw std::runtime_error("invalid Straydog index shape");
@@ -1069,6 +1081,13 @@ void index_select(Device& value, const float* q, const float* keys, const float*
     if (rope_dims) op_span(value, frequencies, checked_floats({rope_dims / 2}), "rope frequencies");
     op_span(value, scores, checked_floats({rows, std::max(groups, scored)}), "index scores");
     op_span(value, out, checked_floats({rows, k}), "top-k indices");
+}
+
+void index_select_launch(Device& value, const float* q, const float* keys, const float* weights, const int32_t* visible, uint64_t rows,
+                         uint64_t groups, uint64_t heads, uint64_t dim, float scale, uint64_t rope_dims, const int32_t* positions,
+                         const float* frequencies, float* scores, uint64_t k, int32_t* out, const int32_t* candidates, uint64_t blocks,
+                         uint64_t block) {
+    const uint64_t scored = candidates ? blocks * block : groups;
     const float* rotated = q;
     if (rope_dims) {
         // q itself stays as it was: the rotated copy lives in the device's workspace
@@ -1089,6 +1108,15 @@ void index_select(Device& value, const float* q, const float* keys, const float*
     else
         top_k_kernel<<<unsigned(rows), TOPK_THREADS, 0, value.stream>>>(scores, size_t(groups), stride, size_t(k), out);
     SD_CHECK(hipGetLastError());
+}
+
+void index_select(Device& value, const float* q, const float* keys, const float* weights, const int32_t* visible, uint64_t rows,
+                  uint64_t groups, uint64_t heads, uint64_t dim, float scale, uint64_t rope_dims, const int32_t* positions,
+                  const float* frequencies, float* scores, uint64_t k, int32_t* out, const int32_t* candidates, uint64_t blocks,
+                  uint64_t block) {
+    index_select_check(value, q, keys, weights, visible, rows, groups, heads, dim, rope_dims, positions, frequencies, scores, k, out, candidates, blocks, block);
+    index_select_launch(value, q, keys, weights, visible, rows, groups, heads, dim, scale, rope_dims, positions, frequencies, scores, k, out, candidates,
+                        blocks, block);
 }
 
 }  // namespace
@@ -1197,11 +1225,13 @@ int sd_op_index_select_proj(void* handle, const void* proj_weights, int proj_kin
                             uint64_t rope_dims, const int32_t* positions, const float* frequencies, float* scores, uint64_t k, int32_t* out,
                             const int32_t* candidates, uint64_t blocks, uint64_t block) {
     SD_OP_BEGIN
-    if (!heads || heads > 64) throw std::runtime_error("invalid Straydog index shape");
-    index_projection(value, proj_weights, proj_kind, proj_cols, x, heads, weights);
+    // every argument of both halves is checked before the projection, which overwrites `weights`, is queued
+    const size_t row_bytes = index_projection_check(value, proj_weights, proj_kind, proj_cols, x, heads, weights);
+    index_select_check(value, q, keys, weights, visible, 1, groups, heads, dim, rope_dims, positions, frequencies, scores, k, out, candidates, blocks, block);
+    index_projection_launch(value, proj_weights, proj_kind, proj_cols, x, heads, weights, row_bytes);
     SD_CHECK(hipGetLastError());
-    index_select(value, q, keys, weights, visible, 1, groups, heads, dim, scale, rope_dims, positions, frequencies, scores, k, out, candidates, blocks,
-                 block);
+    index_select_launch(value, q, keys, weights, visible, 1, groups, heads, dim, scale, rope_dims, positions, frequencies, scores, k, out, candidates, blocks,
+                        block);
     SD_OP_END
 }
 

@@ -91,11 +91,32 @@ def test_stubs_fail_cleanly(library):
     assert len(stubs) > 250
     for name, kind in stubs:
         function = getattr(library, name)
+        if kind == "STR":
+            continue            # (text results: test_text_results_are_never_null)
         function.restype, expected = results[kind]
         function.argtypes = None
         # arguments are ignored (the caller owns them in the C calling convention): pass a few, as a bound caller would
         assert function(None, None, ctypes.c_uint64(3), None) == expected, name
         assert library.sd_error().decode() == f"{name} is not implemented in the attention library"
+
+
+def test_text_results_are_never_null(library):
+    # the host reads a text result without a null check (CStr::from_ptr(ffi::sd_cpu_error()) after any failed CPU-engine call,
+    # crates/straydog-engine/src/gpu.rs:3831-3838): every function that answers text answers some, and sd_cpu_error the reason
+    # of the thread's last refusal
+    golden = _golden_symbols()
+    texts = [name for name, (kind, _) in golden.items() if kind == "STR"]
+    assert set(texts) == {"sd_error", "sd_cpu_error", "sd_cpu_experts_isa"}
+    for name in texts:
+        function = getattr(library, name)
+        function.restype, function.argtypes = ctypes.c_char_p, None
+    library.sd_cpu_experts_create.restype, library.sd_cpu_experts_create.argtypes = ctypes.c_void_p, None
+    assert library.sd_cpu_experts_create(ctypes.c_uint32(4), ctypes.c_uint32(0)) is None
+    assert library.sd_cpu_error() == b"sd_cpu_experts_create is not implemented in the attention library"
+    assert library.sd_cpu_error() == library.sd_error()
+    isa = library.sd_cpu_experts_isa(None)
+    assert isa is not None and b"sd_cpu_experts_isa is not implemented" in isa
+    assert library.sd_error() is not None
 
 
 def test_backend_refuses_a_missing_library(tmp_path):

@@ -244,3 +244,71 @@ def test_a_pool_in_mapped_host_memory_attends_to_the_same_bits(gpu, oracle):
     assert not gpu.read_buffer(large, 0, np.uint8, 1 << 20).any() and not gpu.read_buffer(small, 0, np.uint8, 4096).any()
     for b in (large, other, small):
         gpu.release(b)
+
+
+def test_a_recorded_step_runs_after_the_page_moves_queued_before_it(gpu, oracle):
+    """A decode step recorded as a graph reads the pages its sequence holds when it is replayed: a replay queued right after a
+    resume (onto other pages) or a stage comes after the copies that fill them, and gives the eager call's bits."""
+    context, length = 16384, 16000
+    pages = context // PAGE
+    cache, *_ = gpu.kv_cache(2 * pages, PAGE, KVH, DIM, ROW, 2, context)
+    gpu.kv_cache_host(cache, 2 * pages)
+    rng = np.random.default_rng(75)
+    pool, table, stride = gpu.kv_cache_view(cache)
+    gpu.kv_cache_reserve(cache, 0, length)
+    k = rng.standard_normal((1, length, KVH, DIM)).astype(np.float32)
+    v = rng.standard_normal((1, length, KVH, DIM)).astype(np.float32)
+    q = rng.standard_normal((1, 1, HEADS, DIM)).astype(np.float32)
+    kb, vb, zero, qb, pb = (gpu.upload(a) for a in (k, v, np.zeros(1, np.int32), q, np.array([length - 1], np.int32)))
+    gpu.kv_write(pool, table, stride, zero.base(), kb.base(), vb.base(), False, 1, length)
+    out = gpu.buffer(q.size * 4)
+    scratch = gpu.buffer(gpu.paged_attention_scratch(1, 1, HEADS, DIM, context))
+
+    def step(view):
+        gpu.paged_attention(view[0], view[1], view[2], pb.base(), context, qb.base(), False, 1, 1, HEADS, 0.09, out.base(), False, scratch)
+
+    def result():
+        return gpu.read_buffer(out, 0, np.float32, q.size)
+
+    step((pool, table, stride))
+    eager = result()
+    gpu.graph_begin()
+    step((pool, table, stride))
+    gpu.graph_end(31, True)
+    for turn in range(3):
+        # the sequence leaves, another takes (and writes) the pages it held, and it comes back onto other pages
+        gpu.kv_cache_park(cache, 0)
+        gpu.kv_cache_reserve(cache, 1, length)
+        gpu.kv_write(pool, table + stride * 4, stride, zero.base(), vb.base(), kb.base(), False, 1, length)
+        gpu.kv_cache_resume(cache, 0)
+        gpu.write_buffer(out, 0, np.zeros(q.size, np.float32))
+        assert gpu.graph_run(31)
+        assert np.array_equal(result(), eager), f"replay {turn} right after a resume"
+        gpu.kv_cache_truncate(cache, 1, 0)
+    # the same through the stage: the view's pool is the stage, whose rows a staging refills
+    gpu.kv_cache_park(cache, 0)
+    page_bytes = 2 * KVH * PAGE * ROW
+    stage_rows = pages * page_bytes // 4096 + 1
+    stage = gpu.buffer(stage_rows * 4096)
+    gpu.kv_stage(stage.base(), stage_rows)
+    view = gpu.kv_cache_stage(cache, 0, length)
+    step(view)
+    assert np.array_equal(result(), eager), "the same rows, read from the stage"
+    gpu.graph_begin()
+    step(view)
+    gpu.graph_end(32, True)
+    gpu.kv_cache_reserve(cache, 1, 4 * PAGE)
+    gpu.kv_write(pool, table + stride * 4, stride, zero.base(), vb.base(), kb.base(), False, 1, 4 * PAGE)
+    for turn in range(3):
+        gpu.kv_cache_park(cache, 1)
+        gpu.kv_cache_stage(cache, 1, 4 * PAGE)              # the stage now holds the other sequence's first pages
+        gpu.kv_cache_resume(cache, 1)
+        again = gpu.kv_cache_stage(cache, 0, length)
+        assert again[0].pages == view[0].pages and again[1] == view[1]
+        gpu.write_buffer(out, 0, np.zeros(q.size, np.float32))
+        assert gpu.graph_run(32)
+        assert np.array_equal(result(), eager), f"replay {turn} right after a staging"
+    gpu.release(stage)
+    for b in (kb, vb, zero, qb, pb, out, scratch):
+        gpu.release(b)
+    gpu.kv_cache_destroy(cache)

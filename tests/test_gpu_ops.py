@@ -335,6 +335,14 @@ def test_an_index_select_with_its_projection_matches_the_two_ops(gpu, oracle):
         gpu.index_select_proj((mb.base(), 30, 5004), xb.base(), qb.base(), kb.base(), w.base(), vb.base(), groups, heads, dim, scale, rope, s.base(), k, o.base())
     with pytest.raises(StraydogError, match="outside"):
         gpu.index_select_proj((mb.base(), 30, width), xb.at(4 * 100), qb.base(), kb.base(), w.base(), vb.base(), groups, heads, dim, scale, rope, s.base(), k, o.base())
+    # a shape the selection half refuses is refused before the projection half has written the weights (gpu/kernels.cpp:5626-5640)
+    marks = np.full(heads, 7.25, np.float32)
+    gpu.write_buffer(w, 0, marks)
+    with pytest.raises(StraydogError, match="invalid Straydog index shape"):
+        gpu.index_select_proj((mb.base(), 30, width), xb.base(), qb.base(), kb.base(), w.base(), vb.base(), groups, heads, dim, scale, rope, s.base(), 0, o.base())
+    with pytest.raises(StraydogError, match="outside"):
+        gpu.index_select_proj((mb.base(), 30, width), xb.base(), qb.base(), kb.base(), w.base(), vb.base(), groups, heads, dim, scale, rope, s.base(), k + 1, o.base())
+    assert np.array_equal(_read(gpu, w, np.float32, heads), marks)
     for b in (mb, w, s, o, fb, xb, qb, kb, pb, vb):
         gpu.release(b)
 

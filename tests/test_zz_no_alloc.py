@@ -24,13 +24,31 @@ def _both(gpu, work):
     work.step()
     want = gpu.read_buffer(work.out_buffer, 0, np.uint8, count).copy()
     gpu.write_buffer(work.out_buffer, 0, np.full(count, 0x5a, np.uint8))
-    used_before = gpu.memory()[0]
+    used_before, state_before = gpu.memory()[0], gpu.device_state()
     gpu.paged_attention_static(work.pool, work.table_buffer.base(), work.table_stride, work.position_buffer.base(), work.max_context,
                                work.q_buffer.base(), work.q_f16, work.seqs, work.span, work.heads, work.scale, work.out_buffer.base(),
                                work.out_f16)
     got = gpu.read_buffer(work.out_buffer, 0, np.uint8, count).copy()
+    # nothing allocated: neither in the handle's own accounting, nor as the driver sees the device, nor as workspace or events
     assert gpu.memory()[0] == used_before
+    assert gpu.device_state() == state_before
     return got, want
+
+
+def test_static_entry_first_call_on_a_fresh_handle():
+    # the handle's very first launch is the static entry's: whatever it sets up for itself (LDS limits) allocates nothing either
+    with backend() as fresh:
+        work = PagedWorkload(fresh, [900, 4100, 33], span=1, heads=32, kv_heads=4, dim=128, seed=20)
+        count = work.seqs * work.span * work.heads * work.dim * 2
+        state_before = fresh.device_state()
+        fresh.paged_attention_static(work.pool, work.table_buffer.base(), work.table_stride, work.position_buffer.base(), work.max_context,
+                                     work.q_buffer.base(), work.q_f16, work.seqs, work.span, work.heads, work.scale, work.out_buffer.base(),
+                                     work.out_f16)
+        got = fresh.read_buffer(work.out_buffer, 0, np.uint8, count).copy()
+        assert fresh.device_state() == state_before
+        work.step()
+        assert np.array_equal(got, fresh.read_buffer(work.out_buffer, 0, np.uint8, count))
+        work.release()
 
 
 def test_static_entry_equals_the_scratch_entry_twice_in_a_row(gpu, oracle):
