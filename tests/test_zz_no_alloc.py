@@ -17,6 +17,13 @@ def gpu():
         yield handle
 
 
+def _nothing_allocated(before, after):
+    """Device memory as the driver reports it has not shrunk (it may grow: memory released earlier comes back late), and the
+    handle's workspace and its timing events are what they were."""
+    assert after[0] >= before[0], f"the device's free memory fell by {before[0] - after[0]} bytes"
+    assert after[1:] == before[1:]
+
+
 def _both(gpu, work):
     """Output bytes of the scratch-argument entry point and of the static one, on the same inputs."""
     count = work.seqs * work.span * work.heads * work.dim * (2 if work.out_f16 else 4)
@@ -31,7 +38,7 @@ def _both(gpu, work):
     got = gpu.read_buffer(work.out_buffer, 0, np.uint8, count).copy()
     # nothing allocated: neither in the handle's own accounting, nor as the driver sees the device, nor as workspace or events
     assert gpu.memory()[0] == used_before
-    assert gpu.device_state() == state_before
+    _nothing_allocated(state_before, gpu.device_state())
     return got, want
 
 
@@ -45,7 +52,7 @@ def test_static_entry_first_call_on_a_fresh_handle():
                                      work.q_buffer.base(), work.q_f16, work.seqs, work.span, work.heads, work.scale, work.out_buffer.base(),
                                      work.out_f16)
         got = fresh.read_buffer(work.out_buffer, 0, np.uint8, count).copy()
-        assert fresh.device_state() == state_before
+        _nothing_allocated(state_before, fresh.device_state())
         work.step()
         assert np.array_equal(got, fresh.read_buffer(work.out_buffer, 0, np.uint8, count))
         work.release()
