@@ -98,6 +98,25 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
                         const int32_t* positions, uint64_t max_context, const void* q, int q_f16, uint64_t seqs, uint64_t span,
                         uint64_t heads, float scale, void* out, int out_f16, void* scratch, uint64_t scratch_bytes);
 
+/* A prompt chunk in one call: the chunk's K/V rows appended to the cache and its queries attended -- the K/V write and the
+ * attention stage of the reference's prompt passes (write_attention_kv gpu/kernels.cpp:79-98, then qsa_prompt_attention
+ * gpu/qsa_prompt_attention.hpp:47-213, 220-234, inside sd_prefill_span) with the dense selection 0..position.  The bits of
+ * sdx_kv_write followed by sdx_paged_attention on the same arguments (cache bytes and outputs; 128 columns, Q8_0 or FP16 rows),
+ * in two launches where those take three, and without unpacking the prompt's earlier rows again at every chunk: the FP16 operand
+ * tiles of the cached rows, which sdx_paged_attention rebuilds in the handle's workspace on every call, live in `tiles`, device
+ * memory of sdx_prefill_tiles_bytes(seqs, kv_heads, 128, max_context) bytes that the caller keeps between the chunks of a prompt.
+ *   keys/values  [seqs][span][kv_heads][dim] FP32 (kv_f16 = 0) or FP16 (1), rows for positions[s] .. positions[s] + span - 1; both
+ *                null when the rows are in the cache already (the call then only attends)
+ *   valid        device, int32 [seqs], or null: the leading positions of each sequence whose tiles `tiles` still holds from earlier
+ *                calls on the same cache rows (in a chunked prefill: positions itself -- everything before this chunk); null or 0
+ *                rebuilds every tile.  A position above positions[s] counts as positions[s].
+ * Rows at positions >= max_context are neither stored nor attended. */
+uint64_t sdx_prefill_tiles_bytes(uint64_t seqs, uint64_t kv_heads, uint64_t dim, uint64_t max_context);
+int sdx_prefill_chunk(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
+                      uint64_t max_context, const void* keys, const void* values, int kv_f16, const void* q, int q_f16, uint64_t seqs,
+                      uint64_t span, uint64_t heads, float scale, void* out, int out_f16, void* tiles, uint64_t tiles_bytes,
+                      const int32_t* valid);
+
 /* The same attention for callers that cannot allocate device memory or pass a scratch buffer: code under graph capture, tight
  * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The split partial results live in
  * an area of sdx_paged_attention_static_bytes() bytes (16 MiB) that the library itself holds on every GPU it runs on until the

@@ -282,6 +282,17 @@ class Backend:
                                                 q, int(q_f16), seqs, span, heads, scale, out, int(out_f16), scratch.pointer,
                                                 scratch.size))
 
+    def prefill_tiles_bytes(self, seqs, kv_heads, dim, max_context):
+        return int(self.lib.sdx_prefill_tiles_bytes(seqs, kv_heads, dim, max_context))
+
+    def prefill_chunk(self, pool, page_table, table_stride, positions, max_context, keys, values, kv_f16, q, q_f16, seqs, span, heads, scale,
+                      out, out_f16, tiles, valid=None):
+        """A prompt chunk in one call: K/V append (keys/values may be None) + causal attention; `tiles` (a Buffer) keeps the cached
+        rows' operand tiles between chunks, `valid` the device array of positions whose tiles are still good."""
+        self.check(self.lib.sdx_prefill_chunk(self.handle, ctypes.byref(pool), page_table, table_stride, positions, max_context, keys, values,
+                                              int(kv_f16), q, int(q_f16), seqs, span, heads, scale, out, int(out_f16), tiles.pointer, tiles.size,
+                                              valid))
+
     def paged_attention_static(self, pool, page_table, table_stride, positions, max_context, q, q_f16, seqs, span, heads, scale, out,
                                out_f16):
         """sdx_paged_attention with the partial results in the library's own area: the call allocates nothing."""

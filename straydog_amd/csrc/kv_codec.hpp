@@ -15,6 +15,24 @@ __device__ __forceinline__ float kv_value(const uint8_t* row, unsigned column, u
     return __half2float(reinterpret_cast<const __half*>(row)[column]);
 }
 
+// The Q8_0 encoding of four consecutive values of a 32-value block: their four bytes and the block's scale.  The 8 lanes that
+// hold the block are adjacent (lane % 8 = quad within the block) and must all call this together.
+__device__ __forceinline__ void kv_quad_q8(const float (&x)[4], uint32_t& word, __half& scale16) {
+    float top = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
+    top = fmaxf(top, __shfl_xor(top, 1));
+    top = fmaxf(top, __shfl_xor(top, 2));
+    top = fmaxf(top, __shfl_xor(top, 4));
+    scale16 = __float2half_rn(top / 127.0f);
+    const float scale = __half2float(scale16);
+    word = 0;
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int q = scale > 0.0f ? __float2int_rn(x[i] / scale) : 0;
+        q = q > 127 ? 127 : q < -127 ? -127 : q;
+        word |= uint32_t(uint8_t(int8_t(q))) << (8 * i);
+    }
+}
+
 // Four consecutive values (column a multiple of 4) stored into a row.  The 8 lanes that hold one 32-value block
 // are adjacent (lane % 8 = quad within the block) and must all call this together.
 __device__ __forceinline__ void kv_store_quad(uint8_t* row, unsigned quad, unsigned dim, bool q8, const float (&x)[4], bool live) {
@@ -27,19 +45,9 @@ __device__ __forceinline__ void kv_store_quad(uint8_t* row, unsigned quad, unsig
         *reinterpret_cast<uint2*>(row + quad * 8) = packed;
         return;
     }
-    float top = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
-    top = fmaxf(top, __shfl_xor(top, 1));
-    top = fmaxf(top, __shfl_xor(top, 2));
-    top = fmaxf(top, __shfl_xor(top, 4));
-    const __half scale16 = __float2half_rn(top / 127.0f);
-    const float scale = __half2float(scale16);
-    uint32_t word = 0;
-    #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        int q = scale > 0.0f ? __float2int_rn(x[i] / scale) : 0;
-        q = q > 127 ? 127 : q < -127 ? -127 : q;
-        word |= uint32_t(uint8_t(int8_t(q))) << (8 * i);
-    }
+    uint32_t word;
+    __half scale16;
+    kv_quad_q8(x, word, scale16);
     if (!live) return;
     *reinterpret_cast<uint32_t*>(row + quad * 4) = word;
     if (quad % 8 == 0) *reinterpret_cast<__half*>(row + dim + quad / 8 * 2) = scale16;

@@ -23,6 +23,10 @@ void validate_pool(Device& d, const sdx_kv_pool* pool);
 void prefill_attention(Device& d, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
                        uint64_t max_context, const void* q, int q_f16, uint64_t seqs, uint64_t span, uint64_t heads, float scale, void* out,
                        int out_f16);
+void prefill_chunk(Device& d, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
+                   uint64_t max_context, const void* keys, const void* values, int kv_f16, const void* q, int q_f16, uint64_t seqs, uint64_t span,
+                   uint64_t heads, float scale, void* out, int out_f16, void* tiles, const int32_t* valid);
+uint64_t prefill_tiles_bytes(uint64_t seqs, uint64_t kv_heads, uint64_t max_context);
 }
 using namespace sd;
 using namespace sd::paged;
@@ -577,6 +581,38 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
     SD_OP_BEGIN
     paged_attention(value, pool, page_table, table_stride, positions, max_context, q, q_f16, seqs, span, heads, scale, out, out_f16,
                     static_cast<float*>(scratch), scratch_bytes, false);
+    SD_OP_END
+}
+
+uint64_t sdx_prefill_tiles_bytes(uint64_t seqs, uint64_t kv_heads, uint64_t dim, uint64_t max_context) {
+    try { return dim == 128 && seqs && kv_heads && max_context ? prefill_tiles_bytes(seqs, kv_heads, max_context) : 0; }
+    catch (const std::exception&) { return 0; }
+}
+
+int sdx_prefill_chunk(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
+                      uint64_t max_context, const void* keys, const void* values, int kv_f16, const void* q, int q_f16, uint64_t seqs, uint64_t span,
+                      uint64_t heads, float scale, void* out, int out_f16, void* tiles, uint64_t tiles_bytes, const int32_t* valid) {
+    SD_OP_BEGIN
+    validate_pool(value, pool);
+    if (pool->dim != 128) throw std::runtime_error("Straydog prefill chunk: rows of 128 columns only");
+    if (!(scale > 0.0f) || !seqs || seqs > 65535 || !span || !heads || heads % pool->kv_heads || !max_context || max_context > (uint64_t(1) << 30) ||
+        !table_stride || max_context > table_stride * pool->page_tokens || !keys != !values)
+        throw std::runtime_error("invalid Straydog prefill chunk shape");
+    op_span(value, page_table, checked_floats({seqs, table_stride}), "a page table");
+    op_span(value, positions, checked_floats({seqs}), "query positions");
+    if (valid) op_span(value, valid, checked_floats({seqs}), "valid tile positions");
+    if (keys) {
+        op_span(value, keys, checked_product({seqs, span, pool->kv_heads, pool->dim, kv_f16 ? 2u : 4u}), "new keys");
+        op_span(value, values, checked_product({seqs, span, pool->kv_heads, pool->dim, kv_f16 ? 2u : 4u}), "new values");
+    }
+    op_span(value, q, checked_product({seqs, span, heads, pool->dim, q_f16 ? 2u : 4u}), "attention queries");
+    op_span(value, out, checked_product({seqs, span, heads, pool->dim, out_f16 ? 2u : 4u}), "an attention output");
+    const uint64_t need = prefill_tiles_bytes(seqs, pool->kv_heads, max_context);
+    if (!tiles || tiles_bytes < need) throw std::runtime_error("Straydog prefill chunk: the tile buffer is too small");
+    if (uintptr_t(tiles) % 16) throw std::runtime_error("Straydog prefill chunk: the tile buffer must lie on a 16-byte boundary");
+    op_span(value, tiles, size_t(need), "prefill tiles");
+    prefill_chunk(value, pool, page_table, table_stride, positions, max_context, keys, values, kv_f16, q, q_f16, seqs, span, heads, scale, out, out_f16,
+                  tiles, valid);
     SD_OP_END
 }
 

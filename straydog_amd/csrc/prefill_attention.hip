@@ -20,6 +20,7 @@
 //     keys of every step and one the last 32, each with its own online softmax, merged through LDS at the end; the
 //     workgroups with the longest walks are dispatched first.
 #include "paged_rows.hpp"
+#include "kv_codec.hpp"
 
 #include <type_traits>
 
@@ -383,81 +384,139 @@ constexpr int TILE_KEYS = 64;
 typedef float float2v __attribute__((ext_vector_type(2)));
 template<int DIM> constexpr int tile_bytes() { return 2 * TILE_KEYS * DIM * 2; }
 
-template<int DIM, bool Q8>
-__global__ void __launch_bounds__(256) unpack_tiles_kernel(PrefillArgs args, uint8_t* tiles_out, unsigned tiles_per_seq) {
+// A chunk's new rows may come with the call (IN: 1 FP32, 2 FP16; 0: none): then the kernel is also the K/V writer -- a new row
+// is encoded (kv_encode's bits) into its page and, from the same bytes, into the tile, where otherwise it would be read back from
+// the page.  `valid` (device, may be null): the leading positions of each sequence whose tiles the buffer still holds from
+// earlier chunks; a tile that lies wholly below it is left as it is.
+struct AppendArgs {
+    const void* keys;
+    const void* values;
+    const int32_t* valid;
+};
+// A workgroup builds a quarter of a tile: the K block's or the V^T block's share of 32 of the tile's 64 keys.
+constexpr int PART_KEYS = 32, TILE_PARTS = 2 * (TILE_KEYS / PART_KEYS);
+template<int DIM, bool Q8, int IN>
+__global__ void __launch_bounds__(256) unpack_tiles_kernel(PrefillArgs args, uint8_t* tiles_out, unsigned tiles_per_seq, AppendArgs append) {
     constexpr int ROW = Q8 ? DIM + DIM / 16 : 2 * DIM, KT = TILE_KEYS * DIM * 2, PIECES = DIM / 8;
-    static_assert(DIM == 128, "a K row is 16 pieces, a V^T row 16 units");
-    const int tile = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z, t = threadIdx.x;
-    const int cached = min(first_position(args.positions, unsigned(seq), args.max_context) + int(args.span), args.max_context), key0 = tile * TILE_KEYS;
-    if (key0 >= cached) return;
+    static_assert(DIM == 128 && PART_KEYS == 32, "a K row is 16 pieces, a V^T row 16 units; a 16-byte piece of V^T holds keys of one half");
+    const int tile = blockIdx.x / TILE_PARTS, value = blockIdx.x / 2 % 2, half = blockIdx.x % 2, kvh = blockIdx.y, seq = blockIdx.z, t = threadIdx.x;
+    const int position = first_position(args.positions, unsigned(seq), args.max_context);
+    const int cached = min(position + int(args.span), args.max_context), key0 = tile * TILE_KEYS + half * PART_KEYS;
+    if (tile * TILE_KEYS >= cached) return;
+    if (append.valid && (tile + 1) * TILE_KEYS <= min(max(append.valid[seq], 0), position)) return;
     const int32_t* table = args.page_table + size_t(seq) * args.table_stride;
-    const size_t plane_bytes = size_t(args.page_tokens) * ROW;
+    const size_t plane_bytes = size_t(args.page_tokens) * ROW, plane = (value ? args.kv_heads : 0) + kvh;
     uint8_t* out = tiles_out + ((size_t(seq) * args.kv_heads + kvh) * tiles_per_seq + tile) * tile_bytes<DIM>();
-    // The tile's raw rows come into LDS first, by 8-byte words that follow one another through a row and from row to row of
-    // a page (the small pieces the layouts below are made of would each be a memory access of their own otherwise).
-    __shared__ __attribute__((aligned(16))) uint8_t raw[2][TILE_KEYS][ROW];
-    constexpr int WORDS = ROW / 8;
-    constexpr int ALL = 2 * TILE_KEYS * WORDS, MINE = (ALL + 255) / 256;
+    // The part's raw rows come into LDS first, by 8-byte words that follow one another through a row and from row to row of
+    // a page (the small pieces the layouts below are made of would each be a memory access of their own otherwise).  Rows past
+    // the sequence's end are never read: they become zeros below.
+    __shared__ __attribute__((aligned(16))) uint8_t raw[PART_KEYS][ROW];
+    const auto row_in_pool = [&](int token) {
+        return const_cast<uint8_t*>(args.pages) + (size_t(pool_page(table[token / int(args.page_tokens)], args.page_last)) * 2 * args.kv_heads + plane) * plane_bytes +
+               size_t(token % int(args.page_tokens)) * ROW;
+    };
+    constexpr int WORDS = ROW / 8, ALL = PART_KEYS * WORDS, MINE = (ALL + 255) / 256;
     uint2 held[MINE];
+    bool old[MINE];
     #pragma unroll
     for (int j = 0; j < MINE; ++j) {                        // all of a thread's words are asked for before the first is stored
-        const int word = min(t + 256 * j, ALL - 1);
-        const int value = word / (TILE_KEYS * WORDS), key = word / WORDS % TILE_KEYS, at = word % WORDS;
-        const int token = min(key0 + key, cached - 1);
-        const uint8_t* row = args.pages + (size_t(pool_page(table[token / int(args.page_tokens)], args.page_last)) * 2 * args.kv_heads + (value ? args.kv_heads : 0) + kvh) * plane_bytes +
-                             size_t(token % int(args.page_tokens)) * ROW;
-        held[j] = *reinterpret_cast<const uint2*>(row + 8 * at);
+        const int word = min(t + 256 * j, ALL - 1), key = word / WORDS, at = word % WORDS, token = key0 + key;
+        old[j] = t + 256 * j < ALL && token < cached && !(IN && token >= position);            // (a new row is not in its page yet)
+        held[j] = old[j] ? *reinterpret_cast<const uint2*>(row_in_pool(token) + 8 * at) : uint2{0u, 0u};
     }
-    #pragma unroll
-    for (int j = 0; j < MINE; ++j) {
-        const int word = t + 256 * j;
-        if (word < ALL) *reinterpret_cast<uint2*>(&raw[0][0][0] + 8 * word) = held[j];
-    }
-    __syncthreads();
-    const auto row_of = [&](int key, bool value) -> const uint8_t* { return raw[value ? 1 : 0][key]; };
-    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-    // K: a thread takes pieces of 8 columns; rows past the sequence's end become zeros
-    #pragma unroll
-    for (int j = 0; j < TILE_KEYS * PIECES / 256; ++j) {
-        const int piece = t + 256 * j, key = piece / PIECES, c = piece % PIECES;
-        const uint8_t* row = row_of(key, false);
-        half8 values;
-        if (Q8) {
-            const uint2 bytes = *reinterpret_cast<const uint2*>(row + 8 * c);
-            const _Float16 scale = *reinterpret_cast<const _Float16*>(row + DIM + 2 * (c / 4));
-            #pragma unroll
-            for (int i = 0; i < 8; ++i) values[i] = (_Float16)float(int8_t((i < 4 ? bytes.x : bytes.y) >> (8 * (i & 3)))) * scale;
-        } else values = *reinterpret_cast<const half8*>(row + 16 * c);
-        if (key0 + key >= cached) values = half8{};
-        *reinterpret_cast<half8*>(out + key * (2 * DIM) + ((c ^ (key & 15)) * 16)) = values;
-    }
-    // V^T: a thread takes 4 keys x 4 columns
-    #pragma unroll
-    for (int j = 0; j < (TILE_KEYS / 4) * (DIM / 4) / 256; ++j) {
-        const int block = t + 256 * j, keys4 = block % (TILE_KEYS / 4), cols4 = block / (TILE_KEYS / 4);
-        _Float16 v[4][4];       // [key][column]
+    [[maybe_unused]] float x[PART_KEYS * (DIM / 4) / 256][4];
+    if (IN) {
+        // the new rows among the part's keys: four values a thread, the eight threads of a 32-value block side by side
+        constexpr int QUADS = DIM / 4;
+        const void* source = value ? append.values : append.keys;
         #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const uint8_t* row = row_of(4 * keys4 + e, true);
-            const bool live = key0 + 4 * keys4 + e < cached;
-            if (Q8) {
-                const uint32_t bytes = *reinterpret_cast<const uint32_t*>(row + 4 * cols4);
-                const _Float16 scale = *reinterpret_cast<const _Float16*>(row + DIM + 2 * (cols4 / 8));
-                #pragma unroll
-                for (int c = 0; c < 4; ++c) v[e][c] = live ? (_Float16)float(int8_t(bytes >> (8 * c))) * scale : (_Float16)0.0f;
+        for (int j = 0; j < PART_KEYS * QUADS / 256; ++j) {
+            const int index = t + 256 * j, key = index / QUADS, quad = index % QUADS, token = key0 + key;
+            const bool live = token >= position && token < cached;
+            const size_t first = ((size_t(seq) * args.span + size_t(live ? token - position : 0)) * args.kv_heads + kvh) * DIM + 4 * quad;
+            if (IN == 2) {
+                const uint2 bits = *reinterpret_cast<const uint2*>(static_cast<const __half*>(source) + first);
+                const __half2 a = *reinterpret_cast<const __half2*>(&bits.x), b = *reinterpret_cast<const __half2*>(&bits.y);
+                x[j][0] = __low2float(a); x[j][1] = __high2float(a); x[j][2] = __low2float(b); x[j][3] = __high2float(b);
             } else {
-                const half4 four = *reinterpret_cast<const half4*>(row + 8 * cols4);
-                #pragma unroll
-                for (int c = 0; c < 4; ++c) v[e][c] = live ? four[c] : (_Float16)0.0f;
+                const float4 four = *reinterpret_cast<const float4*>(static_cast<const float*>(source) + first);
+                x[j][0] = four.x; x[j][1] = four.y; x[j][2] = four.z; x[j][3] = four.w;
             }
         }
+    }
+    #pragma unroll
+    for (int j = 0; j < MINE; ++j)
+        if (old[j]) *reinterpret_cast<uint2*>(&raw[0][0] + 8 * (t + 256 * j)) = held[j];
+    if (IN) {
+        constexpr int QUADS = DIM / 4;
         #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int column = 4 * cols4 + c;
-            // keys 32 part + 16 h + 4 g + (0..3) go to piece 4 part + g, its first (h = 0) or second 8 bytes
-            const int piece = 4 * (keys4 / 8) + keys4 % 4, second = (keys4 / 4) % 2;
-            *reinterpret_cast<half4*>(out + KT + column * (2 * TILE_KEYS) + ((piece ^ ((column >> 1) & 7)) * 16) + 8 * second) = half4{v[0][c], v[1][c], v[2][c], v[3][c]};
+        for (int j = 0; j < PART_KEYS * QUADS / 256; ++j) {
+            const int index = t + 256 * j, key = index / QUADS, quad = index % QUADS, token = key0 + key;
+            const bool live = token >= position && token < cached;
+            uint8_t* page_row = row_in_pool(live ? token : position);
+            if (Q8) {
+                uint32_t word;
+                __half scale16;
+                kv_quad_q8(x[j], word, scale16);
+                if (live) {
+                    *reinterpret_cast<uint32_t*>(page_row + quad * 4) = word;
+                    *reinterpret_cast<uint32_t*>(raw[key] + quad * 4) = word;
+                    if (quad % 8 == 0) {
+                        *reinterpret_cast<__half*>(page_row + DIM + quad / 8 * 2) = scale16;
+                        *reinterpret_cast<__half*>(raw[key] + DIM + quad / 8 * 2) = scale16;
+                    }
+                }
+            } else {
+                kv_store_quad(page_row, unsigned(quad), DIM, false, x[j], live);
+                kv_store_quad(raw[key], unsigned(quad), DIM, false, x[j], live);
+            }
         }
+    }
+    __syncthreads();
+    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+    if (!value) {
+        // K: a thread takes pieces of 8 columns; rows past the sequence's end become zeros
+        #pragma unroll
+        for (int j = 0; j < PART_KEYS * PIECES / 256; ++j) {
+            const int piece = t + 256 * j, key = piece / PIECES, c = piece % PIECES, tile_key = half * PART_KEYS + key;
+            const uint8_t* row = raw[key];
+            half8 values;
+            if (Q8) {
+                const uint2 bytes = *reinterpret_cast<const uint2*>(row + 8 * c);
+                const _Float16 scale = *reinterpret_cast<const _Float16*>(row + DIM + 2 * (c / 4));
+                #pragma unroll
+                for (int i = 0; i < 8; ++i) values[i] = (_Float16)float(int8_t((i < 4 ? bytes.x : bytes.y) >> (8 * (i & 3)))) * scale;
+            } else values = *reinterpret_cast<const half8*>(row + 16 * c);
+            if (key0 + key >= cached) values = half8{};
+            *reinterpret_cast<half8*>(out + tile_key * (2 * DIM) + ((c ^ (tile_key & 15)) * 16)) = values;
+        }
+        return;
+    }
+    // V^T: a thread takes 4 keys x 4 columns
+    static_assert((PART_KEYS / 4) * (DIM / 4) == 256, "one block of 4 keys x 4 columns a thread");
+    const int keys4 = t % (PART_KEYS / 4), cols4 = t / (PART_KEYS / 4);
+    _Float16 v[4][4];       // [key][column]
+    #pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const uint8_t* row = raw[4 * keys4 + e];
+        const bool live = key0 + 4 * keys4 + e < cached;
+        if (Q8) {
+            const uint32_t bytes = *reinterpret_cast<const uint32_t*>(row + 4 * cols4);
+            const _Float16 scale = *reinterpret_cast<const _Float16*>(row + DIM + 2 * (cols4 / 8));
+            #pragma unroll
+            for (int c = 0; c < 4; ++c) v[e][c] = live ? (_Float16)float(int8_t(bytes >> (8 * c))) * scale : (_Float16)0.0f;
+        } else {
+            const half4 four = *reinterpret_cast<const half4*>(row + 8 * cols4);
+            #pragma unroll
+            for (int c = 0; c < 4; ++c) v[e][c] = live ? four[c] : (_Float16)0.0f;
+        }
+    }
+    #pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int column = 4 * cols4 + c;
+        // keys 32 half + 16 h + 4 g + (0..3) go to piece 4 half + g, its first (h = 0) or second 8 bytes
+        const int piece = 4 * half + keys4 % 4, second = keys4 / 4;
+        *reinterpret_cast<half4*>(out + KT + column * (2 * TILE_KEYS) + ((piece ^ ((column >> 1) & 7)) * 16) + 8 * second) = half4{v[0][c], v[1][c], v[2][c], v[3][c]};
     }
 }
 
@@ -705,13 +764,18 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     }
 }
 
+// `tiles`: where the cached rows' FP16 tiles go -- the device's workspace, rebuilt whole on every call, or a buffer the caller
+// keeps between the chunks of a prompt (then `append` may carry the chunk's new rows and the count of positions still valid).
 template<int DIM, int QT, bool Q8>
-void launch_dense(Device& d, const PrefillArgs& args, unsigned seqs) {
+void launch_dense(Device& d, const PrefillArgs& args, unsigned seqs, uint8_t* tiles, const AppendArgs& append, int input) {
     const unsigned tiles_per_seq = unsigned((args.max_context + TILE_KEYS - 1) / TILE_KEYS);
-    auto* tiles = static_cast<uint8_t*>(workspace(d, checked_product({seqs, args.kv_heads, tiles_per_seq, uint64_t(tile_bytes<DIM>())})));
+    if (!tiles) tiles = static_cast<uint8_t*>(workspace(d, checked_product({seqs, args.kv_heads, tiles_per_seq, uint64_t(tile_bytes<DIM>())})));
     constexpr int shared = 4 * tile_bytes<DIM>();
     raise_shared_limit(d, reinterpret_cast<const void*>(&prefill_dense_kernel<DIM, QT>), shared);
-    unpack_tiles_kernel<DIM, Q8><<<dim3(tiles_per_seq, args.kv_heads, seqs), 256, 0, d.stream>>>(args, tiles, tiles_per_seq);
+    const dim3 grid(tiles_per_seq * TILE_PARTS, args.kv_heads, seqs);
+    if (input == 2) unpack_tiles_kernel<DIM, Q8, 2><<<grid, 256, 0, d.stream>>>(args, tiles, tiles_per_seq, append);
+    else if (input == 1) unpack_tiles_kernel<DIM, Q8, 1><<<grid, 256, 0, d.stream>>>(args, tiles, tiles_per_seq, append);
+    else unpack_tiles_kernel<DIM, Q8, 0><<<grid, 256, 0, d.stream>>>(args, tiles, tiles_per_seq, append);
     const unsigned runs = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
     timed_launch(d, &prefill_dense_kernel<DIM, QT>, dim3((runs + 1) / 2, args.kv_heads, seqs), dim3(TEAM * 64), shared, args, tiles, tiles_per_seq);
 }
@@ -746,8 +810,33 @@ void prefill_attention(Device& d, const sdx_kv_pool* pool, const int32_t* page_t
     args.page_last = unsigned(std::min<uint64_t>(pool->page_count - 1, 0x7fffffffu));
     args.out = out; args.out_f16 = out_f16;
     const bool q8 = pool->row_bytes != 2 * pool->dim;
-    if (pool->dim == 128) { if (q8) launch_dense<128, 2, true>(d, args, unsigned(seqs)); else launch_dense<128, 2, false>(d, args, unsigned(seqs)); }
-    else { if (q8) launch<256, 1, true, 2>(d, args, unsigned(seqs)); else launch<256, 1, false, 2>(d, args, unsigned(seqs)); }
+    if (pool->dim == 128) {
+        if (q8) launch_dense<128, 2, true>(d, args, unsigned(seqs), nullptr, AppendArgs{}, 0); else launch_dense<128, 2, false>(d, args, unsigned(seqs), nullptr, AppendArgs{}, 0);
+    } else { if (q8) launch<256, 1, true, 2>(d, args, unsigned(seqs)); else launch<256, 1, false, 2>(d, args, unsigned(seqs)); }
+}
+
+// A prompt chunk in one call: the chunk's K/V rows appended (when given) and its queries attended, the cached rows' tiles kept in
+// the caller's buffer from chunk to chunk.  128 columns.
+void prefill_chunk(Device& d, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
+                   uint64_t max_context, const void* keys, const void* values, int kv_f16, const void* q, int q_f16, uint64_t seqs, uint64_t span,
+                   uint64_t heads, float scale, void* out, int out_f16, void* tiles, const int32_t* valid) {
+    PrefillArgs args{};
+    args.pages = static_cast<const uint8_t*>(pool->pages);
+    args.page_tokens = pool->page_tokens; args.kv_heads = pool->kv_heads; args.heads = unsigned(heads);
+    args.group = unsigned(heads / pool->kv_heads); args.span = unsigned(span);
+    args.page_table = page_table; args.table_stride = size_t(table_stride); args.positions = positions;
+    args.q = q; args.q_f16 = q_f16; args.scale_log2 = scale * 1.44269504088896341f;
+    args.rows = unsigned(span * args.group); args.max_context = int(max_context);
+    args.page_last = unsigned(std::min<uint64_t>(pool->page_count - 1, 0x7fffffffu));
+    args.out = out; args.out_f16 = out_f16;
+    const AppendArgs append{keys, values, valid};
+    const int input = keys ? (kv_f16 ? 2 : 1) : 0;
+    if (pool->row_bytes != 2 * pool->dim) launch_dense<128, 2, true>(d, args, unsigned(seqs), static_cast<uint8_t*>(tiles), append, input);
+    else launch_dense<128, 2, false>(d, args, unsigned(seqs), static_cast<uint8_t*>(tiles), append, input);
+}
+
+uint64_t prefill_tiles_bytes(uint64_t seqs, uint64_t kv_heads, uint64_t max_context) {
+    return checked_product({seqs, kv_heads, (max_context + TILE_KEYS - 1) / TILE_KEYS, uint64_t(tile_bytes<128>())});
 }
 
 // The union walk of a prompt chunk (256 columns): `tokens` rows of one sequence from position `base`, each tile of 64 query rows

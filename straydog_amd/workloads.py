@@ -118,6 +118,7 @@ class PrefillWorkload:
         gpu.fill_normal(self.v.base(), tokens * kv_heads * dim, stream(seed, 2), 1)
         gpu.fill_normal(self.q.base(), tokens * heads * dim, stream(seed, 3), 1)
         self.scratch = gpu.buffer(max(gpu.paged_attention_scratch(1, chunk, heads, dim, tokens), 4))
+        self.tiles = None
         gpu.synchronize()
 
     def step(self):
@@ -128,6 +129,18 @@ class PrefillWorkload:
                        True, 1, self.chunk)
             g.paged_attention(self.pool, self.table_buffer.base(), self.table.shape[1], self.starts.at(4 * c), self.tokens,
                               self.q.at(q_at), True, 1, self.chunk, self.heads, self.scale, self.out.at(q_at), True, self.scratch)
+
+    def step_chunks(self):
+        """The same prompt through sdx_prefill_chunk: K/V append and attention in one call a chunk, the cached rows' operand
+        tiles kept between the chunks (everything before a chunk is valid: `valid` is the chunk's own position)."""
+        g = self.gpu
+        if self.tiles is None:
+            self.tiles = g.buffer(g.prefill_tiles_bytes(1, self.kv_heads, self.dim, self.tokens))
+        for c in range(self.tokens // self.chunk):
+            kv_at, q_at = c * self.chunk * self.kv_heads * self.dim * 2, c * self.chunk * self.heads * self.dim * 2
+            g.prefill_chunk(self.pool, self.table_buffer.base(), self.table.shape[1], self.starts.at(4 * c), self.tokens, self.k.at(kv_at),
+                            self.v.at(kv_at), True, self.q.at(q_at), True, 1, self.chunk, self.heads, self.scale, self.out.at(q_at), True,
+                            self.tiles, self.starts.at(4 * c))
 
     def flops(self):
         # causal only: 2 products x 2 flops per (query row, visible key, column)
@@ -144,8 +157,9 @@ class PrefillWorkload:
         return self.gpu.read_buffer(buffer, 0, np.float16, count).astype(np.float32)
 
     def release(self):
-        for b in (self.pool_buffer, self.table_buffer, self.starts, self.k, self.v, self.q, self.out, self.scratch):
-            self.gpu.release(b)
+        for b in (self.pool_buffer, self.table_buffer, self.starts, self.k, self.v, self.q, self.out, self.scratch, self.tiles):
+            if b is not None:
+                self.gpu.release(b)
 
 
 class SparseWorkload:
