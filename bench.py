@@ -21,6 +21,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+SETTLE_MS = 60.0            # untimed device time of the same steps before every timed pass
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense FP16/BF16 MFMA, published
 
@@ -58,6 +59,20 @@ def timed(gpu, step, steps, warmup):
     for _ in range(warmup):
         step()
     gpu.synchronize()
+    # The box's clocks settle under tens of milliseconds of the same load, whatever --warmup says: the same steps go on, untimed,
+    # until SETTLE_MS of device time have passed (in stretches between two events, so that the queue never runs dry inside one).
+    settled, settle_steps, stretch = 0.0, 0, 4
+    while settled < SETTLE_MS and settle_steps < 20000:
+        begin = gpu.event()
+        for _ in range(stretch):
+            step()
+        end = gpu.event()
+        took = gpu.elapsed_ms(begin, end)
+        gpu.events_clear()
+        settled += took
+        settle_steps += stretch
+        stretch = max(4, min(2000, int(stretch * 10.0 / max(took, 1e-3))))        # about 10 ms a stretch
+    timed.settle_ms, timed.settle_steps = settled, settle_steps
     begin = gpu.event()
     for _ in range(steps):
         step()
@@ -113,6 +128,7 @@ def paged_result(gpu, work, steps, warmup):
         "algorithmic_bytes": size, "gbps": size / ms / 1e6, "frac_of_hbm_peak": size / ms / 1e6 / HBM_PEAK_GBPS,
         "kernel_gbps": None if kernel_ms is None else size / kernel_ms / 1e6,
         "tokens_per_s": work.seqs * work.span / (ms * 1e-3), "tflops": work.flops() / ms / 1e9,
+        "settle_ms": timed.settle_ms, "settle_steps": timed.settle_steps,
     }
 
 
@@ -145,10 +161,10 @@ def cpu_baseline_paged(work, sample_seqs, threads, budget_seconds=12.0):
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    # (the defaults: 200 untimed steps are ~25 ms of the same load -- the memory and fabric clocks of the box take tens of
-    # milliseconds of sustained traffic to settle, and a pass timed after 10 steps reads 1.5-4 % low)
+    # (the memory and fabric clocks of the box take tens of milliseconds of sustained traffic to settle, and a pass timed after
+    # 10 steps reads 1.5-4 % low: whatever --warmup is, every timed pass comes after SETTLE_MS more of the same steps)
     parser.add_argument("--steps", type=int, default=100)
-    parser.add_argument("--warmup", type=int, default=200)
+    parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--workload", default="config1")
     parser.add_argument("--no-also", action="store_true", help="measure only the named workload")
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -231,7 +247,9 @@ def main():
     def run_sparse(with_cpu=True):
         work = workloads.SparseWorkload(gpu)
         ms_index, bounds_ms = timed(gpu, work.step_index, max(args.steps // 5, 3), short_warmup)
+        settle_ms = timed.settle_ms
         ms_attention, gather_ms = timed(gpu, work.step_attention, max(args.steps // 5, 3), short_warmup)
+        settle_ms += timed.settle_ms
         size, keys = work.algorithmic_bytes(), work.batch * work.context * work.index_dim * 2
         sparse_baseline = cpu_baseline_sparse(work) if with_cpu and not args.no_cpu else None
         work.release()
@@ -241,7 +259,7 @@ def main():
                 "kernel_us": None if bounds_ms is None else bounds_ms * 1e3, "key_bytes": keys,
                 "gather_kernel_us": None if gather_ms is None else gather_ms * 1e3,
                 "algorithmic_bytes": size, "gbps": size / total / 1e6, "frac_of_hbm_peak": size / total / 1e6 / HBM_PEAK_GBPS,
-                "cpu_baseline": sparse_baseline}
+                "settle_ms": settle_ms, "cpu_baseline": sparse_baseline}
 
     def cpu_baseline_prefill(work, tokens=(2040, 4090, 6140, 8184), rows=8):
         """The oracle on `rows` consecutive query tokens near the end of each chunk (each attends the cache up to its own position),
@@ -269,18 +287,22 @@ def main():
                 "max_abs_error_vs_oracle_on_sample": error}
 
     def run_prefill(with_cpu=True):
+        # a step = the prompt's four chunks through sdx_prefill_chunk (K/V append + attention in one call a chunk, the cached rows'
+        # operand tiles kept between chunks); the same prompt through sdx_kv_write + sdx_paged_attention is timed beside it
         work = workloads.PrefillWorkload(gpu)
         steps = max(args.steps // 5, 3)
-        ms, kernel_ms = timed(gpu, work.step, steps, short_warmup)
+        separate_ms, _ = timed(gpu, work.step, steps, short_warmup)
+        ms, kernel_ms = timed(gpu, work.step_chunks, steps, short_warmup)
         flops, size = work.flops(), work.algorithmic_bytes()
         prefill_baseline = cpu_baseline_prefill(work) if with_cpu and not args.no_cpu else None
         work.release()
-        # the timed kernel launches are the 4 attention kernels of a step (not the K/V writer, not the kernel that unpacks the tiles)
+        # the timed kernel launches are the 4 attention kernels of a step (not the kernel that appends the rows and builds the tiles)
         return {"ms_per_step": ms, "us_per_step": ms * 1e3, "kernel_us": None if kernel_ms is None else kernel_ms * 4e3, "flops": flops,
                 "tflops": flops / ms / 1e9, "frac_of_mfma_peak": flops / ms / 1e9 / MFMA_PEAK_TFLOPS,
                 "kernel_tflops": None if kernel_ms is None else flops / (4 * kernel_ms) / 1e9,
+                "us_per_step_separate_calls": separate_ms * 1e3,
                 "algorithmic_bytes": size, "gbps": size / ms / 1e6, "frac_of_hbm_peak": size / ms / 1e6 / HBM_PEAK_GBPS,
-                "tokens_per_s": work.tokens / (ms * 1e-3), "cpu_baseline": prefill_baseline}
+                "tokens_per_s": work.tokens / (ms * 1e-3), "settle_ms": timed.settle_ms, "cpu_baseline": prefill_baseline}
 
     def run_block_index():
         # Qwen's block indexer (scores + choice of 512 blocks) at 242K tokens: a decode row, and a prefill chunk of 256 rows
@@ -396,7 +418,7 @@ def main():
                     "measured_mfma_tflops_live_operands": measured_mfma_ceiling(gpu, True)}
     line = {
         "metric": "Q8_0 decode-attn HBM GB/s", "value": main_result["gbps"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": main_result.get("ms_per_step", main_result["us_per_step"] / 1e3), "higher_is_better": True,
+        "warmup": args.warmup, "settle_ms": main_result.get("settle_ms"), "ms_per_step": main_result.get("ms_per_step", main_result["us_per_step"] / 1e3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "int8 K/V x fp16 MFMA, fp32 accumulate", "data": "synthetic",
         "config": {"workload": names[args.workload], "batch": 32 if args.workload.startswith("config1") else None},
         "tokens_per_s": main_result.get("tokens_per_s"), "frac_of_hbm_peak": main_result["frac_of_hbm_peak"],
