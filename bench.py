@@ -351,9 +351,29 @@ def main():
                 stage.release()
         return out
 
+    def run_host_resident():
+        # the selection-list attention of rows at 242K tokens when the sequence's K/V rows are not in HBM: read over the bus entry by
+        # entry (a pool in mapped host memory), or through the union of the selected blocks gathered into a VRAM stage first
+        # (sdx_kv_cache_gather over a sequence parked in the cache's host tier); the same rows from HBM beside them, same bits
+        out = {}
+        for name, rows, similar in (("decode_row", 1, False), ("verify_rows_5", 5, False), ("prefill_chunk_256_similar_queries", 256, True)):
+            work = workloads.HostResidentWorkload(gpu, rows, similar)
+            resident_ms, _ = timed(gpu, work.step_resident, max(args.steps // 5, 3), 2)
+            want = work.read_output()
+            bus_ms, _ = timed(gpu, work.step_over_the_bus, 3, 1)
+            same = bool(np.array_equal(work.read_output(), want))
+            work.park()
+            gathered_ms, _ = timed(gpu, work.step_gathered, 3, 1)
+            same = same and bool(np.array_equal(work.read_output(), want))
+            out[name] = {"rows": rows, "resident_in_hbm_us": resident_ms * 1e3, "read_over_the_bus_us": bus_ms * 1e3, "union_gathered_us": gathered_ms * 1e3,
+                         "union_positions": work.union_positions, "gather_calls": work.gather_calls, "selected_positions": rows * 2051,
+                         "same_bits_as_resident": same}
+            work.release()
+        return out
+
     if args.workload == "block_index":
         # the Qwen block indexer alone (what profiles/block_index_242k.md traces): not a BASELINE config, no headline metric
-        print(json.dumps({"workload": "Qwen block indexer at 242K tokens", "steps": args.steps, **run_block_index()}))
+        print(json.dumps({"workload": "Qwen block indexer at 242K tokens", "steps": args.steps, **run_block_index(), "host_resident_242k": run_host_resident()}))
         gpu.close()
         return
     if args.workload == "config4":
@@ -399,6 +419,8 @@ def main():
                                                "traffic": PROFILED_TRAFFIC["config4"][0], "kernel": "index_interval_kernel<64>", "kernel_us": also["config4"]["kernel_us"]}
         also["block_index_242k"] = run_block_index()
         also["block_index_242k"]["workload"] = "Qwen block indexer: 4x128 index heads, 60.5K complete blocks of a 262144-token context, top 512 blocks"
+        also["host_resident_242k"] = run_host_resident()
+        also["host_resident_242k"]["workload"] = "selection-list attention at 242K tokens (24q/2kv heads, 256 columns, Q8_0) over K/V rows that are not in HBM"
 
     kernel_us = main_result.get("kernel_us")
     achieved = main_result["algorithmic_bytes"] / (kernel_us * 1e-6) / 1e9 if kernel_us else main_result["gbps"]

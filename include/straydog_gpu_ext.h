@@ -84,6 +84,23 @@ int sdx_kv_cache_stage(void* handle, void* cache, uint64_t sequence, uint64_t to
 int sdx_kv_cache_unstage(void* handle, void* cache, uint64_t sequence, uint64_t first, uint64_t count);
 int sdx_kv_cache_grow(void* handle, void* cache, uint64_t pages);
 int sdx_kv_cache_residency(void* handle, void* cache, uint64_t sequence, uint64_t* parked, uint64_t* host_pages_free, uint64_t* staged_pages);
+/* The union gather for a sparse (selection-list) pass over a sequence whose rows are not in HBM -- the reference's qsa_mark_selection,
+ * qsa_place_union, qsa_gather_union and qsa_renumber_selection as qsa_attention_gathered drives them (gpu/sparse_attention_compute.hpp:
+ * 677-733, gpu/prefill_batch.hpp:224-254, kv_union_count gpu/kv_stage.hpp:166-172).  The blocks of four positions that the selections
+ * of query rows first .. first + rows - 1 name (entries that count by sdx_selected_attention's rule, row r at position base + r) are
+ * copied once, in block order, from the sequence's pages -- the host tier of a parked sequence, read over the bus, or the pool -- into
+ * the VRAM stage registered with sd_kv_stage, and the lists are renumbered to the places there (renumbered: [.][selected] floats at
+ * the same rows; an entry that does not count becomes -1): a row then attends the same keys and values in the same order, the same
+ * bits, through pool / page_table / table_stride (the stage in the pool's page layout) with the same context, positions and counts:
+ *     sdx_selected_attention(handle, pool, page_table, context, base + first, NULL, renumbered + first * selected, selected,
+ *                            counts + first, q of row first, ..., *taken rows, ...)
+ * *taken: how many of the rows the stage holds the union of -- the rows are halved until their union fits (0: the stage is too small
+ * for a single row's selection; nothing was gathered); the caller attends those and calls again from first + *taken.  *union_rows
+ * (may be null): the positions gathered.  The union's size is read back from the device at each attempt (the call waits for the
+ * stream, as the reference's does), so it cannot be recorded into a graph; what the stage held before is forgotten. */
+int sdx_kv_cache_gather(void* handle, void* cache, uint64_t sequence, uint64_t context, uint64_t base, const float* indices, uint64_t selected,
+                        const float* counts, uint64_t first, uint64_t rows, float* renumbered, uint64_t* taken, uint64_t* union_rows, sdx_kv_pool* pool,
+                        const int32_t** page_table, uint64_t* table_stride);
 
 /* Causal grouped-query attention over the paged cache: the attention step of a decode (span 1), a speculative
  * verify (span <= 8) or a prefill chunk (any span), i.e. qsa_decode_parts/qsa_decode_merge, qsa_flash and

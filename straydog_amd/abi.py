@@ -100,6 +100,8 @@ SIGNATURES = {
     "sdx_kv_cache_unstage": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64]),
     "sdx_kv_cache_grow": (c_int, [c_void_p, c_void_p, c_u64]),
     "sdx_kv_cache_residency": (c_int, [c_void_p, c_void_p, c_u64, _P(c_u64), _P(c_u64), _P(c_u64)]),
+    "sdx_kv_cache_gather": (c_int, [c_void_p, c_void_p, c_u64, c_u64, c_u64, c_void_p, c_u64, c_void_p, c_u64, c_u64, c_void_p, _P(c_u64), _P(c_u64), _P(KvPool),
+                                    _P(c_void_p), _P(c_u64)]),
     "sdx_kv_write": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_void_p, c_void_p, c_int, c_u64, c_u64]),
     "sdx_paged_attention_scratch": (c_u64, [c_u64, c_u64, c_u64, c_u64, c_u64]),
     "sdx_paged_attention": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_u64, c_void_p, c_int, c_u64, c_u64, c_u64,

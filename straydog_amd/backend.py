@@ -247,6 +247,15 @@ class Backend:
         self.check(self.lib.sdx_kv_cache_stage(self.handle, cache, sequence, tokens, ctypes.byref(pool), ctypes.byref(table), ctypes.byref(stride)))
         return pool, table.value, stride.value
 
+    def kv_cache_gather(self, cache, sequence, context, base, indices, selected, counts, first, rows, renumbered):
+        """The union of the selections of rows first .. first + rows - 1 copied into the VRAM stage and the lists renumbered:
+        (rows taken, positions gathered, pool struct, device page table, table stride)."""
+        taken, gathered = abi.c_u64(), abi.c_u64()
+        pool, table, stride = abi.KvPool(), ctypes.c_void_p(), abi.c_u64()
+        self.check(self.lib.sdx_kv_cache_gather(self.handle, cache, sequence, context, base, indices, selected, counts, first, rows, renumbered,
+                                                ctypes.byref(taken), ctypes.byref(gathered), ctypes.byref(pool), ctypes.byref(table), ctypes.byref(stride)))
+        return taken.value, gathered.value, pool, table.value, stride.value
+
     def kv_cache_unstage(self, cache, sequence, first, count):
         self.check(self.lib.sdx_kv_cache_unstage(self.handle, cache, sequence, first, count))
 

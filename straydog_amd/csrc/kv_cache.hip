@@ -116,6 +116,108 @@ void copy_rows(KvCache& c, Device& d, int32_t source, int32_t copy, size_t rows)
                                 hipMemcpyDeviceToDevice, d.stream));
 }
 
+
+// ---- the union gather (reference gpu/sparse_attention_compute.hpp:677-733) ------------------------------------------------
+// Rows of a sequence whose pages are not in HBM would be read over the bus entry by entry, by every query row that names them.
+// Instead the blocks of four rows that the rows' selections name are copied once, in block order, into the VRAM stage, and each
+// selection is renumbered to the places there: a row reads the same keys and values in the same order, from HBM.
+
+// marks[block] = 1 for every block of four positions that an entry which counts names (the rule of the selection-list attention:
+// entry j < min(selected, counts[row]) counts iff 0 <= raw <= base + row and raw < context).  A workgroup a row.
+__global__ void __launch_bounds__(256) union_mark_kernel(const float* indices, const float* counts, size_t selected, size_t first, size_t base, size_t context,
+                                                         uint32_t* marks) {
+    const size_t row = first + blockIdx.x;
+    const float* list = indices + row * selected;
+    const float stated = counts[row];
+    const size_t count = stated > 0.0f ? min(selected, size_t(stated)) : 0;
+    const float limit = float(base + row);
+    for (size_t j = threadIdx.x; j < count; j += 256) {
+        const float raw = list[j];
+        if (raw >= 0.0f && raw <= limit && raw < float(context)) marks[size_t(raw) / 4] = 1u;
+    }
+}
+
+// The union's places, in two launches of a workgroup per 1024 blocks: first each stretch's count of marked blocks, then
+// marks[block] becomes the number of marked blocks before it, blocks[place] the block in that place, marks[end] the union's size.
+__global__ void __launch_bounds__(1024) union_count_kernel(const uint32_t* marks, size_t end, uint32_t* stretch_counts) {
+    __shared__ uint32_t wave_sums[16];
+    const size_t block = size_t(blockIdx.x) * 1024 + threadIdx.x;
+    const bool marked = block < end && marks[block] != 0;
+    const uint64_t votes = __ballot(marked);
+    if ((threadIdx.x & 63) == 0) wave_sums[threadIdx.x >> 6] = uint32_t(__popcll(votes));
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t total = 0;
+        #pragma unroll
+        for (int w = 0; w < 16; ++w) total += wave_sums[w];
+        stretch_counts[blockIdx.x] = total;
+    }
+}
+__global__ void __launch_bounds__(1024) union_place_kernel(uint32_t* marks, size_t end, const uint32_t* stretch_counts, uint32_t* blocks) {
+    __shared__ uint32_t wave_sums[16];
+    __shared__ uint32_t before_stretch;
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t block = size_t(blockIdx.x) * 1024 + threadIdx.x;
+    const bool marked = block < end && marks[block] != 0;
+    const uint64_t votes = __ballot(marked);
+    if (lane == 0) wave_sums[wave] = uint32_t(__popcll(votes));
+    if (wave == 15) {
+        // the stretches before this one, added up by one wave
+        uint32_t sum = 0;
+        for (unsigned i = lane; i < blockIdx.x; i += 64) sum += stretch_counts[i];
+        #pragma unroll
+        for (unsigned offset = 32; offset; offset >>= 1) sum += __shfl_xor(sum, offset);
+        if (lane == 0) before_stretch = sum;
+    }
+    __syncthreads();
+    uint32_t at = before_stretch + uint32_t(__popcll(votes & ((uint64_t(1) << lane) - 1)));
+    #pragma unroll
+    for (unsigned w = 0; w < 16; ++w) if (w < wave) at += wave_sums[w];
+    if (block < end) {
+        marks[block] = at;
+        if (marked) blocks[at] = uint32_t(block);
+    }
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 1023) marks[end] = at + (marked ? 1u : 0u);
+}
+
+// Place p's four rows of every plane, from the sequence's pages (in HBM, or in the cache's host tier: over the bus) into
+// positions 4p .. 4p + 3 of the stage, which has the pool's page layout.  A workgroup a place, 16 bytes a thread at a time (four
+// rows of a plane follow one another and start on a 16-byte boundary: a block never straddles a page).
+__global__ void __launch_bounds__(256) union_gather_kernel(const uint8_t* source, const int32_t* table, unsigned page_last, unsigned page_tokens, unsigned planes,
+                                                           unsigned row_bytes, const uint32_t* blocks, uint8_t* stage) {
+    const size_t place = blockIdx.x, block = blocks[place];
+    const size_t pieces = size_t(4) * row_bytes / 16, plane_bytes = size_t(page_tokens) * row_bytes;
+    const size_t from_token = block * 4, to_token = place * 4;
+    const unsigned entry = unsigned(table[from_token / page_tokens]);
+    const uint8_t* from = source + size_t(min(entry, page_last)) * planes * plane_bytes + (from_token % page_tokens) * row_bytes;
+    uint8_t* to = stage + (to_token / page_tokens) * planes * plane_bytes + (to_token % page_tokens) * row_bytes;
+    for (size_t i = threadIdx.x; i < planes * pieces; i += 256) {
+        const size_t plane = i / pieces, piece = i % pieces;
+        reinterpret_cast<uint4*>(to + plane * plane_bytes)[piece] = reinterpret_cast<const uint4*>(from + plane * plane_bytes)[piece];
+    }
+}
+
+// The rows' lists renumbered to the union's places; an entry that does not count becomes -1 (which never counts).
+__global__ void __launch_bounds__(256) union_renumber_kernel(const float* indices, const float* counts, size_t selected, size_t first, size_t base, size_t context,
+                                                             const uint32_t* places, float* renumbered) {
+    const size_t row = first + blockIdx.x;
+    const float* list = indices + row * selected;
+    float* out = renumbered + row * selected;
+    const float stated = counts[row];
+    const size_t count = stated > 0.0f ? min(selected, size_t(stated)) : 0;
+    const float limit = float(base + row);
+    for (size_t j = threadIdx.x; j < selected; j += 256) {
+        const float raw = list[j];
+        const bool counted = j < count && raw >= 0.0f && raw <= limit && raw < float(context);
+        out[j] = counted ? float(size_t(places[size_t(raw) / 4]) * 4 + size_t(raw) % 4) : -1.0f;
+    }
+}
+
+__global__ void __launch_bounds__(256) union_clear_kernel(uint32_t* words, size_t count) {
+    const size_t i = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (i < count) words[i] = 0u;
+}
+
 }  // namespace
 
 extern "C" {
@@ -409,6 +511,71 @@ int sdx_kv_cache_residency(void* handle, void* cache, uint64_t sequence, uint64_
     if (parked) *parked = c.parked[sequence];
     if (host_pages_free) *host_pages_free = c.free_host.size();
     if (staged_pages) *staged_pages = value.kv_stage_owner == &c && value.kv_stage_sequence == sequence ? value.kv_stage_pages : 0;
+    SD_OP_END
+}
+
+int sdx_kv_cache_gather(void* handle, void* cache, uint64_t sequence, uint64_t context, uint64_t base, const float* indices, uint64_t selected,
+                        const float* counts, uint64_t first, uint64_t rows, float* renumbered, uint64_t* taken, uint64_t* union_rows, sdx_kv_pool* pool,
+                        const int32_t** page_table, uint64_t* table_stride) {
+    SD_OP_BEGIN
+    KvCache& c = cache_of(value, cache);
+    check_sequence(c, sequence);
+    if (value.recording) throw std::runtime_error("Straydog K/V cache: the union gather reads its size back and cannot be recorded");
+    const size_t bytes = page_bytes(c), room = value.kv_stage ? value.kv_stage_bytes / bytes : 0, tokens = c.pool.page_tokens;
+    if (!room) throw std::runtime_error("Straydog K/V cache: no K/V stage is registered (sd_kv_stage)");
+    if (!rows || rows > 65535 || !selected || selected > (uint64_t(1) << 20) || !context || context > (uint64_t(1) << 24) || !taken || first > (uint64_t(1) << 24) ||
+        base > (uint64_t(1) << 24) || base + first + rows > context)
+        throw std::runtime_error("invalid Straydog union gather");
+    if (pages_for(c, context) > c.held[sequence]) throw std::runtime_error("Straydog K/V cache: the sequence holds fewer rows");
+    op_span(value, indices, checked_floats({first + rows, selected}), "selection lists");
+    op_span(value, counts, checked_floats({first + rows}), "selection counts");
+    op_span(value, renumbered, checked_floats({first + rows, selected}), "renumbered selection lists");
+    if (!c.stage_table) {
+        std::vector<int32_t> places(c.stride);
+        for (size_t i = 0; i < c.stride; ++i) places[i] = int32_t(i);
+        c.stage_table = static_cast<int32_t*>(allocate(value, c.stride * sizeof(int32_t), false));
+        upload(value, c.stage_table, places.data(), c.stride * sizeof(int32_t));
+    }
+    // where the sequence's pages are: the host tier (the device's table row then names host pages) or the pool
+    const bool parked = c.parked[sequence] != 0;
+    const uint8_t* source = parked ? c.host : static_cast<const uint8_t*>(c.pool.pages);
+    const unsigned page_last = unsigned((parked ? c.host_pages : size_t(c.pool.page_count)) - 1);
+    if (parked) upload_entries(c, sequence, 0, c.held[sequence]);
+    kv_settle(value);                   // (a parked sequence's rows may still be on their way to the host tier)
+    forget_stage(value, c, sequence);
+    value.kv_stage_owner = nullptr; value.kv_stage_pages = 0;         // what the stage held, a prefix of some sequence, is gone
+    const size_t end = size_t((base + first + rows - 1) / 4 + 1), capacity = room * tokens;
+    const unsigned stretches = checked_blocks(end, 1024);
+    uint32_t* marks = static_cast<uint32_t*>(workspace(value, checked_floats({2 * uint64_t(end) + 2 + stretches})));
+    uint32_t* blocks = marks + end + 1;
+    uint32_t* stretch_counts = blocks + end;
+    // as many of the rows as the stage holds the union of: halved until it fits (the union's size is read back each time)
+    size_t count = size_t(rows);
+    uint32_t total = 0;
+    for (;;) {
+        union_clear_kernel<<<checked_blocks(end + 1), 256, 0, value.stream>>>(marks, end + 1);
+        union_mark_kernel<<<unsigned(count), 256, 0, value.stream>>>(indices, counts, size_t(selected), size_t(first), size_t(base), size_t(context), marks);
+        union_count_kernel<<<stretches, 1024, 0, value.stream>>>(marks, end, stretch_counts);
+        union_place_kernel<<<stretches, 1024, 0, value.stream>>>(marks, end, stretch_counts, blocks);
+        SD_CHECK(hipGetLastError());
+        SD_CHECK(hipMemcpyAsync(value.arena, marks + end, 4, hipMemcpyDeviceToHost, value.stream));
+        SD_CHECK(hipStreamSynchronize(value.stream));
+        std::memcpy(&total, value.arena, 4);
+        if (size_t(total) * 4 <= capacity || count == 1) break;
+        count = (count + 1) / 2;
+    }
+    if (size_t(total) * 4 > capacity) count = 0;        // (a stage too small for one row's selection: nothing is gathered)
+    if (count) {
+        if (total)
+            union_gather_kernel<<<total, 256, 0, value.stream>>>(source, c.table + size_t(sequence) * c.stride, page_last, c.pool.page_tokens, 2 * c.pool.kv_heads,
+                                                                c.pool.row_bytes, blocks, static_cast<uint8_t*>(value.kv_stage));
+        union_renumber_kernel<<<unsigned(count), 256, 0, value.stream>>>(indices, counts, size_t(selected), size_t(first), size_t(base), size_t(context), marks, renumbered);
+    }
+    *taken = count;
+    if (union_rows) *union_rows = count ? uint64_t(total) * 4 : 0;
+    if (pool) *pool = sdx_kv_pool{value.kv_stage, room, c.pool.page_tokens, c.pool.kv_heads, c.pool.dim, c.pool.row_bytes};
+    if (page_table) *page_table = c.stage_table;
+    if (table_stride) *table_stride = c.stride;
     SD_OP_END
 }
 

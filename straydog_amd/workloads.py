@@ -312,6 +312,85 @@ class BlockIndexWorkload:
             self.gpu.release(self.union_scratch)
 
 
+class HostResidentWorkload:
+    """A sparse (selection-list) pass over a Qwen-shaped sequence at 242K tokens whose K/V rows are not in HBM: the same rows'
+    selections attended (a) from the pool in HBM, (b) from a pool in mapped host memory, every selected row read over the bus,
+    (c) from a sequence parked in the cache's host tier, through the union of the selected blocks gathered into a VRAM stage
+    (sdx_kv_cache_gather).  The selections are the block indexer's own (BlockIndexWorkload)."""
+
+    def __init__(self, gpu, steps, similar=False, base=242000, heads=24, kv_heads=2, row_bytes=272, page_tokens=256, stage_positions=65536, seed=11):
+        self.gpu, self.steps, self.base, self.heads, self.kv_heads = gpu, steps, base, heads, kv_heads
+        self.context = base + steps
+        pages = (self.context + page_tokens - 1) // page_tokens
+        self.index = BlockIndexWorkload(gpu, steps, base=base)
+        if similar:
+            self.index.similar_queries()
+        self.index.step()
+        self.cache, *_ = gpu.kv_cache(pages, page_tokens, kv_heads, 256, row_bytes, 1, pages * page_tokens)
+        gpu.kv_cache_host(self.cache, pages)
+        gpu.kv_cache_reserve(self.cache, 0, self.context)
+        self.pool, self.table, self.stride = gpu.kv_cache_view(self.cache)
+        k, start = gpu.buffer(8192 * kv_heads * 256 * 2), gpu.buffer(4)
+        for first in range(0, self.context, 8192):
+            gpu.fill_normal(k.base(), 8192 * kv_heads * 256, stream(seed, 3 + first), 1)
+            gpu.write_buffer(start, 0, np.array([first], dtype=np.int32))
+            gpu.kv_write(self.pool, self.table, self.stride, start.base(), k.base(), k.base(), True, 1, min(8192, self.context - first))
+        page_bytes = 2 * kv_heads * page_tokens * row_bytes
+        # the same bytes in mapped host memory, under the same page table
+        from . import abi
+        self.mapped = gpu.host_state(pages * page_bytes)
+        gpu.copy(self.mapped.base(), self.pool.pages, pages * page_bytes)
+        self.mapped_pool = abi.KvPool(self.mapped.base(), pages, page_tokens, kv_heads, 256, row_bytes)
+        self.stage = gpu.buffer(stage_positions // page_tokens * page_bytes)
+        gpu.kv_stage(self.stage.base(), self.stage.size // 4096)
+        self.q = gpu.buffer(steps * heads * 256 * 2)
+        gpu.fill_normal(self.q.base(), steps * heads * 256, stream(seed, 4), 1)
+        self.out = gpu.buffer(steps * heads * 256 * 2)
+        self.renumbered = gpu.buffer(steps * 2052 * 4)
+        self.scratch = gpu.buffer(gpu.selected_attention_scratch(steps, kv_heads, 2052))
+        self.parked, self.union_positions, self.gather_calls = False, 0, 0
+        gpu.synchronize()
+        gpu.release(k); gpu.release(start)
+
+    def _attend(self, pool, table, first=0, rows=None, indices=None):
+        rows = self.steps if rows is None else rows
+        indices = self.index.indices if indices is None else indices
+        self.gpu.selected_attention(pool, table, self.context, self.base + first, indices.at(first * 2052 * 4), 2052, self.index.counts.at(first * 4),
+                                    self.q.at(first * self.heads * 256 * 2), True, rows, self.heads, 0.0625, self.out.at(first * self.heads * 256 * 2), True,
+                                    self.scratch)
+
+    def step_resident(self):
+        self._attend(self.pool, self.table)
+
+    def step_over_the_bus(self):
+        self._attend(self.mapped_pool, self.table)
+
+    def park(self):
+        self.gpu.kv_cache_park(self.cache, 0)
+        self.parked = True
+
+    def step_gathered(self):
+        first, self.union_positions, self.gather_calls = 0, 0, 0
+        while first < self.steps:
+            taken, gathered, view, table, _ = self.gpu.kv_cache_gather(self.cache, 0, self.context, self.base, self.index.indices.base(), 2052,
+                                                                      self.index.counts.base(), first, self.steps - first, self.renumbered.base())
+            if not taken:
+                raise RuntimeError("the stage does not hold one row's selection")
+            self._attend(view, table, first, taken, self.renumbered)
+            first += taken
+            self.union_positions += gathered
+            self.gather_calls += 1
+
+    def read_output(self):
+        return self.gpu.read_buffer(self.out, 0, np.float16, self.steps * self.heads * 256)
+
+    def release(self):
+        self.index.release()
+        for b in (self.mapped, self.stage, self.q, self.out, self.renumbered, self.scratch):
+            self.gpu.release(b)
+        self.gpu.kv_cache_destroy(self.cache)
+
+
 class QwenStageWorkload:
     """The whole attention stage of a Qwen decode / verification pass in one call (sdx_qsa_decode_attend) at 242K tokens:
     24 query / 2 K/V heads of 256 columns, Q8_0 rows in the reference's state layout, 4 x 128 index heads."""

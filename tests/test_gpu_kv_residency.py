@@ -312,3 +312,106 @@ def test_a_recorded_step_runs_after_the_page_moves_queued_before_it(gpu, oracle)
     for b in (kb, vb, zero, qb, pb, out, scratch):
         gpu.release(b)
     gpu.kv_cache_destroy(cache)
+
+
+def _selections(rng, base, rows, context, blocks=512):
+    """Selection lists as the Qwen block selection leaves them: `blocks` complete blocks of four positions in block order, then
+    the positions of the row's incomplete block; floats, with the counts."""
+    selected = 4 * blocks + 4
+    indices = np.full((rows, selected), -7.0, np.float32)
+    counts = np.zeros(rows, np.float32)
+    for r in range(rows):
+        position = base + r
+        complete = (position + 1) // 4
+        chosen = np.sort(rng.choice(complete, size=min(blocks, complete), replace=False))
+        listed = (chosen[:, None] * 4 + np.arange(4)[None, :]).reshape(-1)
+        tail = np.arange(complete * 4, position + 1)
+        entries = np.concatenate([listed, tail]).astype(np.float32)
+        indices[r, :entries.size] = entries
+        counts[r] = entries.size
+    return indices, counts, selected
+
+
+def test_a_sparse_pass_over_a_parked_sequence_gathers_the_union_of_its_selections(gpu, oracle):
+    """The union gather (the reference's qsa_attention_gathered, gpu/prefill_batch.hpp:224-254): a Qwen-shaped sequence of 242K
+    tokens is attended through selection lists where it lives in HBM, then parked in host memory and attended again through the
+    blocks its selections name, copied into a small VRAM stage and renumbered: the same bits, for a decode row, a verification span
+    and a run of prompt rows whose union the stage only holds a few rows of at a time."""
+    page, kvh, dim, row, heads, context = 256, 2, 256, 272, 24, 242000
+    pages = (context + page - 1) // page
+    rng = np.random.default_rng(76)
+    cache, *_ = gpu.kv_cache(pages + 1, page, kvh, dim, row, 2, pages * page)
+    gpu.kv_cache_host(cache, pages)
+    gpu.kv_cache_reserve(cache, 0, context)
+    pool, table, stride = gpu.kv_cache_view(cache)
+    # the rows: seeded values drawn on the device, appended a stretch at a time
+    stretch = 16384
+    kb, vb, pb = gpu.buffer(stretch * kvh * dim * 2), gpu.buffer(stretch * kvh * dim * 2), gpu.buffer(4)
+    for at in range(0, context, stretch):
+        count = min(stretch, context - at)
+        gpu.fill_normal(kb.base(), count * kvh * dim, 1000 + at, 1)
+        gpu.fill_normal(vb.base(), count * kvh * dim, 5000 + at, 1)
+        gpu.write_buffer(pb, 0, np.array([at], np.int32))
+        gpu.kv_write(pool, table, stride, pb.base(), kb.base(), vb.base(), True, 1, count)
+    stage_pages = 48                                                     # 12288 positions: a decode row names 2052, five rows about 10200
+    page_bytes = 2 * kvh * page * row
+    stage = gpu.buffer(stage_pages * page_bytes)
+    gpu.kv_stage(stage.base(), stage_pages * page_bytes // 4096)
+    scale = 1.0 / 16.0
+    cases = []
+    for rows, base in ((1, context - 1), (5, context - 5), (40, context - 40)):
+        indices, counts, selected = _selections(rng, base, rows, context)
+        if rows == 5:
+            # entries that do not count stay out of the union: a position after the row's own, a negative one, entries past the count
+            indices[1, 3] = float(base + 1 + 3)
+            indices[2, 0] = -1.0
+            counts[3] = 1000.0
+        q = rng.standard_normal((rows, heads, dim)).astype(np.float32)
+        ib, cb, qb = gpu.upload(indices), gpu.upload(counts), gpu.upload(q)
+        out = gpu.buffer(rows * heads * dim * 4)
+        scratch = gpu.buffer(gpu.selected_attention_scratch(rows, kvh, selected))
+        gpu.selected_attention(pool, table, context, base, ib.base(), selected, cb.base(), qb.base(), False, rows, heads, scale, out.base(), False, scratch)
+        resident = gpu.read_buffer(out, 0, np.float32, rows * heads * dim)
+        assert np.all(np.isfinite(resident)) and np.abs(resident).max() > 0
+        cases.append((rows, base, selected, ib, cb, qb, out, scratch, resident, indices, counts))
+    gpu.kv_cache_park(cache, 0)
+    assert gpu.kv_cache_residency(cache, 0)[0]
+    for rows, base, selected, ib, cb, qb, out, scratch, resident, indices, counts in cases:
+        renumbered = gpu.buffer(rows * selected * 4)
+        gpu.write_buffer(out, 0, np.zeros(rows * heads * dim, np.float32))
+        first, calls = 0, 0
+        while first < rows:
+            taken, gathered, view, view_table, view_stride = gpu.kv_cache_gather(cache, 0, context, base, ib.base(), selected, cb.base(), first, rows - first,
+                                                                                renumbered.base())
+            assert 1 <= taken <= rows - first and 0 < gathered <= stage_pages * page and view.pages == stage.base()
+            gpu.selected_attention(view, view_table, context, base + first, renumbered.at(first * selected * 4), selected, cb.at(first * 4),
+                                   qb.at(first * heads * dim * 4), False, taken, heads, scale, out.at(first * heads * dim * 4), False, scratch)
+            first += taken
+            calls += 1
+        assert np.array_equal(gpu.read_buffer(out, 0, np.float32, rows * heads * dim), resident), f"{rows} rows from the stage"
+        assert calls == 1 if rows <= 5 else calls > 1, "the long run's union does not fit the stage at once"
+        listed = gpu.read_buffer(renumbered, 0, np.float32, rows * selected).reshape(rows, selected)
+        if rows == 5:
+            # the lists' places follow block order, and what did not count is -1
+            assert listed[1, 3] == -1.0 and listed[2, 0] == -1.0 and np.all(listed[3, 1000:] == -1.0) and np.all(listed[0, int(counts[0]):] == -1.0)
+            kept = listed[0, :int(counts[0])]
+            assert np.all(np.diff(kept) > 0) and np.all(kept <= indices[0, :int(counts[0])])
+        for b in (renumbered, ib, cb, qb, out, scratch):
+            gpu.release(b)
+    # a stage too small for one row's selection takes nothing and says so
+    gpu.release(stage)
+    small = gpu.buffer(4 * page_bytes)
+    gpu.kv_stage(small.base(), 4 * page_bytes // 4096)
+    indices, counts, selected = _selections(rng, context - 1, 1, context)
+    ib, cb, rb = gpu.upload(indices), gpu.upload(counts), gpu.buffer(selected * 4)
+    taken, gathered, *_ = gpu.kv_cache_gather(cache, 0, context, context - 1, ib.base(), selected, cb.base(), 0, 1, rb.base())
+    assert (taken, gathered) == (0, 0)
+    with pytest.raises(StraydogError, match="invalid Straydog union gather"):
+        gpu.kv_cache_gather(cache, 0, context, context, ib.base(), selected, cb.base(), 0, 1, rb.base())
+    with pytest.raises(StraydogError, match="holds fewer rows"):
+        gpu.kv_cache_gather(cache, 1, context, 0, ib.base(), selected, cb.base(), 0, 1, rb.base())
+    # back in HBM the sequence is what it was
+    gpu.kv_cache_resume(cache, 0)
+    for b in (small, ib, cb, rb, kb, vb, pb):
+        gpu.release(b)
+    gpu.kv_cache_destroy(cache)
