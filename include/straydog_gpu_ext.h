@@ -214,6 +214,20 @@ uint64_t sdx_qsa_decode_attend_scratch(uint64_t steps, uint64_t heads, uint64_t 
 int sdx_qsa_decode_attend(void* handle, const sdx_qsa_state* state, float* projections, uint64_t stride, uint64_t steps, const uint32_t* positions,
                           const uint32_t* ropes, void* scratch, uint64_t scratch_bytes, float* attended);
 
+/* The attention stage of a prompt chunk in one call: the stage of the reference's qsa_prefill for a span of rows at the consecutive
+ * positions base .. base + steps - 1 (gpu/sparse_attention.hpp:444-506: qsa_normalize, the K/V write, qsa_pool + qsa_save_history
+ * :497-501, the selection -- qsa_iv_chunk gpu/qsa_interval.hpp:601-626 past 32768 positions, qsa_index_exact before --, the
+ * attention over each row's selection gpu/qsa_prompt_attention.hpp:220-234 and qsa_gate).  projections as for sdx_qsa_decode_attend
+ * (index queries normalised in place); rope positions are the positions.  The values of the separate entry points, bit for bit:
+ * sdx_qsa_normalize on queries, keys and index queries, sdx_kv_write, sdx_qsa_pool over the span, sdx_qsa_index_interval,
+ * sdx_selected_attention with the gate.  attended: [steps][heads][256] FP32.  scratch: sdx_qsa_prefill_attend_scratch bytes on a
+ * 256-byte boundary; its tail holds the interval scheme's packed keys, which are carried from chunk to chunk when the caller passes
+ * the same scratch and the `valid` its last call left (host, in and out, may be null; 0 after the pooled keys' earlier blocks
+ * changed), as for sdx_qsa_index_interval. */
+uint64_t sdx_qsa_prefill_attend_scratch(uint64_t steps, uint64_t heads, uint64_t kv_heads, uint64_t context);
+int sdx_qsa_prefill_attend(void* handle, const sdx_qsa_state* state, float* projections, uint64_t stride, uint64_t steps, uint64_t base, void* scratch,
+                           uint64_t scratch_bytes, uint64_t* valid, float* attended);
+
 /* Selection-list attention over K/V rows of 256 columns (Q8_0 or FP16): the reference's qsa_attention / qsa_attention_rows
  * (gpu/sparse_attention_compute.hpp:609-647: qsa_decode_parts :41-135 + qsa_decode_merge :139-170) followed by qsa_gate
  * (gpu/sparse_attention.hpp:439-442).  Row r, at position base + r (or *dynamic_base + r, a device-resident position),

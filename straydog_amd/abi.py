@@ -127,6 +127,8 @@ SIGNATURES = {
                                              c_u64, c_u64, c_float, c_void_p, c_u64, c_u64, c_void_p, c_int, c_void_p, c_u64]),
     "sdx_qsa_decode_attend_scratch": (c_u64, [c_u64, c_u64, c_u64, c_u64]),
     "sdx_qsa_decode_attend": (c_int, [c_void_p, _P(QsaState), c_void_p, c_u64, c_u64, c_void_p, c_void_p, c_void_p, c_u64, c_void_p]),
+    "sdx_qsa_prefill_attend_scratch": (c_u64, [c_u64, c_u64, c_u64, c_u64]),
+    "sdx_qsa_prefill_attend": (c_int, [c_void_p, _P(QsaState), c_void_p, c_u64, c_u64, c_u64, c_void_p, c_u64, _P(c_u64), c_void_p]),
     "sdx_index_projection": (c_int, [c_void_p, c_void_p, c_int, c_u64, c_void_p, c_u64, c_void_p]),
     "sdx_index_score_bounds": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float, c_void_p, c_void_p]),
     "sdx_index_top_k": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_u64, c_u64, c_u64, c_u64, c_float, c_void_p,

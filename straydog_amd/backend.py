@@ -339,6 +339,17 @@ class Backend:
         self.check(self.lib.sdx_qsa_decode_attend(self.handle, ctypes.byref(state), projections, stride, steps, positions, ropes, scratch.pointer,
                                                   scratch.size, attended))
 
+    def qsa_prefill_attend_scratch(self, steps, heads, kv_heads, context):
+        return int(self.lib.sdx_qsa_prefill_attend_scratch(steps, heads, kv_heads, context))
+
+    def qsa_prefill_attend(self, state, projections, stride, steps, base, scratch, attended, valid=None):
+        """A prompt chunk's attention stage in one call; `valid` is a one-element list (the interval scheme's packed blocks, in and out)."""
+        held = abi.c_u64(valid[0] if valid else 0)
+        self.check(self.lib.sdx_qsa_prefill_attend(self.handle, ctypes.byref(state), projections, stride, steps, base, scratch.pointer, scratch.size,
+                                                   ctypes.byref(held) if valid is not None else None, attended))
+        if valid is not None:
+            valid[0] = held.value
+
     def index_top_k(self, q_index, keys, weights, visible, batch, groups, heads, dim, scale, scores, k, indices):
         self.check(self.lib.sdx_index_top_k(self.handle, q_index, keys, weights, visible, batch, groups, heads, dim, scale, scores,
                                             k, indices))

@@ -67,19 +67,19 @@ __device__ __forceinline__ float pooled_mean(const float* incoming, size_t incom
 }
 
 // One workgroup of 128 threads per block completed by the span.
-__global__ void __launch_bounds__(COLUMNS) pool_kernel(const float* incoming, const float* history, const float* norm, size_t pool, size_t base,
-                                                       float* blocks) {
+__global__ void __launch_bounds__(COLUMNS) pool_kernel(const float* incoming, size_t incoming_stride, const float* history, const float* norm, size_t pool,
+                                                       size_t base, float* blocks) {
     __shared__ float values[256], sums[256];
     const size_t block = base / 4 + blockIdx.x, begin = block * 4;
     const unsigned c = threadIdx.x;
-    blocks[c * pool + block] = normalized(pooled_mean(incoming, COLUMNS, history, begin, base, c), norm, COLUMNS, begin, values, sums);
+    blocks[c * pool + block] = normalized(pooled_mean(incoming, incoming_stride, history, begin, base, c), norm, COLUMNS, begin, values, sums);
 }
 
-__global__ void __launch_bounds__(256) save_history_kernel(const float* incoming, size_t base, size_t steps, float* history) {
+__global__ void __launch_bounds__(256) save_history_kernel(const float* incoming, size_t incoming_stride, size_t base, size_t steps, float* history) {
     const size_t i = threadIdx.x + size_t(blockIdx.x) * 256, kept = steps < 4 ? steps : 4;
     if (i >= kept * COLUMNS) return;
     const size_t token = steps - kept + i / COLUMNS;
-    history[((base + token) % RING) * COLUMNS + i % COLUMNS] = incoming[token * COLUMNS + i % COLUMNS];
+    history[((base + token) % RING) * COLUMNS + i % COLUMNS] = incoming[token * incoming_stride + i % COLUMNS];
 }
 
 __device__ __forceinline__ float positive_sum(const float (&dot)[HEADS]) {
@@ -590,7 +590,8 @@ struct StageArgs {
     size_t stride;
     const float *q_norm, *k_norm, *index_q_norm, *index_k_norm;
     unsigned heads, kv_heads, steps;
-    const uint32_t *positions, *ropes;
+    const uint32_t *positions, *ropes;   // device-resident positions of the rows, or null: row r is at base + r
+    size_t base;
     uint8_t* pages;
     unsigned page_tokens, row_bytes;
     const int32_t* page_table;
@@ -604,7 +605,7 @@ __global__ void __launch_bounds__(256) stage_prepare_kernel(StageArgs a) {
     __shared__ float values[256], sums[256];
     __shared__ __align__(16) float key[256];
     const unsigned block = blockIdx.x, c = threadIdx.x;
-    const size_t row = blockIdx.y, pos = a.positions[row], rope = a.ropes[row];
+    const size_t row = blockIdx.y, pos = a.positions ? a.positions[row] : a.base + row, rope = a.ropes ? a.ropes[row] : a.base + row;
     float* own = a.projections + row * a.stride;
     const size_t keys_at = size_t(a.heads) * 512, values_at = keys_at + size_t(a.kv_heads) * 256, index_at = keys_at + size_t(a.kv_heads) * 512;
     if (block < a.heads) {
@@ -655,6 +656,7 @@ void launch_rows(Device& d, const float* queries, size_t stride, const float* bl
 }  // namespace
 
 namespace sd {
+void validate_pool(Device& d, const sdx_kv_pool* pool);     // kv_write.hip
 // block_interval.hip
 size_t interval_scratch_bytes(size_t steps, size_t pool);
 bool interval_serves(size_t base);
@@ -695,8 +697,8 @@ int sdx_qsa_pool(void* handle, const float* incoming, float* history, const floa
     op_span(value, norm, COLUMNS * 4, "sdx_qsa_pool norm");
     op_span(value, blocks, checked_floats({pool, uint64_t(COLUMNS)}), "sdx_qsa_pool blocks");
     const size_t completed = (base + steps) / 4 - base / 4;
-    if (completed) pool_kernel<<<checked_blocks(completed, 1), COLUMNS, 0, value.stream>>>(incoming, history, norm, pool, base, blocks);
-    save_history_kernel<<<checked_blocks(std::min<size_t>(steps, 4) * COLUMNS), 256, 0, value.stream>>>(incoming, base, steps, history);
+    if (completed) pool_kernel<<<checked_blocks(completed, 1), COLUMNS, 0, value.stream>>>(incoming, COLUMNS, history, norm, pool, base, blocks);
+    save_history_kernel<<<checked_blocks(std::min<size_t>(steps, 4) * COLUMNS), 256, 0, value.stream>>>(incoming, COLUMNS, base, steps, history);
     SD_OP_END
 }
 
@@ -812,7 +814,7 @@ int sdx_qsa_decode_attend(void* handle, const sdx_qsa_state* state, float* proje
             throw std::runtime_error("sdx_qsa_decode_attend: 1..8 rows of heads x 512 + K/V heads x 512 + 640 projections, K/V rows of 256 columns");
         if (!state->page_table && kv.page_tokens < context) throw std::runtime_error("sdx_qsa_decode_attend: without a page table one page must hold the context");
         if (state->page_table) op_span(value, state->page_table, checked_floats({(context + kv.page_tokens - 1) / kv.page_tokens}), "a page table");
-        op_span(value, kv.pages, checked_product({kv.page_count, 2, kv.kv_heads, kv.page_tokens, kv.row_bytes}), "a K/V pool");
+        validate_pool(value, state->kv);        // (the rows are written below: page moves queued so far come first)
         op_span(value, state->blocks, checked_floats({pool, uint64_t(COLUMNS)}), "pooled index keys");
         op_span(value, state->history, size_t(RING) * COLUMNS * 4, "the index history");
         op_span(value, state->q_norm, 256 * 4, "a query norm weight");
@@ -847,6 +849,77 @@ int sdx_qsa_decode_attend(void* handle, const sdx_qsa_state* state, float* proje
     if (sdx_qsa_index(handle, projections + index_at, stride, state->blocks, pool, 0, positions, steps, 2052, scores, indices, counts) < 0) return -1;
     return sdx_selected_attention(handle, state->kv, state->page_table, state->context, 0, positions, indices, 2052, counts, queries, 0, steps, heads, 0.0625f,
                                   projections + 256, 512, stride, attended, 0, partial, sdx_selected_attention_scratch(steps, state->kv->kv_heads, 2052));
+}
+
+uint64_t sdx_qsa_prefill_attend_scratch(uint64_t steps, uint64_t heads, uint64_t kv_heads, uint64_t context) {
+    try {
+        const uint64_t pool = context / 4 + 1;
+        const uint64_t first = (checked_floats({steps, heads * 256 + pool + 2052 + 1}) + 255) & ~uint64_t(255);
+        const uint64_t partial = (sdx_selected_attention_scratch(steps, kv_heads, 2052) + 255) & ~uint64_t(255);
+        return first + partial + sdx_qsa_index_interval_scratch(steps, pool);
+    } catch (const std::exception&) { return 0; }
+}
+
+int sdx_qsa_prefill_attend(void* handle, const sdx_qsa_state* state, float* projections, uint64_t stride, uint64_t steps, uint64_t base, void* scratch,
+                           uint64_t scratch_bytes, uint64_t* valid, float* attended) {
+    size_t index_at = 0;
+    uint64_t pool = 0;
+    {
+        SD_OP_BEGIN
+        if (!state || !state->kv) throw std::runtime_error("sdx_qsa_prefill_attend: no state");
+        const sdx_kv_pool& kv = *state->kv;
+        const uint64_t heads = state->heads, context = state->context;
+        pool = context / 4 + 1;
+        if (kv.dim != 256 || !heads || heads % kv.kv_heads || heads / kv.kv_heads > 16 || !steps || steps > 4096 || !context || context > (uint64_t(1) << 24) ||
+            base + steps > context || stride < heads * 512 + uint64_t(kv.kv_heads) * 512 + HEADS * COLUMNS + COLUMNS)
+            throw std::runtime_error("sdx_qsa_prefill_attend: 1..4096 rows of heads x 512 + K/V heads x 512 + 640 projections inside the context, K/V rows of 256 columns");
+        if (!state->page_table && kv.page_tokens < context) throw std::runtime_error("sdx_qsa_prefill_attend: without a page table one page must hold the context");
+        if (state->page_table) op_span(value, state->page_table, checked_floats({(context + kv.page_tokens - 1) / kv.page_tokens}), "a page table");
+        validate_pool(value, state->kv);
+        op_span(value, state->blocks, checked_floats({pool, uint64_t(COLUMNS)}), "pooled index keys");
+        op_span(value, state->history, size_t(RING) * COLUMNS * 4, "the index history");
+        op_span(value, state->q_norm, 256 * 4, "a query norm weight");
+        op_span(value, state->k_norm, 256 * 4, "a key norm weight");
+        op_span(value, state->index_q_norm, COLUMNS * 4, "an index query norm weight");
+        op_span(value, state->index_k_norm, COLUMNS * 4, "an index key norm weight");
+        op_span(value, projections, checked_floats({steps - 1, stride}) + (heads * 512 + uint64_t(kv.kv_heads) * 512 + 640) * 4, "projections");
+        op_span(value, attended, checked_floats({steps, heads, 256}), "an attention output");
+        const uint64_t need = sdx_qsa_prefill_attend_scratch(steps, heads, kv.kv_heads, context);
+        if (!need || scratch_bytes < need) throw std::runtime_error("sdx_qsa_prefill_attend: scratch too small (see sdx_qsa_prefill_attend_scratch)");
+        if (uintptr_t(scratch) % 256) throw std::runtime_error("sdx_qsa_prefill_attend: the scratch must lie on a 256-byte boundary");
+        op_span(value, scratch, need, "stage scratch");
+        StageArgs args{};
+        args.projections = projections; args.stride = stride;
+        args.q_norm = state->q_norm; args.k_norm = state->k_norm; args.index_q_norm = state->index_q_norm; args.index_k_norm = state->index_k_norm;
+        args.heads = unsigned(heads); args.kv_heads = kv.kv_heads; args.steps = unsigned(steps); args.positions = nullptr; args.ropes = nullptr; args.base = size_t(base);
+        args.pages = static_cast<uint8_t*>(kv.pages); args.page_tokens = kv.page_tokens; args.row_bytes = kv.row_bytes; args.page_table = state->page_table; args.page_count = size_t(kv.page_count);
+        args.context = context; args.queries = static_cast<float*>(scratch); args.blocks = state->blocks; args.history = state->history; args.pool = pool;
+        // 1. rows normalised and turned, K/V rows appended (no workgroup of the grid pools: the span's blocks are pooled at once below)
+        stage_prepare_kernel<<<dim3(unsigned(heads + kv.kv_heads + HEADS), unsigned(steps)), 256, 0, value.stream>>>(args);
+        SD_CHECK(hipGetLastError());
+        // 2. the blocks the span completes, and the ring's newest rows
+        index_at = heads * 512 + size_t(kv.kv_heads) * 512;
+        const float* incoming = projections + index_at + HEADS * COLUMNS;
+        const size_t completed = size_t((base + steps) / 4 - base / 4);
+        if (completed) pool_kernel<<<checked_blocks(completed, 1), COLUMNS, 0, value.stream>>>(incoming, size_t(stride), state->history, state->index_k_norm, size_t(pool), size_t(base), state->blocks);
+        save_history_kernel<<<checked_blocks(std::min<size_t>(steps, 4) * COLUMNS), 256, 0, value.stream>>>(incoming, size_t(stride), size_t(base), size_t(steps), state->history);
+        SD_CHECK(hipGetLastError());
+    } catch (const std::exception& e) { ::sd::last_error = e.what(); return -1; }
+    }
+    // 3. the rows' selections (by intervals past 32768 positions, the packed keys carried from chunk to chunk in the scratch);
+    // 4. each row over its selection, gated
+    const uint64_t heads = state->heads, kv_heads = state->kv->kv_heads;
+    float* queries = static_cast<float*>(scratch);
+    float* scores = queries + steps * heads * 256;
+    float* indices = scores + steps * pool;
+    float* counts = indices + steps * 2052;
+    uint8_t* partial = reinterpret_cast<uint8_t*>((reinterpret_cast<uintptr_t>(counts + steps) + 255) & ~uintptr_t(255));
+    const uint64_t partial_bytes = sdx_selected_attention_scratch(steps, kv_heads, 2052);
+    uint8_t* interval = partial + ((partial_bytes + 255) & ~uint64_t(255));
+    if (sdx_qsa_index_interval(handle, projections + index_at, stride, state->blocks, pool, base, steps, 2052, scores, indices, counts, interval,
+                               sdx_qsa_index_interval_scratch(steps, pool), valid) < 0) return -1;
+    return sdx_selected_attention(handle, state->kv, state->page_table, state->context, base, nullptr, indices, 2052, counts, queries, 0, steps, heads, 0.0625f,
+                                  projections + 256, 512, stride, attended, 0, partial, partial_bytes);
 }
 
 }  // extern "C"

@@ -159,6 +159,49 @@ def test_qwen_decode_stage_recorded(gpu, oracle):
         assert np.abs(_read(gpu, recorded["attended"], np.float32, heads * 256)).max() > 0
 
 
+def test_prompt_chunk_stage_recorded(gpu, oracle):
+    # sdx_qsa_prefill_attend recorded once at a position past 32768 (the selection by intervals); replays on new projections give
+    # the bits of eager calls on a twin state
+    rng = np.random.default_rng(16)
+    heads, kv_heads, context, first, row_bytes, steps = 24, 2, 36864, 34000, 272, 24
+    pool_blocks, stride = context // 4 + 1, 24 * 512 + 2 * 512 + 640
+    blocks = np.zeros((128, pool_blocks), dtype=np.float32)
+    blocks[:, :first // 4] = rng.standard_normal((128, first // 4)).astype(np.float32)
+    history = rng.standard_normal((16, 128)).astype(np.float32)
+    norms = [(0.4 + 1.2 * rng.random(n)).astype(np.float32) for n in (256, 256, 128, 128)]
+    cached = rng.integers(0, 256, context * 4 * row_bytes, dtype=np.uint8)
+    cached.reshape(-1, row_bytes)[:, 256:] = np.tile(np.frombuffer(np.float16(0.01).tobytes(), np.uint8), 8)
+
+    def twin():
+        kv, buffer = gpu.kv_pool(1, context, kv_heads, 256, row_bytes)
+        gpu.write_buffer(buffer, 0, cached)
+        s = dict(kv=kv, buffer=buffer, projections=gpu.buffer(steps * stride * 4), blocks=gpu.upload(blocks), history=gpu.upload(history),
+                 norms=[gpu.upload(n) for n in norms], attended=gpu.buffer(steps * heads * 256 * 4),
+                 scratch=gpu.buffer(gpu.qsa_prefill_attend_scratch(steps, heads, kv_heads, context)))
+        s["state"] = gpu.qsa_state(kv, None, context, s["blocks"].base(), s["history"].base(), *[n.base() for n in s["norms"]], heads)
+        return s
+
+    def call(s):
+        gpu.qsa_prefill_attend(s["state"], s["projections"].base(), stride, steps, first, s["scratch"], s["attended"].base())
+    recorded, eager, warm = twin(), twin(), twin()
+    gpu.write_buffer(warm["projections"], 0, rng.standard_normal(steps * stride).astype(np.float32))
+    call(warm)                               # a first call outside the recording
+    gpu.graph_begin()
+    call(recorded)
+    gpu.graph_end(19)
+    for turn in range(3):
+        rows = (rng.standard_normal(steps * stride) * 2).astype(np.float32)
+        for s in (recorded, eager):
+            gpu.write_buffer(s["projections"], 0, rows)
+        assert gpu.graph_run(19)
+        call(eager)
+        for what, count, dtype in (("attended", steps * heads * 256, np.float32), ("blocks", blocks.size, np.float32), ("history", history.size, np.float32),
+                                   ("buffer", cached.size, np.uint8)):
+            a, b = _read(gpu, recorded[what], dtype, count), _read(gpu, eager[what], dtype, count)
+            assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), f"replay {turn}: {what}"
+        assert np.abs(_read(gpu, recorded["attended"], np.float32, steps * heads * 256)).max() > 0
+
+
 def test_graphs_are_dropped_when_the_workspace_moves(gpu, oracle):
     # ops that use the handle's workspace bake its address into a recorded graph; when a later, larger call makes the workspace
     # grow (and move), the kept graphs are dropped: sd_graph_run answers "none stored" and the caller records again, instead of

@@ -559,3 +559,86 @@ def test_decode_stage_in_one_call_equals_its_parts(gpu, oracle, row_bytes, paged
         a, b = got[what], want[what]
         assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), what
     assert np.all(np.isfinite(got["attended"])) and np.abs(got["attended"]).max() > 0
+
+
+@pytest.mark.parametrize("row_bytes,paged,context,first,spans", [(272, True, 4096, 1990, (100,)), (512, False, 40960, 36001, (64, 37))])
+def test_prompt_chunk_stage_in_one_call_equals_its_parts(gpu, oracle, row_bytes, paged, context, first, spans):
+    # sdx_qsa_prefill_attend (the stage of qsa_prefill, gpu/sparse_attention.hpp:444-506): normalised rows, K/V bytes, pooled blocks
+    # and ring equal those of sdx_qsa_normalize + sdx_kv_write + sdx_qsa_pool over the span, and the attended rows equal
+    # sdx_qsa_index_interval + sdx_selected_attention (gated) on them, bit for bit: before the 512-block line and across it with
+    # the exact kernels, and past 32768 positions by intervals, the packed keys carried from one chunk to the next
+    rng = np.random.default_rng(context + first)
+    heads, kv_heads = 24, 2
+    pool_blocks, stride = context // 4 + 1, 24 * 512 + 2 * 512 + 640 + 5
+    norms = [(0.4 + 1.2 * rng.random(n)).astype(np.float32) for n in (256, 256, 128, 128)]
+    blocks = np.zeros((128, pool_blocks), dtype=np.float32)
+    blocks[:, :first // 4] = rng.standard_normal((128, first // 4)).astype(np.float32)
+    history = rng.standard_normal((16, 128)).astype(np.float32)
+    page_tokens = 256 if paged else context
+    pages = context // page_tokens
+    order = rng.permutation(pages).astype(np.int32)
+    if row_bytes == 272:
+        filled = rng.integers(0, 256, pages * 4 * page_tokens * row_bytes, dtype=np.uint8)
+        rows = filled.reshape(-1, 272)
+        rows[:, 256:] = np.tile(np.frombuffer(np.float16(0.01).tobytes(), np.uint8), 8)
+    else:
+        filled = rng.standard_normal(pages * 4 * page_tokens * 256).astype(np.float16).view(np.uint8)
+    most = max(spans)
+
+    def fresh():
+        kv, buffer = gpu.kv_pool(pages, page_tokens, kv_heads, 256, row_bytes)
+        gpu.write_buffer(buffer, 0, filled)
+        return dict(kv=kv, buffer=buffer, table=gpu.upload(order) if paged else None, projections=gpu.buffer(most * stride * 4), blocks=gpu.upload(blocks),
+                    history=gpu.upload(history), norms=[gpu.upload(n) for n in norms], attended=gpu.buffer(most * heads * 256 * 4))
+
+    def read_state(s, steps):
+        return dict(kv=_read(gpu, s["buffer"], np.uint8, filled.size), blocks=_read(gpu, s["blocks"], np.float32, blocks.size),
+                    history=_read(gpu, s["history"], np.float32, history.size), projections=_read(gpu, s["projections"], np.float32, steps * stride),
+                    attended=_read(gpu, s["attended"], np.float32, steps * heads * 256))
+    one, two = fresh(), fresh()
+    state = gpu.qsa_state(one["kv"], one["table"].base() if paged else None, context, one["blocks"].base(), one["history"].base(),
+                          *[n.base() for n in one["norms"]], heads)
+    scratch = gpu.buffer(gpu.qsa_prefill_attend_scratch(most, heads, kv_heads, context))
+    valid_one, valid_two = [0], [0]
+    queries, keys, values = gpu.buffer(most * heads * 256 * 4), gpu.buffer(most * kv_heads * 256 * 4), gpu.buffer(most * kv_heads * 256 * 4)
+    index_keys = gpu.buffer(most * 128 * 4)
+    scores, indices, counts = gpu.buffer(most * pool_blocks * 4), gpu.buffer(most * 2052 * 4), gpu.buffer(most * 4)
+    interval = gpu.buffer(gpu.qsa_index_interval_scratch(most, pool_blocks))
+    partial = gpu.buffer(gpu.selected_attention_scratch(most, kv_heads, 2052))
+    table_two = two["table"].base() if paged else gpu.upload(np.zeros(1, np.int32)).base()
+    at = first
+    for steps in spans:
+        projections = (rng.standard_normal((steps, stride)) * 2).astype(np.float32)
+        # one call
+        gpu.write_buffer(one["projections"], 0, projections)
+        gpu.qsa_prefill_attend(state, one["projections"].base(), stride, steps, at, scratch, one["attended"].base(), valid_one)
+        got = read_state(one, steps)
+        # the parts
+        gpu.write_buffer(two["projections"], 0, projections)
+        base = two["projections"].base()
+        for r in range(steps):
+            row = base + r * stride * 4
+            gpu.qsa_normalize(row, two["norms"][0].base(), 1, heads, 256, 512, at + r, queries.at(r * heads * 256 * 4))
+            gpu.qsa_normalize(row + heads * 512 * 4, two["norms"][1].base(), 1, kv_heads, 256, 256, at + r, keys.at(r * kv_heads * 256 * 4))
+            gpu.qsa_normalize(row + (heads * 512 + kv_heads * 512) * 4, two["norms"][2].base(), 1, 4, 128, 128, at + r, row + (heads * 512 + kv_heads * 512) * 4)
+        gpu.write_buffer(values, 0, np.ascontiguousarray(projections[:, heads * 512 + kv_heads * 256:heads * 512 + kv_heads * 512]))
+        gpu.write_buffer(index_keys, 0, np.ascontiguousarray(projections[:, heads * 512 + kv_heads * 512 + 512:heads * 512 + kv_heads * 512 + 640]))
+        start = gpu.upload(np.array([at], dtype=np.int32))
+        gpu.kv_write(two["kv"], table_two, pages, start.base(), keys.base(), values.base(), False, 1, steps)
+        gpu.qsa_pool(index_keys.base(), two["history"].base(), two["norms"][3].base(), pool_blocks, at, steps, two["blocks"].base())
+        gpu.qsa_index_interval(base + (heads * 512 + kv_heads * 512) * 4, stride, two["blocks"].base(), pool_blocks, at, steps, 2052, scores.base(), indices.base(),
+                               counts.base(), interval, valid_two)
+        gpu.selected_attention(two["kv"], two["table"].base() if paged else None, context, at, indices.base(), 2052, counts.base(), queries.base(), False,
+                               steps, heads, 0.0625, two["attended"].base(), False, partial, gate=base + 256 * 4, gate_stride=512, gate_row_stride=stride)
+        want = read_state(two, steps)
+        for what in ("kv", "blocks", "history", "projections", "attended"):
+            assert np.array_equal(got[what].view(np.uint8), want[what].view(np.uint8)), f"{what} after the chunk at {at}"
+        assert valid_one == valid_two and np.all(np.isfinite(got["attended"])) and np.abs(got["attended"]).max() > 0
+        gpu.release(start)
+        at += steps
+    if first >= 32768:
+        assert valid_one[0] > 0, "past 32768 positions the packed keys are carried to the next chunk"
+    with pytest.raises(RuntimeError, match="scratch too small"):
+        gpu.qsa_prefill_attend(state, one["projections"].base(), stride, most, first, gpu.buffer(4096), one["attended"].base())
+    with pytest.raises(RuntimeError, match="inside the context"):
+        gpu.qsa_prefill_attend(state, one["projections"].base(), stride, most, context - 1, scratch, one["attended"].base())
