@@ -129,6 +129,12 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
  *                rebuilds every tile.  A position above positions[s] counts as positions[s].
  * Rows at positions >= max_context are neither stored nor attended. */
 uint64_t sdx_prefill_tiles_bytes(uint64_t seqs, uint64_t kv_heads, uint64_t dim, uint64_t max_context);
+/* Which of the two prompt kernels takes spans at 128 columns on this handle from now on: waves of 64 query rows, one a SIMD, the
+ * queries and output accumulators in the accumulation registers (the default), or waves of 32 rows, two a SIMD.  Same rows a
+ * workgroup, same tiles, same grid; the results agree to rounding, not bit for bit (a row's reference maximum is raised when any
+ * row of its wave asks for it).  No counterpart in the reference: a tuning switch, kept so that either kernel can be measured
+ * and tested beside the other.  Anything but 32 or 64 is refused. */
+int sdx_prefill_wave_rows(void* handle, uint64_t rows);
 int sdx_prefill_chunk(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
                       uint64_t max_context, const void* keys, const void* values, int kv_f16, const void* q, int q_f16, uint64_t seqs,
                       uint64_t span, uint64_t heads, float scale, void* out, int out_f16, void* tiles, uint64_t tiles_bytes,

@@ -107,6 +107,7 @@ SIGNATURES = {
     "sdx_paged_attention": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_u64, c_void_p, c_int, c_u64, c_u64, c_u64,
                                     c_float, c_void_p, c_int, c_void_p, c_u64]),
     "sdx_prefill_tiles_bytes": (c_u64, [c_u64, c_u64, c_u64, c_u64]),
+    "sdx_prefill_wave_rows": (c_int, [c_void_p, c_u64]),
     "sdx_prefill_chunk": (c_int, [c_void_p, _P(KvPool), c_void_p, c_u64, c_void_p, c_u64, c_void_p, c_void_p, c_int, c_void_p, c_int, c_u64, c_u64,
                                   c_u64, c_float, c_void_p, c_int, c_void_p, c_u64, c_void_p]),
     "sdx_paged_attention_static_bytes": (c_u64, []),

@@ -294,6 +294,10 @@ class Backend:
     def prefill_tiles_bytes(self, seqs, kv_heads, dim, max_context):
         return int(self.lib.sdx_prefill_tiles_bytes(seqs, kv_heads, dim, max_context))
 
+    def prefill_wave_rows(self, rows):
+        """Waves of 64 query rows (the default) or of 32 for the prompt kernel at 128 columns, on this handle from now on."""
+        self.check(self.lib.sdx_prefill_wave_rows(self.handle, rows))
+
     def prefill_chunk(self, pool, page_table, table_stride, positions, max_context, keys, values, kv_f16, q, q_f16, seqs, span, heads, scale,
                       out, out_f16, tiles, valid=None):
         """A prompt chunk in one call: K/V append (keys/values may be None) + causal attention; `tiles` (a Buffer) keeps the cached

@@ -50,6 +50,8 @@ struct Device {
     uint8_t* arena = nullptr;                       // page-locked staging, io_arena_bytes
     uint32_t kv_row = 272;                          // sd_kv_format: 272 (Q8_0) or 512 (FP16)
     unsigned compute_units = 0;
+    // Query rows a wave of the prompt kernel holds at 128 columns: 64 (one wave a SIMD) or 32 (two); sdx_prefill_wave_rows.
+    uint32_t prefill_wave_rows = 64;
     // Workspaces the attention ops own (allocated on first use, outside any graph capture).
     void* sequence_input = nullptr; size_t sequence_input_bytes = 0;
     void* sequence_output = nullptr; size_t sequence_output_bytes = 0;

@@ -589,6 +589,13 @@ uint64_t sdx_prefill_tiles_bytes(uint64_t seqs, uint64_t kv_heads, uint64_t dim,
     catch (const std::exception&) { return 0; }
 }
 
+int sdx_prefill_wave_rows(void* handle, uint64_t rows) {
+    SD_OP_BEGIN
+    if (rows != 32 && rows != 64) throw std::runtime_error("a wave of the Straydog prompt kernel holds 32 or 64 rows");
+    value.prefill_wave_rows = uint32_t(rows);
+    SD_OP_END
+}
+
 int sdx_prefill_chunk(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
                       uint64_t max_context, const void* keys, const void* values, int kv_f16, const void* q, int q_f16, uint64_t seqs, uint64_t span,
                       uint64_t heads, float scale, void* out, int out_f16, void* tiles, uint64_t tiles_bytes, const int32_t* valid) {

@@ -22,6 +22,7 @@
 #include "paged_rows.hpp"
 #include "kv_codec.hpp"
 
+#include <cstdlib>
 #include <type_traits>
 
 using namespace sd;
@@ -764,6 +765,271 @@ __global__ void __launch_bounds__(TEAM * 64) __attribute__((amdgpu_waves_per_eu(
     }
 }
 
+// ---- the same walk with 64 rows a wave ---------------------------------------------------------------------------------------
+// One wave a SIMD (four a workgroup) holds four 16-row tiles: two of the run counted from the span's end and two of its mirror
+// image from the start, so a wave is its own pair and every SIMD has work as long as the workgroup has.  An operand read from
+// LDS then feeds four products where it fed two: what a compute unit reads from LDS per product is halved, and LDS traffic
+// (operand reads and the tiles' arrival) is what the products compete with.  The wave needs about 330 registers; which of them
+// live in the accumulation half of the register file is said here, by writing the products as instructions with register
+// classes: the queries (only ever a B operand) and the output accumulators (only ever written by products) do, everything the
+// vector arithmetic touches does not -- left to itself the compiler puts every product's result there and copies scores back
+// and forth (2.6 copies a product, measured).  The compiler then does not know these instructions for products, so what it would
+// have kept apart is kept apart here: a vector instruction's result waits two states before a product reads it (s_nop 1 ahead of
+// the first product that follows one), a product's result is read by vector instructions only a step later (or after a wait
+// written out), and a product that adds to another's result comes at least three products after it.
+template<bool AFTER_VECTOR>
+__device__ __forceinline__ void score_first(floatx4& d, const half8& k, const half8& q, const floatx4& c) {
+    if (AFTER_VECTOR) asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(k), "a"(q), "v"(c));
+    else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(k), "a"(q), "v"(c));
+}
+__device__ __forceinline__ void score_more(floatx4& d, const half8& k, const half8& q) { asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(d) : "v"(k), "a"(q)); }
+template<bool AFTER_VECTOR>
+__device__ __forceinline__ void output_more(floatx4& d, const half8& v, const words4& p) {
+    if (AFTER_VECTOR) asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(d) : "v"(v), "v"(p));
+    else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(d) : "v"(v), "v"(p));
+}
+// (after products whose results vector instructions read at once: longer than any product takes)
+__device__ __forceinline__ void products_done() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+
+template<int DIM>
+__global__ void __launch_bounds__(GROUPS * 64) __attribute__((amdgpu_waves_per_eu(1, 1))) prefill_dense64_kernel(PrefillArgs args, const uint8_t* tiles_in,
+                                                                                                            unsigned tiles_per_seq) {
+    constexpr int QT = 4, BLOCKS = DIM / 32, TILES = DIM / 16, KT = TILE_KEYS * DIM * 2, TILE = tile_bytes<DIM>();
+    constexpr int PAIR_ROWS = 32, GROUP_ROWS = GROUPS * PAIR_ROWS, RING = 4, PER = TILE / 1024 / GROUPS, SUB = 32;
+    static_assert(TILE % (1024 * GROUPS) == 0 && RING * TILE <= 160 * 1024 - 1024 && TILE_KEYS == 2 * SUB && BLOCKS == 4 && TILES == 8, "a tile is two steps of a wave");
+    const int kvh = blockIdx.y, seq = blockIdx.z;
+    const int thread = threadIdx.x, lane = thread & 63, wave = __builtin_amdgcn_readfirstlane(thread >> 6), li = lane & 15, g = lane >> 4;
+    const int position = first_position(args.positions, unsigned(seq), args.max_context);
+    const int cached = min(position + int(args.span), args.max_context);
+    const int runs = (int(args.rows) + GROUP_ROWS - 1) / GROUP_ROWS;
+    const int late = runs - 1 - int(blockIdx.x), early = int(blockIdx.x);
+    const int group_last = min(int(args.rows), (late + 1) * GROUP_ROWS) - 1;
+    const int keys = min(position + group_last / int(args.group) + 1, cached);
+    // the wave's two pairs of tiles: pair 0 of the late run, pair 1 of the early one
+    int row0[2], wave_first[2], steps[2];
+    #pragma unroll
+    for (int p = 0; p < 2; ++p) {
+        row0[p] = (p == 0 ? late : early) * GROUP_ROWS + wave * PAIR_ROWS;
+        const bool idle = row0[p] >= int(args.rows) || (p == 1 && early == late);
+        wave_first[p] = position + row0[p] / int(args.group);
+        const int wave_last = min(position + (min(int(args.rows), row0[p] + PAIR_ROWS) - 1) / int(args.group), keys - 1);
+        steps[p] = idle ? 0 : wave_last / SUB + 1;
+    }
+    if (steps[0] < steps[1]) {      // (the late run's quarter may lie past the span's last row: the longer walk is pair 0's)
+        const int r = row0[0], f = wave_first[0], n = steps[0];
+        row0[0] = row0[1]; wave_first[0] = wave_first[1]; steps[0] = steps[1];
+        row0[1] = r; wave_first[1] = f; steps[1] = n;
+    }
+    extern __shared__ __attribute__((aligned(16))) uint8_t stages[];              // [RING][K block | V^T block]
+    const uint8_t* const source = tiles_in + (size_t(seq) * args.kv_heads + kvh) * tiles_per_seq * TILE + 1024 * PER * wave + 16 * lane;
+    const int last_tile = (keys - 1) / TILE_KEYS;
+    const auto copy_in = [&](int tile) {
+        const uint8_t* from = source + size_t(min(tile, last_tile)) * TILE;
+        uint8_t* stage = stages + (tile % RING) * TILE + 1024 * PER * wave;
+        #pragma unroll
+        for (int k = 0; k < PER; ++k) load_to_lds<false>(from + 1024 * k, stage + 1024 * k);
+    };
+    #pragma unroll
+    for (int ahead = 0; ahead < RING - 1; ++ahead) copy_in(ahead);
+    half8 qf[QT][BLOCKS];          // the queries times scale * log2 e: a score is a base-2 exponent
+    int limit[QT];
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int row = row0[qt / 2] + (qt % 2) * 16 + li;
+        const bool real = row < int(args.rows) && steps[qt / 2] > 0;
+        const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
+        limit[qt] = real ? position + span_row : 0x7fffffff;                      // a padding row masks nothing
+        const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
+        #pragma unroll
+        for (int b = 0; b < BLOCKS; ++b) {
+            half8 value = {};
+            if (real) {
+                if (args.q_f16) {
+                    const half8 raw = *reinterpret_cast<const half8*>(static_cast<const _Float16*>(args.q) + at + 32 * b + 8 * g);
+                    #pragma unroll
+                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)(float(raw[i]) * args.scale_log2);
+                } else {
+                    const float* from = static_cast<const float*>(args.q) + at + 32 * b + 8 * g;
+                    #pragma unroll
+                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)(from[i] * args.scale_log2);
+                }
+            }
+            // (the queries are only ever a product's B operand: they live in the accumulation registers, where a product reads them
+            // as well, and leave the vector registers to what the vector arithmetic touches)
+            asm volatile("; queries of tile %1 block %2" : "=a"(qf[qt][b]) : "n"(qt), "n"(b), "0"(value));
+        }
+    }
+    floatx4 acc[QT][TILES], start[QT][2];
+    float l[QT], ref[QT];
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        l[qt] = 0.0f; ref[qt] = 0.0f;
+        start[qt][0] = start[qt][1] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj) asm volatile("; zero" : "=a"(acc[qt][jj]) : "0"(floatx4{0.0f, 0.0f, 0.0f, 0.0f}));
+    }
+    const auto crosses = [&](int p, int u) { return SUB * u + SUB - 1 > wave_first[p]; };
+    // the starting values of a pair's step that crosses its diagonal (every later step of the pair does)
+    const auto veil = [&](int p, int u) {
+        asm volatile("; the step crosses the diagonal" ::: "memory");
+        #pragma unroll
+        for (int q = 0; q < 2; ++q)
+            #pragma unroll
+            for (int t = 0; t < 2; ++t)
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) start[2 * p + q][t][r] = SUB * u + 16 * t + 4 * g + r > limit[2 * p + q] ? -INFINITY : ref[2 * p + q];
+    };
+    // K operands of step u and the scores they give a pair, relative to its references (not pipelined: the start and the rare raise)
+    const auto scores = [&](int p, int u, floatx4 (&s)[QT][2]) {
+        const uint8_t* const kblock = stages + ((u >> 1) % RING) * TILE + (u & 1) * (SUB * 2 * DIM);
+        half8 k[2][BLOCKS];
+        #pragma unroll
+        for (int t = 0; t < 2; ++t)
+            #pragma unroll
+            for (int b = 0; b < BLOCKS; ++b) k[t][b] = *reinterpret_cast<const half8*>(kblock + (16 * t + li) * (2 * DIM) + (((4 * b + g) ^ li) * 16));
+        #pragma unroll
+        for (int b = 0; b < BLOCKS; ++b)
+            #pragma unroll
+            for (int t = 0; t < 2; ++t)
+                #pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    if (b == 0) score_first<true>(s[2 * p + q][t], k[t][b], qf[2 * p + q][b], start[2 * p + q][t]);      // (the starting values may have been written just now)
+                    else score_more(s[2 * p + q][t], k[t][b], qf[2 * p + q][b]);
+                }
+        products_done();
+    };
+    const auto raise = [&](auto first, int p, int u, floatx4 (&s)[QT][2]) {
+        asm volatile("; new reference maxima" ::: "memory");
+        if (!decltype(first)::value) products_done();       // (the accumulators scaled below were written by products just now)
+        #pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int qt = 2 * p + q;
+            float most = s[qt][0][0];
+            #pragma unroll
+            for (int t = 0; t < 2; ++t)
+                #pragma unroll
+                for (int r = 0; r < 4; ++r) most = fmaxf(most, s[qt][t][r]);
+            const float top = row_max(most);
+            const float delta = decltype(first)::value ? top : fmaxf(top, 0.0f);
+            ref[qt] -= delta;
+            start[qt][0] -= delta; start[qt][1] -= delta;
+            if (!decltype(first)::value) {
+                const float alpha = __builtin_amdgcn_exp2f(-delta);
+                l[qt] *= alpha;
+                #pragma unroll
+                for (int jj = 0; jj < TILES; ++jj) {
+                    const floatx4 scaled = acc[qt][jj] * alpha;
+                    asm volatile("; scaled" : "=a"(acc[qt][jj]) : "0"(scaled));     // (back into the accumulation registers)
+                }
+            }
+        }
+        scores(p, u, s);
+    };
+    half8 ka[2][BLOCKS];           // the K operands of the step after the one whose weights are being formed: read a step ahead
+    const auto read_k = [&](int u, int t, int b) {
+        const uint8_t* const kblock = stages + ((u >> 1) % RING) * TILE + (u & 1) * (SUB * 2 * DIM);
+        ka[t][b] = *reinterpret_cast<const half8*>(kblock + (16 * t + li) * (2 * DIM) + (((4 * b + g) ^ li) * 16));
+    };
+    half8 va[TILES];               // the V^T operands of the step whose weights are being formed
+    const auto meet = [&](int tile) {
+        wait_loads<PER * (RING - 3)>();
+        ring_barrier();
+        copy_in(tile + RING - 1);
+    };
+    // One step of one pair p: weights of step u from `now`, scores of step u + 1 into `next`, the products of step u, the largest
+    // score of step u + 1.  READS_V: this pair is the step's first (it fetches the V^T operands and, on even steps, meets the
+    // workgroup); READS_K: it is the step's last (it fetches the K operands of the step after the next).
+    const auto advance = [&](auto reads_v, auto reads_k, auto even, int p, int u, floatx4 (&now)[QT][2], floatx4 (&next)[QT][2]) {
+        constexpr bool READS_V = decltype(reads_v)::value, READS_K = decltype(reads_k)::value;
+        if (crosses(p, u + 1)) veil(p, u + 1);
+        const uint8_t* const vblock = stages + ((u >> 1) % RING) * TILE + KT;
+        const int part = u & 1, q0 = 2 * p, q1 = 2 * p + 1;
+        __builtin_amdgcn_sched_barrier(0);
+        words4 pw[2];
+        float w0[8], w1[8];
+        const auto packed = [&](float first, float second) { return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{first, second}, half2v)); };
+        #pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int b = i / 4, t = (i / 2) % 2, q = i % 2;
+            // (the starting values may have been written by the veil just above: the four products that read them wait two states)
+            if (b == 0) score_first<true>(next[q0 + q][t], ka[t][b], qf[q0 + q][b], start[q0 + q][t]); else score_more(next[q0 + q][t], ka[t][b], qf[q0 + q][b]);
+            const int e = i / 2;
+            if (i % 2 == 0) w0[e] = __builtin_amdgcn_exp2f(now[q0][e / 4][e % 4]);
+            else {
+                l[q0] += w0[e];
+                if (e % 2) pw[0][e / 2] = packed(w0[e - 1], w0[e]);
+            }
+            if (READS_V && i < 8) va[i] = *reinterpret_cast<const half8*>(vblock + (16 * i + li) * (2 * TILE_KEYS) + (((4 * part + g) ^ (li >> 1)) * 16));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (READS_V && decltype(even)::value) meet(u >> 1);        // the step after the next reads the next tile
+        __builtin_amdgcn_sched_barrier(0);
+        #pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (j == 0) output_more<true>(acc[q0][j], va[j], pw[0]); else output_more<false>(acc[q0][j], va[j], pw[0]);
+            w1[j] = __builtin_amdgcn_exp2f(now[q1][j / 4][j % 4]);
+            if (j % 2) pw[1][j / 2] = packed(w1[j - 1], w1[j]);
+            if (READS_K) read_k(u + 2, j % 2, j / 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        float most = next[q0][0][0];
+        #pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (j == 0) output_more<true>(acc[q1][j], va[j], pw[1]); else output_more<false>(acc[q1][j], va[j], pw[1]);
+            l[q1] += w1[j];
+            most = fmaxf(fmaxf(most, next[q0 + j / 4][(j / 2) % 2][2 * (j % 2)]), next[q0 + j / 4][(j / 2) % 2][2 * (j % 2) + 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (__builtin_expect(__any(most > SLACK), 0)) raise(std::false_type{}, p, u + 1, next);
+    };
+    floatx4 even[QT][2], odd[QT][2];
+    wait_loads<PER * (RING - 2)>();
+    ring_barrier();
+    #pragma unroll
+    for (int p = 0; p < 2; ++p)
+        if (steps[p] > 0) {
+            if (crosses(p, 0)) veil(p, 0);
+            scores(p, 0, even);
+            raise(std::true_type{}, p, 0, even);
+        }
+    #pragma unroll
+    for (int b = 0; b < BLOCKS; ++b)
+        #pragma unroll
+        for (int t = 0; t < 2; ++t) read_k(1, t, b);
+    // Whole tiles (two steps each): first those both pairs walk, then those only the longer pair walks.  A pair's last tile may
+    // hold a step past its rows' last key: every score of it is masked, it adds nothing, and the loops stay free of branches.
+    const int both = steps[1] == 0 ? 0 : min((steps[1] + 1) / 2, last_tile + 1);
+    int tile = 0;
+    for (; tile < both; ++tile) {
+        advance(std::true_type{}, std::false_type{}, std::true_type{}, 0, 2 * tile, even, odd);
+        advance(std::false_type{}, std::true_type{}, std::true_type{}, 1, 2 * tile, even, odd);
+        advance(std::true_type{}, std::false_type{}, std::false_type{}, 0, 2 * tile + 1, odd, even);
+        advance(std::false_type{}, std::true_type{}, std::false_type{}, 1, 2 * tile + 1, odd, even);
+    }
+    for (; tile <= last_tile; ++tile) {
+        advance(std::true_type{}, std::true_type{}, std::true_type{}, 0, 2 * tile, even, odd);
+        advance(std::true_type{}, std::true_type{}, std::false_type{}, 0, 2 * tile + 1, odd, even);
+    }
+
+    products_done();
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int row = row0[qt / 2] + (qt % 2) * 16 + li;
+        const float inverse = 1.0f / row_sum(l[qt]);
+        if (steps[qt / 2] == 0 || row >= int(args.rows)) continue;
+        const int span_row = row / int(args.group), head = kvh * int(args.group) + row % int(args.group);
+        const size_t first = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM + 4 * g;
+        #pragma unroll
+        for (int jj = 0; jj < TILES; ++jj) {
+            const floatx4 value = acc[qt][jj] * inverse;
+            if (args.out_f16) {
+                typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+                *reinterpret_cast<half4*>(static_cast<_Float16*>(args.out) + first + 16 * jj) = half4{(_Float16)value[0], (_Float16)value[1], (_Float16)value[2], (_Float16)value[3]};
+            } else *reinterpret_cast<floatx4*>(static_cast<float*>(args.out) + first + 16 * jj) = value;
+        }
+    }
+}
+
 // `tiles`: where the cached rows' FP16 tiles go -- the device's workspace, rebuilt whole on every call, or a buffer the caller
 // keeps between the chunks of a prompt (then `append` may carry the chunk's new rows and the count of positions still valid).
 template<int DIM, int QT, bool Q8>
@@ -777,7 +1043,10 @@ void launch_dense(Device& d, const PrefillArgs& args, unsigned seqs, uint8_t* ti
     else if (input == 1) unpack_tiles_kernel<DIM, Q8, 1><<<grid, 256, 0, d.stream>>>(args, tiles, tiles_per_seq, append);
     else unpack_tiles_kernel<DIM, Q8, 0><<<grid, 256, 0, d.stream>>>(args, tiles, tiles_per_seq, append);
     const unsigned runs = (args.rows + GROUPS * QT * 16 - 1) / (GROUPS * QT * 16);
-    timed_launch(d, &prefill_dense_kernel<DIM, QT>, dim3((runs + 1) / 2, args.kv_heads, seqs), dim3(TEAM * 64), shared, args, tiles, tiles_per_seq);
+    if (d.prefill_wave_rows == 64) {        // (the same rows a workgroup, the same tiles, the same grid: four waves of 64 rows for eight of 32)
+        raise_shared_limit(d, reinterpret_cast<const void*>(&prefill_dense64_kernel<DIM>), shared);
+        timed_launch(d, &prefill_dense64_kernel<DIM>, dim3((runs + 1) / 2, args.kv_heads, seqs), dim3(GROUPS * 64), shared, args, tiles, tiles_per_seq);
+    } else timed_launch(d, &prefill_dense_kernel<DIM, QT>, dim3((runs + 1) / 2, args.kv_heads, seqs), dim3(TEAM * 64), shared, args, tiles, tiles_per_seq);
 }
 
 template<int DIM, int QT, bool Q8, int OCC>

@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from gpu_util import backend, close_enough, make_pool
+from straydog_amd.backend import StraydogError
 
 pytestmark = pytest.mark.gpu
 
@@ -217,6 +218,33 @@ def test_prefill_in_chunks_equals_prefill_at_once(gpu, oracle):
         part = _run(gpu, pool, table, tb, [c * chunk], q[:, c * chunk:(c + 1) * chunk], chunk, heads, scale, True, False,
                     max_context=tokens)
         assert np.array_equal(part, whole[:, c * chunk:(c + 1) * chunk])     # the same keys in the same order: the same bits
+    gpu.release(buffer); gpu.release(tb)
+
+
+def test_waves_of_64_rows_and_of_32(gpu, oracle):
+    # The prompt kernel at 128 columns exists twice: waves of 64 query rows (queries and accumulators in the accumulation registers,
+    # the default) and waves of 32.  Each meets the oracle; they agree to the rounding of the FP16 weights.  An odd number of
+    # 128-row runs (the middle run is its own partner), rows past the span's end in the last run, several contexts, growing scores.
+    rng = np.random.default_rng(404)
+    dim, row_bytes, page_tokens, heads, kv_heads, span = 128, 136, 64, 24, 2, 203
+    contexts = [0, 100, 701]
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, [c + span for c in contexts], kv_heads, dim, page_tokens, row_bytes)
+    q = (rng.standard_normal((len(contexts), span, heads, dim)) * rng.choice([0.3, 1.0, 1.5], size=(len(contexts), span, heads, 1)))
+    q = q.astype(np.float16).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array(contexts, np.int32), q, scale)
+    try:
+        gpu.prefill_wave_rows(32)
+        narrow = _run(gpu, pool, table, tb, contexts, q, span, heads, scale, True, False)
+        gpu.prefill_wave_rows(64)
+        wide = _run(gpu, pool, table, tb, contexts, q, span, heads, scale, True, False)
+        with pytest.raises(StraydogError, match="32 or 64 rows"):
+            gpu.prefill_wave_rows(48)
+    finally:
+        gpu.prefill_wave_rows(64)
+    close_enough(narrow, want, "waves of 32 rows")
+    close_enough(wide, want, "waves of 64 rows")
+    assert np.abs(narrow - wide).max() < 1e-3
     gpu.release(buffer); gpu.release(tb)
 
 
