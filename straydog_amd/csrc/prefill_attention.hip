@@ -821,13 +821,25 @@ __global__ void __launch_bounds__(GROUPS * 64) __attribute__((amdgpu_waves_per_e
         row0[1] = r; wave_first[1] = f; steps[1] = n;
     }
     extern __shared__ __attribute__((aligned(16))) uint8_t stages[];              // [RING][K block | V^T block]
-    const uint8_t* const source = tiles_in + (size_t(seq) * args.kv_heads + kvh) * tiles_per_seq * TILE + 1024 * PER * wave + 16 * lane;
+    const uint8_t* const source = tiles_in + (size_t(seq) * args.kv_heads + kvh) * tiles_per_seq * TILE;        // (the wave's: scalar)
     const int last_tile = (keys - 1) / TILE_KEYS;
+    // A tile's eight pieces of a wave as one run of instructions: the tile's address is the wave's (scalar registers), a lane adds
+    // its own constant offset, the pieces differ by the instruction's offset, which moves both ends.
+    static_assert(PER == 8, "two runs of four pieces");
+    const uint32_t lane_offset = 1024 * PER * wave + 16 * lane, lane_offset_high = lane_offset + 4096;
+    const uint32_t wave_stage = __builtin_amdgcn_readfirstlane(lds_address(stages)) + 1024 * PER * wave;
     const auto copy_in = [&](int tile) {
-        const uint8_t* from = source + size_t(min(tile, last_tile)) * TILE;
-        uint8_t* stage = stages + (tile % RING) * TILE + 1024 * PER * wave;
-        #pragma unroll
-        for (int k = 0; k < PER; ++k) load_to_lds<false>(from + 1024 * k, stage + 1024 * k);
+        const uint64_t from = uint64_t(source + size_t(min(tile, last_tile)) * TILE);
+        const uint32_t to = wave_stage + (tile % RING) * TILE;
+        uint32_t keep;
+        asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %3, %2\n\tglobal_load_lds_dwordx4 %3, %2 offset:1024\n\t"
+                     "global_load_lds_dwordx4 %3, %2 offset:2048\n\tglobal_load_lds_dwordx4 %3, %2 offset:3072\n\t"
+                     "s_add_u32 m0, %1, 0x1000\n\ts_nop 0\n\t"
+                     "global_load_lds_dwordx4 %4, %2\n\tglobal_load_lds_dwordx4 %4, %2 offset:1024\n\t"
+                     "global_load_lds_dwordx4 %4, %2 offset:2048\n\tglobal_load_lds_dwordx4 %4, %2 offset:3072\n\t"
+                     "s_mov_b32 m0, %0"
+                     : "=&s"(keep) : "s"(to), "s"(from), "v"(lane_offset), "v"(lane_offset_high) : "memory", "scc");
     };
     #pragma unroll
     for (int ahead = 0; ahead < RING - 1; ++ahead) copy_in(ahead);
@@ -878,6 +890,7 @@ __global__ void __launch_bounds__(GROUPS * 64) __attribute__((amdgpu_waves_per_e
             for (int t = 0; t < 2; ++t)
                 #pragma unroll
                 for (int r = 0; r < 4; ++r) start[2 * p + q][t][r] = SUB * u + 16 * t + 4 * g + r > limit[2 * p + q] ? -INFINITY : ref[2 * p + q];
+        asm volatile("s_nop 1" ::: "memory");      // (the products that read these come right behind)
     };
     // K operands of step u and the scores they give a pair, relative to its references (not pipelined: the start and the rare raise)
     const auto scores = [&](int p, int u, floatx4 (&s)[QT][2]) {
@@ -948,16 +961,19 @@ __global__ void __launch_bounds__(GROUPS * 64) __attribute__((amdgpu_waves_per_e
         words4 pw[2];
         float w0[8], w1[8];
         const auto packed = [&](float first, float second) { return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2v{first, second}, half2v)); };
+        // (the weights' exponentials are written as instructions too: the compiler then keeps no wait state after each for the vector
+        // instruction that reads it -- a product always lies between them here)
+        const auto weight = [&](float score) { float w; asm volatile("v_exp_f32 %0, %1" : "=v"(w) : "v"(score)); return w; };
         #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int b = i / 4, t = (i / 2) % 2, q = i % 2;
-            // (the starting values may have been written by the veil just above: the four products that read them wait two states)
-            if (b == 0) score_first<true>(next[q0 + q][t], ka[t][b], qf[q0 + q][b], start[q0 + q][t]); else score_more(next[q0 + q][t], ka[t][b], qf[q0 + q][b]);
+            if (b == 0) score_first<false>(next[q0 + q][t], ka[t][b], qf[q0 + q][b], start[q0 + q][t]); else score_more(next[q0 + q][t], ka[t][b], qf[q0 + q][b]);
             const int e = i / 2;
-            if (i % 2 == 0) w0[e] = __builtin_amdgcn_exp2f(now[q0][e / 4][e % 4]);
+            if (i % 2 == 0) w0[e] = weight(now[q0][e / 4][e % 4]);
             else {
-                l[q0] += w0[e];
+                __builtin_amdgcn_sched_barrier(0);      // (the exponential of the slot before and the sum that reads it: the product between them)
                 if (e % 2) pw[0][e / 2] = packed(w0[e - 1], w0[e]);
+                l[q0] += w0[e];
             }
             if (READS_V && i < 8) va[i] = *reinterpret_cast<const half8*>(vblock + (16 * i + li) * (2 * TILE_KEYS) + (((4 * part + g) ^ (li >> 1)) * 16));
             __builtin_amdgcn_sched_barrier(0);
@@ -966,8 +982,11 @@ __global__ void __launch_bounds__(GROUPS * 64) __attribute__((amdgpu_waves_per_e
         __builtin_amdgcn_sched_barrier(0);
         #pragma unroll
         for (int j = 0; j < 8; ++j) {
+            w1[j] = weight(now[q1][j / 4][j % 4]);
+            __builtin_amdgcn_sched_barrier(0);
+            // (the first product reads weights packed two instructions ago: more wait states)
             if (j == 0) output_more<true>(acc[q0][j], va[j], pw[0]); else output_more<false>(acc[q0][j], va[j], pw[0]);
-            w1[j] = __builtin_amdgcn_exp2f(now[q1][j / 4][j % 4]);
+            __builtin_amdgcn_sched_barrier(0);
             if (j % 2) pw[1][j / 2] = packed(w1[j - 1], w1[j]);
             if (READS_K) read_k(u + 2, j % 2, j / 2);
             __builtin_amdgcn_sched_barrier(0);
@@ -975,9 +994,10 @@ __global__ void __launch_bounds__(GROUPS * 64) __attribute__((amdgpu_waves_per_e
         float most = next[q0][0][0];
         #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            if (j == 0) output_more<true>(acc[q1][j], va[j], pw[1]); else output_more<false>(acc[q1][j], va[j], pw[1]);
             l[q1] += w1[j];
             most = fmaxf(fmaxf(most, next[q0 + j / 4][(j / 2) % 2][2 * (j % 2)]), next[q0 + j / 4][(j / 2) % 2][2 * (j % 2) + 1]);
+            if (j == 0) __builtin_amdgcn_sched_barrier(0);      // (the first product reads weights packed just now: the two instructions above first)
+            output_more<false>(acc[q1][j], va[j], pw[1]);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (__builtin_expect(__any(most > SLACK), 0)) raise(std::false_type{}, p, u + 1, next);
