@@ -34,7 +34,7 @@ PROFILED_TRAFFIC = {
     "config1_32k": (1147.5e6, "profiles/paged_attention_q8_d128_decode_config1_32k.md"),
     "config0": (2.61e6, "profiles/paged_attention_q8_d128_decode_config0.md"),
     "config3": (1157.7e6, "profiles/paged_attention_q8_d128_verify_config3.md"),
-    "config2": (117.1e6, "profiles/prefill_dense_d128_config2.md"),        # prefill_dense_kernel, averaged over a prompt's four launches
+    "config2": (117.3e6, "profiles/prefill_dense_d128_config2.md"),        # prefill_dense64_kernel, averaged over a prompt's four launches
     "config4": (278.0e6, "profiles/sparse_path_config4.md"),               # index_interval_kernel
 }
 
@@ -406,7 +406,7 @@ def main():
             also["config2"]["traffic"], also["config2"]["traffic_source"] = PROFILED_TRAFFIC["config2"]
             achieved = also["config2"]["kernel_tflops"] or also["config2"]["tflops"]
             also["config2"]["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
-                                           "traffic": PROFILED_TRAFFIC["config2"][0], "kernel": "prefill_dense_kernel<128,2>", "kernel_us": also["config2"]["kernel_us"]}
+                                           "traffic": PROFILED_TRAFFIC["config2"][0], "kernel": "prefill_dense64_kernel<128>", "kernel_us": also["config2"]["kernel_us"]}
             also["config2"]["measured_mfma_tflops"] = measured_mfma_ceiling(gpu, False)
             also["config2"]["measured_mfma_tflops_live_operands"] = measured_mfma_ceiling(gpu, True)
         if args.workload != "config4":
@@ -435,7 +435,7 @@ def main():
     if args.workload == "config2":
         achieved = main_result["kernel_tflops"] or main_result["tflops"]
         roofline = {"bound": "mfma", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
-                    "traffic": PROFILED_TRAFFIC["config2"][0], "traffic_source": PROFILED_TRAFFIC["config2"][1], "kernel": "prefill_dense_kernel<128,2>", "kernel_us": kernel_us,
+                    "traffic": PROFILED_TRAFFIC["config2"][0], "traffic_source": PROFILED_TRAFFIC["config2"][1], "kernel": "prefill_dense64_kernel<128>", "kernel_us": kernel_us,
                     "measured_mfma_tflops": measured_mfma_ceiling(gpu, False),
                     "measured_mfma_tflops_live_operands": measured_mfma_ceiling(gpu, True)}
     line = {
