@@ -158,16 +158,24 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
                 for (int at = valid * ROW + 4 * lane; at < SLAB; at += 256) *reinterpret_cast<uint32_t*>(stage + part * SLAB + at) = 0u;
         load_step<DIM>(rows, stage, stage + SLAB, li, g);
     };
-    // The step's two slabs copied into the stage, 1 KiB per instruction, lanes past a slab's end switched off.
+    // The step's two slabs copied into the stage, 1 KiB per instruction and up to four instructions a run (the slab's address is
+    // the wave's: scalar registers; a lane adds 16 * lane), lanes past a slab's end switched off.
+    const uint32_t lane_bytes = 16 * lane;
     const auto copy_in = [&](uint8_t* stage, int page, int in_page) {
-        const uint8_t* base = args.pages + (size_t(pool_page(page, args.page_last)) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(in_page) * ROW + 16 * lane;
+        const uint8_t* base = args.pages + (size_t(pool_page(page, args.page_last)) * 2 * args.kv_heads + kvh) * plane_bytes + size_t(in_page) * ROW;
+        const uint32_t to = __builtin_amdgcn_readfirstlane(lds_address(stage));
+        constexpr int WHOLE = SLAB / 1024, REST = SLAB % 1024;
         #pragma unroll
         for (int part = 0; part < 2; ++part) {
             const uint8_t* from = base + size_t(part ? args.kv_heads : 0) * plane_bytes;
             #pragma unroll
-            for (int j = 0; j < (SLAB + 1023) / 1024; ++j)
-                if (1024 * j + 1024 <= SLAB || 16 * lane + 1024 * j < SLAB)
-                    load_to_lds<true>(from + 1024 * j, stage + part * SLAB + 1024 * j);
+            for (int j = 0; j < WHOLE; j += 4) {
+                if (WHOLE - j >= 4) load_run_to_lds<true, 4>(from + 1024 * j, to + part * SLAB + 1024 * j, lane_bytes);
+                else if (WHOLE - j == 3) load_run_to_lds<true, 3>(from + 1024 * j, to + part * SLAB + 1024 * j, lane_bytes);
+                else if (WHOLE - j == 2) load_run_to_lds<true, 2>(from + 1024 * j, to + part * SLAB + 1024 * j, lane_bytes);
+                else load_run_to_lds<true, 1>(from + 1024 * j, to + part * SLAB + 1024 * j, lane_bytes);
+            }
+            if (REST && int(lane_bytes) < REST) load_run_to_lds<true, 1>(from + 1024 * WHOLE, to + part * SLAB + 1024 * WHOLE, lane_bytes);
         }
     };
 

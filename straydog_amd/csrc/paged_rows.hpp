@@ -88,6 +88,34 @@ __device__ __forceinline__ void load_to_lds(const void* from, const void* to) {
     if (STREAM) asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt\n\ts_mov_b32 m0, %0" : "=&s"(keep) : "v"(from), "s"(base) : "memory");
     else asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0" : "=&s"(keep) : "v"(from), "s"(base) : "memory");
 }
+// N (1 to 4) consecutive 1 KiB pieces as one run of instructions: `from` is an address the whole wave shares (it travels in scalar
+// registers), a lane adds `lane_offset` (16 * lane, or that plus a constant), the pieces are told apart by the instruction's
+// offset, which moves the global and the LDS address alike; M0 is set once.  No vector instruction forms an address.
+template<bool STREAM, int N>
+__device__ __forceinline__ void load_run_to_lds(const void* from, uint32_t to, uint32_t lane_offset) {
+    static_assert(N >= 1 && N <= 4, "an instruction's offset reaches 4095 bytes");
+    const uint64_t source = uint64_t(uintptr_t(from));
+    uint32_t keep;
+#define SD_RUN_HEAD "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+#define SD_RUN_LOAD(offset, hint) "global_load_lds_dwordx4 %3, %2 offset:" #offset hint "\n\t"
+#define SD_RUN_TAIL "s_mov_b32 m0, %0"
+#define SD_RUN(body) asm volatile(SD_RUN_HEAD body SD_RUN_TAIL : "=&s"(keep) : "s"(to), "s"(source), "v"(lane_offset) : "memory")
+    if (STREAM) {
+        if (N == 1) SD_RUN(SD_RUN_LOAD(0, " nt"));
+        if (N == 2) SD_RUN(SD_RUN_LOAD(0, " nt") SD_RUN_LOAD(1024, " nt"));
+        if (N == 3) SD_RUN(SD_RUN_LOAD(0, " nt") SD_RUN_LOAD(1024, " nt") SD_RUN_LOAD(2048, " nt"));
+        if (N == 4) SD_RUN(SD_RUN_LOAD(0, " nt") SD_RUN_LOAD(1024, " nt") SD_RUN_LOAD(2048, " nt") SD_RUN_LOAD(3072, " nt"));
+    } else {
+        if (N == 1) SD_RUN(SD_RUN_LOAD(0, ""));
+        if (N == 2) SD_RUN(SD_RUN_LOAD(0, "") SD_RUN_LOAD(1024, ""));
+        if (N == 3) SD_RUN(SD_RUN_LOAD(0, "") SD_RUN_LOAD(1024, "") SD_RUN_LOAD(2048, ""));
+        if (N == 4) SD_RUN(SD_RUN_LOAD(0, "") SD_RUN_LOAD(1024, "") SD_RUN_LOAD(2048, "") SD_RUN_LOAD(3072, ""));
+    }
+#undef SD_RUN
+#undef SD_RUN_TAIL
+#undef SD_RUN_LOAD
+#undef SD_RUN_HEAD
+}
 // The loads the compiler knows of (queries and the like) are waited for once, before the first hidden load is issued:
 // its own wait for them would otherwise sit at their first use inside the loop and wait for the hidden loads as well.
 __device__ __forceinline__ void settle_loads() { __builtin_amdgcn_s_waitcnt(0x0f70); }
