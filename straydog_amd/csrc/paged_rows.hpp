@@ -163,8 +163,15 @@ __device__ __forceinline__ void load_step(RowLoad<DIM, true>& r, const uint8_t* 
     #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const int token = e < 4 ? e : 12 + e;       // the lane's tokens are 4g + {0..3, 16..19}
-        #pragma unroll
-        for (int w = 0; w < W / 4; ++w) r.v[e][w] = *reinterpret_cast<const uint32_t*>(vrow + token * ROW + W * li + 4 * w);
+        // (the lane's W bytes of a row lie at a multiple of W: one read, at a 16-bit distance from the lane's first row -- as single
+        // words the reads pair up with 1 KiB of reach and every few rows want an address of their own)
+        if (W == 8) {
+            const uint2 words = *reinterpret_cast<const uint2*>(vrow + token * ROW + W * li);
+            r.v[e][0] = words.x; r.v[e][1] = words.y;
+        } else {
+            const uint4 words = *reinterpret_cast<const uint4*>(vrow + token * ROW + W * li);
+            r.v[e][0] = words.x; r.v[e][1] = words.y; r.v[e][W / 4 - 2] = words.z; r.v[e][W / 4 - 1] = words.w;
+        }
         r.vscale[e] = *reinterpret_cast<const uint16_t*>(vrow + token * ROW + DIM + 2 * ((W * li) / 32));
     }
 }
