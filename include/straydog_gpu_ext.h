@@ -131,8 +131,8 @@ int sdx_paged_attention(void* handle, const sdx_kv_pool* pool, const int32_t* pa
 uint64_t sdx_prefill_tiles_bytes(uint64_t seqs, uint64_t kv_heads, uint64_t dim, uint64_t max_context);
 /* Which of the two prompt kernels takes spans at 128 columns on this handle from now on: waves of 64 query rows, one a SIMD, the
  * queries and output accumulators in the accumulation registers (the default), or waves of 32 rows, two a SIMD.  Same rows a
- * workgroup, same tiles, same grid; the results agree to rounding, not bit for bit (a row's reference maximum is raised when any
- * row of its wave asks for it).  No counterpart in the reference: a tuning switch, kept so that either kernel can be measured
+ * workgroup, same tiles, same grid; only agreement to rounding is promised, though the bits have been the same in every case tried
+ * (the 32 rows that raise their reference maxima together are the same in both).  No counterpart in the reference: a tuning switch, kept so that either kernel can be measured
  * and tested beside the other.  Anything but 32 or 64 is refused. */
 int sdx_prefill_wave_rows(void* handle, uint64_t rows);
 int sdx_prefill_chunk(void* handle, const sdx_kv_pool* pool, const int32_t* page_table, uint64_t table_stride, const int32_t* positions,
