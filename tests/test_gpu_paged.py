@@ -114,9 +114,11 @@ def test_ragged_batched_decode(gpu, oracle, dim, fmt, heads, kv_heads):
         gpu.release(b)
 
 
-@pytest.mark.parametrize("span,heads,kv_heads", [(5, 32, 4), (8, 8, 2), (2, 16, 1), (4, 16, 1)])
+@pytest.mark.parametrize("span,heads,kv_heads", [(5, 32, 4), (8, 8, 2), (2, 16, 1), (4, 16, 1), (8, 32, 4), (7, 32, 4), (13, 8, 2), (5, 24, 2)])
 def test_verify_span_rows(gpu, oracle, span, heads, kv_heads):
-    # BASELINE config 3 in small: span rows attend all of the context and causally inside the span
+    # BASELINE config 3 in small: span rows attend all of the context and causally inside the span.  (Spans of 7 and 8 at eight
+    # heads a group, 13 at four and 5 at twelve are the four-tile variant: 49 to 64 rows a K/V head, the last tile full, short, or
+    # starting in the middle of a token's heads.)
     rng = np.random.default_rng(31 + span)
     dim, row_bytes, page_tokens = 128, 136, 64
     contexts = [0, 27, 64, 300, 1029]
