@@ -203,7 +203,8 @@ __device__ __forceinline__ void load_step(RowLoad<DIM, false>& r, const uint8_t*
 template<int DIM>
 __device__ __forceinline__ half8 key_operand(const RowLoad<DIM, true>& r, int t, int b) {
     const uint32_t pairs = r.kscale[t][b / 2];
-    const half2v scale = as_half2((b & 1) ? byte_perm(pairs, pairs, 0x03020302u) : byte_perm(pairs, pairs, 0x01000100u));
+    const _Float16 one = (b & 1) ? as_half2(pairs).y : as_half2(pairs).x;      // (which half of the word a packed multiply reads is part of the instruction)
+    const half2v scale = {one, one};
     const uint32_t magic = 0x64646464u;
     const uint32_t lo = r.k[t][b].x ^ 0x80808080u, hi = r.k[t][b].y ^ 0x80808080u;
     const half2v a0 = magic_to_half2(byte_perm(magic, lo, 0x04010400u), scale);
