@@ -94,7 +94,11 @@ __device__ __forceinline__ void load_to_lds(const void* from, const void* to) {
 template<bool STREAM, int N>
 __device__ __forceinline__ void load_run_to_lds(const void* from, uint32_t to, uint32_t lane_offset) {
     static_assert(N >= 1 && N <= 4, "an instruction's offset reaches 4095 bytes");
-    const uint64_t source = uint64_t(uintptr_t(from));
+    // (said to be the wave's in a way the compiler sees: where it cannot tell that the address is the same in every lane it would
+    // hand over vector registers)
+    const uint64_t given = uint64_t(uintptr_t(from));
+    const uint64_t source = uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(given))))) |
+                            uint64_t(uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(given >> 32))))) << 32;
     uint32_t keep;
 #define SD_RUN_HEAD "s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
 #define SD_RUN_LOAD(offset, hint) "global_load_lds_dwordx4 %3, %2 offset:" #offset hint "\n\t"
