@@ -202,6 +202,45 @@ def test_prompt_chunk_stage_recorded(gpu, oracle):
         assert np.abs(_read(gpu, recorded["attended"], np.float32, steps * heads * 256)).max() > 0
 
 
+def test_prompt_chunk_call_recorded(gpu, oracle):
+    # sdx_prefill_chunk -- a chunk's K/V append, its tiles and its attention -- recorded once and replayed chunk after chunk of a
+    # prompt as the device-resident positions advance: every replay's cache bytes and outputs against the oracle
+    rng = np.random.default_rng(12)
+    seqs, heads, kv_heads, dim, page_tokens, row_bytes, span, chunks = 2, 16, 2, 128, 64, 136, 96, 4
+    begins = [0, 40]                        # the second sequence's prompt starts behind 40 cached tokens
+    capacity = [b + chunks * span for b in begins]
+    pool, buffer, host, table, table_buffer = make_pool(gpu, oracle, rng, capacity, kv_heads, dim, page_tokens, row_bytes)
+    max_context = max(capacity)
+    positions = gpu.upload(np.array(begins, dtype=np.int32))
+    kb, vb = gpu.buffer(seqs * span * kv_heads * dim * 2), gpu.buffer(seqs * span * kv_heads * dim * 2)
+    qb, out = gpu.buffer(seqs * span * heads * dim * 2), gpu.buffer(seqs * span * heads * dim * 4)
+    tiles = gpu.buffer(gpu.prefill_tiles_bytes(seqs, kv_heads, dim, max_context))
+    valid = gpu.upload(np.zeros(seqs, dtype=np.int32))      # what the tiles hold: nothing before the first chunk, then the positions
+
+    def call():
+        gpu.prefill_chunk(pool, table_buffer.base(), table.shape[1], positions.base(), max_context, kb.base(), vb.base(), True, qb.base(), True,
+                          seqs, span, heads, 0.088, out.base(), False, tiles, valid.base())
+    gpu.graph_begin()
+    call()
+    gpu.graph_end(11)
+    for turn in range(chunks):
+        at = np.array([b + turn * span for b in begins], dtype=np.int32)
+        k = rng.standard_normal((seqs, span, kv_heads, dim)).astype(np.float16)
+        v = rng.standard_normal((seqs, span, kv_heads, dim)).astype(np.float16)
+        q = rng.standard_normal((seqs, span, heads, dim)).astype(np.float16)
+        for b, a in ((positions, at), (kb, k), (vb, v), (qb, q)):
+            gpu.write_buffer(b, 0, a)
+        gpu.write_buffer(valid, 0, at if turn else np.zeros(seqs, dtype=np.int32))
+        assert gpu.graph_run(11)
+        got = _read(gpu, out, np.float32, q.size).reshape(q.shape)
+        oracle.kv_write(host, row_bytes, page_tokens, kv_heads, dim, table, at, k.astype(np.float32), v.astype(np.float32))
+        want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, at, q.astype(np.float32), 0.088)
+        close_enough(got, want, f"replay {turn}")
+        assert np.array_equal(_read(gpu, buffer, np.uint8, host.size), host), "the appended rows"
+    for b in (buffer, table_buffer, positions, kb, vb, qb, out, tiles, valid):
+        gpu.release(b)
+
+
 def test_graphs_are_dropped_when_the_workspace_moves(gpu, oracle):
     # ops that use the handle's workspace bake its address into a recorded graph; when a later, larger call makes the workspace
     # grow (and move), the kept graphs are dropped: sd_graph_run answers "none stored" and the caller records again, instead of
