@@ -131,12 +131,37 @@ __device__ __forceinline__ half2v as_half2(uint32_t bits) { return __builtin_bit
 // v_perm_b32: byte i of the result is byte sel[i] of the 8 bytes {high, low} (0-3 = low's bytes, 4-7 = high's, 0x0c = 0x00).
 __device__ __forceinline__ uint32_t byte_perm(uint32_t high, uint32_t low, uint32_t sel) { return __builtin_amdgcn_perm(high, low, sel); }
 
-// Two bytes u (an int8 xor 0x80) sitting in FP16 patterns 0x64uu: 0x6400 | u is the FP16 1024 + u exactly; minus 1152 leaves the
-// signed byte; one rounding by the block scale (the reference's qsa_q8_half16, gpu/qsa_prompt_attention.hpp:15-33).
-__device__ __forceinline__ half2v magic_to_half2(uint32_t pattern, half2v scale) {
-    const half2v bias = {(_Float16)1152.0f, (_Float16)1152.0f};
-    return (as_half2(pattern) - bias) * scale;
+// Int8 bytes as the FP16 integers they are, then one rounding by the block scale (the reference's qsa_q8_half16,
+// gpu/qsa_prompt_attention.hpp:15-33).  A byte is converted where it lies: v_cvt_f16_i16 with a byte of the source word
+// sign-extended as its operand and one half of the result register as its destination (the other half kept) -- an
+// instruction an element and no byte shuffling, against 1.25 an element for the bytes placed into 0x64uu patterns (v_perm, xor)
+// and the patterns' bias subtracted.  Written as one run per operand: a register's two halves are written four instructions
+// apart and a wait state follows the run, because a result written to half a register may not be read by the next vector
+// instruction (the compiler keeps that distance for its own instructions, not for these).
+#define SD_BYTE_LOW(to, from, byte) "v_cvt_f16_i16_sdwa " to ", sext(" from ") dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_" #byte "\n\t"
+#define SD_BYTE_HIGH(to, from, byte) "v_cvt_f16_i16_sdwa " to ", sext(" from ") dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_" #byte "\n\t"
+// the eight bytes of two words, in order
+__device__ __forceinline__ void bytes_in_a_row(uint32_t low, uint32_t high, uint32_t (&pairs)[4]) {
+    asm(SD_BYTE_LOW("%0", "%4", 0) SD_BYTE_LOW("%1", "%4", 2) SD_BYTE_LOW("%2", "%5", 0) SD_BYTE_LOW("%3", "%5", 2)
+        SD_BYTE_HIGH("%0", "%4", 1) SD_BYTE_HIGH("%1", "%4", 3) SD_BYTE_HIGH("%2", "%5", 1) SD_BYTE_HIGH("%3", "%5", 3) "s_nop 0"
+        : "=&v"(pairs[0]), "=&v"(pairs[1]), "=&v"(pairs[2]), "=&v"(pairs[3]) : "v"(low), "v"(high));
 }
+// byte BYTE of eight words, in order
+template<int BYTE>
+__device__ __forceinline__ void bytes_in_a_column(const uint32_t (&words)[8], uint32_t (&pairs)[4]) {
+#define SD_COLUMN(byte) \
+    asm(SD_BYTE_LOW("%0", "%4", byte) SD_BYTE_LOW("%1", "%6", byte) SD_BYTE_LOW("%2", "%8", byte) SD_BYTE_LOW("%3", "%10", byte) \
+        SD_BYTE_HIGH("%0", "%5", byte) SD_BYTE_HIGH("%1", "%7", byte) SD_BYTE_HIGH("%2", "%9", byte) SD_BYTE_HIGH("%3", "%11", byte) "s_nop 0" \
+        : "=&v"(pairs[0]), "=&v"(pairs[1]), "=&v"(pairs[2]), "=&v"(pairs[3]) \
+        : "v"(words[0]), "v"(words[1]), "v"(words[2]), "v"(words[3]), "v"(words[4]), "v"(words[5]), "v"(words[6]), "v"(words[7]))
+    if (BYTE == 0) SD_COLUMN(0);
+    if (BYTE == 1) SD_COLUMN(1);
+    if (BYTE == 2) SD_COLUMN(2);
+    if (BYTE == 3) SD_COLUMN(3);
+#undef SD_COLUMN
+}
+#undef SD_BYTE_HIGH
+#undef SD_BYTE_LOW
 
 template<int DIM, bool Q8> struct RowLoad;
 
@@ -206,15 +231,12 @@ __device__ __forceinline__ void load_step(RowLoad<DIM, false>& r, const uint8_t*
 // The A operand of S^T = K . Q^T for tile t, block b.
 template<int DIM>
 __device__ __forceinline__ half8 key_operand(const RowLoad<DIM, true>& r, int t, int b) {
-    const uint32_t pairs = r.kscale[t][b / 2];
-    const _Float16 one = (b & 1) ? as_half2(pairs).y : as_half2(pairs).x;      // (which half of the word a packed multiply reads is part of the instruction)
+    const uint32_t scales = r.kscale[t][b / 2];
+    const _Float16 one = (b & 1) ? as_half2(scales).y : as_half2(scales).x;      // (which half of the word a packed multiply reads is part of the instruction)
     const half2v scale = {one, one};
-    const uint32_t magic = 0x64646464u;
-    const uint32_t lo = r.k[t][b].x ^ 0x80808080u, hi = r.k[t][b].y ^ 0x80808080u;
-    const half2v a0 = magic_to_half2(byte_perm(magic, lo, 0x04010400u), scale);
-    const half2v a1 = magic_to_half2(byte_perm(magic, lo, 0x04030402u), scale);
-    const half2v a2 = magic_to_half2(byte_perm(magic, hi, 0x04010400u), scale);
-    const half2v a3 = magic_to_half2(byte_perm(magic, hi, 0x04030402u), scale);
+    uint32_t pairs[4];
+    bytes_in_a_row(r.k[t][b].x, r.k[t][b].y, pairs);
+    const half2v a0 = as_half2(pairs[0]) * scale, a1 = as_half2(pairs[1]) * scale, a2 = as_half2(pairs[2]) * scale, a3 = as_half2(pairs[3]) * scale;
     return half8{a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
 }
 template<int DIM>
@@ -233,13 +255,18 @@ __device__ __forceinline__ void value_scales(const RowLoad<DIM, false>&, ValueSc
 // The A operand of O^T += V^T . P^T for output tile jj: column W*li + jj of the lane's 8 tokens.
 template<int DIM>
 __device__ __forceinline__ half8 value_operand(const RowLoad<DIM, true>& r, const ValueScales<DIM>& s, int jj) {
-    half2v out[4];
     const int word = jj / 4;
-    // bytes (jj % 4) of tokens e (low half) and e + 1 (high half), zero bytes between; the xor turns them into 0x64uu patterns
-    const uint32_t sel = 0x0c000c00u | uint32_t(jj % 4) | (uint32_t(4 + jj % 4) << 16);
+    const uint32_t words[8] = {r.v[0][word], r.v[1][word], r.v[2][word], r.v[3][word], r.v[4][word], r.v[5][word], r.v[6][word], r.v[7][word]};
+    uint32_t pairs[4];
+    switch (jj % 4) {
+        case 0: bytes_in_a_column<0>(words, pairs); break;
+        case 1: bytes_in_a_column<1>(words, pairs); break;
+        case 2: bytes_in_a_column<2>(words, pairs); break;
+        default: bytes_in_a_column<3>(words, pairs); break;
+    }
+    half2v out[4];
     #pragma unroll
-    for (int e = 0; e < 8; e += 2)
-        out[e / 2] = magic_to_half2(byte_perm(r.v[e + 1][word], r.v[e][word], sel) ^ 0x64806480u, s.pair[e / 2]);
+    for (int e = 0; e < 4; ++e) out[e] = as_half2(pairs[e]) * s.pair[e];
     return half8{out[0].x, out[0].y, out[1].x, out[1].y, out[2].x, out[2].y, out[3].x, out[3].y};
 }
 template<int DIM>
