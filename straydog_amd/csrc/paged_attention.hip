@@ -134,11 +134,16 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
     const table_ptr table = (table_ptr)(args.page_table + size_t(seq) * args.table_stride);
     const size_t plane_bytes = size_t(args.page_tokens) * ROW;
 
-    floatx4 acc[QT][TILES];
+    // With several query tiles the kernel is bound by its vector instructions and the matrix cores have time to spare: a row's sum
+    // of weights is then one more product a tile and step -- the weights against a block of ones, every row of the result the sum,
+    // every one of a row's four lanes holding all of it -- instead of eight additions a tile.
+    constexpr bool SUMS_BY_PRODUCT = QT >= 2 && DIM == 128;      // (at 256 columns the registers are all taken)
+    floatx4 acc[QT][TILES], sums[SUMS_BY_PRODUCT ? QT : 1];
     float m[QT], l[QT];
     #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
         m[qt] = NEG_BIG; l[qt] = 0.0f;
+        if (SUMS_BY_PRODUCT) sums[qt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
         #pragma unroll
         for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
@@ -283,6 +288,7 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
                 const float alpha = __builtin_amdgcn_exp2f((m[qt] - m_new) * args.scale_log2);
                 m[qt] = m_new;
                 l[qt] *= alpha;
+                if (SUMS_BY_PRODUCT) sums[qt] *= alpha;
                 #pragma unroll
                 for (int jj = 0; jj < TILES; ++jj) acc[qt][jj] *= alpha;
             }
@@ -298,11 +304,14 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
                 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const float w = __builtin_amdgcn_exp2f(fmaf(s[qt][t][r], args.scale_log2, offset));
-                    sum += w;
+                    if (!SUMS_BY_PRODUCT) sum += w;
                     p[4 * t + r] = (_Float16)w;
                 }
             pb[qt] = p;
-            l[qt] += sum;
+            if (SUMS_BY_PRODUCT) {
+                const _Float16 one = (_Float16)1.0f;
+                sums[qt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(half8{one, one, one, one, one, one, one, one}, p, sums[qt], 0, 0, 0);
+            } else l[qt] += sum;
         }
         // O^T tiles: columns (rows of the tile, W*row + jj) x query rows
         ValueScales<DIM> vs;
@@ -318,6 +327,9 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
     // Merge the waves, two by two, through LDS: waves 2 and 3 hand their maxima, sums and unnormalised outputs to waves 0 and
     // 1, then wave 1 hands its own to wave 0.  Corresponding lanes hold corresponding elements, so a value goes from lane to
     // lane ([register][lane] in LDS, no bank conflicts), and the area is two waves' registers: it fits the stages it overlays.
+    if (SUMS_BY_PRODUCT)
+        #pragma unroll
+        for (int qt = 0; qt < QT; ++qt) l[qt] = sums[qt][0];
     __syncthreads();    // the stages are free
     constexpr int STRIDE = DIM + 2, HELD = QT * (TILES * 4 + 2);
     const int lane_after = fresh_lane(), li_after = lane_after & 15, g_after = lane_after >> 4;   // (again: nothing of this is worked out before the loop)
@@ -361,7 +373,7 @@ __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu
         float* out = args.partial + (size_t(blockIdx.x) + size_t(seq) * args.kv_heads + kvh) * args.rows * STRIDE;
         #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
-            const float sum = row_sum(l[qt]);
+            const float sum = SUMS_BY_PRODUCT ? l[qt] : row_sum(l[qt]);       // (a sum formed by products is whole in each of the row's lanes)
             const int row = qt * 16 + li_after;
             if (row < int(args.rows)) {
                 float* to = out + size_t(row) * STRIDE;

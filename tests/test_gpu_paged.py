@@ -135,7 +135,9 @@ def test_verify_span_rows(gpu, oracle, span, heads, kv_heads):
         single = _run(gpu, pool, table, tb, [c + r for c in contexts], q[:, r:r + 1], 1, heads, scale, True, False,
                       max_context=max(lengths))
         close_enough(single[:, 0], want[:, r], f"row {r} alone")
-        assert np.abs(single[:, 0] - got[:, r]).max() < 2e-4
+        # (not the same bits: with several query tiles a row's sum is the sum of its weights as rounded to FP16, the ones the
+        # values are multiplied by, formed by a product; the decode variant adds the weights before they are rounded)
+        assert np.abs(single[:, 0] - got[:, r]).max() < 5e-4
     gpu.release(buffer); gpu.release(tb)
 
 
