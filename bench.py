@@ -30,9 +30,9 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense FP16/BF16 MFMA, published
 # counters read for the library's 1 GiB copy kernel), kept here so that the bench line carries them; `traffic_source` names the
 # summary.  A counter run cannot share a process with the timed passes.
 PROFILED_TRAFFIC = {
-    "config1": (626.9e6, "profiles/paged_attention_q8_d128_decode_config1.md"),
-    "config1_32k": (1147.5e6, "profiles/paged_attention_q8_d128_decode_config1_32k.md"),
-    "config0": (2.61e6, "profiles/paged_attention_q8_d128_decode_config0.md"),
+    "config1": (626.8e6, "profiles/paged_attention_q8_d128_decode_config1.md"),
+    "config1_32k": (1147.4e6, "profiles/paged_attention_q8_d128_decode_config1_32k.md"),
+    "config0": (2.60e6, "profiles/paged_attention_q8_d128_decode_config0.md"),
     "config3": (1157.6e6, "profiles/paged_attention_q8_d128_verify_config3.md"),
     "config2": (117.3e6, "profiles/prefill_dense_d128_config2.md"),        # prefill_dense64_kernel, averaged over a prompt's four launches
     "config4": (278.0e6, "profiles/sparse_path_config4.md"),               # index_interval_kernel
