@@ -799,10 +799,29 @@ __global__ void __launch_bounds__(GROUPS * 64) __attribute__((amdgpu_waves_per_e
     static_assert(TILE % (1024 * GROUPS) == 0 && RING * TILE <= 160 * 1024 - 1024 && TILE_KEYS == 2 * SUB && BLOCKS == 4 && TILES == 8, "a tile is two steps of a wave");
     const int kvh = blockIdx.y, seq = blockIdx.z;
     const int thread = threadIdx.x, lane = thread & 63, wave = __builtin_amdgcn_readfirstlane(thread >> 6), li = lane & 15, g = lane >> 4;
-    const int position = first_position(args.positions, unsigned(seq), args.max_context);
-    const int cached = min(position + int(args.span), args.max_context);
     const int runs = (int(args.rows) + GROUP_ROWS - 1) / GROUP_ROWS;
     const int late = runs - 1 - int(blockIdx.x), early = int(blockIdx.x);
+    // The queries are asked for first: where they lie does not depend on the sequence's position, whose own trip from memory
+    // everything else waits for.  (Tiles 0 and 1 are the late run's, 2 and 3 the early run's; a row past the last stands for the last.)
+    half8 raw16[QT][BLOCKS];
+    float raw32[QT][BLOCKS][8];
+    #pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int row = min(((qt / 2 == 0 ? late : early) * GROUP_ROWS + wave * PAIR_ROWS) + (qt % 2) * 16 + li, int(args.rows) - 1);
+        const int span_row = row / int(args.group), head = kvh * int(args.group) + row % int(args.group);
+        const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
+        #pragma unroll
+        for (int b = 0; b < BLOCKS; ++b) {
+            if (args.q_f16) raw16[qt][b] = *reinterpret_cast<const half8*>(static_cast<const _Float16*>(args.q) + at + 32 * b + 8 * g);
+            else {
+                const float* from = static_cast<const float*>(args.q) + at + 32 * b + 8 * g;
+                #pragma unroll
+                for (int i = 0; i < 8; ++i) raw32[qt][b][i] = from[i];
+            }
+        }
+    }
+    const int position = first_position(args.positions, unsigned(seq), args.max_context);
+    const int cached = min(position + int(args.span), args.max_context);
     const int group_last = min(int(args.rows), (late + 1) * GROUP_ROWS) - 1;
     const int keys = min(position + group_last / int(args.group) + 1, cached);
     // the wave's two pairs of tiles: pair 0 of the late run, pair 1 of the early one
@@ -815,7 +834,8 @@ __global__ void __launch_bounds__(GROUPS * 64) __attribute__((amdgpu_waves_per_e
         const int wave_last = min(position + (min(int(args.rows), row0[p] + PAIR_ROWS) - 1) / int(args.group), keys - 1);
         steps[p] = idle ? 0 : wave_last / SUB + 1;
     }
-    if (steps[0] < steps[1]) {      // (the late run's quarter may lie past the span's last row: the longer walk is pair 0's)
+    const bool swapped = steps[0] < steps[1];
+    if (swapped) {      // (the late run's quarter may lie past the span's last row: the longer walk is pair 0's)
         const int r = row0[0], f = wave_first[0], n = steps[0];
         row0[0] = row0[1]; wave_first[0] = wave_first[1]; steps[0] = steps[1];
         row0[1] = r; wave_first[1] = f; steps[1] = n;
@@ -849,21 +869,18 @@ __global__ void __launch_bounds__(GROUPS * 64) __attribute__((amdgpu_waves_per_e
     for (int qt = 0; qt < QT; ++qt) {
         const int row = row0[qt / 2] + (qt % 2) * 16 + li;
         const bool real = row < int(args.rows) && steps[qt / 2] > 0;
-        const int span_row = real ? row / int(args.group) : 0, head = kvh * int(args.group) + (real ? row % int(args.group) : 0);
-        limit[qt] = real ? position + span_row : 0x7fffffff;                      // a padding row masks nothing
-        const size_t at = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM;
+        limit[qt] = real ? position + row / int(args.group) : 0x7fffffff;         // a padding row masks nothing
         #pragma unroll
         for (int b = 0; b < BLOCKS; ++b) {
             half8 value = {};
             if (real) {
                 if (args.q_f16) {
-                    const half8 raw = *reinterpret_cast<const half8*>(static_cast<const _Float16*>(args.q) + at + 32 * b + 8 * g);
+                    const half8 raw = swapped ? raw16[qt ^ 2][b] : raw16[qt][b];
                     #pragma unroll
                     for (int i = 0; i < 8; ++i) value[i] = (_Float16)(float(raw[i]) * args.scale_log2);
                 } else {
-                    const float* from = static_cast<const float*>(args.q) + at + 32 * b + 8 * g;
                     #pragma unroll
-                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)(from[i] * args.scale_log2);
+                    for (int i = 0; i < 8; ++i) value[i] = (_Float16)((swapped ? raw32[qt ^ 2][b][i] : raw32[qt][b][i]) * args.scale_log2);
                 }
             }
             // (the queries are only ever a product's B operand: they live in the accumulation registers, where a product reads them
