@@ -1043,28 +1043,39 @@ __global__ void __launch_bounds__(GROUPS * 64) __attribute__((amdgpu_waves_per_e
         advance(std::true_type{}, std::false_type{}, std::false_type{}, 0, 2 * tile + 1, odd, even);
         advance(std::false_type{}, std::true_type{}, std::false_type{}, 1, 2 * tile + 1, odd, even);
     }
+    // A pair's rows normalised and written.  The shorter pair's leave as soon as it is done, while the longer one walks on: the
+    // launch's outputs then do not all reach memory at once as every workgroup ends.
+    const auto deliver = [&](int p) {
+        #pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int qt = 2 * p + q, row = row0[p] + q * 16 + li;
+            const float inverse = 1.0f / row_sum(l[qt]);
+            if (steps[p] == 0 || row >= int(args.rows)) continue;
+            const int span_row = row / int(args.group), head = kvh * int(args.group) + row % int(args.group);
+            const size_t first = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM + 4 * g;
+            #pragma unroll
+            for (int jj = 0; jj < TILES; ++jj) {
+                const floatx4 value = acc[qt][jj] * inverse;
+                if (args.out_f16) {
+                    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+                    *reinterpret_cast<half4*>(static_cast<_Float16*>(args.out) + first + 16 * jj) = half4{(_Float16)value[0], (_Float16)value[1], (_Float16)value[2], (_Float16)value[3]};
+                } else *reinterpret_cast<floatx4*>(static_cast<float*>(args.out) + first + 16 * jj) = value;
+            }
+        }
+    };
+    const bool early_leaves = tile <= last_tile;        // (the longer pair has tiles of its own left)
+    if (early_leaves) {
+        products_done();
+        deliver(1);
+    }
     for (; tile <= last_tile; ++tile) {
         advance(std::true_type{}, std::true_type{}, std::true_type{}, 0, 2 * tile, even, odd);
         advance(std::true_type{}, std::true_type{}, std::false_type{}, 0, 2 * tile + 1, odd, even);
     }
 
     products_done();
-    #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-        const int row = row0[qt / 2] + (qt % 2) * 16 + li;
-        const float inverse = 1.0f / row_sum(l[qt]);
-        if (steps[qt / 2] == 0 || row >= int(args.rows)) continue;
-        const int span_row = row / int(args.group), head = kvh * int(args.group) + row % int(args.group);
-        const size_t first = ((size_t(seq) * args.span + span_row) * args.heads + head) * DIM + 4 * g;
-        #pragma unroll
-        for (int jj = 0; jj < TILES; ++jj) {
-            const floatx4 value = acc[qt][jj] * inverse;
-            if (args.out_f16) {
-                typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-                *reinterpret_cast<half4*>(static_cast<_Float16*>(args.out) + first + 16 * jj) = half4{(_Float16)value[0], (_Float16)value[1], (_Float16)value[2], (_Float16)value[3]};
-            } else *reinterpret_cast<floatx4*>(static_cast<float*>(args.out) + first + 16 * jj) = value;
-        }
-    }
+    deliver(0);
+    if (!early_leaves) deliver(1);
 }
 
 // `tiles`: where the cached rows' FP16 tiles go -- the device's workspace, rebuilt whole on every call, or a buffer the caller
