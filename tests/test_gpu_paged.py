@@ -141,6 +141,27 @@ def test_verify_span_rows(gpu, oracle, span, heads, kv_heads):
     gpu.release(buffer); gpu.release(tb)
 
 
+@pytest.mark.parametrize("dim,fmt,span,heads,kv_heads", [(128, "f16", 3, 16, 2), (128, "f16", 5, 32, 4), (128, "f16", 8, 32, 4),
+                                                         (256, "q8", 2, 24, 2), (256, "f16", 2, 24, 2)])
+def test_verify_span_rows_of_other_formats(gpu, oracle, dim, fmt, span, heads, kv_heads):
+    # The few-rows kernel's variants of two, three and four query tiles over FP16 rows, and of two tiles over 256 columns: the
+    # same walk as over Q8_0 rows of 128 columns with other row loads (and, at 128 columns, the rows' sums formed by a product).
+    rng = np.random.default_rng(900 + dim + span)
+    row_bytes = (dim + dim // 16) if fmt == "q8" else 2 * dim
+    page_tokens = 64
+    contexts = [0, 31, 64, 290, 1100]
+    lengths = [c + span for c in contexts]
+    pool, buffer, host, table, tb = make_pool(gpu, oracle, rng, lengths, kv_heads, dim, page_tokens, row_bytes,
+                                              dtype=np.float32 if fmt == "q8" else np.float16)
+    q = rng.standard_normal((len(lengths), span, heads, dim)).astype(np.float16).astype(np.float32)
+    scale = 1.0 / np.sqrt(dim)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array(contexts, np.int32), q, scale)
+    for q_f16, out_f16 in ((True, False), (False, True)):
+        got = _run(gpu, pool, table, tb, contexts, q, span, heads, scale, q_f16, out_f16)
+        close_enough(got, want, f"span {span} of {fmt} rows, {dim} columns")
+    gpu.release(buffer); gpu.release(tb)
+
+
 @pytest.mark.parametrize("dim,fmt,span,heads,kv_heads", [(128, "q8", 40, 32, 4), (128, "q8", 100, 8, 1), (128, "f16", 33, 16, 2),
                                                          (256, "q8", 24, 24, 2), (256, "f16", 9, 24, 2), (128, "q8", 9, 4, 4)])
 @pytest.mark.parametrize("page_tokens", [64, 32])
