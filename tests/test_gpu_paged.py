@@ -229,6 +229,38 @@ def test_prefill_with_scores_that_keep_growing(gpu, oracle, fmt):
     gpu.release(buffer); gpu.release(tb)
 
 
+@pytest.mark.parametrize("fmt,span", [("q8", 5), ("q8", 8), ("f16", 3), ("f16", 8)])
+def test_verify_span_with_scores_that_keep_growing(gpu, oracle, fmt, span):
+    # The same rising keys under the few-rows kernel at two, three and four query tiles: a row's reference moves many times along
+    # the walk, and what was summed by then -- the outputs and, with several tiles, the sums of weights a product forms -- is scaled
+    # each time.  (A workgroup's share is 256 tokens here, along which a score rises by up to 16 in the exponent: a wave moves its
+    # references once or twice after the first step.)
+    rng = np.random.default_rng(191 + span)
+    dim, page_tokens, heads, kv_heads, context = 128, 64, 16, 2, 600
+    row_bytes = (dim + dim // 16) if fmt == "q8" else 2 * dim
+    total = span + context
+    pages = (total + page_tokens - 1) // page_tokens
+    table = rng.permutation(pages + 1)[:pages].astype(np.int32).reshape(1, pages)
+    host = np.zeros(oracle.pool_bytes(pages + 1, kv_heads, page_tokens, row_bytes), dtype=np.uint8)
+    u = rng.standard_normal(dim).astype(np.float32)
+    u /= np.linalg.norm(u)
+    rise = (np.arange(total, dtype=np.float32) / 8.0)[None, :, None, None] * u[None, None, None, :]
+    k = (rise + 0.3 * rng.standard_normal((1, total, kv_heads, dim))).astype(np.float16).astype(np.float32)
+    v = rng.standard_normal((1, total, kv_heads, dim)).astype(np.float16).astype(np.float32)
+    oracle.kv_write(host, row_bytes, page_tokens, kv_heads, dim, table, np.zeros(1, np.int32), k, v)
+    pool, buffer = gpu.kv_pool(pages + 1, page_tokens, kv_heads, dim, row_bytes)
+    gpu.write_buffer(buffer, 0, host)
+    tb = gpu.upload(table)
+    strength = rng.choice([0.5, 4.0, 30.0] if fmt == "f16" else [0.5, 2.0, 4.0], size=(1, span, heads, 1)).astype(np.float32)
+    q = (strength * u[None, None, None, :] + 0.2 * rng.standard_normal((1, span, heads, dim))).astype(np.float16).astype(np.float32)
+    q[:, :, 3] = 0.0
+    scale = 1.0 / np.sqrt(dim)
+    want = oracle.paged_attention(host, row_bytes, page_tokens, kv_heads, dim, table, np.array([context], np.int32), q, scale)
+    got = _run(gpu, pool, table, tb, [context], q, span, heads, scale, True, False)
+    close_enough(got, want, f"growing scores, span {span}, {fmt}")
+    gpu.release(buffer); gpu.release(tb)
+
+
 def test_prefill_in_chunks_equals_prefill_at_once(gpu, oracle):
     # a prompt prefilled in 4 chunks (each chunk attends the cache so far) gives the rows of one whole-prompt pass
     rng = np.random.default_rng(5)
